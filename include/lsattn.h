@@ -1,0 +1,192 @@
+/*
+ * lsattn.h -- C ABI of the MI355X (gfx950) attention hot path.
+ *
+ * Plain C: device pointers, sizes and element strides only; no torch, no HIP types
+ * (a hipStream_t is passed as `void*`; NULL means the default stream).  Every entry point
+ *   - launches asynchronously on the given stream and returns without a host sync,
+ *   - allocates nothing and keeps no pointer after it returns (the caller owns every
+ *     buffer, scratch included),
+ *   - returns LSATTN_OK or a negative LSATTN_ERR_* code and never aborts or throws.
+ *
+ * Citations name the reference interface each entry point replaces, relative to the
+ * reference tree:
+ *   RING  = loongserve/models/llama/triton_kernel/ring_context_flashattention_nopad.py
+ *   S1CU/S1H = longserve_cuda_kernels/src/flash_decoding_stage1.{cu,h}
+ *   S2CU/S2H = longserve_cuda_kernels/src/flash_decoding_stage2.{cu,h}
+ *   ENTRY = longserve_cuda_kernels/src/entrypoints.cpp
+ */
+#ifndef LSATTN_H
+#define LSATTN_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define LSATTN_OK 0
+#define LSATTN_ERR_INVALID_ARG (-1) /* null pointer, negative size, bad stride            */
+#define LSATTN_ERR_UNSUPPORTED (-2) /* head_dim / dtype / head ratio the kernels lack     */
+#define LSATTN_ERR_LAUNCH (-3)      /* hipGetLastError() after the launch was not success */
+
+/* element types of q/k/v and of `o` outputs */
+#define LSATTN_F16 0
+#define LSATTN_BF16 1
+#define LSATTN_F32 2
+
+#define LSATTN_MAX_PARTS 16
+
+/*
+ * One ring / context-parallel prefill attention step: local Q chunk against one KV chunk.
+ * Replaces context_attention_fwd + _fwd_kernel (RING:13-188, :190-284).
+ *
+ * q [Tq,Hq,D], k/v [Tkv,Hkv,D] with the last dimension contiguous and the token / head
+ * strides given in elements (k and v are usually the two halves of one interleaved
+ * [Tkv,2*Hkv,D] buffer).  The six int32 device vectors of length `batch` carry, per
+ * sequence, the start row, the number of local rows and the global index of the first
+ * local row for q and for the kv chunk; local row m of q has global position
+ * q_first + m*sp_peers, key n has kv_first + n*sp_peers, and key n is visible to row m
+ * iff kv position <= q position and n < kv_len (RING:156-159).  sp_peers = 1 with shard
+ * offsets in the *_first vectors expresses contiguous sharding.
+ */
+typedef struct lsattn_prefill_args {
+  const void* q;
+  const void* k;
+  const void* v;
+  int64_t q_stride_t, q_stride_h;
+  int64_t k_stride_t, k_stride_h;
+  int64_t v_stride_t, v_stride_h;
+  const int32_t* q_b_start_loc;
+  const int32_t* q_b_seq_len;
+  const int32_t* q_first_token_global_idx;
+  const int32_t* kv_b_start_loc;
+  const int32_t* kv_b_seq_len;
+  const int32_t* kv_first_token_global_idx;
+  int32_t batch;
+  int32_t num_q_heads;
+  int32_t num_kv_heads;
+  int32_t head_dim;   /* 128 */
+  int32_t dtype;      /* LSATTN_F16 or LSATTN_BF16 (q, k, v) */
+  int32_t sp_peers;   /* logical_sp_peers_num, >= 1 */
+  int32_t max_q_len;  /* max over q_b_seq_len (sizes the launch, RING:262) */
+  float sm_scale;     /* natural-domain softmax scale, 1/sqrt(D) in the reference (RING:252) */
+  /* outputs */
+  void* o;            /* [Tq,Hq,D] */
+  int64_t o_stride_t, o_stride_h;
+  int32_t o_dtype;    /* step: LSATTN_F32; step_merge: same as dtype */
+  int32_t reserved;
+  float* lse;         /* step: [Tq,Hq] natural-log LSE, contiguous         */
+  float* m;           /* step_merge: [Tq,Hq] running max, log2 domain       */
+  float* l;           /* step_merge: [Tq,Hq] running sum                    */
+  int64_t ml_stride_t, ml_stride_h; /* strides of m and l (RING:274-275)     */
+} lsattn_prefill_args;
+
+/* Partial of one step from the empty state: o = normalised fp32 output, lse = natural-log
+ * log-sum-exp; rows that see no key get o = 0, lse = -inf.  Uses o (F32), lse. */
+int lsattn_prefill_step(const lsattn_prefill_args* a, void* stream);
+
+/* Drop-in for context_attention_fwd (RING:191-206): folds this step into the running
+ * (o, m, l) state in place with the update of RING:171-188.  Start state is m = -inf,
+ * l = 0; after any number of calls ln2*(m + log2 l) is the natural LSE over all keys
+ * seen and o is the normalised output in o_dtype.  Uses o (dtype of q), m, l. */
+int lsattn_prefill_step_merge(const lsattn_prefill_args* a, void* stream);
+
+/*
+ * Merge n normalised partials (O_i fp32 [rows,D] contiguous, LSE_i [rows]) over disjoint key
+ * sets: LSE = log sum_i exp(LSE_i), O = sum_i exp(LSE_i-LSE) O_i.  Same recurrence as
+ * S2CU:38-48 applied to separately allocated partials (the ring steps of one query chunk).
+ */
+typedef struct lsattn_merge_args {
+  int32_t n_parts; /* 1..LSATTN_MAX_PARTS */
+  int32_t head_dim;
+  int64_t rows;    /* tokens * heads */
+  const float* o_parts[LSATTN_MAX_PARTS];
+  const float* lse_parts[LSATTN_MAX_PARTS];
+  void* o;         /* [rows,D] contiguous */
+  int32_t o_dtype; /* LSATTN_F32 / F16 / BF16 */
+  int32_t reserved;
+  float* lse;      /* [rows] */
+} lsattn_merge_args;
+int lsattn_lse_merge(const lsattn_merge_args* a, void* stream);
+
+/*
+ * Flash-decoding stage 1 over a token-indexed KV pool.  Replaces
+ * LongServe::flash_decoding_stage1 (S1H:7-27, S1CU:187-215) behind ENTRY:103-164.
+ * For request b and block blk with blk*block_seq < b_seqlen[b]:
+ *   mid_o[blk,b,h,:], mid_o_logexpsum[blk,b,h] = normalised partial and natural LSE of
+ *   q[b,h] against pool rows req_to_tokens[b_req_idx[b], blk*BS : min((blk+1)*BS, len)].
+ * Other blocks are left untouched.  Partials are written once, without atomics.
+ */
+typedef struct lsattn_decode_stage1_args {
+  float* mid_o;            /* [num_blocks, batch, Hq, D] contiguous */
+  float* mid_o_logexpsum;  /* [num_blocks, batch, Hq]               */
+  const void* q;           /* [batch, Hq, D] contiguous              */
+  const void* k;           /* [slots, Hkv, D], last dim contiguous   */
+  const void* v;
+  int64_t k_stride_0, k_stride_1; /* elements */
+  int64_t v_stride_0, v_stride_1;
+  float sm_scale;
+  int32_t dtype;           /* LSATTN_F16 or LSATTN_BF16 */
+  const int32_t* req_to_tokens; /* [max_req, max_seq_len] contiguous */
+  const int32_t* b_req_idx;     /* [batch] */
+  const int32_t* b_seqlen;      /* [batch] */
+  int64_t batch;
+  int64_t num_q_heads;
+  int64_t num_kv_heads;
+  int64_t num_blocks;      /* mid_o.size(0) */
+  int64_t head_dim;        /* 128 */
+  int64_t max_seq_len;     /* req_to_tokens.size(1) */
+  int64_t seq_block_size;  /* tokens per partial, >= 1 */
+  int64_t max_len_in_batch;
+} lsattn_decode_stage1_args;
+int lsattn_decode_stage1(const lsattn_decode_stage1_args* a, void* stream);
+
+/*
+ * Flash-decoding stage 2: LSE-weighted merge over the block axis.  Replaces
+ * LongServe::flash_decoding_stage2 (S2H:7-19, S2CU:116-132) behind ENTRY:166-221.
+ * n_b = b_seqlen[b] <= 0 ? 0 : ceil(b_seqlen[b]/block_seq) rows are merged (S2CU:30);
+ * n_b = 0 writes o = 0, out_logexpsum = -inf.
+ */
+typedef struct lsattn_decode_stage2_args {
+  void* o;                 /* [batch, H, D] contiguous */
+  int32_t o_dtype;         /* LSATTN_F16 / BF16 / F32  */
+  int32_t reserved;
+  float* out_logexpsum;    /* [batch, H] */
+  const int32_t* b_seqlen; /* [batch]    */
+  const float* mid_o;            /* [num_seq_blocks, batch, H, D] */
+  const float* mid_o_logexpsum;  /* [num_seq_blocks, batch, H]    */
+  int64_t batch;
+  int64_t num_heads;
+  int64_t num_seq_blocks;
+  int64_t head_dim;        /* 32, 64 or 128 */
+  int64_t block_seq;
+} lsattn_decode_stage2_args;
+int lsattn_decode_stage2(const lsattn_decode_stage2_args* a, void* stream);
+
+/*
+ * Row scatter into the KV pool: dst[dest_index[i]] = src[i] for i < n_rows, bit-exact.
+ * Replaces _fwd_kernel_destindex_copy_kv
+ * (loongserve/common/basemodel/triton_kernel/destindex_copy_kv.py:7-51).
+ * Rows are row_bytes long (a multiple of 16, 16-byte aligned); strides are in bytes.
+ */
+int lsattn_kv_scatter(const void* src, int64_t src_stride_bytes, void* dst, int64_t dst_stride_bytes,
+                      const int32_t* dest_index, int64_t n_rows, int64_t row_bytes, void* stream);
+
+/*
+ * Prefill registration of freshly written slots:
+ *   req_to_tokens[b_req_idx[b], 0:b_seq_len[b]] = mem_index[b_start_loc[b] : +b_seq_len[b]].
+ * Replaces init_req_to_token_indexes (loongserve/common/infer_utils.py:1-13), which loops
+ * on the host after a device-to-host copy.
+ */
+int lsattn_register_tokens(int32_t* req_to_tokens, int64_t max_seq_len, const int32_t* b_req_idx,
+                           const int32_t* b_start_loc, const int32_t* b_seq_len, const int32_t* mem_index,
+                           int64_t batch, int64_t max_len_in_batch, void* stream);
+
+const char* lsattn_strerror(int code);
+int lsattn_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LSATTN_H */

@@ -1,0 +1,24 @@
+"""MI355X-native attention hot path with LoongServe's operator interface.
+
+Prefill: context_attention_fwd (ring / context-parallel step, in-place (o, m, l) state),
+prefill_attention_step (+ lse_merge) for mergeable fp32 partials.
+Decode: longserve_flash_decode_stage1 / stage2,
+longserve_token_decode_attention_flash_decoding, and the extension-module stand-in
+`longserve_cuda_kernels`.  All of them run hand-written gfx950 HIP kernels from
+liblsattn.so; importing this package fails if that library has not been built.
+"""
+from . import _lib
+
+_lib.load()  # fail loudly at import time if the HIP library is missing
+
+from . import longserve_cuda_kernels  # noqa: E402
+from .decoding import (longserve_flash_decode_stage1, longserve_flash_decode_stage2,  # noqa: E402
+                       longserve_token_decode_attention_flash_decoding)
+from .ops import (context_attention_fwd, init_req_to_token_indexes, kv_scatter, lse_merge,  # noqa: E402
+                  prefill_attention_step)
+
+__all__ = [
+    "context_attention_fwd", "prefill_attention_step", "lse_merge", "kv_scatter", "init_req_to_token_indexes",
+    "longserve_flash_decode_stage1", "longserve_flash_decode_stage2",
+    "longserve_token_decode_attention_flash_decoding", "longserve_cuda_kernels",
+]

@@ -1,0 +1,101 @@
+"""ctypes binding of liblsattn.so (the C ABI declared in include/lsattn.h).
+
+The library is the only implementation of the operators in this package: there is no
+CPU or PyTorch fallback.  If the shared object is missing or fails to load, importing
+an operator raises; build it with `python -m loongserve_amd.build`.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "liblsattn.so")
+
+LSATTN_F16, LSATTN_BF16, LSATTN_F32 = 0, 1, 2
+LSATTN_MAX_PARTS = 16
+
+_vp, _i32, _i64, _f32 = C.c_void_p, C.c_int32, C.c_int64, C.c_float
+
+
+class PrefillArgs(C.Structure):
+    _fields_ = [
+        ("q", _vp), ("k", _vp), ("v", _vp),
+        ("q_stride_t", _i64), ("q_stride_h", _i64),
+        ("k_stride_t", _i64), ("k_stride_h", _i64),
+        ("v_stride_t", _i64), ("v_stride_h", _i64),
+        ("q_b_start_loc", _vp), ("q_b_seq_len", _vp), ("q_first_token_global_idx", _vp),
+        ("kv_b_start_loc", _vp), ("kv_b_seq_len", _vp), ("kv_first_token_global_idx", _vp),
+        ("batch", _i32), ("num_q_heads", _i32), ("num_kv_heads", _i32), ("head_dim", _i32),
+        ("dtype", _i32), ("sp_peers", _i32), ("max_q_len", _i32), ("sm_scale", _f32),
+        ("o", _vp), ("o_stride_t", _i64), ("o_stride_h", _i64),
+        ("o_dtype", _i32), ("reserved", _i32),
+        ("lse", _vp), ("m", _vp), ("l", _vp),
+        ("ml_stride_t", _i64), ("ml_stride_h", _i64),
+    ]
+
+
+class MergeArgs(C.Structure):
+    _fields_ = [
+        ("n_parts", _i32), ("head_dim", _i32), ("rows", _i64),
+        ("o_parts", _vp * LSATTN_MAX_PARTS), ("lse_parts", _vp * LSATTN_MAX_PARTS),
+        ("o", _vp), ("o_dtype", _i32), ("reserved", _i32), ("lse", _vp),
+    ]
+
+
+class DecodeStage1Args(C.Structure):
+    _fields_ = [
+        ("mid_o", _vp), ("mid_o_logexpsum", _vp), ("q", _vp), ("k", _vp), ("v", _vp),
+        ("k_stride_0", _i64), ("k_stride_1", _i64), ("v_stride_0", _i64), ("v_stride_1", _i64),
+        ("sm_scale", _f32), ("dtype", _i32),
+        ("req_to_tokens", _vp), ("b_req_idx", _vp), ("b_seqlen", _vp),
+        ("batch", _i64), ("num_q_heads", _i64), ("num_kv_heads", _i64), ("num_blocks", _i64),
+        ("head_dim", _i64), ("max_seq_len", _i64), ("seq_block_size", _i64), ("max_len_in_batch", _i64),
+    ]
+
+
+class DecodeStage2Args(C.Structure):
+    _fields_ = [
+        ("o", _vp), ("o_dtype", _i32), ("reserved", _i32), ("out_logexpsum", _vp), ("b_seqlen", _vp),
+        ("mid_o", _vp), ("mid_o_logexpsum", _vp),
+        ("batch", _i64), ("num_heads", _i64), ("num_seq_blocks", _i64), ("head_dim", _i64), ("block_seq", _i64),
+    ]
+
+
+# every symbol include/lsattn.h declares: name -> (restype, argtypes)
+EXPORTS = {
+    "lsattn_prefill_step": (C.c_int, [C.POINTER(PrefillArgs), _vp]),
+    "lsattn_prefill_step_merge": (C.c_int, [C.POINTER(PrefillArgs), _vp]),
+    "lsattn_lse_merge": (C.c_int, [C.POINTER(MergeArgs), _vp]),
+    "lsattn_decode_stage1": (C.c_int, [C.POINTER(DecodeStage1Args), _vp]),
+    "lsattn_decode_stage2": (C.c_int, [C.POINTER(DecodeStage2Args), _vp]),
+    "lsattn_kv_scatter": (C.c_int, [_vp, _i64, _vp, _i64, _vp, _i64, _i64, _vp]),
+    "lsattn_register_tokens": (C.c_int, [_vp, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _vp]),
+    "lsattn_strerror": (C.c_char_p, [C.c_int]),
+    "lsattn_version": (C.c_int, []),
+}
+
+_lib = None
+
+
+def load():
+    """Load liblsattn.so once and type its entry points.  Raises if it is not built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            "loongserve_amd: %s is missing; there is no fallback implementation. "
+            "Build it with `python -m loongserve_amd.build`." % LIB_PATH)
+    lib = C.CDLL(LIB_PATH)
+    for name, (res, args) in EXPORTS.items():
+        fn = getattr(lib, name)  # AttributeError if the symbol is not exported
+        fn.restype = res
+        fn.argtypes = args
+    _lib = lib
+    return lib
+
+
+def check(rc: int, what: str) -> None:
+    if rc != 0:
+        msg = load().lsattn_strerror(rc).decode()
+        raise RuntimeError("%s failed: %s (code %d)" % (what, msg, rc))

@@ -1,0 +1,365 @@
+// Token-indexed flash decoding for gfx950: stage 1 (gather + split-K partials) and
+// stage 2 (LSE merge over the block axis).
+//
+// Stage 1 replaces flash_decoding_stage1_kernel
+// (longserve_cuda_kernels/src/flash_decoding_stage1.cu:25-143).  Differences by design:
+//   * one wave64 serves one KV head and all (up to 8) query heads of its GQA group, so a
+//     K/V row is fetched once per KV head instead of once per query head;
+//   * a K/V row of 128 16-bit elements is read by 16 lanes x 16 bytes; a wave has four
+//     such lane groups and every group keeps 8 K rows and 8 V rows in flight;
+//   * each lane group runs its own online softmax; groups are merged once per block with
+//     an LSE merge, and the partial is written with plain stores (no atomics), so the
+//     result is deterministic;
+//   * a workgroup walks several consecutive blocks, so the launch is sized for the chip
+//     and not for block_seq.
+#include "common.hip.h"
+
+namespace lsattn {
+
+struct Stage1Params {
+  float* mid_o;
+  float* mid_lse;
+  const void* q;
+  const void* k;
+  const void* v;
+  int64_t k_s0, k_s1, v_s0, v_s1;
+  float scale_log2;  // sm_scale * log2(e)
+  const int32_t* req_to_tokens;
+  const int32_t* b_req_idx;
+  const int32_t* b_seqlen;
+  int64_t batch, hq, hkv, num_blocks, max_seq_len, block_seq, grid_blocks;
+  int32_t blocks_per_wg;  // consecutive blocks walked by one workgroup
+  int32_t tasks;          // hkv * (group / GT) wave tasks
+};
+
+constexpr int kTok = 8;  // K/V rows in flight per 16-lane group
+
+template <typename T, int GT, int NW>
+__global__ __launch_bounds__(NW * 64) void decode_stage1_kernel(Stage1Params p) {
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int grp = lane >> 4;   // which of the 4 row slots of the wave
+  const int sub = lane & 15;   // 16-byte column slot: elements sub*8 .. sub*8+7
+  const int64_t b = blockIdx.z;
+  const int task = blockIdx.y * NW + wave;
+  if (task >= p.tasks) return;
+  const int group = (int)(p.hq / p.hkv);
+  const int sub_groups = group / GT;
+  const int kvh = task / sub_groups;
+  const int qh0 = kvh * group + (task % sub_groups) * GT;
+
+  const int64_t len = p.b_seqlen[b];
+  int64_t nblk = len <= 0 ? 0 : (len + p.block_seq - 1) / p.block_seq;
+  if (nblk > p.grid_blocks) nblk = p.grid_blocks;
+  if (nblk > p.num_blocks) nblk = p.num_blocks;
+  const int64_t blk_begin = (int64_t)blockIdx.x * p.blocks_per_wg;
+  int64_t blk_end = blk_begin + p.blocks_per_wg;
+  if (blk_end > nblk) blk_end = nblk;
+  if (blk_begin >= blk_end) return;
+
+  const int32_t* table = p.req_to_tokens + (int64_t)p.b_req_idx[b] * p.max_seq_len;
+  const char* kbase = (const char*)p.k + ((int64_t)kvh * p.k_s1 + sub * 8) * 2;
+  const char* vbase = (const char*)p.v + ((int64_t)kvh * p.v_s1 + sub * 8) * 2;
+  const int64_t k_row_bytes = p.k_s0 * 2, v_row_bytes = p.v_s0 * 2;
+
+  float qf[GT][8];
+#pragma unroll
+  for (int h = 0; h < GT; h++) {
+    const u32x4 w = *(const u32x4*)((const char*)p.q + ((b * p.hq + qh0 + h) * 128 + sub * 8) * 2);
+    unpack8<T>(w, qf[h]);
+#pragma unroll
+    for (int i = 0; i < 8; i++) qf[h][i] *= p.scale_log2;
+  }
+
+  for (int64_t blk = blk_begin; blk < blk_end; blk++) {
+    const int64_t t0 = blk * p.block_seq;
+    int64_t t1 = t0 + p.block_seq;
+    if (t1 > len) t1 = len;
+
+    float m[GT], l[GT], o[GT][8];
+#pragma unroll
+    for (int h = 0; h < GT; h++) {
+      m[h] = -INFINITY;
+      l[h] = 0.f;
+#pragma unroll
+      for (int i = 0; i < 8; i++) o[h][i] = 0.f;
+    }
+
+    // slot indices of the first batch of rows
+    int32_t slot[kTok];
+#pragma unroll
+    for (int j = 0; j < kTok; j++) {
+      const int64_t tok = t0 + j * 4 + grp;
+      slot[j] = tok < t1 ? table[tok] : -1;
+    }
+
+    for (int64_t it = t0; it < t1; it += 4 * kTok) {
+      u32x4 kr[kTok], vr[kTok];
+#pragma unroll
+      for (int j = 0; j < kTok; j++) {
+        if (slot[j] >= 0) {
+          kr[j] = *(const u32x4*)(kbase + (int64_t)slot[j] * k_row_bytes);
+          vr[j] = *(const u32x4*)(vbase + (int64_t)slot[j] * v_row_bytes);
+        } else {
+          kr[j] = u32x4{0, 0, 0, 0};
+          vr[j] = u32x4{0, 0, 0, 0};
+        }
+      }
+      bool valid[kTok];
+#pragma unroll
+      for (int j = 0; j < kTok; j++) valid[j] = slot[j] >= 0;
+      // prefetch the slot indices of the next batch while the rows are in flight
+#pragma unroll
+      for (int j = 0; j < kTok; j++) {
+        const int64_t tok = it + 4 * kTok + j * 4 + grp;
+        slot[j] = tok < t1 ? table[tok] : -1;
+      }
+
+      float s[kTok][GT];
+#pragma unroll
+      for (int j = 0; j < kTok; j++) {
+        float kf[8];
+        unpack8<T>(kr[j], kf);
+#pragma unroll
+        for (int h = 0; h < GT; h++) {
+          float d = 0.f;
+#pragma unroll
+          for (int i = 0; i < 8; i++) d = __builtin_fmaf(qf[h][i], kf[i], d);
+          d = sum_row16(d);
+          s[j][h] = valid[j] ? d : -INFINITY;
+        }
+      }
+      float pj[kTok][GT];
+#pragma unroll
+      for (int h = 0; h < GT; h++) {
+        float mx = s[0][h];
+#pragma unroll
+        for (int j = 1; j < kTok; j++) mx = fmaxf(mx, s[j][h]);
+        const float m_new = fmaxf(m[h], mx);
+        const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+        const float alpha = __builtin_amdgcn_exp2f(m[h] - m_safe);
+        float ps = 0.f;
+#pragma unroll
+        for (int j = 0; j < kTok; j++) {
+          pj[j][h] = __builtin_amdgcn_exp2f(s[j][h] - m_safe);
+          ps += pj[j][h];
+        }
+        l[h] = l[h] * alpha + ps;
+        m[h] = m_new;
+#pragma unroll
+        for (int i = 0; i < 8; i++) o[h][i] *= alpha;
+      }
+#pragma unroll
+      for (int j = 0; j < kTok; j++) {
+        float vf[8];
+        unpack8<T>(vr[j], vf);
+#pragma unroll
+        for (int h = 0; h < GT; h++)
+#pragma unroll
+          for (int i = 0; i < 8; i++) o[h][i] = __builtin_fmaf(pj[j][h], vf[i], o[h][i]);
+      }
+    }
+
+    // merge the four lane groups and write the block's partial
+#pragma unroll
+    for (int h = 0; h < GT; h++) {
+      float M = fmaxf(m[h], __shfl_xor(m[h], 16));
+      M = fmaxf(M, __shfl_xor(M, 32));
+      const float w = exp2_diff(m[h], M);  // the block holds >= 1 row, so M is finite
+      float L = l[h] * w;
+      L += __shfl_xor(L, 16);
+      L += __shfl_xor(L, 32);
+      float ov[8];
+#pragma unroll
+      for (int i = 0; i < 8; i++) {
+        float x = o[h][i] * w;
+        x += __shfl_xor(x, 16);
+        x += __shfl_xor(x, 32);
+        ov[i] = x;
+      }
+      if (grp == 0) {
+        const float inv = 1.f / L;
+        const int64_t row = (blk * p.batch + b) * p.hq + qh0 + h;
+        f32x4* dst = (f32x4*)(p.mid_o + row * 128 + sub * 8);
+        dst[0] = f32x4{ov[0] * inv, ov[1] * inv, ov[2] * inv, ov[3] * inv};
+        dst[1] = f32x4{ov[4] * inv, ov[5] * inv, ov[6] * inv, ov[7] * inv};
+        if (sub == 0) p.mid_lse[row] = (M + __builtin_amdgcn_logf(L)) * kLn2;
+      }
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------
+// Stage 2: grid (batch, heads); SL slices of D/4 lanes walk the block axis in parallel
+// (the reference walks it serially, flash_decoding_stage2.cu:38-48), then merge through LDS.
+// ------------------------------------------------------------------------------------
+struct Stage2Params {
+  void* o;
+  float* out_lse;
+  const int32_t* b_seqlen;
+  const float* mid_o;
+  const float* mid_lse;
+  int64_t batch, heads, num_seq_blocks, block_seq;
+};
+
+template <typename OT> __device__ __forceinline__ void store4(void* base, int64_t elem, const f32x4& v);
+template <> __device__ __forceinline__ void store4<float>(void* base, int64_t elem, const f32x4& v) {
+  *(f32x4*)((float*)base + elem) = v;
+}
+template <> __device__ __forceinline__ void store4<F16>(void* base, int64_t elem, const f32x4& v) {
+  *(u32x2*)((uint16_t*)base + elem) = u32x2{pack2<F16>(v[0], v[1]), pack2<F16>(v[2], v[3])};
+}
+template <> __device__ __forceinline__ void store4<BF16>(void* base, int64_t elem, const f32x4& v) {
+  *(u32x2*)((uint16_t*)base + elem) = u32x2{pack2<BF16>(v[0], v[1]), pack2<BF16>(v[2], v[3])};
+}
+
+template <typename OT, int D>
+__global__ __launch_bounds__(256) void decode_stage2_kernel(Stage2Params p) {
+  constexpr int LPR = D / 4;      // lanes per row (float4 each)
+  constexpr int SL = 256 / LPR;   // slices walking the block axis
+  const int64_t b = blockIdx.x, h = blockIdx.y;
+  const int slice = threadIdx.x / LPR, c = threadIdx.x % LPR;
+  const int64_t len = p.b_seqlen[b];
+  int64_t n = len <= 0 ? 0 : (len + p.block_seq - 1) / p.block_seq;
+  if (n > p.num_seq_blocks) n = p.num_seq_blocks;
+  const int64_t row_stride = p.batch * p.heads;
+  const int64_t row0 = b * p.heads + h;
+
+  float M = -INFINITY, L = 0.f;
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  for (int64_t i = slice; i < n; i += SL) {
+    const int64_t row = i * row_stride + row0;
+    const float lse = p.mid_lse[row];
+    const f32x4 tv = *(const f32x4*)(p.mid_o + row * D + c * 4);
+    if (lse == -INFINITY) continue;  // an empty partial contributes nothing
+    const float Mn = fmaxf(M, lse);
+    const float so = exp2_diff(M * kLog2e, Mn * kLog2e);
+    const float sn = __builtin_amdgcn_exp2f((lse - Mn) * kLog2e);
+    acc = acc * so + tv * sn;
+    L = L * so + sn;
+    M = Mn;
+  }
+  __shared__ float sM[SL], sL[SL];
+  __shared__ f32x4 sAcc[SL][LPR];
+  if (c == 0) {
+    sM[slice] = M;
+    sL[slice] = L;
+  }
+  sAcc[slice][c] = acc;
+  __syncthreads();
+  if (slice == 0) {
+    float Mt = -INFINITY;
+#pragma unroll
+    for (int s = 0; s < SL; s++) Mt = fmaxf(Mt, sM[s]);
+    float Lt = 0.f;
+    f32x4 a = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < SL; s++) {
+      const float w = exp2_diff(sM[s] * kLog2e, Mt * kLog2e);
+      Lt += sL[s] * w;
+      a += sAcc[s][c] * w;
+    }
+    const float inv = Lt > 0.f ? 1.f / Lt : 0.f;
+    store4<OT>(p.o, row0 * D + c * 4, a * inv);
+    if (c == 0) p.out_lse[row0] = Lt > 0.f ? Mt + __builtin_amdgcn_logf(Lt) * kLn2 : -INFINITY;
+  }
+}
+
+template <typename T, int GT>
+static int launch_stage1(const lsattn_decode_stage1_args* a, hipStream_t st) {
+  constexpr int NW = 8;
+  Stage1Params p;
+  p.mid_o = a->mid_o;
+  p.mid_lse = a->mid_o_logexpsum;
+  p.q = a->q;
+  p.k = a->k;
+  p.v = a->v;
+  p.k_s0 = a->k_stride_0;
+  p.k_s1 = a->k_stride_1;
+  p.v_s0 = a->v_stride_0;
+  p.v_s1 = a->v_stride_1;
+  p.scale_log2 = a->sm_scale * kLog2e;
+  p.req_to_tokens = a->req_to_tokens;
+  p.b_req_idx = a->b_req_idx;
+  p.b_seqlen = a->b_seqlen;
+  p.batch = a->batch;
+  p.hq = a->num_q_heads;
+  p.hkv = a->num_kv_heads;
+  p.num_blocks = a->num_blocks;
+  p.max_seq_len = a->max_seq_len;
+  p.block_seq = a->seq_block_size;
+  p.grid_blocks = (a->max_len_in_batch + a->seq_block_size - 1) / a->seq_block_size;  // stage1.cu:211
+  const int group = (int)(a->num_q_heads / a->num_kv_heads);
+  p.tasks = (int)a->num_kv_heads * (group / GT);
+  const int wgs_y = (p.tasks + NW - 1) / NW;
+  // tokens per workgroup: at least ~1024, and few enough workgroups-per-launch to stay cheap
+  int64_t per_wg = (1024 + a->seq_block_size - 1) / a->seq_block_size;
+  if (per_wg < 1) per_wg = 1;
+  int64_t nblk = p.grid_blocks < a->num_blocks ? p.grid_blocks : a->num_blocks;
+  if (nblk < 1) return LSATTN_OK;
+  p.blocks_per_wg = (int32_t)per_wg;
+  const int64_t chunks = (nblk + per_wg - 1) / per_wg;
+  if (chunks > 0x7fffffff || a->batch > 65535 || wgs_y > 65535) return LSATTN_ERR_INVALID_ARG;
+  dim3 grid((unsigned)chunks, (unsigned)wgs_y, (unsigned)a->batch);
+  hipLaunchKernelGGL((decode_stage1_kernel<T, GT, NW>), grid, dim3(NW * 64), 0, st, p);
+  return check_launch();
+}
+
+template <typename T> static int dispatch_stage1(const lsattn_decode_stage1_args* a, hipStream_t st) {
+  const int group = (int)(a->num_q_heads / a->num_kv_heads);
+  if (group % 4 == 0) return launch_stage1<T, 4>(a, st);
+  if (group % 2 == 0) return launch_stage1<T, 2>(a, st);
+  return launch_stage1<T, 1>(a, st);
+}
+
+}  // namespace lsattn
+
+using namespace lsattn;
+
+extern "C" int lsattn_decode_stage1(const lsattn_decode_stage1_args* a, void* stream) {
+  if (!a || !a->mid_o || !a->mid_o_logexpsum || !a->q || !a->k || !a->v || !a->req_to_tokens || !a->b_req_idx ||
+      !a->b_seqlen)
+    return LSATTN_ERR_INVALID_ARG;
+  if (a->batch < 0 || a->num_q_heads <= 0 || a->num_kv_heads <= 0 || a->num_blocks < 0 || a->seq_block_size < 1 ||
+      a->max_len_in_batch < 0 || a->max_seq_len < 0)
+    return LSATTN_ERR_INVALID_ARG;
+  if (a->num_q_heads % a->num_kv_heads != 0) return LSATTN_ERR_INVALID_ARG;
+  // 16-byte row loads: strides must keep every row 16-byte aligned
+  if (a->k_stride_0 % 8 || a->k_stride_1 % 8 || a->v_stride_0 % 8 || a->v_stride_1 % 8) return LSATTN_ERR_INVALID_ARG;
+  if (((uintptr_t)a->k | (uintptr_t)a->v | (uintptr_t)a->q | (uintptr_t)a->mid_o) & 15) return LSATTN_ERR_INVALID_ARG;
+  if (a->head_dim != 128) return LSATTN_ERR_UNSUPPORTED;  // as flash_decoding_stage1.cu:210
+  if (a->batch == 0 || a->num_blocks == 0 || a->max_len_in_batch == 0) return LSATTN_OK;
+  hipStream_t st = (hipStream_t)stream;
+  if (a->dtype == LSATTN_F16) return dispatch_stage1<F16>(a, st);
+  if (a->dtype == LSATTN_BF16) return dispatch_stage1<BF16>(a, st);
+  return LSATTN_ERR_UNSUPPORTED;
+}
+
+template <typename OT> static int dispatch_stage2(const Stage2Params& p, int64_t D, dim3 grid, hipStream_t st) {
+  switch (D) {
+    case 32: hipLaunchKernelGGL((decode_stage2_kernel<OT, 32>), grid, dim3(256), 0, st, p); break;
+    case 64: hipLaunchKernelGGL((decode_stage2_kernel<OT, 64>), grid, dim3(256), 0, st, p); break;
+    case 128: hipLaunchKernelGGL((decode_stage2_kernel<OT, 128>), grid, dim3(256), 0, st, p); break;
+    default: return LSATTN_ERR_UNSUPPORTED;
+  }
+  return check_launch();
+}
+
+extern "C" int lsattn_decode_stage2(const lsattn_decode_stage2_args* a, void* stream) {
+  if (!a || !a->o || !a->out_logexpsum || !a->b_seqlen || !a->mid_o || !a->mid_o_logexpsum) return LSATTN_ERR_INVALID_ARG;
+  if (a->batch < 0 || a->num_heads <= 0 || a->num_seq_blocks < 0 || a->block_seq < 1) return LSATTN_ERR_INVALID_ARG;
+  if (((uintptr_t)a->o | (uintptr_t)a->mid_o) & 15) return LSATTN_ERR_INVALID_ARG;
+  if (a->head_dim != 32 && a->head_dim != 64 && a->head_dim != 128) return LSATTN_ERR_UNSUPPORTED;
+  if (a->batch == 0) return LSATTN_OK;
+  if (a->num_heads > 65535) return LSATTN_ERR_INVALID_ARG;
+  Stage2Params p{a->o, a->out_logexpsum, a->b_seqlen, a->mid_o, a->mid_o_logexpsum,
+                 a->batch, a->num_heads, a->num_seq_blocks, a->block_seq};
+  dim3 grid((unsigned)a->batch, (unsigned)a->num_heads);
+  hipStream_t st = (hipStream_t)stream;
+  switch (a->o_dtype) {
+    case LSATTN_F32: return dispatch_stage2<float>(p, a->head_dim, grid, st);
+    case LSATTN_F16: return dispatch_stage2<F16>(p, a->head_dim, grid, st);
+    case LSATTN_BF16: return dispatch_stage2<BF16>(p, a->head_dim, grid, st);
+    default: return LSATTN_ERR_UNSUPPORTED;
+  }
+}

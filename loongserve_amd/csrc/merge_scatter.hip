@@ -1,0 +1,155 @@
+// HBM-bound helpers around the attention kernels: LSE merge of separately allocated
+// prefill partials, KV-pool row scatter, and prefill slot registration.
+#include "common.hip.h"
+
+namespace lsattn {
+
+struct MergeParams {
+  int32_t n;
+  int64_t rows;
+  const float* o[LSATTN_MAX_PARTS];
+  const float* lse[LSATTN_MAX_PARTS];
+  void* out;
+  float* out_lse;
+};
+
+template <typename OT> __device__ __forceinline__ void put4(void* base, int64_t elem, const f32x4& v);
+template <> __device__ __forceinline__ void put4<float>(void* base, int64_t elem, const f32x4& v) {
+  *(f32x4*)((float*)base + elem) = v;
+}
+template <> __device__ __forceinline__ void put4<F16>(void* base, int64_t elem, const f32x4& v) {
+  *(u32x2*)((uint16_t*)base + elem) = u32x2{pack2<F16>(v[0], v[1]), pack2<F16>(v[2], v[3])};
+}
+template <> __device__ __forceinline__ void put4<BF16>(void* base, int64_t elem, const f32x4& v) {
+  *(u32x2*)((uint16_t*)base + elem) = u32x2{pack2<BF16>(v[0], v[1]), pack2<BF16>(v[2], v[3])};
+}
+
+// one thread per (row, 4 consecutive output elements); same recurrence as
+// flash_decoding_stage2.cu:38-48 with the partials living in separate buffers
+template <typename OT, int D>
+__global__ __launch_bounds__(256) void lse_merge_kernel(MergeParams p) {
+  constexpr int LPR = D / 4;
+  const int64_t gid = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t row = gid / LPR;
+  const int c = (int)(gid % LPR);
+  if (row >= p.rows) return;
+  float M = -INFINITY;
+  for (int i = 0; i < p.n; i++) M = fmaxf(M, p.lse[i][row]);
+  float L = 0.f;
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  if (M != -INFINITY) {
+    for (int i = 0; i < p.n; i++) {
+      const float w = __builtin_amdgcn_exp2f((p.lse[i][row] - M) * kLog2e);
+      if (w == 0.f) continue;
+      L += w;
+      acc += *(const f32x4*)(p.o[i] + row * D + c * 4) * w;
+    }
+  }
+  const float inv = L > 0.f ? 1.f / L : 0.f;
+  put4<OT>(p.out, row * D + c * 4, acc * inv);
+  if (c == 0) p.out_lse[row] = L > 0.f ? M + __builtin_amdgcn_logf(L) * kLn2 : -INFINITY;
+}
+
+// dst[dest_index[i]] = src[i]; 16 bytes per lane, consecutive lanes cover one row
+__global__ __launch_bounds__(256) void kv_scatter_kernel(const char* __restrict__ src, int64_t src_stride,
+                                                         char* __restrict__ dst, int64_t dst_stride,
+                                                         const int32_t* __restrict__ dest_index, int64_t n_rows,
+                                                         int32_t chunks_per_row) {
+  const int64_t gid = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t row = gid / chunks_per_row;
+  const int c = (int)(gid % chunks_per_row);
+  if (row >= n_rows) return;
+  const u32x4 w = *(const u32x4*)(src + row * src_stride + (int64_t)c * 16);
+  *(u32x4*)(dst + (int64_t)dest_index[row] * dst_stride + (int64_t)c * 16) = w;
+}
+
+__global__ __launch_bounds__(256) void register_tokens_kernel(int32_t* __restrict__ req_to_tokens, int64_t max_seq_len,
+                                                              const int32_t* __restrict__ b_req_idx,
+                                                              const int32_t* __restrict__ b_start_loc,
+                                                              const int32_t* __restrict__ b_seq_len,
+                                                              const int32_t* __restrict__ mem_index) {
+  const int64_t b = blockIdx.y;
+  const int64_t j = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (j >= b_seq_len[b]) return;
+  req_to_tokens[(int64_t)b_req_idx[b] * max_seq_len + j] = mem_index[(int64_t)b_start_loc[b] + j];
+}
+
+template <typename OT> static int launch_merge(const MergeParams& p, int D, hipStream_t st) {
+  const int64_t threads = p.rows * (D / 4);
+  const int64_t blocks = (threads + 255) / 256;
+  if (blocks > 0x7fffffff) return LSATTN_ERR_INVALID_ARG;
+  switch (D) {
+    case 32: hipLaunchKernelGGL((lse_merge_kernel<OT, 32>), dim3((unsigned)blocks), dim3(256), 0, st, p); break;
+    case 64: hipLaunchKernelGGL((lse_merge_kernel<OT, 64>), dim3((unsigned)blocks), dim3(256), 0, st, p); break;
+    case 128: hipLaunchKernelGGL((lse_merge_kernel<OT, 128>), dim3((unsigned)blocks), dim3(256), 0, st, p); break;
+    default: return LSATTN_ERR_UNSUPPORTED;
+  }
+  return check_launch();
+}
+
+}  // namespace lsattn
+
+using namespace lsattn;
+
+extern "C" int lsattn_lse_merge(const lsattn_merge_args* a, void* stream) {
+  if (!a || a->n_parts < 1 || a->n_parts > LSATTN_MAX_PARTS || a->rows < 0 || !a->o || !a->lse) return LSATTN_ERR_INVALID_ARG;
+  MergeParams p;
+  p.n = a->n_parts;
+  p.rows = a->rows;
+  for (int i = 0; i < LSATTN_MAX_PARTS; i++) {
+    p.o[i] = i < a->n_parts ? a->o_parts[i] : nullptr;
+    p.lse[i] = i < a->n_parts ? a->lse_parts[i] : nullptr;
+    if (i < a->n_parts && (!p.o[i] || !p.lse[i] || ((uintptr_t)p.o[i] & 15))) return LSATTN_ERR_INVALID_ARG;
+  }
+  if ((uintptr_t)a->o & 15) return LSATTN_ERR_INVALID_ARG;
+  p.out = a->o;
+  p.out_lse = a->lse;
+  if (a->rows == 0) return LSATTN_OK;
+  hipStream_t st = (hipStream_t)stream;
+  switch (a->o_dtype) {
+    case LSATTN_F32: return launch_merge<float>(p, a->head_dim, st);
+    case LSATTN_F16: return launch_merge<F16>(p, a->head_dim, st);
+    case LSATTN_BF16: return launch_merge<BF16>(p, a->head_dim, st);
+    default: return LSATTN_ERR_UNSUPPORTED;
+  }
+}
+
+extern "C" int lsattn_kv_scatter(const void* src, int64_t src_stride_bytes, void* dst, int64_t dst_stride_bytes,
+                                 const int32_t* dest_index, int64_t n_rows, int64_t row_bytes, void* stream) {
+  if (!src || !dst || !dest_index || n_rows < 0 || row_bytes <= 0) return LSATTN_ERR_INVALID_ARG;
+  if (row_bytes % 16 || src_stride_bytes % 16 || dst_stride_bytes % 16 || (((uintptr_t)src | (uintptr_t)dst) & 15))
+    return LSATTN_ERR_INVALID_ARG;
+  if (n_rows == 0) return LSATTN_OK;
+  const int64_t cpr = row_bytes / 16;
+  const int64_t blocks = (n_rows * cpr + 255) / 256;
+  if (blocks > 0x7fffffff || cpr > 0x7fffffff) return LSATTN_ERR_INVALID_ARG;
+  hipLaunchKernelGGL(kv_scatter_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (const char*)src,
+                     src_stride_bytes, (char*)dst, dst_stride_bytes, dest_index, n_rows, (int32_t)cpr);
+  return check_launch();
+}
+
+extern "C" int lsattn_register_tokens(int32_t* req_to_tokens, int64_t max_seq_len, const int32_t* b_req_idx,
+                                      const int32_t* b_start_loc, const int32_t* b_seq_len, const int32_t* mem_index,
+                                      int64_t batch, int64_t max_len_in_batch, void* stream) {
+  if (!req_to_tokens || !b_req_idx || !b_start_loc || !b_seq_len || !mem_index || batch < 0 || max_len_in_batch < 0 ||
+      max_len_in_batch > max_seq_len)
+    return LSATTN_ERR_INVALID_ARG;
+  if (batch == 0 || max_len_in_batch == 0) return LSATTN_OK;
+  if (batch > 65535) return LSATTN_ERR_INVALID_ARG;
+  dim3 grid((unsigned)((max_len_in_batch + 255) / 256), (unsigned)batch);
+  hipLaunchKernelGGL(register_tokens_kernel, grid, dim3(256), 0, (hipStream_t)stream, req_to_tokens, max_seq_len,
+                     b_req_idx, b_start_loc, b_seq_len, mem_index);
+  return check_launch();
+}
+
+extern "C" const char* lsattn_strerror(int code) {
+  switch (code) {
+    case LSATTN_OK: return "ok";
+    case LSATTN_ERR_INVALID_ARG: return "invalid argument (null pointer, bad size, stride or alignment)";
+    case LSATTN_ERR_UNSUPPORTED: return "unsupported head_dim, dtype or head ratio";
+    case LSATTN_ERR_LAUNCH: return "kernel launch failed";
+    default: return "unknown error";
+  }
+}
+
+extern "C" int lsattn_version(void) { return 1; }

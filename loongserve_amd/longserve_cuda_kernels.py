@@ -1,0 +1,99 @@
+"""Stand-in for the `longserve_cuda_kernels` extension module (decode entry points only).
+
+Exports flash_decoding_stage1 / flash_decoding_stage2 with the argument order and the
+tensor checks of longserve_cuda_kernels/src/entrypoints.cpp:103-221 (exported at
+:237-238).  A failed check raises ValueError instead of aborting the process
+(the reference calls __assert_fail, longserve_cuda_kernels/src/common.h:29-32).
+Beyond the reference: q/k/v may be bfloat16, and stage-2 `o` may be bfloat16.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import math
+
+import torch
+
+from . import _lib
+from .ops import _DT, _stream
+
+
+def _req(cond: bool, what: str) -> None:
+    if not cond:
+        raise ValueError("longserve_cuda_kernels: check failed: " + what)
+
+
+@torch.inference_mode()
+def flash_decoding_stage1(mid_o, mid_o_logexpsum, q, k, v, req_to_tokens, b_req_idx, b_seqlen,
+                          max_len_in_batch: int, seq_block_size: int) -> None:
+    # ENTRY:115-122
+    _req(mid_o.is_contiguous(), "mid_o.is_contiguous()")
+    _req(mid_o_logexpsum.is_contiguous(), "mid_o_logexpsum.is_contiguous()")
+    _req(q.is_contiguous(), "q.is_contiguous()")
+    _req(k.stride(2) == 1, "k.stride(2) == 1")
+    _req(v.stride(2) == 1, "v.stride(2) == 1")
+    _req(req_to_tokens.is_contiguous(), "req_to_tokens.is_contiguous()")
+    _req(b_req_idx.is_contiguous(), "b_req_idx.is_contiguous()")
+    _req(b_seqlen.is_contiguous(), "b_seqlen.is_contiguous()")
+    # ENTRY:124-131
+    for t, d, n in ((mid_o, 4, "mid_o"), (mid_o_logexpsum, 3, "mid_o_logexpsum"), (q, 3, "q"), (k, 3, "k"), (v, 3, "v"),
+                    (req_to_tokens, 2, "req_to_tokens"), (b_req_idx, 1, "b_req_idx"), (b_seqlen, 1, "b_seqlen")):
+        _req(t.dim() == d, "%s.dim() == %d" % (n, d))
+        _req(t.is_cuda, "%s on the GPU" % n)
+    # ENTRY:133-140 (bfloat16 accepted in addition to half)
+    _req(mid_o.dtype == torch.float32, "mid_o float32")
+    _req(mid_o_logexpsum.dtype == torch.float32, "mid_o_logexpsum float32")
+    _req(q.dtype in (torch.float16, torch.bfloat16), "q half or bfloat16")
+    _req(k.dtype == q.dtype and v.dtype == q.dtype, "k, v dtype == q dtype")
+    _req(req_to_tokens.dtype == torch.int32, "req_to_tokens int32")
+    _req(b_req_idx.dtype == torch.int32, "b_req_idx int32")
+    _req(b_seqlen.dtype == torch.int32, "b_seqlen int32")
+    # shapes are inferred from mid_o as in ENTRY:155-160; make the implied relations explicit
+    B, Hq, D = mid_o.size(1), mid_o.size(2), mid_o.size(3)
+    _req(tuple(q.shape) == (B, Hq, D), "q.shape == mid_o.shape[1:]")
+    _req(tuple(mid_o_logexpsum.shape) == tuple(mid_o.shape[:3]), "mid_o_logexpsum.shape == mid_o.shape[:3]")
+    _req(k.size(1) == v.size(1) and k.size(2) == D and v.size(2) == D, "k/v head shapes")
+    _req(b_req_idx.size(0) == B and b_seqlen.size(0) == B, "b_req_idx/b_seqlen length == batch")
+    _req(seq_block_size >= 1, "seq_block_size >= 1")
+    a = _lib.DecodeStage1Args()
+    a.mid_o, a.mid_o_logexpsum = mid_o.data_ptr(), mid_o_logexpsum.data_ptr()
+    a.q, a.k, a.v = q.data_ptr(), k.data_ptr(), v.data_ptr()
+    a.k_stride_0, a.k_stride_1 = k.stride(0), k.stride(1)
+    a.v_stride_0, a.v_stride_1 = v.stride(0), v.stride(1)
+    a.sm_scale = 1.0 / math.sqrt(q.size(2))  # ENTRY:142
+    a.dtype = _DT[q.dtype]
+    a.req_to_tokens, a.b_req_idx, a.b_seqlen = req_to_tokens.data_ptr(), b_req_idx.data_ptr(), b_seqlen.data_ptr()
+    a.batch, a.num_q_heads, a.num_kv_heads = B, Hq, k.size(1)
+    a.num_blocks, a.head_dim, a.max_seq_len = mid_o.size(0), D, req_to_tokens.size(1)
+    a.seq_block_size, a.max_len_in_batch = int(seq_block_size), int(max_len_in_batch)
+    _lib.check(_lib.load().lsattn_decode_stage1(C.byref(a), _stream()), "lsattn_decode_stage1")
+
+
+@torch.inference_mode()
+def flash_decoding_stage2(o, out_logexpsum, b_seqlen, mid_o, mid_o_logexpsum, block_seq: int) -> None:
+    # ENTRY:174-190
+    for t, d, n in ((o, 3, "o"), (out_logexpsum, 2, "out_logexpsum"), (b_seqlen, 1, "b_seqlen"), (mid_o, 4, "mid_o"),
+                    (mid_o_logexpsum, 3, "mid_o_logexpsum")):
+        _req(t.is_contiguous(), "%s.is_contiguous()" % n)
+        _req(t.dim() == d, "%s.dim() == %d" % (n, d))
+        _req(t.is_cuda, "%s on the GPU" % n)
+    _req(o.dtype in (torch.float16, torch.float32, torch.bfloat16), "o half, bfloat16 or float")
+    _req(out_logexpsum.dtype == torch.float32, "out_logexpsum float32")
+    _req(b_seqlen.dtype == torch.int32, "b_seqlen int32")
+    _req(mid_o.dtype == torch.float32, "mid_o float32")
+    _req(mid_o_logexpsum.dtype == torch.float32, "mid_o_logexpsum float32")
+    B, H, D = mid_o.size(1), mid_o.size(2), mid_o.size(3)
+    _req(tuple(o.shape) == (B, H, D), "o.shape == mid_o.shape[1:]")
+    _req(tuple(out_logexpsum.shape) == (B, H), "out_logexpsum.shape == [batch, heads]")
+    _req(tuple(mid_o_logexpsum.shape) == tuple(mid_o.shape[:3]), "mid_o_logexpsum.shape == mid_o.shape[:3]")
+    _req(b_seqlen.size(0) == B, "b_seqlen length == batch")
+    _req(block_seq >= 1, "block_seq >= 1")
+    a = _lib.DecodeStage2Args()
+    a.o, a.o_dtype, a.out_logexpsum, a.b_seqlen = o.data_ptr(), _DT[o.dtype], out_logexpsum.data_ptr(), b_seqlen.data_ptr()
+    a.mid_o, a.mid_o_logexpsum = mid_o.data_ptr(), mid_o_logexpsum.data_ptr()
+    a.batch, a.num_heads, a.num_seq_blocks, a.head_dim, a.block_seq = B, H, mid_o.size(0), D, int(block_seq)
+    _lib.check(_lib.load().lsattn_decode_stage2(C.byref(a), _stream()), "lsattn_decode_stage2")
+
+
+def hello_world() -> None:
+    """Load check, as ENTRY:231-232."""
+    print("Hello world from loongserve_amd.longserve_cuda_kernels (liblsattn v%d)!" % _lib.load().lsattn_version())

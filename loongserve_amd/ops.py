@@ -1,0 +1,200 @@
+"""Operators of the attention hot path, with the reference's Python signatures.
+
+Each function validates its tensors, extracts raw device pointers / strides and calls the
+C ABI in liblsattn.so on the current PyTorch HIP stream.  Nothing here computes on the
+host and nothing falls back to PyTorch math.
+
+Reference call sites (relative to the reference tree):
+  loongserve/models/llama/layer_infer/longserve_transformer_layer_infer.py:11-14 imports
+  context_attention_fwd, longserve_flash_decode_stage1/2 and
+  longserve_token_decode_attention_flash_decoding; :146-160, :272-281, :293-308, :360-367
+  call them.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import math
+from typing import List, Optional, Sequence, Tuple
+
+import torch
+
+from . import _lib
+from ._lib import LSATTN_BF16, LSATTN_F16, LSATTN_F32
+
+_DT = {torch.float16: LSATTN_F16, torch.bfloat16: LSATTN_BF16, torch.float32: LSATTN_F32}
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _dev(t: torch.Tensor, name: str) -> None:
+    if not t.is_cuda:
+        raise ValueError("%s must live on the GPU (got %s)" % (name, t.device))
+
+
+def _i32vec(t: torch.Tensor, name: str, n: Optional[int] = None) -> None:
+    _dev(t, name)
+    if t.dtype != torch.int32 or t.dim() != 1 or not t.is_contiguous():
+        raise ValueError("%s must be a contiguous 1-D int32 tensor" % name)
+    if n is not None and t.shape[0] != n:
+        raise ValueError("%s must have %d entries" % (name, n))
+
+
+def _prefill_args(q, k, v, o, q_b_start_loc, q_b_seq_len, q_first, kv_b_start_loc, kv_b_seq_len, kv_first,
+                  peers: int, max_q_len: int, sm_scale: Optional[float]) -> _lib.PrefillArgs:
+    for t, n in ((q, "q"), (k, "k"), (v, "v"), (o, "o")):
+        _dev(t, n)
+        if t.dim() != 3:
+            raise ValueError("%s must be [tokens, heads, head_dim]" % n)
+        if t.stride(2) != 1:
+            raise ValueError("%s must be contiguous in head_dim" % n)
+    Lq, Lk, Lv = q.shape[-1], k.shape[-1], v.shape[-1]
+    # RING:248-250
+    assert Lq == Lk and Lk == Lv
+    assert Lk in {16, 32, 64, 128}
+    if q.dtype not in (torch.float16, torch.bfloat16) or k.dtype != q.dtype or v.dtype != q.dtype:
+        raise ValueError("q, k, v must share dtype float16 or bfloat16")
+    if k.shape[1] != v.shape[1] or q.shape[1] % k.shape[1] != 0:
+        raise ValueError("bad head counts: Hq=%d Hkv=%d" % (q.shape[1], k.shape[1]))
+    if o.shape != q.shape:
+        raise ValueError("o must have the shape of q")
+    B = q_b_seq_len.shape[0]
+    for t, n in ((q_b_start_loc, "q_b_start_loc"), (q_b_seq_len, "q_b_seq_len"), (q_first, "q_first_token_global_idx"),
+                 (kv_b_start_loc, "kv_b_start_loc"), (kv_b_seq_len, "kv_b_seq_len"), (kv_first, "kv_first_token_global_idx")):
+        _i32vec(t, n, B)
+    a = _lib.PrefillArgs()
+    a.q, a.k, a.v = q.data_ptr(), k.data_ptr(), v.data_ptr()
+    a.q_stride_t, a.q_stride_h = q.stride(0), q.stride(1)
+    a.k_stride_t, a.k_stride_h = k.stride(0), k.stride(1)
+    a.v_stride_t, a.v_stride_h = v.stride(0), v.stride(1)
+    a.q_b_start_loc, a.q_b_seq_len, a.q_first_token_global_idx = q_b_start_loc.data_ptr(), q_b_seq_len.data_ptr(), q_first.data_ptr()
+    a.kv_b_start_loc, a.kv_b_seq_len, a.kv_first_token_global_idx = kv_b_start_loc.data_ptr(), kv_b_seq_len.data_ptr(), kv_first.data_ptr()
+    a.batch, a.num_q_heads, a.num_kv_heads, a.head_dim = B, q.shape[1], k.shape[1], Lq
+    a.dtype = _DT[q.dtype]
+    a.sp_peers = int(peers)
+    a.max_q_len = int(max_q_len)
+    a.sm_scale = (1.0 / (Lq ** 0.5)) if sm_scale is None else float(sm_scale)  # RING:252
+    a.o = o.data_ptr()
+    a.o_stride_t, a.o_stride_h = o.stride(0), o.stride(1)
+    a.o_dtype = _DT[o.dtype]
+    return a
+
+
+@torch.inference_mode()
+def context_attention_fwd(q, k, v, o, q_b_start_loc, q_b_seq_len, q_first_token_global_idx,
+                          kv_b_start_loc, kv_b_seq_len, kv_first_token_global_idx,
+                          logical_sp_peers_num: int, max_q_b_seq_len: int, m, l) -> None:
+    """One ring-attention step folded in place into (o, m, l); signature of RING:191-206.
+
+    Call it repeatedly with the same local q/o/m/l and a different kv chunk each time.
+    Start from m = -inf, l = 0 (o need not be zeroed).  After k calls o is the
+    normalised attention output over all keys seen and ln2*(m + log2 l) their LSE.
+    """
+    a = _prefill_args(q, k, v, o, q_b_start_loc, q_b_seq_len, q_first_token_global_idx, kv_b_start_loc,
+                      kv_b_seq_len, kv_first_token_global_idx, logical_sp_peers_num, max_q_b_seq_len, None)
+    if o.dtype != q.dtype:
+        raise ValueError("o must have the dtype of q")
+    for t, n in ((m, "m"), (l, "l")):
+        _dev(t, n)
+        if t.dtype != torch.float32 or t.dim() != 2 or tuple(t.shape) != (q.shape[0], q.shape[1]):
+            raise ValueError("%s must be float32 [tokens, q_heads]" % n)
+    if m.stride() != l.stride():
+        raise ValueError("m and l must share strides")
+    a.m, a.l = m.data_ptr(), l.data_ptr()
+    a.ml_stride_t, a.ml_stride_h = m.stride(0), m.stride(1)
+    _lib.check(_lib.load().lsattn_prefill_step_merge(C.byref(a), _stream()), "lsattn_prefill_step_merge")
+
+
+@torch.inference_mode()
+def prefill_attention_step(q, k, v, q_b_start_loc, q_b_seq_len, q_first_token_global_idx,
+                           kv_b_start_loc, kv_b_seq_len, kv_first_token_global_idx,
+                           logical_sp_peers_num: int, max_q_b_seq_len: int,
+                           out: Optional[torch.Tensor] = None, lse: Optional[torch.Tensor] = None,
+                           sm_scale: Optional[float] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+    """One step as a mergeable partial: (O fp32 [Tq,Hq,D] normalised, LSE fp32 [Tq,Hq]).
+
+    Same inputs as context_attention_fwd; rows that see no key get O = 0, LSE = -inf.
+    """
+    if out is None:
+        out = torch.empty(q.shape, dtype=torch.float32, device=q.device)
+    if lse is None:
+        lse = torch.empty(q.shape[:2], dtype=torch.float32, device=q.device)
+    if out.dtype != torch.float32 or lse.dtype != torch.float32 or not lse.is_contiguous():
+        raise ValueError("out and lse must be float32, lse contiguous")
+    a = _prefill_args(q, k, v, out, q_b_start_loc, q_b_seq_len, q_first_token_global_idx, kv_b_start_loc,
+                      kv_b_seq_len, kv_first_token_global_idx, logical_sp_peers_num, max_q_b_seq_len, sm_scale)
+    a.lse = lse.data_ptr()
+    _lib.check(_lib.load().lsattn_prefill_step(C.byref(a), _stream()), "lsattn_prefill_step")
+    return out, lse
+
+
+@torch.inference_mode()
+def lse_merge(parts: Sequence[Tuple[torch.Tensor, torch.Tensor]], out: Optional[torch.Tensor] = None,
+              lse: Optional[torch.Tensor] = None, out_dtype: torch.dtype = torch.float32):
+    """Merge partials [(O_i fp32 [..., D], LSE_i [...])] over disjoint key sets -> (O, LSE)."""
+    n = len(parts)
+    if not 1 <= n <= _lib.LSATTN_MAX_PARTS:
+        raise ValueError("1..%d partials" % _lib.LSATTN_MAX_PARTS)
+    o0, l0 = parts[0]
+    a = _lib.MergeArgs()
+    for i, (oi, li) in enumerate(parts):
+        _dev(oi, "partial O")
+        if oi.dtype != torch.float32 or li.dtype != torch.float32 or not oi.is_contiguous() or not li.is_contiguous():
+            raise ValueError("partials must be contiguous float32")
+        if oi.shape != o0.shape or li.shape != l0.shape or oi.shape[:-1] != li.shape:
+            raise ValueError("partials must share shapes")
+        a.o_parts[i] = oi.data_ptr()
+        a.lse_parts[i] = li.data_ptr()
+    if out is None:
+        out = torch.empty(o0.shape, dtype=out_dtype, device=o0.device)
+    if lse is None:
+        lse = torch.empty(l0.shape, dtype=torch.float32, device=o0.device)
+    if not out.is_contiguous() or not lse.is_contiguous() or out.shape != o0.shape or lse.dtype != torch.float32:
+        raise ValueError("bad output tensors")
+    a.n_parts, a.head_dim, a.rows = n, o0.shape[-1], l0.numel()
+    a.o, a.o_dtype, a.lse = out.data_ptr(), _DT[out.dtype], lse.data_ptr()
+    _lib.check(_lib.load().lsattn_lse_merge(C.byref(a), _stream()), "lsattn_lse_merge")
+    return out, lse
+
+
+@torch.inference_mode()
+def kv_scatter(src: torch.Tensor, dest_index: torch.Tensor, pool: torch.Tensor) -> None:
+    """pool[dest_index[i]] = src[i] (bit-exact row scatter into the token-indexed pool).
+
+    Semantics of destindex_copy_kv
+    (loongserve/common/basemodel/triton_kernel/destindex_copy_kv.py:31-51).
+    """
+    _dev(src, "src"); _dev(pool, "pool"); _i32vec(dest_index, "dest_index", src.shape[0])
+    if src.dtype != pool.dtype or src.shape[1:] != pool.shape[1:]:
+        raise ValueError("src and pool rows must match")
+    if not src[0].is_contiguous() or not pool[0].is_contiguous():
+        raise ValueError("rows must be contiguous")
+    row_bytes = src[0].numel() * src.element_size()
+    rc = _lib.load().lsattn_kv_scatter(src.data_ptr(), src.stride(0) * src.element_size(), pool.data_ptr(),
+                                       pool.stride(0) * pool.element_size(), dest_index.data_ptr(),
+                                       src.shape[0], row_bytes, _stream())
+    _lib.check(rc, "lsattn_kv_scatter")
+
+
+@torch.inference_mode()
+def init_req_to_token_indexes(req_to_token_indexs, b_req_idx, b_seq_len, alloc_mem_index,
+                              b_start_loc: Optional[torch.Tensor] = None, max_len_in_batch: Optional[int] = None) -> None:
+    """req_to_token_indexs[req_b, 0:len_b] = alloc_mem_index[start_b : start_b+len_b] on the device.
+
+    Signature of loongserve/common/infer_utils.py:1 plus two optional arguments that avoid
+    a host round trip (packed start offsets and the longest length)."""
+    _dev(req_to_token_indexs, "req_to_token_indexs")
+    if req_to_token_indexs.dtype != torch.int32 or not req_to_token_indexs.is_contiguous():
+        raise ValueError("req_to_token_indexs must be contiguous int32")
+    B = b_req_idx.shape[0]
+    _i32vec(b_req_idx, "b_req_idx", B); _i32vec(b_seq_len, "b_seq_len", B); _i32vec(alloc_mem_index, "alloc_mem_index")
+    if b_start_loc is None:
+        b_start_loc = (torch.cumsum(b_seq_len, 0, dtype=torch.int32) - b_seq_len).to(torch.int32)
+    if max_len_in_batch is None:
+        max_len_in_batch = int(b_seq_len.max().item()) if B else 0
+    _i32vec(b_start_loc, "b_start_loc", B)
+    rc = _lib.load().lsattn_register_tokens(req_to_token_indexs.data_ptr(), req_to_token_indexs.shape[1],
+                                            b_req_idx.data_ptr(), b_start_loc.data_ptr(), b_seq_len.data_ptr(),
+                                            alloc_mem_index.data_ptr(), B, max_len_in_batch, _stream())
+    _lib.check(rc, "lsattn_register_tokens")

@@ -1,0 +1,96 @@
+"""CPU-only checks of the drop-in boundary: the C-ABI library loads and exports every
+symbol include/lsattn.h declares, and argument validation rejects bad input without
+touching a GPU."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "lsattn.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(lsattn_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from loongserve_amd import _lib
+    lib = _lib.load()
+    names = _declared_symbols()
+    assert len(names) >= 9
+    assert set(names) == set(_lib.EXPORTS), (names, sorted(_lib.EXPORTS))
+    for n in names:
+        assert getattr(lib, n) is not None
+    assert lib.lsattn_version() >= 1
+    assert lib.lsattn_strerror(0) == b"ok"
+    assert b"invalid" in lib.lsattn_strerror(-1)
+
+
+def test_struct_layout_matches_header():
+    # compile a tiny C program against the header and compare sizeof / offsetof with ctypes
+    import subprocess
+    import tempfile
+    from loongserve_amd import _lib
+    src = r'''
+#include <stdio.h>
+#include <stddef.h>
+#include "lsattn.h"
+int main(void) {
+  printf("%zu %zu %zu %zu\n", sizeof(lsattn_prefill_args), sizeof(lsattn_merge_args),
+         sizeof(lsattn_decode_stage1_args), sizeof(lsattn_decode_stage2_args));
+  printf("%zu %zu %zu %zu\n", offsetof(lsattn_prefill_args, sm_scale), offsetof(lsattn_prefill_args, ml_stride_h),
+         offsetof(lsattn_decode_stage1_args, req_to_tokens), offsetof(lsattn_decode_stage2_args, block_seq));
+  return 0;
+}'''
+    with tempfile.TemporaryDirectory() as d:
+        c = os.path.join(d, "t.c")
+        open(c, "w").write(src)
+        exe = os.path.join(d, "t")
+        subprocess.check_call(["gcc", "-std=c99", "-I", os.path.join(ROOT, "include"), c, "-o", exe])
+        out = subprocess.check_output([exe]).decode().split()
+    sizes = [int(x) for x in out[:4]]
+    offs = [int(x) for x in out[4:]]
+    assert sizes == [C.sizeof(_lib.PrefillArgs), C.sizeof(_lib.MergeArgs), C.sizeof(_lib.DecodeStage1Args),
+                     C.sizeof(_lib.DecodeStage2Args)]
+    assert offs == [_lib.PrefillArgs.sm_scale.offset, _lib.PrefillArgs.ml_stride_h.offset,
+                    _lib.DecodeStage1Args.req_to_tokens.offset, _lib.DecodeStage2Args.block_seq.offset]
+
+
+def test_validation_rejects_bad_arguments_without_gpu():
+    from loongserve_amd import _lib
+    lib = _lib.load()
+    a = _lib.PrefillArgs()  # all null
+    assert lib.lsattn_prefill_step(C.byref(a), None) == -1
+    assert lib.lsattn_prefill_step(None, None) == -1
+    d1 = _lib.DecodeStage1Args()
+    assert lib.lsattn_decode_stage1(C.byref(d1), None) == -1
+    d2 = _lib.DecodeStage2Args()
+    assert lib.lsattn_decode_stage2(C.byref(d2), None) == -1
+    m = _lib.MergeArgs()
+    assert lib.lsattn_lse_merge(C.byref(m), None) == -1
+    assert lib.lsattn_kv_scatter(None, 0, None, 0, None, 0, 0, None) == -1
+    # unsupported head_dim is reported as such (pointers are fake but never dereferenced)
+    fake = 0x1000
+    for f in ("q", "k", "v", "o", "lse", "q_b_start_loc", "q_b_seq_len", "q_first_token_global_idx", "kv_b_start_loc",
+              "kv_b_seq_len", "kv_first_token_global_idx"):
+        setattr(a, f, fake)
+    a.batch, a.num_q_heads, a.num_kv_heads, a.head_dim, a.sp_peers, a.max_q_len = 1, 4, 2, 64, 1, 8
+    a.o_dtype = _lib.LSATTN_F32
+    assert lib.lsattn_prefill_step(C.byref(a), None) == -2
+    a.head_dim, a.num_kv_heads = 128, 3
+    assert lib.lsattn_prefill_step(C.byref(a), None) == -1
+
+
+def test_python_wrappers_reject_cpu_tensors():
+    import torch
+    import loongserve_amd as lsa
+    q = torch.zeros(4, 2, 128, dtype=torch.float16)
+    i = torch.zeros(1, dtype=torch.int32)
+    with pytest.raises(ValueError):
+        lsa.prefill_attention_step(q, q, q, i, i, i, i, i, i, 1, 4, out=torch.zeros(4, 2, 128), lse=torch.zeros(4, 2))
+    with pytest.raises(ValueError):
+        lsa.longserve_cuda_kernels.flash_decoding_stage1(torch.zeros(1, 1, 2, 128), torch.zeros(1, 1, 2), q[:1], q, q,
+                                                         torch.zeros(1, 4, dtype=torch.int32), i, i, 4, 4)

@@ -1,0 +1,115 @@
+"""GPU parity of token-indexed flash decoding against the CPU oracle (through the C ABI)."""
+import math
+
+import pytest
+import torch
+
+from oracle import attn_oracle as orc
+from tests.helpers import assert_lse_close, assert_o_close, decode_case
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("Hq,Hkv,BS", [(32, 8, 256), (4, 4, 64), (16, 8, 16), (10, 5, 128), (12, 4, 256), (8, 1, 32)])
+def test_stage1_stage2_vs_oracle(lsa, dtype, Hq, Hkv, BS):
+    print("case", dtype, Hq, Hkv, BS, flush=True)
+    B, D = 5, 128
+    lens = [700, 1, 256, 33, 1025]
+    q, kv, table, b_req, b_len = decode_case(100, B, Hq, Hkv, D, lens, 3000, dtype)
+    k, v = kv[:, :Hkv], kv[:, Hkv:]
+    nblk = (max(lens) + BS - 1) // BS
+    mid_o = torch.full((nblk, B, Hq, D), float("nan"))
+    mid_l = torch.full((nblk, B, Hq), float("nan"))
+    orc.decode_stage1(q, k, v, table, b_req, b_len, max(lens), mid_o, mid_l, BS)
+    kvd = kv.to(DEV)
+    mo_d = torch.full((nblk, B, Hq, D), float("nan"), device=DEV)
+    ml_d = torch.full((nblk, B, Hq), float("nan"), device=DEV)
+    lsa.longserve_flash_decode_stage1(q.to(DEV), kvd[:, :Hkv], kvd[:, Hkv:], table.to(DEV), b_req.to(DEV),
+                                      b_len.to(DEV), max(lens), mo_d, ml_d, BS)
+    torch.cuda.synchronize()
+    # blocks past a request's length are left untouched, like the reference
+    written = ~torch.isnan(mid_l)
+    assert torch.equal(torch.isnan(ml_d.cpu()), ~written)
+    mo_c, ml_c = mo_d.cpu(), ml_d.cpu()
+    assert_o_close(torch.where(written[..., None], mo_c, torch.zeros(())), torch.where(written[..., None], mid_o, torch.zeros(())),
+                   "mid_o")
+    assert_lse_close(ml_c[written], mid_l[written], "mid_lse")
+    for odt in (torch.float32, dtype):
+        o_d = torch.empty(B, Hq, D, dtype=odt, device=DEV)
+        l_d = torch.empty(B, Hq, device=DEV)
+        lsa.longserve_flash_decode_stage2(mo_d, ml_d, b_len.to(DEV), o_d, l_d, BS)
+        torch.cuda.synchronize()
+        o_ref, l_ref = orc.decode_full(q, k, v, table, b_req, b_len)
+        if odt == torch.bfloat16:
+            assert_o_close(o_d, o_ref, "o bf16 out", max_abs=4e-3, rel=4e-3)  # 8-bit mantissa output
+        else:
+            assert_o_close(o_d, o_ref, "o")
+        assert_lse_close(l_d, l_ref, "lse")
+
+
+def test_gather_indices_bit_exact(lsa):
+    # q = 0 and V[slot] = ordinal code of the slot: the set of gathered slots is read back from O*len
+    B, H, D = 3, 2, 128
+    lens = [37, 300, 1000]
+    q, kv, table, b_req, b_len = decode_case(200, B, H, H, D, lens, 1500)
+    q.zero_()
+    kv[:, H:, :] = (torch.arange(1500, dtype=torch.float32) % 2048)[:, None, None].to(torch.float16)
+    kv[:, H:, 1] = 1.0
+    kvd = kv.to(DEV)
+    BS = 256
+    nblk = (max(lens) + BS - 1) // BS
+    mo = torch.zeros(nblk, B, H, D, device=DEV)
+    ml = torch.zeros(nblk, B, H, device=DEV)
+    o, lse = lsa.longserve_token_decode_attention_flash_decoding(q.to(DEV), table.to(DEV), b_req.to(DEV), b_len.to(DEV),
+                                                                 mo, ml, B, max(lens), H, D, kvd[:, :H], kvd[:, H:], BS)
+    torch.cuda.synchronize()
+    assert o.dtype == torch.float32
+    for b in range(B):
+        slots = table[int(b_req[b]), :lens[b]].long()
+        want = float(kv[slots, H, 0].float().sum())
+        got = float(o[b, 0, 0]) * lens[b]
+        assert abs(got - want) <= 1e-4 * max(want, 1.0) + 0.5, (got, want)
+        assert abs(float(o[b, 1, 1]) - 1.0) < 1e-6
+        assert abs(float(lse[b, 0]) - math.log(lens[b])) < 1e-5
+
+
+def test_multi_instance_decode_with_empty_peer(lsa):
+    # each request's KV split over 3 instances; one peer holds nothing for one request
+    from loongserve_amd.simulate import DecodeInstance, multi_instance_decode
+    B, Hq, Hkv, D = 4, 8, 2, 128
+    lens = [900, 64, 333, 2000]
+    q, kv, table, b_req, b_len = decode_case(300, B, Hq, Hkv, D, lens, 4000)
+    o_ref, l_ref = orc.decode_full(q, kv[:, :Hkv], kv[:, Hkv:], table, b_req, b_len)
+    cuts = [[300, 600], [0, 64], [111, 111], [700, 1300]]  # ranges: master [0,c0), peer1 [c0,c1), peer2 [c1,len)
+    kvd = kv.to(DEV)
+    insts = []
+    for r in range(3):
+        t = torch.full_like(table, orc.INT32_PAD)
+        ln = []
+        for b in range(B):
+            lo = [0, cuts[b][0], cuts[b][1]][r]
+            hi = [cuts[b][0], cuts[b][1], lens[b]][r]
+            t[int(b_req[b]), :hi - lo] = table[int(b_req[b]), lo:hi]
+            ln.append(hi - lo)
+        insts.append(DecodeInstance(kvd, t.to(DEV), b_req.to(DEV), torch.tensor(ln, dtype=torch.int32, device=DEV), max(ln)))
+    o, lse = multi_instance_decode(q.to(DEV), insts, Hkv)
+    torch.cuda.synchronize()
+    assert o.dtype == torch.float16
+    assert_o_close(o, o_ref, "multi-instance o")
+    assert_lse_close(lse, l_ref, "multi-instance lse")
+
+
+def test_stage2_empty_request_defined(lsa):
+    B, H, D = 2, 4, 128
+    mo = torch.randn(3, B, H, D, device=DEV)
+    ml = torch.randn(3, B, H, device=DEV)
+    o = torch.full((B, H, D), 7.0, device=DEV)
+    l = torch.full((B, H), 7.0, device=DEV)
+    lsa.longserve_flash_decode_stage2(mo, ml, torch.tensor([0, 3], dtype=torch.int32, device=DEV), o, l, 1)
+    torch.cuda.synchronize()
+    assert torch.all(o[0] == 0) and torch.all(torch.isinf(l[0]) & (l[0] < 0))
+    o_ref, l_ref = orc.lse_merge([(mo[i, 1].cpu(), ml[i, 1].cpu()) for i in range(3)])
+    assert_o_close(o[1], o_ref, "o", max_abs=1e-5, rel=1e-5)
+    assert_lse_close(l[1], l_ref, "lse", rel=1e-5)

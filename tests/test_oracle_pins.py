@@ -1,0 +1,295 @@
+"""Pins for the CPU oracle (oracle/attn_oracle.py).
+
+The reference holds no golden vectors for this path and its only prefill self-test is
+stale, so every oracle function is checked here against something it was NOT written
+from: a library routine, a brute-force float64 loop, a closed-form special case or an
+algebraic invariant.  A dropped term, a wrong sign, a transposed operand or an off-by-one
+in the mask fails at least one of these.
+"""
+import math
+
+import pytest
+import torch
+
+from oracle import attn_oracle as orc
+
+
+def _meta(lens, firsts=None):
+    lens = torch.tensor(lens, dtype=torch.int32)
+    start = (torch.cumsum(lens, 0) - lens).to(torch.int32)
+    firsts = torch.zeros_like(lens) if firsts is None else torch.tensor(firsts, dtype=torch.int32)
+    return start, lens, firsts
+
+
+def _rand(shape, seed, dtype=torch.float16):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g) * 0.5).to(dtype)
+
+
+def brute_force_step(q, k, v, qs, ql, qf, ks, kl, kf, P):
+    """float64 loops, written from the definition: key n visible to row m iff
+    kf + n*P <= qf + m*P; softmax over visible keys of q.k/sqrt(D)."""
+    Tq, Hq, D = q.shape
+    Hkv = k.shape[1]
+    O = [[[0.0] * D for _ in range(Hq)] for _ in range(Tq)]
+    LSE = [[-math.inf] * Hq for _ in range(Tq)]
+    for b in range(len(ql)):
+        for m in range(int(ql[b])):
+            for h in range(Hq):
+                hk = h // (Hq // Hkv)
+                sc = []
+                for n in range(int(kl[b])):
+                    if int(kf[b]) + n * P <= int(qf[b]) + m * P:
+                        dot = sum(float(q[int(qs[b]) + m, h, d]) * float(k[int(ks[b]) + n, hk, d]) for d in range(D))
+                        sc.append((n, dot / math.sqrt(D)))
+                if not sc:
+                    continue
+                mx = max(s for _, s in sc)
+                den = sum(math.exp(s - mx) for _, s in sc)
+                LSE[int(qs[b]) + m][h] = mx + math.log(den)
+                for n, s in sc:
+                    w = math.exp(s - mx) / den
+                    for d in range(D):
+                        O[int(qs[b]) + m][h][d] += w * float(v[int(ks[b]) + n, hk, d])
+    return torch.tensor(O, dtype=torch.float64), torch.tensor(LSE, dtype=torch.float64)
+
+
+@pytest.mark.parametrize("P,qf,kf", [(1, [0, 0], [0, 0]), (1, [7, 3], [2, 0]), (3, [1, 2], [2, 0]), (4, [0, 3], [3, 1])])
+def test_attn_step_vs_brute_force(P, qf, kf):
+    Hq, Hkv, D = 4, 2, 8
+    qs, ql, qf_t = _meta([5, 3], qf)
+    ks, kl, kf_t = _meta([7, 4], kf)
+    q, k, v = _rand((8, Hq, D), 1), _rand((11, Hkv, D), 2), _rand((11, Hkv, D), 3)
+    O, LSE = orc.attn_step(q, k, v, qs, ql, qf_t, ks, kl, kf_t, P, dtype=torch.float64)
+    Ob, Lb = brute_force_step(q, k, v, qs, ql, qf_t, ks, kl, kf_t, P)
+    assert torch.allclose(O, Ob, atol=1e-12)
+    assert torch.equal(torch.isinf(LSE), torch.isinf(Lb))
+    fin = ~torch.isinf(Lb)
+    assert torch.allclose(LSE[fin], Lb[fin], atol=1e-12)
+    # rows that see nothing: O = 0, LSE = -inf
+    assert torch.all(O[~fin] == 0)
+
+
+def test_attn_step_vs_library_sdpa_causal():
+    T, H, D = 193, 6, 64
+    q, k, v = _rand((T, H, D), 4), _rand((T, 2, D), 5), _rand((T, 2, D), 6)
+    s, l, f = _meta([T])
+    O, LSE = orc.attn_step(q, k, v, s, l, f, s, l, f, 1)
+    kk = k.float().repeat_interleave(3, dim=1).permute(1, 0, 2)
+    vv = v.float().repeat_interleave(3, dim=1).permute(1, 0, 2)
+    ref = torch.nn.functional.scaled_dot_product_attention(q.float().permute(1, 0, 2)[None], kk[None], vv[None],
+                                                           is_causal=True)[0].permute(1, 0, 2)
+    assert torch.allclose(O, ref, atol=2e-6, rtol=1e-5)
+    sc = torch.einsum("thd,shd->hts", q.float(), kk.permute(1, 0, 2)) / math.sqrt(D)
+    sc = sc.masked_fill(torch.triu(torch.ones(T, T, dtype=torch.bool), 1), float("-inf"))
+    assert torch.allclose(LSE, torch.logsumexp(sc, -1).permute(1, 0), atol=1e-5)
+
+
+def test_special_cases_single_key_zero_q_constant_v():
+    H, D = 2, 16
+    s1, l1, f1 = _meta([1])
+    q, k, v = _rand((1, H, D), 7), _rand((1, H, D), 8), _rand((1, H, D), 9)
+    O, LSE = orc.attn_step(q, k, v, s1, l1, f1, s1, l1, f1, 1)
+    assert torch.allclose(O, v.float(), atol=1e-7)                      # single visible key: O = V
+    assert torch.allclose(LSE[0], (q.float() * k.float()).sum(-1)[0] / math.sqrt(D), atol=1e-6)
+    T = 9
+    s, l, f = _meta([T])
+    k, v = _rand((T, H, D), 10), _rand((T, H, D), 11)
+    O, LSE = orc.attn_step(torch.zeros(T, H, D, dtype=torch.float16), k, v, s, l, f, s, l, f, 1)
+    cm = torch.cumsum(v.float(), 0) / torch.arange(1, T + 1)[:, None, None]
+    assert torch.allclose(O, cm, atol=1e-6)                             # q = 0: running mean of V
+    assert torch.allclose(LSE, torch.log(torch.arange(1, T + 1).float())[:, None].expand(T, H), atol=1e-6)
+    vc = torch.full((T, H, D), 0.25, dtype=torch.float16)
+    O, _ = orc.attn_step(_rand((T, H, D), 12), k, vc, s, l, f, s, l, f, 1)
+    assert torch.allclose(O, vc.float(), atol=1e-6)                     # constant V: O = V
+
+
+def _shard_contiguous(k, v, lens, nshard, rng):
+    """Random contiguous partition of each sequence over nshard nodes (the recipe of the
+    reference's own self-test, ring_context_flashattention_nopad.py:354-371)."""
+    B = len(lens)
+    starts = [0]
+    for n in lens:
+        starts.append(starts[-1] + n)
+    cuts = []
+    for b in range(B):
+        c = sorted(int(x) for x in torch.randint(0, lens[b] + 1, (nshard - 1,), generator=rng))
+        cuts.append([0] + c + [lens[b]])
+    shards = []
+    for j in range(nshard):
+        ks, vs, sl, fi = [], [], [], []
+        for b in range(B):
+            a, e = cuts[b][j], cuts[b][j + 1]
+            ks.append(k[starts[b] + a:starts[b] + e])
+            vs.append(v[starts[b] + a:starts[b] + e])
+            sl.append(e - a)
+            fi.append(a)
+        st, ln, fr = _meta(sl, fi)
+        shards.append((torch.cat(ks), torch.cat(vs), st, ln, fr))
+    return shards
+
+
+def test_ring_equals_monolithic_reference_recipe():
+    # B=2, Hq=40, Hkv=4, D=128, KV contiguously partitioned over 8 nodes: RING:324-371
+    g = torch.Generator().manual_seed(0)
+    lens = [int(x) for x in torch.randint(1, 300, (2,), generator=g)]
+    T, Hq, Hkv, D = sum(lens), 40, 4, 128
+    q, k, v = _rand((T, Hq, D), 20), _rand((T, Hkv, D), 21), _rand((T, Hkv, D), 22)
+    s, l, f = _meta(lens)
+    O_full, LSE_full = orc.attn_step(q, k, v, s, l, f, s, l, f, 1)
+    shards = _shard_contiguous(k, v, lens, 8, g)
+    parts = [orc.attn_step(q, ks, vs, s, l, f, st, ln, fr, 1) for ks, vs, st, ln, fr in shards]
+    O, LSE = orc.lse_merge(parts)
+    assert torch.allclose(O, O_full, atol=2e-6)
+    assert torch.allclose(LSE, LSE_full, atol=2e-6)
+    # step order does not matter (commutativity / associativity of the LSE merge)
+    O2, LSE2 = orc.lse_merge(parts[::-1])
+    assert torch.allclose(O2, O, atol=2e-6) and torch.allclose(LSE2, LSE, atol=2e-6)
+    # in-place (o, m, l) state of the reference operator gives the same answer
+    o = torch.zeros(T, Hq, D, dtype=torch.float32)
+    m = torch.full((T, Hq), float("-inf"))
+    ll = torch.zeros(T, Hq)
+    for ks, vs, st, ln, fr in shards:
+        orc.context_attention_fwd(q, ks, vs, o, s, l, f, st, ln, fr, 1, max(lens), m, ll)
+    assert torch.allclose(o, O_full, atol=3e-6)
+    assert torch.allclose(orc.state_lse(m, ll).float(), LSE_full, atol=1e-5)
+
+
+def test_striped_equals_contiguous():
+    T, H, D, P = 37, 2, 16, 4
+    q, k, v = _rand((T, H, D), 30), _rand((T, H, D), 31), _rand((T, H, D), 32)
+    s, l, f = _meta([T])
+    O_full, LSE_full = orc.attn_step(q, k, v, s, l, f, s, l, f, 1)
+    O = torch.zeros_like(O_full)
+    LSE = torch.zeros_like(LSE_full)
+    for r in range(P):  # rank r owns tokens r, r+P, ... (loongserve/longserve_server/io_struct.py:78-81)
+        qi = q[r::P]
+        qs_, ql_, qf_ = _meta([qi.shape[0]], [r])
+        parts = []
+        for j in range(P):
+            kj, vj = k[j::P], v[j::P]
+            ks_, kl_, kf_ = _meta([kj.shape[0]], [j])
+            parts.append(orc.attn_step(qi, kj, vj, qs_, ql_, qf_, ks_, kl_, kf_, P))
+        o_r, l_r = orc.lse_merge(parts)
+        O[r::P], LSE[r::P] = o_r, l_r
+    assert torch.allclose(O, O_full, atol=2e-6)
+    assert torch.allclose(LSE, LSE_full, atol=2e-6)
+
+
+def test_merge_with_empty_partial_is_identity():
+    O = _rand((5, 2, 8), 40, torch.float32)
+    L = _rand((5, 2), 41, torch.float32)
+    e = (torch.zeros_like(O), torch.full_like(L, float("-inf")))
+    O2, L2 = orc.lse_merge([(O, L), e])
+    assert torch.allclose(O2, O) and torch.allclose(L2, L)
+    O3, L3 = orc.lse_merge([e, e])
+    assert torch.all(O3 == 0) and torch.all(torch.isinf(L3))
+
+
+def _decode_case(seed, B, Hq, Hkv, D, lens, pool):
+    g = torch.Generator().manual_seed(seed)
+    q = _rand((B, Hq, D), seed + 1)
+    kv = _rand((pool, 2 * Hkv, D), seed + 2)
+    perm = torch.randperm(pool, generator=g).to(torch.int32)
+    max_seq = max(max(lens), 1) + 3
+    table = torch.full((B + 2, max_seq), orc.INT32_PAD, dtype=torch.int32)
+    b_req = torch.randperm(B + 2, generator=g)[:B].to(torch.int32)
+    off = 0
+    for b in range(B):
+        table[int(b_req[b]), :lens[b]] = perm[off:off + lens[b]]
+        off += lens[b]
+    return q, kv, table, b_req, torch.tensor(lens, dtype=torch.int32)
+
+
+@pytest.mark.parametrize("BS", [1, 16, 64, 256])
+def test_decode_stage1_stage2_vs_dense(BS):
+    B, Hq, Hkv, D = 3, 8, 2, 128
+    lens = [300, 1, 77]
+    q, kv, table, b_req, b_len = _decode_case(50, B, Hq, Hkv, D, lens, 500)
+    k, v = kv[:, :Hkv], kv[:, Hkv:]
+    nblk = (max(lens) + BS - 1) // BS
+    mid_o = torch.full((nblk, B, Hq, D), float("nan"))
+    mid_l = torch.full((nblk, B, Hq), float("nan"))
+    o = torch.empty(B, Hq, D)
+    lse = torch.empty(B, Hq)
+    orc.decode_stage1(q, k, v, table, b_req, b_len, max(lens), mid_o, mid_l, BS)
+    orc.decode_stage2(mid_o, mid_l, b_len, o, lse, BS)
+    # independent dense computation with torch.softmax on explicitly gathered rows
+    for b in range(B):
+        rows = table[int(b_req[b]), :lens[b]].long()
+        kk = k[rows].float().repeat_interleave(Hq // Hkv, 1)
+        vv = v[rows].float().repeat_interleave(Hq // Hkv, 1)
+        s = torch.einsum("hd,nhd->hn", q[b].float(), kk) / math.sqrt(D)
+        ref = torch.einsum("hn,nhd->hd", torch.softmax(s, -1), vv)
+        assert torch.allclose(o[b], ref, atol=2e-6)
+        assert torch.allclose(lse[b], torch.logsumexp(s, -1), atol=1e-5)
+    of, lf = orc.decode_full(q, k, v, table, b_req, b_len)
+    assert torch.allclose(of, o, atol=2e-6) and torch.allclose(lf, lse, atol=1e-5)
+
+
+def test_decode_gather_is_bit_exact_identity_code():
+    # q = 0 and V rows that encode their own slot number: O * len is the sum of the
+    # gathered slot ids, and the gathered rows themselves compare bit-for-bit
+    B, H, D = 2, 1, 128
+    lens = [5, 9]
+    q, kv, table, b_req, b_len = _decode_case(60, B, H, H, D, lens, 64)
+    q.zero_()
+    kv[:, H:, :] = torch.arange(64, dtype=torch.float16)[:, None, None]
+    k, v = kv[:, :H], kv[:, H:]
+    o, lse = orc.decode_full(q, k, v, table, b_req, b_len)
+    for b in range(B):
+        slots = table[int(b_req[b]), :lens[b]].long()
+        assert torch.equal(orc.gather_rows(v, table, int(b_req[b]), 0, lens[b]), v[slots])
+        assert abs(float(o[b, 0, 0]) * lens[b] - float(slots.sum())) < 1e-3
+        assert abs(float(lse[b, 0]) - math.log(lens[b])) < 1e-6
+
+
+def test_decode_empty_request_and_merge_trick():
+    # a peer that holds nothing for a request contributes (0, -inf); block_seq=1 stage 2 merges
+    # instance partials and split-K blocks alike (longserve_model.py:514-516, stage2.cu:30)
+    B, Hq, Hkv, D = 2, 4, 4, 128
+    lens = [40, 25]
+    q, kv, table, b_req, b_len = _decode_case(70, B, Hq, Hkv, D, lens, 100)
+    k, v = kv[:, :Hkv], kv[:, Hkv:]
+    full_o, full_l = orc.decode_full(q, k, v, table, b_req, b_len)
+    # split each request: peer holds the first part (request 1: nothing), master the rest
+    cut = [13, 0]
+    t_peer = torch.full_like(table, orc.INT32_PAD)
+    t_master = torch.full_like(table, orc.INT32_PAD)
+    for b in range(B):
+        r = int(b_req[b])
+        t_peer[r, :cut[b]] = table[r, :cut[b]]
+        t_master[r, :lens[b] - cut[b]] = table[r, cut[b]:lens[b]]
+    peer_len = torch.tensor(cut, dtype=torch.int32)
+    master_len = torch.tensor([lens[b] - cut[b] for b in range(B)], dtype=torch.int32)
+    BS, P = 16, 2
+    nblk = (int(master_len.max()) + BS - 1) // BS
+    gm = torch.full((P - 1 + nblk, B, Hq, D), float("nan"))
+    gl = torch.full((P - 1 + nblk, B, Hq), float("nan"))
+    pm = torch.empty(int(peer_len.max()) // BS + 1, B, Hq, D)
+    pl = torch.empty(int(peer_len.max()) // BS + 1, B, Hq)
+    po, plse = orc.token_decode_attention_flash_decoding(q, t_peer, b_req, peer_len, pm, pl, B, int(peer_len.max()),
+                                                         Hq, D, k, v, BS)
+    assert torch.all(po[1] == 0) and torch.all(torch.isinf(plse[1]))
+    gm[0], gl[0] = po, plse
+    orc.decode_stage1(q, k, v, t_master, b_req, master_len, int(master_len.max()), gm[P - 1:], gl[P - 1:], BS)
+    merge_len = ((P - 1) + (master_len + BS - 1) // BS).to(torch.int32)
+    o = torch.empty(B, Hq, D)
+    lse = torch.empty(B, Hq)
+    orc.decode_stage2(gm, gl, merge_len, o, lse, 1)
+    assert torch.allclose(o, full_o, atol=2e-6) and torch.allclose(lse, full_l, atol=1e-5)
+
+
+def test_kv_scatter_and_register():
+    src = _rand((6, 4, 8), 80)
+    pool = torch.zeros(10, 4, 8, dtype=torch.float16)
+    dest = torch.tensor([7, 2, 9, 0, 4, 5], dtype=torch.int32)
+    orc.kv_scatter(src, dest, pool)
+    for i in range(6):
+        assert torch.equal(pool[int(dest[i])], src[i])
+    assert torch.all(pool[[1, 3, 6, 8]] == 0)
+    table = torch.full((4, 5), orc.INT32_PAD, dtype=torch.int32)
+    orc.register_tokens(table, torch.tensor([2, 0]), torch.tensor([0, 4]), torch.tensor([4, 2]), dest)
+    assert table[2].tolist() == [7, 2, 9, 0, orc.INT32_PAD]
+    assert table[0].tolist() == [4, 5] + [orc.INT32_PAD] * 3
+    assert torch.all(table[[1, 3]] == orc.INT32_PAD)
