@@ -17,6 +17,8 @@
 //     straddle the diagonal or the end of the KV chunk;
 //   * workgroup ids are mapped so that the workgroups sharing one KV head run on one XCD
 //     (ids are dealt round-robin to the 8 XCDs) and heavy (late) query tiles start first.
+#include <type_traits>
+
 #include "common.hip.h"
 
 namespace lsattn {
@@ -42,9 +44,11 @@ struct PrefillParams {
   int64_t ml_st, ml_sh;
 };
 
-constexpr int BM = 256;  // query rows per workgroup
-constexpr int BN = 64;   // keys per tile
+constexpr int BM = 256;   // query rows per workgroup (64 per wave)
+constexpr int BN = 64;    // keys per LDS tile
+constexpr int SUB = 32;   // keys per pipeline step (one 32x32 MFMA block row)
 constexpr int NWAVE = 4;
+constexpr float kLazyRescale = 8.f;  // log2 units the running max may lag before O is rescaled
 
 template <typename T> struct Mfma;
 template <> struct Mfma<F16> {
@@ -58,8 +62,8 @@ template <> struct Mfma<BF16> {
   }
 };
 
-// The P V product always runs on the f16 MFMA: P in [0,1] keeps 11 significant bits there
-// (8 as bfloat16, which alone would cost ~1.1e-3 relative error in O).  A bfloat16 V tile is
+// The P V product always runs on the f16 MFMA: P keeps 11 significant bits there (8 as
+// bfloat16, which alone would cost ~1.1e-3 relative error in O).  A bfloat16 V tile is
 // therefore converted to f16 while it is staged into LDS; every bfloat16 value with
 // magnitude in [2^-14, 65504] is exactly representable, larger ones saturate to +-65504.
 template <typename T> __device__ __forceinline__ u32x4 to_pv_operand(const u32x4& w);
@@ -76,6 +80,8 @@ template <> __device__ __forceinline__ u32x4 to_pv_operand<BF16>(const u32x4& w)
   }
   return r;
 }
+template <typename T> struct DirectV { static constexpr bool value = true; };
+template <> struct DirectV<BF16> { static constexpr bool value = false; };
 
 // value of the same register in the other half of the wave (lane ^ 32)
 __device__ __forceinline__ float other_half(float v, int upper) {
@@ -84,15 +90,143 @@ __device__ __forceinline__ float other_half(float v, int upper) {
   return __builtin_bit_cast(float, upper ? r[0] : r[1]);
 }
 
-// physical 16-byte chunk of (row, logical chunk) inside a [64 rows][16 chunks] tile
-__device__ __forceinline__ int swz(int row, int chunk) { return row * 16 + (chunk ^ (((row & 3) << 2) | ((row >> 2) & 3))); }
+// LDS: three K tiles at [0, 48K), two V tiles at [48K, 80K); a tile is [64 rows][16 chunks of 16 bytes] and
+// the chunk index is XORed with swz_bits(row), which makes the row-wise 16-byte K reads and the
+// transposing 8-byte V reads both bank-conflict free.
+constexpr int kTileBytes = BN * 256;
+constexpr int kLdsV = 3 * kTileBytes;
+__device__ __forceinline__ int swz_bits(int row) { return ((row & 3) << 2) | ((row >> 2) & 3); }
 
 typedef __attribute__((address_space(3))) i16x4* lds_i16x4_ptr;
+typedef __attribute__((address_space(3))) void* lds_void_ptr;
+typedef const __attribute__((address_space(1))) void* global_void_ptr;
+
+__device__ __forceinline__ void wait_vmem() { __builtin_amdgcn_s_waitcnt(0x0F70); }  // vmcnt(0) only
+
+// K A-operands of one 32-key sub-tile: 8 x 16 bytes per lane
+__device__ __forceinline__ void load_k_operands(const char* ktile, int kb, const int (&koff)[8], u32x4 (&ka)[8]) {
+#pragma unroll
+  for (int t8 = 0; t8 < 8; t8++) ka[t8] = *(const u32x4*)(ktile + kb * (SUB * 256) + koff[t8]);
+}
+// S^T block row of 32 keys x 64 queries: s[qb] = K[kb*32 .. +32) Q^T
+template <typename T>
+__device__ __forceinline__ void qk_stage(const u32x4 (&ka)[8], const u32x4 (&qreg)[2][8], f32x16 (&s)[2]) {
+#pragma unroll
+  for (int i = 0; i < 16; i++) {
+    s[0][i] = 0.f;
+    s[1][i] = 0.f;
+  }
+#pragma unroll
+  for (int t8 = 0; t8 < 8; t8++) {
+    s[0] = Mfma<T>::run(ka[t8], qreg[0][t8], s[0]);
+    s[1] = Mfma<T>::run(ka[t8], qreg[1][t8], s[1]);
+  }
+}
+
+// V^T A-operands of one 32-key sub-tile through transposing LDS reads
+__device__ __forceinline__ void load_v_operands(const char* vtile, int kb, const int (&voffa)[4], const int (&voffb)[4], u32x4 (&va)[2][4]) {
+#pragma unroll
+  for (int jj = 0; jj < 2; jj++) {
+#pragma unroll
+    for (int db = 0; db < 4; db++) {
+      const char* base = vtile + kb * (SUB * 256) + jj * (16 * 256);
+      const i16x4 xa = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_ptr)(base + voffa[db]));
+      const i16x4 xb = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_ptr)(base + voffb[db]));
+      const u32x2 wa = __builtin_bit_cast(u32x2, xa), wb = __builtin_bit_cast(u32x2, xb);
+      va[jj][db] = u32x4{wa[0], wa[1], wb[0], wb[1]};
+    }
+  }
+}
+// O^T += V^T[., kb*32 .. +32) P^T
+__device__ __forceinline__ void pv_stage(const u32x4 (&va)[2][4], const u32x4 (&pk)[2][2], f32x16 (&oacc)[4][2]) {
+#pragma unroll
+  for (int jj = 0; jj < 2; jj++) {
+#pragma unroll
+    for (int db = 0; db < 4; db++) {
+      oacc[db][0] = Mfma<F16>::run(va[jj][db], pk[0][jj], oacc[db][0]);
+      oacc[db][1] = Mfma<F16>::run(va[jj][db], pk[1][jj], oacc[db][1]);
+    }
+  }
+}
+
+// Online softmax of one 32-key block row for the two query columns of this lane.  The running
+// max only moves when some lane of the wave would otherwise exceed it by 2^kLazyRescale; the
+// factor the O accumulators then owe is returned in alpha (applied by the caller after the
+// P V products that still belong to the old max).
+struct MaskInfo {
+  int64_t n0, kv_len, kf, P, qpos0, qpos1;  // sub-tile start, bounds and the two query positions
+};
+template <bool MASK>
+__device__ __forceinline__ bool softmax_stage(f32x16 (&s)[2], u32x4 (&pk)[2][2], float (&m_run)[2], float (&l_run)[2], float (&alpha)[2],
+                                              float scale_log2, int g, const MaskInfo& mi) {
+  float scaled[2];
+#pragma unroll
+  for (int qb = 0; qb < 2; qb++) {
+    if (MASK) {
+      const int64_t qpos = qb ? mi.qpos1 : mi.qpos0;
+#pragma unroll
+      for (int i = 0; i < 16; i++) {
+        const int64_t n = mi.n0 + (i >> 2) * 8 + 4 * g + (i & 3);
+        const bool vis = (mi.kf + n * mi.P <= qpos) && (n < mi.kv_len);
+        s[qb][i] = vis ? s[qb][i] : -INFINITY;
+      }
+    }
+    float mx = fmaxf(s[qb][0], s[qb][1]);
+#pragma unroll
+    for (int i = 2; i < 16; i += 2) mx = fmaxf(mx, fmaxf(s[qb][i], s[qb][i + 1]));
+    mx = fmaxf(mx, other_half(mx, g));
+    scaled[qb] = mx * scale_log2;
+  }
+  const bool grow = (scaled[0] > m_run[0] + kLazyRescale) || (scaled[1] > m_run[1] + kLazyRescale);
+  const bool any = __builtin_amdgcn_ballot_w64(grow) != 0;
+#pragma unroll
+  for (int qb = 0; qb < 2; qb++) {
+    const float m_new = any ? fmaxf(m_run[qb], scaled[qb]) : m_run[qb];
+    float m_use = m_new;
+    if (MASK) {
+      m_use = (m_new == -INFINITY) ? 0.f : m_new;
+      alpha[qb] = (m_run[qb] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m_run[qb] - m_use);
+    } else {
+      alpha[qb] = __builtin_amdgcn_exp2f(m_run[qb] - m_new);
+    }
+    m_run[qb] = m_new;
+    float pv[16];
+    float ps0 = 0.f, ps1 = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; i += 2) {
+      pv[i] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[qb][i], scale_log2, -m_use));
+      pv[i + 1] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[qb][i + 1], scale_log2, -m_use));
+      ps0 += pv[i];
+      ps1 += pv[i + 1];
+    }
+    l_run[qb] = l_run[qb] * alpha[qb] + (ps0 + ps1);
+#pragma unroll
+    for (int jj = 0; jj < 2; jj++) {
+      u32x4 w;
+#pragma unroll
+      for (int e = 0; e < 4; e++) w[e] = pack2<F16>(pv[8 * jj + 2 * e], pv[8 * jj + 2 * e + 1]);
+      pk[qb][jj] = w;
+    }
+  }
+  return any;
+}
+
+__device__ __forceinline__ void rescale_o(f32x16 (&oacc)[4][2], const float (&alpha)[2]) {
+#pragma unroll
+  for (int db = 0; db < 4; db++)
+#pragma unroll
+    for (int qb = 0; qb < 2; qb++)
+#pragma unroll
+      for (int i = 0; i < 16; i++) {
+        // volatile asm: the multiply cannot be speculated, so the caller's branch around this
+        // (rarely needed) pass over the accumulators stays a branch
+        asm volatile("v_mul_f32 %0, %1, %0" : "+v"(oacc[db][qb][i]) : "v"(alpha[qb]));
+      }
+}
 
 template <typename T, int MODE>  // MODE 0: partial (o fp32, lse)   MODE 1: in-place (o, m, l) update
 __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p) {
-  __shared__ u32x4 lds_k[2][BN * 16];
-  __shared__ u32x4 lds_v[2][BN * 16];
+  __shared__ __attribute__((aligned(1024))) char lds[5 * kTileBytes];
 
   // ---- workgroup -> (sequence, q head, query tile) ----
   const int group = p.hq / p.hkv;
@@ -118,26 +252,27 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
   const int64_t P = p.peers;
 
   const int tid = threadIdx.x;
-  const int lane = tid & 63, wave = tid >> 6;
+  const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int qc = lane & 31, g = lane >> 5;
 
-  // keys visible to the last valid row of the workgroup bound the tile loop
+  // number of keys visible to global position qpos, clamped to the chunk
+  auto visible_keys = [&](int64_t qpos) -> int64_t {
+    const int64_t dq = qpos - kf;
+    int64_t n = dq >= 0 ? dq / P + 1 : 0;
+    return n > kv_len ? kv_len : n;
+  };
   const int64_t m_hi = (m_lo + BM < q_len ? m_lo + BM : q_len) - 1;
-  int64_t n_end = 0;
-  {
-    const int64_t dq = qf + m_hi * P - kf;
-    if (dq >= 0) n_end = dq / P + 1;
-    if (n_end > kv_len) n_end = kv_len;
-  }
-  const int n_tiles = (int)((n_end + BN - 1) / BN);
+  const int nt = (int)((visible_keys(qf + m_hi * P) + BN - 1) / BN);  // LDS tiles the workgroup walks
 
-  // ---- this wave's rows ----
+  // ---- this wave's rows and its sub-tile range ----
   const int64_t m_w0 = m_lo + wave * 64;
+  const bool wave_has_rows = m_w0 < q_len;
   int64_t m_wlast = m_w0 + 63;
   if (m_wlast > q_len - 1) m_wlast = q_len - 1;
-  const int64_t qg_wlast = qf + m_wlast * P;  // largest global position in the wave (may be < row 0 if the wave is empty)
-  const int64_t qg_wfirst = qf + m_w0 * P;
-  const bool wave_has_rows = m_w0 < q_len;
+  // sub-tiles [0, ns_w) hold a key some row of the wave sees; sub-tiles [0, i_mask) are seen
+  // entirely by every row of the wave (no mask needed)
+  const int ns_w = wave_has_rows ? (int)((visible_keys(qf + m_wlast * P) + SUB - 1) / SUB) : 0;
+  const int i_mask = wave_has_rows ? (int)(visible_keys(qf + m_w0 * P) / SUB) : 0;
 
   // Q as B operands: qreg[qb][t] = Q[row qb*32+qc][16t + 8g .. +7]
   u32x4 qreg[2][8];
@@ -150,6 +285,66 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
     for (int t = 0; t < 8; t++) qreg[qb][t] = ok ? *(const u32x4*)(src + t * 32) : u32x4{0, 0, 0, 0};
   }
 
+  // ---- per-lane LDS byte offsets inside a tile ----
+  int koff[8];  // K A-operand: row qc (+32 kb), logical chunk 2*t8+g
+#pragma unroll
+  for (int t8 = 0; t8 < 8; t8++) koff[t8] = qc * 256 + (((2 * t8 + g) ^ swz_bits(qc)) << 4);
+  int voffa[4], voffb[4];  // V^T A-operand via transposing reads: keys base+4g'+(li>>2) and +8
+  {
+    const int blk16 = lane >> 4, li = lane & 15;
+    const int row_a = 4 * (blk16 >> 1) + (li >> 2);
+    const int row_b = row_a + 8;
+#pragma unroll
+    for (int db = 0; db < 4; db++) {
+      const int d_off = db * 32 + (blk16 & 1) * 16 + 4 * (li & 3);
+      voffa[db] = row_a * 256 + (((d_off >> 3) ^ swz_bits(row_a)) << 4) + (d_off & 7) * 2;
+      voffb[db] = row_b * 256 + (((d_off >> 3) ^ swz_bits(row_b)) << 4) + (d_off & 7) * 2;
+    }
+  }
+
+  // ---- global -> LDS staging: wave w owns rows [16w, 16w+16) of every tile, 4 rows per instruction ----
+  const char* kg = (const char*)p.k + (kv_start * p.k_st + (int64_t)kvh * p.k_sh) * 2;
+  const char* vg = (const char*)p.v + (kv_start * p.v_st + (int64_t)kvh * p.v_sh) * 2;
+  const int st_row = lane >> 4;                                  // row inside the group of 4
+  auto stage_src_chunk = [&](int r) { return ((lane & 15) ^ swz_bits(r)) << 4; };  // logical chunk bytes for physical slot
+  // Rows past the chunk are masked later; the row index is clamped so that the data stays finite
+  // and a tile index past the walk (harmless prefetch into a free buffer) stays in bounds.
+  const int last_row = (int)(kv_len - 1);
+  const int64_t k_row_bytes = p.k_st * 2, v_row_bytes = p.v_st * 2;
+  auto load_k_tile = [&](int t) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const int r = 16 * wave + 4 * i + st_row;
+      int n = t * BN + r;
+      n = n > last_row ? last_row : n;
+      __builtin_amdgcn_global_load_lds((global_void_ptr)(kg + n * k_row_bytes + stage_src_chunk(r)),
+                                       (lds_void_ptr)(lds + (t % 3) * kTileBytes + (16 * wave + 4 * i) * 256), 16, 0, 0);
+    }
+  };
+  u32x4 vst[4];
+  auto load_v_tile = [&](int t) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const int r = 16 * wave + 4 * i + st_row;
+      int n = t * BN + r;
+      n = n > last_row ? last_row : n;
+      const char* src = vg + n * v_row_bytes + stage_src_chunk(r);
+      if (DirectV<T>::value) {
+        __builtin_amdgcn_global_load_lds((global_void_ptr)src, (lds_void_ptr)(lds + kLdsV + (t & 1) * kTileBytes + (16 * wave + 4 * i) * 256),
+                                         16, 0, 0);
+      } else {
+        vst[i] = *(const u32x4*)src;
+      }
+    }
+  };
+  auto store_v_tile = [&](int t) {  // only for element types whose V goes through registers
+    if (!DirectV<T>::value) {
+#pragma unroll
+      for (int i = 0; i < 4; i++)
+        *(u32x4*)(lds + kLdsV + (t & 1) * kTileBytes + (16 * wave + 4 * i) * 256 + lane * 16) = to_pv_operand<T>(vst[i]);
+    }
+  };
+
   f32x16 oacc[4][2];
 #pragma unroll
   for (int db = 0; db < 4; db++)
@@ -159,141 +354,103 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
       for (int i = 0; i < 16; i++) oacc[db][qb][i] = 0.f;
   float m_run[2] = {-INFINITY, -INFINITY};
   float l_run[2] = {0.f, 0.f};
+  f32x16 s0[2], s1[2];    // S^T of even / odd sub-tiles
+  u32x4 pk0[2][2], pk1[2][2];  // P^T of even / odd sub-tiles
+  float alpha[2];
+  MaskInfo mi;
+  mi.kv_len = kv_len;
+  mi.kf = kf;
+  mi.P = P;
+  mi.qpos0 = qf + (m_w0 + qc) * P;
+  mi.qpos1 = qf + (m_w0 + 32 + qc) * P;
 
-  // ---- tile staging: thread owns 4 chunks of K and 4 of V per tile ----
-  const char* kg = (const char*)p.k + (kv_start * p.k_st + (int64_t)kvh * p.k_sh) * 2;
-  const char* vg = (const char*)p.v + (kv_start * p.v_st + (int64_t)kvh * p.v_sh) * 2;
-  u32x4 kst[4], vst[4];
-  auto load_tile = [&](int t) {
-    const int64_t n0 = (int64_t)t * BN;
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-      const int cid = i * 256 + tid;
-      const int r = cid >> 4, c = cid & 15;
-      const bool ok = n0 + r < kv_len;
-      kst[i] = ok ? *(const u32x4*)(kg + ((n0 + r) * p.k_st) * 2 + c * 16) : u32x4{0, 0, 0, 0};
-      vst[i] = ok ? *(const u32x4*)(vg + ((n0 + r) * p.v_st) * 2 + c * 16) : u32x4{0, 0, 0, 0};
+  // One pipeline step on sub-tile i: S(i+1) = K(i+1) Q^T, P(i) = softmax(S(i)), O += V(i-1) P(i-1).
+  // PAR is the parity of i: S/P of sub-tile i live in the PAR set, those of i+-1 in the other.
+  // The K operands of sub-tile i+1 were read from LDS during the previous step (ka); this step
+  // reads the V operands of sub-tile i-1 up front and the K operands of sub-tile i+2 while its
+  // P V products run, so no MFMA waits on an LDS read it has just issued.
+  // The FAST form assumes all three stages are live and sub-tile i needs no mask.  The general
+  // form runs the same three stages unconditionally and folds "stage not live" into the mask:
+  // a dead softmax sees an empty key range (P = 0, state untouched), a dead S(i+1) is never
+  // read, and a dead P V product multiplies finite LDS contents by P = 0.
+  u32x4 ka[8];
+  auto step = [&](auto par_tag, auto fast_tag, int i) {
+    constexpr int PAR = decltype(par_tag)::value;
+    constexpr bool FAST = decltype(fast_tag)::value;
+    f32x16(&s_cur)[2] = PAR ? s1 : s0;
+    f32x16(&s_nxt)[2] = PAR ? s0 : s1;
+    u32x4(&pk_cur)[2][2] = PAR ? pk1 : pk0;
+    u32x4(&pk_prv)[2][2] = PAR ? pk0 : pk1;
+    // sub-tile i-1 lives in V tile (i-1)/2, half !PAR; sub-tile i+2 in K tile (i+2)/2, half PAR
+    const char* vtile = lds + kLdsV + (((i - 1) >> 1) & 1) * kTileBytes;
+    const char* ktile2 = lds + (((i + 2) >> 1) % 3) * kTileBytes;
+    if (!FAST) {
+      // a dead stage gets a key range that lies past every chunk, so that nothing is visible
+      mi.n0 = (i >= 0 && i < ns_w) ? (int64_t)i * SUB : ((int64_t)1 << 40);
     }
+    u32x4 va[2][4];
+    load_v_operands(vtile, PAR ^ 1, voffa, voffb, va);
+    qk_stage<T>(ka, qreg, s_nxt);
+    const bool any = softmax_stage<!FAST>(s_cur, pk_cur, m_run, l_run, alpha, p.scale_log2, g, mi);
+    load_k_operands(ktile2, PAR, koff, ka);
+    pv_stage(va, pk_prv, oacc);
+    // P(i) is only consumed by the next step; pin its computation into this step so that it
+    // overlaps this step's MFMAs instead of being sunk to where the MFMA pipe has nothing to do
+    asm volatile("" ::"v"(pk_cur[0][0]), "v"(pk_cur[0][1]), "v"(pk_cur[1][0]), "v"(pk_cur[1][1]), "v"(ka[0]), "v"(ka[7]));
+    if (FAST) {
+      // issue order of the step: one MFMA, at most one LDS read, then the ~6 VALU operations the
+      // matrix pipe hides behind it; the 16 transposing V reads ride on the S^T products, the 8
+      // K reads for the next step on the P V products
+#pragma unroll
+      for (int k = 0; k < 32; k++) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);              // MFMA
+        if (k < 24) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // DS read
+        __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);              // VALU
+      }
+    }
+    if (any) rescale_o(oacc, alpha);
   };
-  auto store_tile = [&](int buf) {
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-      const int cid = i * 256 + tid;
-      const int r = cid >> 4, c = cid & 15;
-      lds_k[buf][swz(r, c)] = kst[i];
-      lds_v[buf][swz(r, c)] = to_pv_operand<T>(vst[i]);
-    }
-  };
-
-  if (n_tiles > 0) {
-    load_tile(0);
-    store_tile(0);
-  }
-  __syncthreads();
-
-  for (int t = 0; t < n_tiles; t++) {
-    const int buf = t & 1;
-    if (t + 1 < n_tiles) load_tile(t + 1);
-
-    const int64_t n0 = (int64_t)t * BN;
-    const int64_t kg0 = kf + n0 * P;                 // global position of the tile's first key
-    const bool active = wave_has_rows && kg0 <= qg_wlast;  // some row of the wave sees some key of the tile
-    if (active) {
-      const bool need_mask = !(kf + (n0 + BN - 1) * P <= qg_wfirst && n0 + BN <= kv_len);
-
-      // ---- S^T = K Q^T ----
-      f32x16 s[2][2];
-#pragma unroll
-      for (int kb = 0; kb < 2; kb++)
-#pragma unroll
-        for (int qb = 0; qb < 2; qb++)
-#pragma unroll
-          for (int i = 0; i < 16; i++) s[kb][qb][i] = 0.f;
-#pragma unroll
-      for (int kb = 0; kb < 2; kb++) {
-#pragma unroll
-        for (int t8 = 0; t8 < 8; t8++) {
-          const u32x4 a = lds_k[buf][swz(kb * 32 + qc, 2 * t8 + g)];
-          s[kb][0] = Mfma<T>::run(a, qreg[0][t8], s[kb][0]);
-          s[kb][1] = Mfma<T>::run(a, qreg[1][t8], s[kb][1]);
-        }
-      }
-
-      // ---- online softmax on the query column owned by this lane ----
-      u32x4 pk[2][4];  // P^T as B operands: pk[qb][u], k-step u = kb*2 + jj
-#pragma unroll
-      for (int qb = 0; qb < 2; qb++) {
-        if (need_mask) {
-          const int64_t qpos = qf + (m_w0 + qb * 32 + qc) * P;
-#pragma unroll
-          for (int kb = 0; kb < 2; kb++)
-#pragma unroll
-            for (int i = 0; i < 16; i++) {
-              const int64_t n = n0 + kb * 32 + (i >> 2) * 8 + 4 * g + (i & 3);
-              const bool vis = (kf + n * P <= qpos) && (n < kv_len);
-              s[kb][qb][i] = vis ? s[kb][qb][i] : -INFINITY;
-            }
-        }
-        float mx = s[0][qb][0];
-#pragma unroll
-        for (int kb = 0; kb < 2; kb++)
-#pragma unroll
-          for (int i = 0; i < 16; i++) mx = fmaxf(mx, s[kb][qb][i]);
-        mx = fmaxf(mx, other_half(mx, g));
-        const float m_new = fmaxf(m_run[qb], mx * p.scale_log2);
-        const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
-        const float alpha = __builtin_amdgcn_exp2f(m_run[qb] - m_safe);
-        m_run[qb] = m_new;
-        float ps = 0.f;
-#pragma unroll
-        for (int kb = 0; kb < 2; kb++) {
-          float pv[16];
-#pragma unroll
-          for (int i = 0; i < 16; i++) {
-            pv[i] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kb][qb][i], p.scale_log2, -m_safe));
-            ps += pv[i];
-          }
-#pragma unroll
-          for (int jj = 0; jj < 2; jj++) {
-            u32x4 w;
-#pragma unroll
-            for (int e = 0; e < 4; e++) w[e] = pack2<F16>(pv[8 * jj + 2 * e], pv[8 * jj + 2 * e + 1]);
-            pk[qb][kb * 2 + jj] = w;
-          }
-        }
-        l_run[qb] = l_run[qb] * alpha + ps;
-#pragma unroll
-        for (int db = 0; db < 4; db++)
-#pragma unroll
-          for (int i = 0; i < 16; i++) oacc[db][qb][i] *= alpha;
-      }
-
-      // ---- O^T += V^T P^T ----
-      const int blk16 = lane >> 4;  // 16-lane block of the transposing read
-      const int li = lane & 15;
-#pragma unroll
-      for (int u = 0; u < 4; u++) {
-        const int kb = u >> 1, jj = u & 1;
-        const int row_a = kb * 32 + jj * 16 + 4 * (blk16 >> 1) + (li >> 2);  // keys base + 4g + 0..3
-        const int row_b = row_a + 8;                                          // keys base + 8 + 4g + 0..3
-#pragma unroll
-        for (int db = 0; db < 4; db++) {
-          const int d_off = db * 32 + (blk16 & 1) * 16 + 4 * (li & 3);  // first of 4 consecutive elements
-          const char* base = (const char*)&lds_v[buf][0];
-          const char* pa = base + swz(row_a, d_off >> 3) * 16 + (d_off & 7) * 2;
-          const char* pb = base + swz(row_b, d_off >> 3) * 16 + (d_off & 7) * 2;
-          const i16x4 va = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_ptr)pa);
-          const i16x4 vb = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_ptr)pb);
-          const u32x2 wa = __builtin_bit_cast(u32x2, va), wb = __builtin_bit_cast(u32x2, vb);
-          const u32x4 a = {wa[0], wa[1], wb[0], wb[1]};
-          oacc[db][0] = Mfma<F16>::run(a, pk[0][u], oacc[db][0]);
-          oacc[db][1] = Mfma<F16>::run(a, pk[1][u], oacc[db][1]);
-        }
-      }
-    }
-
-    if (t + 1 < n_tiles) store_tile(buf ^ 1);
+  auto iteration = [&](auto fast_tag, int it) {
+    // after the barrier K tiles it, it+1 and V tile it-1 are resident; K(it+2) and V(it) are sent on their way
+    wait_vmem();
     __syncthreads();
+    load_k_tile(it + 2);
+    load_v_tile(it);
+    step(std::integral_constant<int, 1>{}, fast_tag, 2 * it - 1);
+    step(std::integral_constant<int, 0>{}, fast_tag, 2 * it);
+    store_v_tile(it);
+  };
+
+  // both V buffers start finite (zero): the general step may multiply them by P = 0 before they are loaded
+  for (int i = tid; i < 2 * kTileBytes / 16; i += NWAVE * 64) *(u32x4*)(lds + kLdsV + i * 16) = u32x4{0, 0, 0, 0};
+#pragma unroll
+  for (int qb = 0; qb < 2; qb++) {
+#pragma unroll
+    for (int jj = 0; jj < 2; jj++) {
+      pk0[qb][jj] = u32x4{0, 0, 0, 0};
+      pk1[qb][jj] = u32x4{0, 0, 0, 0};
+    }
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+      s0[qb][i] = 0.f;
+      s1[qb][i] = 0.f;
+    }
+  }
+  if (nt == 0) {
+    // nothing visible to any row of the workgroup: fall through to the epilogue with the empty state
+  } else {
+  load_k_tile(0);
+  load_k_tile(1);
+  wait_vmem();
+  __syncthreads();
+  load_k_operands(lds, 0, koff, ka);
+  // iterations [1, fast_end) of this wave have all stages live and unmasked
+  int fast_end = ns_w / 2 < (i_mask + 1) / 2 ? ns_w / 2 : (i_mask + 1) / 2;
+  if (fast_end < 1) fast_end = 1;
+  if (fast_end > nt + 1) fast_end = nt + 1;
+  iteration(std::false_type{}, 0);
+  for (int it = 1; it < fast_end; it++) iteration(std::true_type{}, it);
+  for (int it = fast_end; it <= nt; it++) iteration(std::false_type{}, it);
   }
 
   // ---- epilogue ----
