@@ -90,11 +90,12 @@ __device__ __forceinline__ float other_half(float v, int upper) {
   return __builtin_bit_cast(float, upper ? r[0] : r[1]);
 }
 
-// LDS: three K tiles at [0, 48K), two V tiles at [48K, 80K); a tile is [64 rows][16 chunks of 16 bytes] and
-// the chunk index is XORed with swz_bits(row), which makes the row-wise 16-byte K reads and the
+// LDS: two K tiles at [0, 32K), three V tiles at [32K, 80K); a tile is [64 rows][16 chunks of 16 bytes]
+// and the chunk index is XORed with swz_bits(row), which makes the row-wise 16-byte K reads and the
 // transposing 8-byte V reads both bank-conflict free.
 constexpr int kTileBytes = BN * 256;
-constexpr int kLdsV = 3 * kTileBytes;
+constexpr int kLdsV = 2 * kTileBytes;
+constexpr int kLdsBytes = 5 * kTileBytes;
 __device__ __forceinline__ int swz_bits(int row) { return ((row & 3) << 2) | ((row >> 2) & 3); }
 
 typedef __attribute__((address_space(3))) i16x4* lds_i16x4_ptr;
@@ -104,9 +105,13 @@ typedef const __attribute__((address_space(1))) void* global_void_ptr;
 __device__ __forceinline__ void wait_vmem() { __builtin_amdgcn_s_waitcnt(0x0F70); }  // vmcnt(0) only
 
 // K A-operands of one 32-key sub-tile: 8 x 16 bytes per lane
-__device__ __forceinline__ void load_k_operands(const char* ktile, int kb, const int (&koff)[8], u32x4 (&ka)[8]) {
+// koff0 is the lane's byte offset for k-step 0; the swizzle is an XOR on the chunk index, so k-step t8
+// sits at koff0 ^ (t8 << 5).  lds_k_sub is the LDS byte address of the sub-tile (a multiple of 8 KB,
+// so adding the offset never carries into the XORed bits).
+__device__ __forceinline__ void load_k_operands(int lds_k_sub, int koff0, u32x4 (&ka)[8]) {
+  const int base = lds_k_sub + koff0;
 #pragma unroll
-  for (int t8 = 0; t8 < 8; t8++) ka[t8] = *(const u32x4*)(ktile + kb * (SUB * 256) + koff[t8]);
+  for (int t8 = 0; t8 < 8; t8++) ka[t8] = *(const __attribute__((address_space(3))) u32x4*)(base ^ (t8 << 5));
 }
 // S^T block row of 32 keys x 64 queries: s[qb] = K[kb*32 .. +32) Q^T
 template <typename T>
@@ -124,20 +129,22 @@ __device__ __forceinline__ void qk_stage(const u32x4 (&ka)[8], const u32x4 (&qre
 }
 
 // V^T A-operands of one 32-key sub-tile through transposing LDS reads
-__device__ __forceinline__ void load_v_operands(const char* vtile, int kb, const int (&voffa)[4], const int (&voffb)[4], u32x4 (&va)[2][4]) {
+// voffa0 / voffb0 are the lane's byte offsets for d-block 0 (keys base+4g'+r and +8); d-block db sits at
+// offset ^ (db << 6), the second group of 16 keys 4 KB further.
+__device__ __forceinline__ void load_v_operands(int lds_v_sub, int voffa0, int voffb0, u32x4 (&va)[2][4]) {
+  const int base_a = lds_v_sub + voffa0, base_b = lds_v_sub + voffb0;
 #pragma unroll
   for (int jj = 0; jj < 2; jj++) {
 #pragma unroll
     for (int db = 0; db < 4; db++) {
-      const char* base = vtile + kb * (SUB * 256) + jj * (16 * 256);
-      const i16x4 xa = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_ptr)(base + voffa[db]));
-      const i16x4 xb = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_ptr)(base + voffb[db]));
+      const i16x4 xa = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_ptr)((base_a ^ (db << 6)) + jj * (16 * 256)));
+      const i16x4 xb = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_ptr)((base_b ^ (db << 6)) + jj * (16 * 256)));
       const u32x2 wa = __builtin_bit_cast(u32x2, xa), wb = __builtin_bit_cast(u32x2, xb);
       va[jj][db] = u32x4{wa[0], wa[1], wb[0], wb[1]};
     }
   }
 }
-// O^T += V^T[., kb*32 .. +32) P^T
+// O^T += V^T[., 32 keys) P^T
 __device__ __forceinline__ void pv_stage(const u32x4 (&va)[2][4], const u32x4 (&pk)[2][2], f32x16 (&oacc)[4][2]) {
 #pragma unroll
   for (int jj = 0; jj < 2; jj++) {
@@ -154,7 +161,7 @@ __device__ __forceinline__ void pv_stage(const u32x4 (&va)[2][4], const u32x4 (&
 // factor the O accumulators then owe is returned in alpha (applied by the caller after the
 // P V products that still belong to the old max).
 struct MaskInfo {
-  int64_t n0, kv_len, kf, P, qpos0, qpos1;  // sub-tile start, bounds and the two query positions
+  int n0, kv_len, kf, P, qpos0, qpos1;  // sub-tile start, bounds and the two query positions
 };
 template <bool MASK>
 __device__ __forceinline__ bool softmax_stage(f32x16 (&s)[2], u32x4 (&pk)[2][2], float (&m_run)[2], float (&l_run)[2], float (&alpha)[2],
@@ -163,11 +170,11 @@ __device__ __forceinline__ bool softmax_stage(f32x16 (&s)[2], u32x4 (&pk)[2][2],
 #pragma unroll
   for (int qb = 0; qb < 2; qb++) {
     if (MASK) {
-      const int64_t qpos = qb ? mi.qpos1 : mi.qpos0;
+      const int qpos = qb ? mi.qpos1 : mi.qpos0;
 #pragma unroll
       for (int i = 0; i < 16; i++) {
-        const int64_t n = mi.n0 + (i >> 2) * 8 + 4 * g + (i & 3);
-        const bool vis = (mi.kf + n * mi.P <= qpos) && (n < mi.kv_len);
+        const int n = mi.n0 + (i >> 2) * 8 + 4 * g + (i & 3);
+        const bool vis = (n < mi.kv_len) && (mi.kf + n * mi.P <= qpos);
         s[qb][i] = vis ? s[qb][i] : -INFINITY;
       }
     }
@@ -226,7 +233,7 @@ __device__ __forceinline__ void rescale_o(f32x16 (&oacc)[4][2], const float (&al
 
 template <typename T, int MODE>  // MODE 0: partial (o fp32, lse)   MODE 1: in-place (o, m, l) update
 __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p) {
-  __shared__ __attribute__((aligned(1024))) char lds[5 * kTileBytes];
+  __shared__ __attribute__((aligned(1024))) char lds[kLdsBytes];
 
   // ---- workgroup -> (sequence, q head, query tile) ----
   const int group = p.hq / p.hkv;
@@ -243,42 +250,42 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
   const int h = kvh * group + gq;
   const int z = p.nz - 1 - zr;
 
-  const int64_t q_len = p.q_len[b];
-  const int64_t m_lo = (int64_t)z * BM;
+  // token counts and global positions are int32 in the interface; only byte offsets need 64 bits
+  const int q_len = p.q_len[b];
+  const int m_lo = z * BM;
   if (m_lo >= q_len) return;
-  const int64_t kv_len = p.kv_len[b];
+  const int kv_len = p.kv_len[b];
   const int64_t q_start = p.q_start[b], kv_start = p.kv_start[b];
-  const int64_t qf = p.q_first[b], kf = p.kv_first[b];
-  const int64_t P = p.peers;
+  const int qf = p.q_first[b], kf = p.kv_first[b];
+  const int P = p.peers;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int qc = lane & 31, g = lane >> 5;
 
   // number of keys visible to global position qpos, clamped to the chunk
-  auto visible_keys = [&](int64_t qpos) -> int64_t {
-    const int64_t dq = qpos - kf;
-    int64_t n = dq >= 0 ? dq / P + 1 : 0;
+  auto visible_keys = [&](int qpos) -> int {
+    const int dq = qpos - kf;
+    const int n = dq >= 0 ? dq / P + 1 : 0;
     return n > kv_len ? kv_len : n;
   };
-  const int64_t m_hi = (m_lo + BM < q_len ? m_lo + BM : q_len) - 1;
-  const int nt = (int)((visible_keys(qf + m_hi * P) + BN - 1) / BN);  // LDS tiles the workgroup walks
+  const int m_hi = (m_lo + BM < q_len ? m_lo + BM : q_len) - 1;
+  const int nt = (visible_keys(qf + m_hi * P) + BN - 1) / BN;  // LDS tiles the workgroup walks
 
   // ---- this wave's rows and its sub-tile range ----
-  const int64_t m_w0 = m_lo + wave * 64;
+  const int m_w0 = m_lo + wave * 64;
   const bool wave_has_rows = m_w0 < q_len;
-  int64_t m_wlast = m_w0 + 63;
-  if (m_wlast > q_len - 1) m_wlast = q_len - 1;
+  const int m_wlast = m_w0 + 63 > q_len - 1 ? q_len - 1 : m_w0 + 63;
   // sub-tiles [0, ns_w) hold a key some row of the wave sees; sub-tiles [0, i_mask) are seen
   // entirely by every row of the wave (no mask needed)
-  const int ns_w = wave_has_rows ? (int)((visible_keys(qf + m_wlast * P) + SUB - 1) / SUB) : 0;
-  const int i_mask = wave_has_rows ? (int)(visible_keys(qf + m_w0 * P) / SUB) : 0;
+  const int ns_w = wave_has_rows ? (visible_keys(qf + m_wlast * P) + SUB - 1) / SUB : 0;
+  const int i_mask = wave_has_rows ? visible_keys(qf + m_w0 * P) / SUB : 0;
 
   // Q as B operands: qreg[qb][t] = Q[row qb*32+qc][16t + 8g .. +7]
   u32x4 qreg[2][8];
 #pragma unroll
   for (int qb = 0; qb < 2; qb++) {
-    const int64_t m = m_w0 + qb * 32 + qc;
+    const int m = m_w0 + qb * 32 + qc;
     const bool ok = m < q_len;
     const char* src = (const char*)p.q + ((q_start + (ok ? m : 0)) * p.q_st + (int64_t)h * p.q_sh + 8 * g) * 2;
 #pragma unroll
@@ -286,62 +293,76 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
   }
 
   // ---- per-lane LDS byte offsets inside a tile ----
-  int koff[8];  // K A-operand: row qc (+32 kb), logical chunk 2*t8+g
-#pragma unroll
-  for (int t8 = 0; t8 < 8; t8++) koff[t8] = qc * 256 + (((2 * t8 + g) ^ swz_bits(qc)) << 4);
-  int voffa[4], voffb[4];  // V^T A-operand via transposing reads: keys base+4g'+(li>>2) and +8
+  // K A-operand of k-step t8: row qc (+32 for the second half), logical chunk 2*t8+g
+  int koff0 = qc * 256 + ((g ^ swz_bits(qc)) << 4);
+  // V^T A-operand of d-block db via transposing reads: key rows base+4g'+(li>>2) (and +8), 4 consecutive
+  // elements starting at db*32 + (blk16&1)*16 + 4*(li&3)
+  int voffa0, voffb0;
   {
     const int blk16 = lane >> 4, li = lane & 15;
     const int row_a = 4 * (blk16 >> 1) + (li >> 2);
     const int row_b = row_a + 8;
-#pragma unroll
-    for (int db = 0; db < 4; db++) {
-      const int d_off = db * 32 + (blk16 & 1) * 16 + 4 * (li & 3);
-      voffa[db] = row_a * 256 + (((d_off >> 3) ^ swz_bits(row_a)) << 4) + (d_off & 7) * 2;
-      voffb[db] = row_b * 256 + (((d_off >> 3) ^ swz_bits(row_b)) << 4) + (d_off & 7) * 2;
-    }
+    const int d_off = (blk16 & 1) * 16 + 4 * (li & 3);
+    voffa0 = row_a * 256 + (((d_off >> 3) ^ swz_bits(row_a)) << 4) + (d_off & 7) * 2;
+    voffb0 = row_b * 256 + (((d_off >> 3) ^ swz_bits(row_b)) << 4) + (d_off & 7) * 2;
   }
+  const int lds_base = (int)(uintptr_t)(__attribute__((address_space(3))) char*)lds;
 
-  // ---- global -> LDS staging: wave w owns rows [16w, 16w+16) of every tile, 4 rows per instruction ----
+  // ---- global -> LDS staging: wave w owns rows [16w, 16w+16) of every tile, 4 rows per instruction.
+  // The lane that fills physical chunk slot (lane & 15) of row r fetches logical chunk slot ^ swz_bits(r).
   const char* kg = (const char*)p.k + (kv_start * p.k_st + (int64_t)kvh * p.k_sh) * 2;
   const char* vg = (const char*)p.v + (kv_start * p.v_st + (int64_t)kvh * p.v_sh) * 2;
-  const int st_row = lane >> 4;                                  // row inside the group of 4
-  auto stage_src_chunk = [&](int r) { return ((lane & 15) ^ swz_bits(r)) << 4; };  // logical chunk bytes for physical slot
-  // Rows past the chunk are masked later; the row index is clamped so that the data stays finite
-  // and a tile index past the walk (harmless prefetch into a free buffer) stays in bounds.
-  const int last_row = (int)(kv_len - 1);
   const int64_t k_row_bytes = p.k_st * 2, v_row_bytes = p.v_st * 2;
-  auto load_k_tile = [&](int t) {
+  const int st_row = lane >> 4;
+  const int last_row = kv_len - 1;
+  uint32_t k_lane_off[4], v_lane_off[4];  // byte offset of this lane's chunk inside a full tile
+  int st_chunk[4];
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const int r = 16 * wave + 4 * i + st_row;
+    st_chunk[i] = ((lane & 15) ^ swz_bits(r)) << 4;
+    k_lane_off[i] = (uint32_t)(r * k_row_bytes) + st_chunk[i];
+    v_lane_off[i] = (uint32_t)(r * v_row_bytes) + st_chunk[i];
+  }
+  u32x4 vst[4];  // V staging registers (element types whose V is converted on the way)
+  // FULL: every row of tile t exists, so the per-lane offsets are added to a uniform tile base.
+  // Otherwise the row index is clamped (rows past the chunk are masked later, the data only has
+  // to stay finite and in bounds; a tile index past the walk prefetches into a free buffer).
+  auto load_tiles = [&](auto full_tag, int tk, int tv) {
+    constexpr bool FULL = decltype(full_tag)::value;
 #pragma unroll
     for (int i = 0; i < 4; i++) {
       const int r = 16 * wave + 4 * i + st_row;
-      int n = t * BN + r;
-      n = n > last_row ? last_row : n;
-      __builtin_amdgcn_global_load_lds((global_void_ptr)(kg + n * k_row_bytes + stage_src_chunk(r)),
-                                       (lds_void_ptr)(lds + (t % 3) * kTileBytes + (16 * wave + 4 * i) * 256), 16, 0, 0);
-    }
-  };
-  u32x4 vst[4];
-  auto load_v_tile = [&](int t) {
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-      const int r = 16 * wave + 4 * i + st_row;
-      int n = t * BN + r;
-      n = n > last_row ? last_row : n;
-      const char* src = vg + n * v_row_bytes + stage_src_chunk(r);
+      const char* ksrc;
+      const char* vsrc;
+      if (FULL) {
+        // uniform (scalar) tile base + 32-bit per-lane offset
+        const char* kt = kg + (int64_t)tk * BN * k_row_bytes;
+        const char* vt = vg + (int64_t)tv * BN * v_row_bytes;
+        asm volatile("" : "+s"(kt), "+s"(vt));
+        ksrc = kt + k_lane_off[i];
+        vsrc = vt + v_lane_off[i];
+      } else {
+        int nk = tk * BN + r, nv = tv * BN + r;
+        nk = nk > last_row ? last_row : nk;
+        nv = nv > last_row ? last_row : nv;
+        ksrc = kg + nk * k_row_bytes + st_chunk[i];
+        vsrc = vg + nv * v_row_bytes + st_chunk[i];
+      }
+      __builtin_amdgcn_global_load_lds((global_void_ptr)ksrc, (lds_void_ptr)(lds + (tk & 1) * kTileBytes + (16 * wave + 4 * i) * 256), 16, 0, 0);
       if (DirectV<T>::value) {
-        __builtin_amdgcn_global_load_lds((global_void_ptr)src, (lds_void_ptr)(lds + kLdsV + (t & 1) * kTileBytes + (16 * wave + 4 * i) * 256),
+        __builtin_amdgcn_global_load_lds((global_void_ptr)vsrc, (lds_void_ptr)(lds + kLdsV + (tv % 3) * kTileBytes + (16 * wave + 4 * i) * 256),
                                          16, 0, 0);
       } else {
-        vst[i] = *(const u32x4*)src;
+        vst[i] = *(const u32x4*)vsrc;
       }
     }
   };
-  auto store_v_tile = [&](int t) {  // only for element types whose V goes through registers
+  auto store_v_tile = [&](int tv) {  // only for element types whose V goes through registers
     if (!DirectV<T>::value) {
 #pragma unroll
       for (int i = 0; i < 4; i++)
-        *(u32x4*)(lds + kLdsV + (t & 1) * kTileBytes + (16 * wave + 4 * i) * 256 + lane * 16) = to_pv_operand<T>(vst[i]);
+        *(u32x4*)(lds + kLdsV + (tv % 3) * kTileBytes + (16 * wave + 4 * i) * 256 + lane * 16) = to_pv_operand<T>(vst[i]);
     }
   };
 
@@ -354,103 +375,100 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
       for (int i = 0; i < 16; i++) oacc[db][qb][i] = 0.f;
   float m_run[2] = {-INFINITY, -INFINITY};
   float l_run[2] = {0.f, 0.f};
-  f32x16 s0[2], s1[2];    // S^T of even / odd sub-tiles
+  f32x16 s[2];                 // S^T of the sub-tile whose softmax comes next
   u32x4 pk0[2][2], pk1[2][2];  // P^T of even / odd sub-tiles
+  u32x4 va[2][4];              // V^T operands of the sub-tile whose P V product comes next
   float alpha[2];
   MaskInfo mi;
-  mi.kv_len = kv_len;
   mi.kf = kf;
   mi.P = P;
   mi.qpos0 = qf + (m_w0 + qc) * P;
   mi.qpos1 = qf + (m_w0 + 32 + qc) * P;
 
-  // One pipeline step on sub-tile i: S(i+1) = K(i+1) Q^T, P(i) = softmax(S(i)), O += V(i-1) P(i-1).
-  // PAR is the parity of i: S/P of sub-tile i live in the PAR set, those of i+-1 in the other.
-  // The K operands of sub-tile i+1 were read from LDS during the previous step (ka); this step
-  // reads the V operands of sub-tile i-1 up front and the K operands of sub-tile i+2 while its
-  // P V products run, so no MFMA waits on an LDS read it has just issued.
+  // One pipeline step on sub-tile i:  O += V(i-1) P(i-1),  P(i) = softmax(S(i)),  S(i+1) = K(i+1) Q^T.
+  // On entry s holds S(i), va the V operands of sub-tile i-1 and the other-parity pk holds P(i-1).
+  // The step first moves S(i) out of the accumulators and issues the K reads for sub-tile i+1; the
+  // P V products then run on operands that are already in registers while the softmax works, the
+  // S^T products follow, and the V reads for the next step ride on them.  No MFMA waits on an LDS
+  // read issued just before it.
   // The FAST form assumes all three stages are live and sub-tile i needs no mask.  The general
-  // form runs the same three stages unconditionally and folds "stage not live" into the mask:
-  // a dead softmax sees an empty key range (P = 0, state untouched), a dead S(i+1) is never
-  // read, and a dead P V product multiplies finite LDS contents by P = 0.
-  u32x4 ka[8];
+  // form runs the same stages unconditionally and folds "stage not live" into the mask: a dead
+  // softmax sees an empty key range (P = 0, state untouched), a dead S(i+1) is never read, and a
+  // dead P V product multiplies finite LDS contents by P = 0.
   auto step = [&](auto par_tag, auto fast_tag, int i) {
     constexpr int PAR = decltype(par_tag)::value;
     constexpr bool FAST = decltype(fast_tag)::value;
-    f32x16(&s_cur)[2] = PAR ? s1 : s0;
-    f32x16(&s_nxt)[2] = PAR ? s0 : s1;
     u32x4(&pk_cur)[2][2] = PAR ? pk1 : pk0;
     u32x4(&pk_prv)[2][2] = PAR ? pk0 : pk1;
-    // sub-tile i-1 lives in V tile (i-1)/2, half !PAR; sub-tile i+2 in K tile (i+2)/2, half PAR
-    const char* vtile = lds + kLdsV + (((i - 1) >> 1) & 1) * kTileBytes;
-    const char* ktile2 = lds + (((i + 2) >> 1) % 3) * kTileBytes;
+    // sub-tile i+1 lives in K tile (i+1)/2, half !PAR; sub-tile i in V tile i/2, half PAR
+    const int ksub = lds_base + (((i + 1) >> 1) & 1) * kTileBytes + (PAR ^ 1) * (SUB * 256);
+    const int vsub = lds_base + kLdsV + (((i >> 1) + 3) % 3) * kTileBytes + PAR * (SUB * 256);
+    // the per-lane offsets are made opaque here so that the XOR-derived addresses are formed where
+    // they are used instead of being hoisted into sixteen long-lived registers
+    asm volatile("" : "+v"(koff0), "+v"(voffa0), "+v"(voffb0));
     if (!FAST) {
-      // a dead stage gets a key range that lies past every chunk, so that nothing is visible
-      mi.n0 = (i >= 0 && i < ns_w) ? (int64_t)i * SUB : ((int64_t)1 << 40);
+      const bool live = i >= 0 && i < ns_w;
+      mi.n0 = live ? i * SUB : 0;
+      mi.kv_len = live ? kv_len : 0;
     }
-    u32x4 va[2][4];
-    load_v_operands(vtile, PAR ^ 1, voffa, voffb, va);
-    qk_stage<T>(ka, qreg, s_nxt);
-    const bool any = softmax_stage<!FAST>(s_cur, pk_cur, m_run, l_run, alpha, p.scale_log2, g, mi);
-    load_k_operands(ktile2, PAR, koff, ka);
+    // scheduling fences between the three parts keep register live ranges as written: the K
+    // operands are requested first, the softmax shares its part with the P V products, and the
+    // V operands of the next step are requested together with the S^T products
+    f32x16 sv[2] = {s[0], s[1]};
+    u32x4 ka[8];
+    load_k_operands(ksub, koff0, ka);
+    __builtin_amdgcn_sched_barrier(0);
     pv_stage(va, pk_prv, oacc);
-    // P(i) is only consumed by the next step; pin its computation into this step so that it
-    // overlaps this step's MFMAs instead of being sunk to where the MFMA pipe has nothing to do
-    asm volatile("" ::"v"(pk_cur[0][0]), "v"(pk_cur[0][1]), "v"(pk_cur[1][0]), "v"(pk_cur[1][1]), "v"(ka[0]), "v"(ka[7]));
-    if (FAST) {
-      // issue order of the step: one MFMA, at most one LDS read, then the ~6 VALU operations the
-      // matrix pipe hides behind it; the 16 transposing V reads ride on the S^T products, the 8
-      // K reads for the next step on the P V products
-#pragma unroll
-      for (int k = 0; k < 32; k++) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);              // MFMA
-        if (k < 24) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // DS read
-        __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);              // VALU
-      }
-    }
+    const bool any = softmax_stage<!FAST>(sv, pk_cur, m_run, l_run, alpha, p.scale_log2, g, mi);
+    // P(i) and the row sums are only consumed later; pin their computation into this part so that
+    // it overlaps the MFMAs here and does not keep the unpacked probabilities alive
+    asm volatile("" ::"v"(pk_cur[0][0]), "v"(pk_cur[0][1]), "v"(pk_cur[1][0]), "v"(pk_cur[1][1]), "v"(l_run[0]), "v"(l_run[1]),
+                 "v"(m_run[0]), "v"(m_run[1]));
+    __builtin_amdgcn_sched_barrier(0);
+    qk_stage<T>(ka, qreg, s);
+    load_v_operands(vsub, voffa0, voffb0, va);
+    __builtin_amdgcn_sched_barrier(0);
     if (any) rescale_o(oacc, alpha);
   };
   auto iteration = [&](auto fast_tag, int it) {
-    // after the barrier K tiles it, it+1 and V tile it-1 are resident; K(it+2) and V(it) are sent on their way
+    // after the barrier K tile it and V tiles it-1, it are resident; K(it+1) and V(it+1) are sent on their way
     wait_vmem();
     __syncthreads();
-    load_k_tile(it + 2);
-    load_v_tile(it);
+    load_tiles(fast_tag, it + 1, it + 1);
     step(std::integral_constant<int, 1>{}, fast_tag, 2 * it - 1);
     step(std::integral_constant<int, 0>{}, fast_tag, 2 * it);
-    store_v_tile(it);
+    store_v_tile(it + 1);
   };
 
-  // both V buffers start finite (zero): the general step may multiply them by P = 0 before they are loaded
-  for (int i = tid; i < 2 * kTileBytes / 16; i += NWAVE * 64) *(u32x4*)(lds + kLdsV + i * 16) = u32x4{0, 0, 0, 0};
+  if (nt > 0) {
+    // the V buffers and the first V operands start finite (zero): the general step may multiply
+    // them by P = 0 before real data arrives
+    for (int i = tid; i < 3 * kTileBytes / 16; i += NWAVE * 64) *(u32x4*)(lds + kLdsV + i * 16) = u32x4{0, 0, 0, 0};
 #pragma unroll
-  for (int qb = 0; qb < 2; qb++) {
+    for (int qb = 0; qb < 2; qb++) {
 #pragma unroll
-    for (int jj = 0; jj < 2; jj++) {
-      pk0[qb][jj] = u32x4{0, 0, 0, 0};
-      pk1[qb][jj] = u32x4{0, 0, 0, 0};
+      for (int jj = 0; jj < 2; jj++) {
+        pk0[qb][jj] = u32x4{0, 0, 0, 0};
+        pk1[qb][jj] = u32x4{0, 0, 0, 0};
+      }
+#pragma unroll
+      for (int i = 0; i < 16; i++) s[qb][i] = 0.f;
     }
 #pragma unroll
-    for (int i = 0; i < 16; i++) {
-      s0[qb][i] = 0.f;
-      s1[qb][i] = 0.f;
-    }
-  }
-  if (nt == 0) {
-    // nothing visible to any row of the workgroup: fall through to the epilogue with the empty state
-  } else {
-  load_k_tile(0);
-  load_k_tile(1);
-  wait_vmem();
-  __syncthreads();
-  load_k_operands(lds, 0, koff, ka);
-  // iterations [1, fast_end) of this wave have all stages live and unmasked
-  int fast_end = ns_w / 2 < (i_mask + 1) / 2 ? ns_w / 2 : (i_mask + 1) / 2;
-  if (fast_end < 1) fast_end = 1;
-  if (fast_end > nt + 1) fast_end = nt + 1;
-  iteration(std::false_type{}, 0);
-  for (int it = 1; it < fast_end; it++) iteration(std::true_type{}, it);
-  for (int it = fast_end; it <= nt; it++) iteration(std::false_type{}, it);
+    for (int jj = 0; jj < 2; jj++)
+#pragma unroll
+      for (int db = 0; db < 4; db++) va[jj][db] = u32x4{0, 0, 0, 0};
+    __syncthreads();
+    load_tiles(std::false_type{}, 0, 0);
+    store_v_tile(0);
+    // iterations [1, fast_end) of this wave have all stages live and unmasked, and prefetch a full tile
+    int fast_end = ns_w / 2 < (i_mask + 1) / 2 ? ns_w / 2 : (i_mask + 1) / 2;
+    if (fast_end > kv_len / BN - 1) fast_end = kv_len / BN - 1;
+    if (fast_end < 1) fast_end = 1;
+    if (fast_end > nt + 1) fast_end = nt + 1;
+    iteration(std::false_type{}, 0);
+    for (int it = 1; it < fast_end; it++) iteration(std::true_type{}, it);
+    for (int it = fast_end; it <= nt; it++) iteration(std::false_type{}, it);
   }
 
   // ---- epilogue ----
