@@ -9,7 +9,9 @@ from __future__ import annotations
 import ctypes as C
 import os
 
-LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "liblsattn.so")
+# LSATTN_LIB_PATH selects another build of the same library (same C ABI), e.g. one made with
+# different compile-time tuning; the default is the in-tree build next to this file.
+LIB_PATH = os.environ.get("LSATTN_LIB_PATH") or os.path.join(os.path.dirname(os.path.abspath(__file__)), "liblsattn.so")
 
 LSATTN_F16, LSATTN_BF16, LSATTN_F32 = 0, 1, 2
 LSATTN_MAX_PARTS = 16

@@ -39,16 +39,16 @@ def _compile(src: str, extra) -> str:
     return obj
 
 
-def build_all(verbose: bool = False, extra_flags=()) -> str:
+def build_all(verbose: bool = False, extra_flags=(), out: str = LIB_PATH) -> str:
     with ThreadPoolExecutor(max_workers=len(SOURCES)) as ex:
         objs = list(ex.map(lambda s: _compile(s, list(extra_flags)), SOURCES))
-    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-fno-gpu-rdc", *objs, "-o", LIB_PATH]
+    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-fno-gpu-rdc", *objs, "-o", out]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError("link failed:\n%s\n%s" % (" ".join(cmd), r.stderr[-6000:]))
     if verbose:
-        print("built", LIB_PATH)
-    return LIB_PATH
+        print("built", out)
+    return out
 
 
 if __name__ == "__main__":

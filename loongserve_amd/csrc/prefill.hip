@@ -18,6 +18,9 @@
 //   * workgroup ids are mapped so that the workgroups sharing one KV head run on one XCD
 //     (ids are dealt round-robin to the 8 XCDs) and heavy (late) query tiles start first.
 #include <type_traits>
+#ifndef LSATTN_EXP
+#define LSATTN_EXP 0
+#endif
 
 #include "common.hip.h"
 
@@ -90,19 +93,21 @@ __device__ __forceinline__ float other_half(float v, int upper) {
   return __builtin_bit_cast(float, upper ? r[0] : r[1]);
 }
 
-// LDS: two K tiles at [0, 32K), three V tiles at [32K, 80K); a tile is [64 rows][16 chunks of 16 bytes]
+// LDS: a ring of four K tiles at [0, 64K) and a ring of four V tiles at [64K, 128K); a tile is [64 rows][16 chunks of 16 bytes]
 // and the chunk index is XORed with swz_bits(row), which makes the row-wise 16-byte K reads and the
 // transposing 8-byte V reads both bank-conflict free.
 constexpr int kTileBytes = BN * 256;
-constexpr int kLdsV = 2 * kTileBytes;
-constexpr int kLdsBytes = 5 * kTileBytes;
+constexpr int kRing = 4;  // tiles per ring
+constexpr int kLdsV = kRing * kTileBytes;
+constexpr int kLdsBytes = 2 * kRing * kTileBytes;
 __device__ __forceinline__ int swz_bits(int row) { return ((row & 3) << 2) | ((row >> 2) & 3); }
 
 typedef __attribute__((address_space(3))) i16x4* lds_i16x4_ptr;
 typedef __attribute__((address_space(3))) void* lds_void_ptr;
 typedef const __attribute__((address_space(1))) void* global_void_ptr;
 
-__device__ __forceinline__ void wait_vmem() { __builtin_amdgcn_s_waitcnt(0x0F70); }  // vmcnt(0) only
+// s_waitcnt on the vector-memory counter only (expcnt / lgkmcnt fields left at their maximum)
+template <int N> __device__ __forceinline__ void wait_vmem() { __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14)); }
 
 // K A-operands of one 32-key sub-tile: 8 x 16 bytes per lane
 // koff0 is the lane's byte offset for k-step 0; the swizzle is an XOR on the chunk index, so k-step t8
@@ -163,9 +168,11 @@ __device__ __forceinline__ void pv_stage(const u32x4 (&va)[2][4], const u32x4 (&
 struct MaskInfo {
   int n0, kv_len, kf, P, qpos0, qpos1;  // sub-tile start, bounds and the two query positions
 };
+// Part 1 of the softmax: mask (if needed), row max of both query columns, the wave-uniform
+// decision whether the running max moves, and the factors that follow from it.
 template <bool MASK>
-__device__ __forceinline__ bool softmax_stage(f32x16 (&s)[2], u32x4 (&pk)[2][2], float (&m_run)[2], float (&l_run)[2], float (&alpha)[2],
-                                              float scale_log2, int g, const MaskInfo& mi) {
+__device__ __forceinline__ bool softmax_max(f32x16 (&s)[2], float (&m_run)[2], float (&m_use)[2], float (&alpha)[2], float scale_log2, int g,
+                                            const MaskInfo& mi) {
   float scaled[2];
 #pragma unroll
   for (int qb = 0; qb < 2; qb++) {
@@ -189,33 +196,35 @@ __device__ __forceinline__ bool softmax_stage(f32x16 (&s)[2], u32x4 (&pk)[2][2],
 #pragma unroll
   for (int qb = 0; qb < 2; qb++) {
     const float m_new = any ? fmaxf(m_run[qb], scaled[qb]) : m_run[qb];
-    float m_use = m_new;
+    m_use[qb] = m_new;
     if (MASK) {
-      m_use = (m_new == -INFINITY) ? 0.f : m_new;
-      alpha[qb] = (m_run[qb] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m_run[qb] - m_use);
+      m_use[qb] = (m_new == -INFINITY) ? 0.f : m_new;
+      alpha[qb] = (m_run[qb] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m_run[qb] - m_use[qb]);
     } else {
       alpha[qb] = __builtin_amdgcn_exp2f(m_run[qb] - m_new);
     }
     m_run[qb] = m_new;
-    float pv[16];
-    float ps0 = 0.f, ps1 = 0.f;
-#pragma unroll
-    for (int i = 0; i < 16; i += 2) {
-      pv[i] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[qb][i], scale_log2, -m_use));
-      pv[i + 1] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[qb][i + 1], scale_log2, -m_use));
-      ps0 += pv[i];
-      ps1 += pv[i + 1];
-    }
-    l_run[qb] = l_run[qb] * alpha[qb] + (ps0 + ps1);
-#pragma unroll
-    for (int jj = 0; jj < 2; jj++) {
-      u32x4 w;
-#pragma unroll
-      for (int e = 0; e < 4; e++) w[e] = pack2<F16>(pv[8 * jj + 2 * e], pv[8 * jj + 2 * e + 1]);
-      pk[qb][jj] = w;
-    }
   }
   return any;
+}
+// Part 2, one query column: probabilities against m_use, packed to f16 as the B operand of the
+// P V product, and their fp32 row sum.
+__device__ __forceinline__ void softmax_exp(const f32x16& s, float m_use, float alpha, float& l_run, u32x4 (&pk)[2], float scale_log2) {
+  float ps0 = 0.f, ps1 = 0.f;
+#pragma unroll
+  for (int jj = 0; jj < 2; jj++) {
+    u32x4 w;
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[8 * jj + 2 * e], scale_log2, -m_use));
+      const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[8 * jj + 2 * e + 1], scale_log2, -m_use));
+      w[e] = pack2<F16>(p0, p1);
+      ps0 += p0;
+      ps1 += p1;
+    }
+    pk[jj] = w;
+  }
+  l_run = l_run * alpha + (ps0 + ps1);
 }
 
 __device__ __forceinline__ void rescale_o(f32x16 (&oacc)[4][2], const float (&alpha)[2]) {
@@ -328,17 +337,22 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
   // FULL: every row of tile t exists, so the per-lane offsets are added to a uniform tile base.
   // Otherwise the row index is clamped (rows past the chunk are masked later, the data only has
   // to stay finite and in bounds; a tile index past the walk prefetches into a free buffer).
-  auto load_tiles = [&](auto full_tag, int tk, int tv) {
+  auto load_tiles = [&](auto full_tag, int tk, int tv, int i_begin = 0, int i_end = 4) {
     constexpr bool FULL = decltype(full_tag)::value;
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
+    for (int i = i_begin; i < i_end; i++) {
       const int r = 16 * wave + 4 * i + st_row;
       const char* ksrc;
       const char* vsrc;
       if (FULL) {
         // uniform (scalar) tile base + 32-bit per-lane offset
+#if LSATTN_EXP == 7
+        const char* kt = kg + (int64_t)(tk & 3) * BN * k_row_bytes;
+        const char* vt = vg + (int64_t)(tv & 3) * BN * v_row_bytes;
+#else
         const char* kt = kg + (int64_t)tk * BN * k_row_bytes;
         const char* vt = vg + (int64_t)tv * BN * v_row_bytes;
+#endif
         asm volatile("" : "+s"(kt), "+s"(vt));
         ksrc = kt + k_lane_off[i];
         vsrc = vt + v_lane_off[i];
@@ -346,13 +360,27 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
         int nk = tk * BN + r, nv = tv * BN + r;
         nk = nk > last_row ? last_row : nk;
         nv = nv > last_row ? last_row : nv;
+        nv = nv < 0 ? 0 : nv;
         ksrc = kg + nk * k_row_bytes + st_chunk[i];
         vsrc = vg + nv * v_row_bytes + st_chunk[i];
       }
-      __builtin_amdgcn_global_load_lds((global_void_ptr)ksrc, (lds_void_ptr)(lds + (tk & 1) * kTileBytes + (16 * wave + 4 * i) * 256), 16, 0, 0);
+      const int kdst = (tk & (kRing - 1)) * kTileBytes + (16 * wave + 4 * i) * 256;
+      const int vdst = kLdsV + (tv & (kRing - 1)) * kTileBytes + (16 * wave + 4 * i) * 256;
+      if (FULL) {
+        // Issued from inline assembly on purpose: the compiler then does not know that LDS is written
+        // behind its back and does not put a full vector-memory wait in front of every later LDS read
+        // (it cannot tell the ring slots apart).  Completion is tracked by hand: wait_vmem<8>() plus
+        // the workgroup barrier at the top of the iteration in which a slot is first read.
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_base + kdst), "v"(ksrc) : "m0");
+        if (DirectV<T>::value)
+          asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_base + vdst), "v"(vsrc) : "m0");
+        else
+          vst[i] = *(const u32x4*)vsrc;
+        continue;
+      }
+      __builtin_amdgcn_global_load_lds((global_void_ptr)ksrc, (lds_void_ptr)(lds + kdst), 16, 0, 0);
       if (DirectV<T>::value) {
-        __builtin_amdgcn_global_load_lds((global_void_ptr)vsrc, (lds_void_ptr)(lds + kLdsV + (tv % 3) * kTileBytes + (16 * wave + 4 * i) * 256),
-                                         16, 0, 0);
+        __builtin_amdgcn_global_load_lds((global_void_ptr)vsrc, (lds_void_ptr)(lds + vdst), 16, 0, 0);
       } else {
         vst[i] = *(const u32x4*)vsrc;
       }
@@ -362,7 +390,7 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
     if (!DirectV<T>::value) {
 #pragma unroll
       for (int i = 0; i < 4; i++)
-        *(u32x4*)(lds + kLdsV + (tv % 3) * kTileBytes + (16 * wave + 4 * i) * 256 + lane * 16) = to_pv_operand<T>(vst[i]);
+        *(u32x4*)(lds + kLdsV + (tv & (kRing - 1)) * kTileBytes + (16 * wave + 4 * i) * 256 + lane * 16) = to_pv_operand<T>(vst[i]);
     }
   };
 
@@ -375,9 +403,9 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
       for (int i = 0; i < 16; i++) oacc[db][qb][i] = 0.f;
   float m_run[2] = {-INFINITY, -INFINITY};
   float l_run[2] = {0.f, 0.f};
-  f32x16 s[2];                 // S^T of the sub-tile whose softmax comes next
+  f32x16 s0[2], s1[2];         // S^T of even / odd sub-tiles
   u32x4 pk0[2][2], pk1[2][2];  // P^T of even / odd sub-tiles
-  u32x4 va[2][4];              // V^T operands of the sub-tile whose P V product comes next
+  u32x4 ka[8];                 // K operands of the sub-tile whose S^T product comes next
   float alpha[2];
   MaskInfo mi;
   mi.kf = kf;
@@ -385,24 +413,27 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
   mi.qpos0 = qf + (m_w0 + qc) * P;
   mi.qpos1 = qf + (m_w0 + 32 + qc) * P;
 
-  // One pipeline step on sub-tile i:  O += V(i-1) P(i-1),  P(i) = softmax(S(i)),  S(i+1) = K(i+1) Q^T.
-  // On entry s holds S(i), va the V operands of sub-tile i-1 and the other-parity pk holds P(i-1).
-  // The step first moves S(i) out of the accumulators and issues the K reads for sub-tile i+1; the
-  // P V products then run on operands that are already in registers while the softmax works, the
-  // S^T products follow, and the V reads for the next step ride on them.  No MFMA waits on an LDS
-  // read issued just before it.
+  // One pipeline step on sub-tile i:  S(i+1) = K(i+1) Q^T,  P(i) = softmax(S(i)),  O += V(i-1) P(i-1).
+  // The three stages touch three different sub-tiles, so nothing in a step waits for a matrix
+  // product issued in the same step.  PAR is the parity of i: S/P of sub-tile i live in the PAR set,
+  // those of i+-1 in the other.  Part 1 issues the transposing V reads for sub-tile i-1 and the S^T
+  // products on K operands that were read during the previous step; part 2 issues the K reads for
+  // sub-tile i+2, the P V products and the softmax.  Scheduling fences between the parts keep the
+  // register live ranges as written.
   // The FAST form assumes all three stages are live and sub-tile i needs no mask.  The general
   // form runs the same stages unconditionally and folds "stage not live" into the mask: a dead
   // softmax sees an empty key range (P = 0, state untouched), a dead S(i+1) is never read, and a
   // dead P V product multiplies finite LDS contents by P = 0.
-  auto step = [&](auto par_tag, auto fast_tag, int i) {
+  auto step = [&](auto par_tag, auto fast_tag, int i, int tk, int tv) {
     constexpr int PAR = decltype(par_tag)::value;
     constexpr bool FAST = decltype(fast_tag)::value;
+    f32x16(&s_cur)[2] = PAR ? s1 : s0;
+    f32x16(&s_nxt)[2] = PAR ? s0 : s1;
     u32x4(&pk_cur)[2][2] = PAR ? pk1 : pk0;
     u32x4(&pk_prv)[2][2] = PAR ? pk0 : pk1;
-    // sub-tile i+1 lives in K tile (i+1)/2, half !PAR; sub-tile i in V tile i/2, half PAR
-    const int ksub = lds_base + (((i + 1) >> 1) & 1) * kTileBytes + (PAR ^ 1) * (SUB * 256);
-    const int vsub = lds_base + kLdsV + (((i >> 1) + 3) % 3) * kTileBytes + PAR * (SUB * 256);
+    // sub-tile i-1 lives in V tile (i-1)/2, half !PAR; sub-tile i+2 in K tile (i+2)/2, half PAR
+    const int vsub = lds_base + kLdsV + (((i - 1) >> 1) & (kRing - 1)) * kTileBytes + (PAR ^ 1) * (SUB * 256);
+    const int ksub2 = lds_base + (((i + 2) >> 1) & (kRing - 1)) * kTileBytes + PAR * (SUB * 256);
     // the per-lane offsets are made opaque here so that the XOR-derived addresses are formed where
     // they are used instead of being hoisted into sixteen long-lived registers
     asm volatile("" : "+v"(koff0), "+v"(voffa0), "+v"(voffb0));
@@ -411,39 +442,69 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
       mi.n0 = live ? i * SUB : 0;
       mi.kv_len = live ? kv_len : 0;
     }
-    // scheduling fences between the three parts keep register live ranges as written: the K
-    // operands are requested first, the softmax shares its part with the P V products, and the
-    // V operands of the next step are requested together with the S^T products
-    f32x16 sv[2] = {s[0], s[1]};
-    u32x4 ka[8];
-    load_k_operands(ksub, koff0, ka);
-    __builtin_amdgcn_sched_barrier(0);
-    pv_stage(va, pk_prv, oacc);
-    const bool any = softmax_stage<!FAST>(sv, pk_cur, m_run, l_run, alpha, p.scale_log2, g, mi);
+    u32x4 va[2][4];
+    float m_use[2];
+    // part 1: transposing V reads for sub-tile i-1, S^T products, row maxima and the first query column
+    load_v_operands(vsub, voffa0, voffb0, va);
+    qk_stage<T>(ka, qreg, s_nxt);
+    if (FAST) load_tiles(fast_tag, tk, tv, 2 * (PAR ^ 1), 2 * (PAR ^ 1) + 1);
+    const bool any = softmax_max<!FAST>(s_cur, m_run, m_use, alpha, p.scale_log2, g, mi);
+    softmax_exp(s_cur[0], m_use[0], alpha[0], l_run[0], pk_cur[0], p.scale_log2);
     // P(i) and the row sums are only consumed later; pin their computation into this part so that
     // it overlaps the MFMAs here and does not keep the unpacked probabilities alive
-    asm volatile("" ::"v"(pk_cur[0][0]), "v"(pk_cur[0][1]), "v"(pk_cur[1][0]), "v"(pk_cur[1][1]), "v"(l_run[0]), "v"(l_run[1]),
-                 "v"(m_run[0]), "v"(m_run[1]));
+    asm volatile("" ::"v"(pk_cur[0][0]), "v"(pk_cur[0][1]), "v"(l_run[0]), "v"(m_run[0]), "v"(m_run[1]), "v"(alpha[1]), "v"(m_use[1]));
+    if (FAST) {
+#pragma unroll
+      for (int k = 0; k < 16; k++) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // one transposing V read
+        if (k == 5 || k == 11) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // one global->LDS tile load
+        __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);  // VALU
+      }
+    }
     __builtin_amdgcn_sched_barrier(0);
-    qk_stage<T>(ka, qreg, s);
-    load_v_operands(vsub, voffa0, voffb0, va);
+    // part 2: K reads for sub-tile i+2, P V products, the second query column
+    load_k_operands(ksub2, koff0, ka);
+    pv_stage(va, pk_prv, oacc);
+    if (FAST) load_tiles(fast_tag, tk, tv, 2 * (PAR ^ 1) + 1, 2 * (PAR ^ 1) + 2);
+    softmax_exp(s_cur[1], m_use[1], alpha[1], l_run[1], pk_cur[1], p.scale_log2);
+    asm volatile("" ::"v"(pk_cur[1][0]), "v"(pk_cur[1][1]), "v"(l_run[1]));
+    if (FAST) {
+#pragma unroll
+      for (int k = 0; k < 16; k++) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);             // MFMA
+        if (k < 8) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // one K read for the next step
+        if (k == 5 || k == 11) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // one global->LDS tile load
+        __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);             // VALU
+      }
+    }
     __builtin_amdgcn_sched_barrier(0);
     if (any) rescale_o(oacc, alpha);
   };
+  // Iteration `it` runs steps 2it-1 and 2it.  Tiles are requested two iterations before they are
+  // first read: the loads issued at the top of iteration `it` are K(it+3) and V(it+1), and the wait
+  // in front of the barrier only covers the loads issued up to iteration it-2 (each wave issues 8
+  // per iteration and they complete in order), so one iteration's worth of loads stays in flight.
   auto iteration = [&](auto fast_tag, int it) {
-    // after the barrier K tile it and V tiles it-1, it are resident; K(it+1) and V(it+1) are sent on their way
-    wait_vmem();
+#if LSATTN_EXP == 6
+    if (!decltype(fast_tag)::value) {
+      wait_vmem<8>();
+      __syncthreads();
+    }
+#else
+    if (DirectV<T>::value) wait_vmem<8>(); else wait_vmem<0>();
     __syncthreads();
-    load_tiles(fast_tag, it + 1, it + 1);
-    step(std::integral_constant<int, 1>{}, fast_tag, 2 * it - 1);
-    step(std::integral_constant<int, 0>{}, fast_tag, 2 * it);
+#endif
+    // the general form issues the 8 tile loads here; the fast form spreads them over its four parts
+    if (!decltype(fast_tag)::value) load_tiles(fast_tag, it + 3, it + 1);
+    step(std::integral_constant<int, 1>{}, fast_tag, 2 * it - 1, it + 3, it + 1);
+    step(std::integral_constant<int, 0>{}, fast_tag, 2 * it, it + 3, it + 1);
     store_v_tile(it + 1);
   };
 
   if (nt > 0) {
-    // the V buffers and the first V operands start finite (zero): the general step may multiply
-    // them by P = 0 before real data arrives
-    for (int i = tid; i < 3 * kTileBytes / 16; i += NWAVE * 64) *(u32x4*)(lds + kLdsV + i * 16) = u32x4{0, 0, 0, 0};
+    // the V ring starts finite (zero): the general step may multiply it by P = 0 before real data arrives
+    for (int i = tid; i < kRing * kTileBytes / 16; i += NWAVE * 64) *(u32x4*)(lds + kLdsV + i * 16) = u32x4{0, 0, 0, 0};
 #pragma unroll
     for (int qb = 0; qb < 2; qb++) {
 #pragma unroll
@@ -452,18 +513,25 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
         pk1[qb][jj] = u32x4{0, 0, 0, 0};
       }
 #pragma unroll
-      for (int i = 0; i < 16; i++) s[qb][i] = 0.f;
+      for (int i = 0; i < 16; i++) {
+        s0[qb][i] = 0.f;
+        s1[qb][i] = 0.f;
+      }
     }
-#pragma unroll
-    for (int jj = 0; jj < 2; jj++)
-#pragma unroll
-      for (int db = 0; db < 4; db++) va[jj][db] = u32x4{0, 0, 0, 0};
     __syncthreads();
-    load_tiles(std::false_type{}, 0, 0);
+    // K(0..2) and V(0); a V tile index of -1 is a clamped, harmless refill of a slot that is not read live
+    load_tiles(std::false_type{}, 0, -1);
+    store_v_tile(-1);
+    load_tiles(std::false_type{}, 1, -1);
+    store_v_tile(-1);
+    load_tiles(std::false_type{}, 2, 0);
     store_v_tile(0);
-    // iterations [1, fast_end) of this wave have all stages live and unmasked, and prefetch a full tile
+    wait_vmem<0>();
+    __syncthreads();
+    load_k_operands(lds_base, koff0, ka);
+    // iterations [1, fast_end) of this wave have all stages live and unmasked, and prefetch full tiles
     int fast_end = ns_w / 2 < (i_mask + 1) / 2 ? ns_w / 2 : (i_mask + 1) / 2;
-    if (fast_end > kv_len / BN - 1) fast_end = kv_len / BN - 1;
+    if (fast_end > kv_len / BN - 3) fast_end = kv_len / BN - 3;
     if (fast_end < 1) fast_end = 1;
     if (fast_end > nt + 1) fast_end = nt + 1;
     iteration(std::false_type{}, 0);
