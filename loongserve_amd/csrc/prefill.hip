@@ -94,13 +94,15 @@ __device__ __forceinline__ float other_half(float v, int upper) {
 }
 
 // LDS: a ring of four K tiles at [0, 64K) and a ring of four V tiles at [64K, 128K); a tile is [64 rows][16 chunks of 16 bytes]
-// and the chunk index is XORed with swz_bits(row), which makes the row-wise 16-byte K reads and the
-// transposing 8-byte V reads both bank-conflict free.
+// and the chunk index is XORed with swz_bits(row).
 constexpr int kTileBytes = BN * 256;
 constexpr int kRing = 4;  // tiles per ring
 constexpr int kLdsV = kRing * kTileBytes;
 constexpr int kLdsBytes = 2 * kRing * kTileBytes;
-__device__ __forceinline__ int swz_bits(int row) { return ((row & 3) << 2) | ((row >> 2) & 3); }
+// LDS moves 128 bytes per clock: eight lanes of a 16-byte read, sixteen lanes of an 8-byte read.  With
+// this XOR the eight K rows read together land in eight different 16-byte bank groups, and the four
+// V rows of a transposing read (32 contiguous bytes each) land in four different 32-byte groups.
+__device__ __forceinline__ int swz_bits(int row) { return ((row & 3) << 1) | ((row >> 2) & 1); }
 
 typedef __attribute__((address_space(3))) i16x4* lds_i16x4_ptr;
 typedef __attribute__((address_space(3))) void* lds_void_ptr;
@@ -337,8 +339,11 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
   // FULL: every row of tile t exists, so the per-lane offsets are added to a uniform tile base.
   // Otherwise the row index is clamped (rows past the chunk are masked later, the data only has
   // to stay finite and in bounds; a tile index past the walk prefetches into a free buffer).
-  auto load_tiles = [&](auto full_tag, int tk, int tv, int i_begin = 0, int i_end = 4) {
+  auto load_tiles = [&](auto full_tag, int tk, int tv, int i_begin = 0, int i_end = 4, bool do_k = true, bool do_v = true) {
     constexpr bool FULL = decltype(full_tag)::value;
+#if LSATTN_EXP == 12
+    if (FULL) return;
+#endif
 #pragma unroll
     for (int i = i_begin; i < i_end; i++) {
       const int r = 16 * wave + 4 * i + st_row;
@@ -371,11 +376,13 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
         // behind its back and does not put a full vector-memory wait in front of every later LDS read
         // (it cannot tell the ring slots apart).  Completion is tracked by hand: wait_vmem<8>() plus
         // the workgroup barrier at the top of the iteration in which a slot is first read.
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_base + kdst), "v"(ksrc) : "m0");
-        if (DirectV<T>::value)
-          asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_base + vdst), "v"(vsrc) : "m0");
-        else
-          vst[i] = *(const u32x4*)vsrc;
+        if (do_k) asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_base + kdst), "v"(ksrc) : "m0");
+        if (do_v) {
+          if (DirectV<T>::value)
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_base + vdst), "v"(vsrc) : "m0");
+          else
+            vst[i] = *(const u32x4*)vsrc;
+        }
         continue;
       }
       __builtin_amdgcn_global_load_lds((global_void_ptr)ksrc, (lds_void_ptr)(lds + kdst), 16, 0, 0);
@@ -444,41 +451,125 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
     }
     u32x4 va[2][4];
     float m_use[2];
-    // part 1: transposing V reads for sub-tile i-1, S^T products, row maxima and the first query column
-    load_v_operands(vsub, voffa0, voffb0, va);
-    qk_stage<T>(ka, qreg, s_nxt);
-    if (FAST) load_tiles(fast_tag, tk, tv, 2 * (PAR ^ 1), 2 * (PAR ^ 1) + 1);
-    const bool any = softmax_max<!FAST>(s_cur, m_run, m_use, alpha, p.scale_log2, g, mi);
-    softmax_exp(s_cur[0], m_use[0], alpha[0], l_run[0], pk_cur[0], p.scale_log2);
-    // P(i) and the row sums are only consumed later; pin their computation into this part so that
-    // it overlaps the MFMAs here and does not keep the unpacked probabilities alive
-    asm volatile("" ::"v"(pk_cur[0][0]), "v"(pk_cur[0][1]), "v"(l_run[0]), "v"(m_run[0]), "v"(m_run[1]), "v"(alpha[1]), "v"(m_use[1]));
-    if (FAST) {
+    bool any;
+    if (!FAST) {
+      // part 1: transposing V reads for sub-tile i-1, S^T products, row maxima and the first query column
+      load_v_operands(vsub, voffa0, voffb0, va);
+      qk_stage<T>(ka, qreg, s_nxt);
+      any = softmax_max<true>(s_cur, m_run, m_use, alpha, p.scale_log2, g, mi);
+      softmax_exp(s_cur[0], m_use[0], alpha[0], l_run[0], pk_cur[0], p.scale_log2);
+      __builtin_amdgcn_sched_barrier(0);
+      // part 2: K reads for sub-tile i+2, P V products, the second query column
+      load_k_operands(ksub2, koff0, ka);
+      pv_stage(va, pk_prv, oacc);
+      softmax_exp(s_cur[1], m_use[1], alpha[1], l_run[1], pk_cur[1], p.scale_log2);
+      __builtin_amdgcn_sched_barrier(0);
+    } else {
+      // Hand-placed form: each part is cut into 8 chunks of two MFMAs that share an A operand, the LDS
+      // reads issued that far ahead of their use, and a share of the softmax; a scheduling fence after
+      // every chunk keeps the issue order as written, so that consecutive MFMAs never chain on one
+      // accumulator and the matrix pipe always has vector work to hide behind.
+      const float sc = p.scale_log2;
+      float sv0[16], sv1[16];
+      float mx0 = -INFINITY, mx1 = -INFINITY;
+      float ps0 = 0.f, ps1 = 0.f;
+      const int va_base_a = vsub + voffa0, va_base_b = vsub + voffb0;
+      const int ka_base = ksub2 + koff0;
+      // ---- part 1: S(i+1) = K(i+1) Q^T, V reads for sub-tile i-1, maxima of S(i), query column 0 ----
 #pragma unroll
-      for (int k = 0; k < 16; k++) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
-        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // one transposing V read
-        if (k == 5 || k == 11) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // one global->LDS tile load
-        __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);  // VALU
-      }
-    }
-    __builtin_amdgcn_sched_barrier(0);
-    // part 2: K reads for sub-tile i+2, P V products, the second query column
-    load_k_operands(ksub2, koff0, ka);
-    pv_stage(va, pk_prv, oacc);
-    if (FAST) load_tiles(fast_tag, tk, tv, 2 * (PAR ^ 1) + 1, 2 * (PAR ^ 1) + 2);
-    softmax_exp(s_cur[1], m_use[1], alpha[1], l_run[1], pk_cur[1], p.scale_log2);
-    asm volatile("" ::"v"(pk_cur[1][0]), "v"(pk_cur[1][1]), "v"(l_run[1]));
-    if (FAST) {
+      for (int c = 0; c < 8; c++) {
+        if (c == 0) {
+          const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+          s_nxt[0] = Mfma<T>::run(ka[0], qreg[0][0], zero);
+          s_nxt[1] = Mfma<T>::run(ka[0], qreg[1][0], zero);
+        } else {
+          s_nxt[0] = Mfma<T>::run(ka[c], qreg[0][c], s_nxt[0]);
+          s_nxt[1] = Mfma<T>::run(ka[c], qreg[1][c], s_nxt[1]);
+        }
+        {
+          const int jj = c >> 2, db = c & 3;
+#if LSATTN_EXP == 10
+          va[jj][db] = u32x4{(uint32_t)va_base_a, (uint32_t)va_base_b, (uint32_t)jj, (uint32_t)db};
+#else
+          const i16x4 xa = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_ptr)((va_base_a ^ (db << 6)) + jj * (16 * 256)));
+          const i16x4 xb = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_ptr)((va_base_b ^ (db << 6)) + jj * (16 * 256)));
+          const u32x2 wa = __builtin_bit_cast(u32x2, xa), wb = __builtin_bit_cast(u32x2, xb);
+          va[jj][db] = u32x4{wa[0], wa[1], wb[0], wb[1]};
+#endif
+        }
+        if (c == 2 || c == 5) load_tiles(fast_tag, tk, tv, 2 * (PAR ^ 1), 2 * (PAR ^ 1) + 1, c == 2, c == 5);
+        if (c < 4) {
+          // S(i) leaves the accumulators, 8 values per chunk, and feeds the row maxima
 #pragma unroll
-      for (int k = 0; k < 16; k++) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);             // MFMA
-        if (k < 8) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // one K read for the next step
-        if (k == 5 || k == 11) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // one global->LDS tile load
-        __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);             // VALU
+          for (int e = 4 * c; e < 4 * c + 4; e++) {
+            sv0[e] = s_cur[0][e];
+            sv1[e] = s_cur[1][e];
+          }
+          mx0 = fmaxf(fmaxf(mx0, fmaxf(sv0[4 * c], sv0[4 * c + 1])), fmaxf(sv0[4 * c + 2], sv0[4 * c + 3]));
+          mx1 = fmaxf(fmaxf(mx1, fmaxf(sv1[4 * c], sv1[4 * c + 1])), fmaxf(sv1[4 * c + 2], sv1[4 * c + 3]));
+          asm volatile("" : "+v"(mx0), "+v"(mx1));
+        } else {
+          if (c == 4) {
+            mx0 = fmaxf(mx0, other_half(mx0, g)) * sc;
+            mx1 = fmaxf(mx1, other_half(mx1, g)) * sc;
+            const bool grow = (mx0 > m_run[0] + kLazyRescale) || (mx1 > m_run[1] + kLazyRescale);
+            any = __builtin_amdgcn_ballot_w64(grow) != 0;
+            const float mn0 = any ? fmaxf(m_run[0], mx0) : m_run[0];
+            const float mn1 = any ? fmaxf(m_run[1], mx1) : m_run[1];
+            alpha[0] = __builtin_amdgcn_exp2f(m_run[0] - mn0);
+            alpha[1] = __builtin_amdgcn_exp2f(m_run[1] - mn1);
+            m_run[0] = m_use[0] = mn0;
+            m_run[1] = m_use[1] = mn1;
+          }
+          // query column 0: 4 probabilities per chunk -> 2 packed words
+          const int e0 = 4 * (c - 4);
+          float pr[4];
+#pragma unroll
+#if LSATTN_EXP == 9
+          for (int e = 0; e < 4; e++) pr[e] = __builtin_fmaf(sv0[e0 + e], sc, -m_use[0]);
+#else
+          for (int e = 0; e < 4; e++) pr[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(sv0[e0 + e], sc, -m_use[0]));
+#endif
+          ps0 += (pr[0] + pr[1]) + (pr[2] + pr[3]);
+          const uint32_t w0 = pack2<F16>(pr[0], pr[1]), w1 = pack2<F16>(pr[2], pr[3]);
+          // elements e0..e0+3 are words (e0/2, e0/2+1) of the 8-word row: pk[jj = word/4][word%4]
+          pk_cur[0][(e0 >> 3)][(e0 >> 1) & 3] = w0;
+          pk_cur[0][(e0 >> 3)][((e0 >> 1) & 3) + 1] = w1;
+          asm volatile("" : "+v"(ps0));
+        }
+        __builtin_amdgcn_sched_barrier(0);
       }
+      l_run[0] = l_run[0] * alpha[0] + ps0;
+      // ---- part 2: O += V(i-1) P(i-1), K reads for sub-tile i+2, query column 1 ----
+#pragma unroll
+      for (int c = 0; c < 8; c++) {
+        {
+          const int jj = c >> 2, db = c & 3;
+          oacc[db][0] = Mfma<F16>::run(va[jj][db], pk_prv[0][jj], oacc[db][0]);
+          oacc[db][1] = Mfma<F16>::run(va[jj][db], pk_prv[1][jj], oacc[db][1]);
+        }
+#if LSATTN_EXP == 11
+        ka[c] = u32x4{(uint32_t)ka_base, (uint32_t)c, 0u, 0u};
+#else
+        ka[c] = *(const __attribute__((address_space(3))) u32x4*)(ka_base ^ (c << 5));
+#endif
+        if (c == 2 || c == 5) load_tiles(fast_tag, tk, tv, 2 * (PAR ^ 1) + 1, 2 * (PAR ^ 1) + 2, c == 2, c == 5);
+        {
+#if LSATTN_EXP == 9
+          const float p0 = __builtin_fmaf(sv1[2 * c], sc, -m_use[1]);
+          const float p1 = __builtin_fmaf(sv1[2 * c + 1], sc, -m_use[1]);
+#else
+          const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sv1[2 * c], sc, -m_use[1]));
+          const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(sv1[2 * c + 1], sc, -m_use[1]));
+#endif
+          ps1 += p0 + p1;
+          pk_cur[1][c >> 2][c & 3] = pack2<F16>(p0, p1);
+          asm volatile("" : "+v"(ps1));
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      l_run[1] = l_run[1] * alpha[1] + ps1;
     }
-    __builtin_amdgcn_sched_barrier(0);
     if (any) rescale_o(oacc, alpha);
   };
   // Iteration `it` runs steps 2it-1 and 2it.  Tiles are requested two iterations before they are
@@ -535,6 +626,9 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
     if (fast_end < 1) fast_end = 1;
     if (fast_end > nt + 1) fast_end = nt + 1;
     iteration(std::false_type{}, 0);
+    // nothing the compiler tracks on the vector-memory counter may be pending when the fast loop is
+    // entered, or it protects the loop header with a full wait that would also drain the prefetch
+    wait_vmem<0>();
     for (int it = 1; it < fast_end; it++) iteration(std::true_type{}, it);
     for (int it = fast_end; it <= nt; it++) iteration(std::false_type{}, it);
   }
