@@ -476,40 +476,41 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
       const int va_base_a = vsub + voffa0, va_base_b = vsub + voffb0;
       const int ka_base = ksub2 + koff0;
       // ---- part 1: S(i+1) = K(i+1) Q^T, V reads for sub-tile i-1, maxima of S(i), query column 0 ----
+      u32x2 vlo[2][4], vhi[2][4];
+      float pr0[16];
 #pragma unroll
-      for (int c = 0; c < 8; c++) {
+      for (int k = 0; k < 16; k++) {
+        const int c = k >> 1, qb = k & 1;
         if (c == 0) {
           const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-          s_nxt[0] = Mfma<T>::run(ka[0], qreg[0][0], zero);
-          s_nxt[1] = Mfma<T>::run(ka[0], qreg[1][0], zero);
+          s_nxt[qb] = Mfma<T>::run(ka[0], qreg[qb][0], zero);
         } else {
-          s_nxt[0] = Mfma<T>::run(ka[c], qreg[0][c], s_nxt[0]);
-          s_nxt[1] = Mfma<T>::run(ka[c], qreg[1][c], s_nxt[1]);
+          s_nxt[qb] = Mfma<T>::run(ka[c], qreg[qb][c], s_nxt[qb]);
         }
         {
+          // one transposing read per chunk: the pair (keys +0..3, keys +8..11) of V operand c
           const int jj = c >> 2, db = c & 3;
-#if LSATTN_EXP == 10
-          va[jj][db] = u32x4{(uint32_t)va_base_a, (uint32_t)va_base_b, (uint32_t)jj, (uint32_t)db};
-#else
-          const i16x4 xa = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_ptr)((va_base_a ^ (db << 6)) + jj * (16 * 256)));
-          const i16x4 xb = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_ptr)((va_base_b ^ (db << 6)) + jj * (16 * 256)));
-          const u32x2 wa = __builtin_bit_cast(u32x2, xa), wb = __builtin_bit_cast(u32x2, xb);
-          va[jj][db] = u32x4{wa[0], wa[1], wb[0], wb[1]};
-#endif
+          const int base = qb ? va_base_b : va_base_a;
+          const i16x4 x = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_ptr)((base ^ (db << 6)) + jj * (16 * 256)));
+          if (qb) vhi[jj][db] = __builtin_bit_cast(u32x2, x); else vlo[jj][db] = __builtin_bit_cast(u32x2, x);
         }
-        if (c == 2 || c == 5) load_tiles(fast_tag, tk, tv, 2 * (PAR ^ 1), 2 * (PAR ^ 1) + 1, c == 2, c == 5);
-        if (c < 4) {
-          // S(i) leaves the accumulators, 8 values per chunk, and feeds the row maxima
+        if (k == 5 || k == 11) load_tiles(fast_tag, tk, tv, 2 * (PAR ^ 1), 2 * (PAR ^ 1) + 1, k == 5, k == 11);
+        if (k < 8) {
+          // S(i) leaves the accumulators, 4 values per chunk, and feeds the row maxima
+          const int e0 = 4 * (k >> 1);
+          if (qb == 0) {
 #pragma unroll
-          for (int e = 4 * c; e < 4 * c + 4; e++) {
-            sv0[e] = s_cur[0][e];
-            sv1[e] = s_cur[1][e];
+            for (int e = e0; e < e0 + 4; e++) sv0[e] = s_cur[0][e];
+            mx0 = fmaxf(fmaxf(mx0, fmaxf(sv0[e0], sv0[e0 + 1])), fmaxf(sv0[e0 + 2], sv0[e0 + 3]));
+            asm volatile("" : "+v"(mx0));
+          } else {
+#pragma unroll
+            for (int e = e0; e < e0 + 4; e++) sv1[e] = s_cur[1][e];
+            mx1 = fmaxf(fmaxf(mx1, fmaxf(sv1[e0], sv1[e0 + 1])), fmaxf(sv1[e0 + 2], sv1[e0 + 3]));
+            asm volatile("" : "+v"(mx1));
           }
-          mx0 = fmaxf(fmaxf(mx0, fmaxf(sv0[4 * c], sv0[4 * c + 1])), fmaxf(sv0[4 * c + 2], sv0[4 * c + 3]));
-          mx1 = fmaxf(fmaxf(mx1, fmaxf(sv1[4 * c], sv1[4 * c + 1])), fmaxf(sv1[4 * c + 2], sv1[4 * c + 3]));
-          asm volatile("" : "+v"(mx0), "+v"(mx1));
         } else {
-          if (c == 4) {
+          if (k == 8) {
             mx0 = fmaxf(mx0, other_half(mx0, g)) * sc;
             mx1 = fmaxf(mx1, other_half(mx1, g)) * sc;
             const bool grow = (mx0 > m_run[0] + kLazyRescale) || (mx1 > m_run[1] + kLazyRescale);
@@ -521,20 +522,12 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
             m_run[0] = m_use[0] = mn0;
             m_run[1] = m_use[1] = mn1;
           }
-          // query column 0: 4 probabilities per chunk -> 2 packed words
-          const int e0 = 4 * (c - 4);
-          float pr[4];
-#pragma unroll
-#if LSATTN_EXP == 9
-          for (int e = 0; e < 4; e++) pr[e] = __builtin_fmaf(sv0[e0 + e], sc, -m_use[0]);
-#else
-          for (int e = 0; e < 4; e++) pr[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(sv0[e0 + e], sc, -m_use[0]));
-#endif
-          ps0 += (pr[0] + pr[1]) + (pr[2] + pr[3]);
-          const uint32_t w0 = pack2<F16>(pr[0], pr[1]), w1 = pack2<F16>(pr[2], pr[3]);
-          // elements e0..e0+3 are words (e0/2, e0/2+1) of the 8-word row: pk[jj = word/4][word%4]
-          pk_cur[0][(e0 >> 3)][(e0 >> 1) & 3] = w0;
-          pk_cur[0][(e0 >> 3)][((e0 >> 1) & 3) + 1] = w1;
+          // query column 0: 2 probabilities per chunk -> 1 packed word
+          const int e0 = 2 * (k - 8);
+          const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sv0[e0], sc, -m_use[0]));
+          const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(sv0[e0 + 1], sc, -m_use[0]));
+          ps0 += p0 + p1;
+          pk_cur[0][(e0 >> 3)][(e0 >> 1) & 3] = pack2<F16>(p0, p1);
           asm volatile("" : "+v"(ps0));
         }
         __builtin_amdgcn_sched_barrier(0);
@@ -542,28 +535,24 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
       l_run[0] = l_run[0] * alpha[0] + ps0;
       // ---- part 2: O += V(i-1) P(i-1), K reads for sub-tile i+2, query column 1 ----
 #pragma unroll
-      for (int c = 0; c < 8; c++) {
+      for (int k = 0; k < 16; k++) {
+        const int c = k >> 1, qb = k & 1;
         {
           const int jj = c >> 2, db = c & 3;
-          oacc[db][0] = Mfma<F16>::run(va[jj][db], pk_prv[0][jj], oacc[db][0]);
-          oacc[db][1] = Mfma<F16>::run(va[jj][db], pk_prv[1][jj], oacc[db][1]);
+          const u32x4 a = {vlo[jj][db][0], vlo[jj][db][1], vhi[jj][db][0], vhi[jj][db][1]};
+          oacc[db][qb] = Mfma<F16>::run(a, pk_prv[qb][jj], oacc[db][qb]);
         }
-#if LSATTN_EXP == 11
-        ka[c] = u32x4{(uint32_t)ka_base, (uint32_t)c, 0u, 0u};
-#else
-        ka[c] = *(const __attribute__((address_space(3))) u32x4*)(ka_base ^ (c << 5));
-#endif
-        if (c == 2 || c == 5) load_tiles(fast_tag, tk, tv, 2 * (PAR ^ 1) + 1, 2 * (PAR ^ 1) + 2, c == 2, c == 5);
+        if (qb == 0) ka[c] = *(const __attribute__((address_space(3))) u32x4*)(ka_base ^ (c << 5));
+        if (k == 5 || k == 11) load_tiles(fast_tag, tk, tv, 2 * (PAR ^ 1) + 1, 2 * (PAR ^ 1) + 2, k == 5, k == 11);
         {
-#if LSATTN_EXP == 9
-          const float p0 = __builtin_fmaf(sv1[2 * c], sc, -m_use[1]);
-          const float p1 = __builtin_fmaf(sv1[2 * c + 1], sc, -m_use[1]);
-#else
-          const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sv1[2 * c], sc, -m_use[1]));
-          const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(sv1[2 * c + 1], sc, -m_use[1]));
-#endif
-          ps1 += p0 + p1;
-          pk_cur[1][c >> 2][c & 3] = pack2<F16>(p0, p1);
+          // query column 1: 1 probability per chunk, packed every second chunk
+          const float pe = __builtin_amdgcn_exp2f(__builtin_fmaf(sv1[k], sc, -m_use[1]));
+          ps1 += pe;
+          if (qb == 0) {
+            pr0[c] = pe;
+          } else {
+            pk_cur[1][c >> 2][c & 3] = pack2<F16>(pr0[c], pe);
+          }
           asm volatile("" : "+v"(ps1));
         }
         __builtin_amdgcn_sched_barrier(0);
