@@ -268,7 +268,7 @@ def main():
             "config": {"workload": "config 3: token-indexed decode, batch 64, ctx U[4096,32768], GQA 32/8, head_dim 128, fp16, "
                                    "2.5M-slot scattered pool; stage1 (split-K, block_seq %d) + stage2" % d.BS,
                        "tokens": d.tokens, "algorithmic_gb_per_step": d.bytes / 1e9, "step_stats": st},
-            "roofline": {"kernel": "decode_stage1_kernel<F16,4,8>", "bound": "hbm", "achieved": ach, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+            "roofline": {"kernel": "decode_stage1_kernel<F16,4,4>", "bound": "hbm", "achieved": ach, "peak": PEAK_HBM_GBS, "unit": "GB/s",
                          "frac": ach / PEAK_HBM_GBS, "traffic": None, "per_launch_ms": s1},
         }
         if not args.no_cpu:

@@ -34,6 +34,15 @@ struct Stage1Params {
 
 constexpr int kTok = 8;  // K/V rows in flight per 16-lane group
 
+// sum over two packed 16-bit products with fp32 accumulation (v_dot2c_f32_f16 / v_dot2c_f32_bf16)
+template <typename T> __device__ __forceinline__ float dot2acc(uint32_t a, uint32_t b, float c);
+template <> __device__ __forceinline__ float dot2acc<F16>(uint32_t a, uint32_t b, float c) {
+  return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, a), __builtin_bit_cast(f16x2, b), c, false);
+}
+template <> __device__ __forceinline__ float dot2acc<BF16>(uint32_t a, uint32_t b, float c) {
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a), __builtin_bit_cast(bf16x2, b), c, false);
+}
+
 template <typename T, int GT, int NW>
 __global__ __launch_bounds__(NW * 64) void decode_stage1_kernel(Stage1Params p) {
   const int lane = threadIdx.x & 63;
@@ -62,19 +71,16 @@ __global__ __launch_bounds__(NW * 64) void decode_stage1_kernel(Stage1Params p) 
   const char* vbase = (const char*)p.v + ((int64_t)kvh * p.v_s1 + sub * 8) * 2;
   const int64_t k_row_bytes = p.k_s0 * 2, v_row_bytes = p.v_s0 * 2;
 
-  float qf[GT][8];
+  // q stays packed (8 elements = 4 words per head and lane); the scale is applied to the reduced dot
+  u32x4 qw[GT];
 #pragma unroll
-  for (int h = 0; h < GT; h++) {
-    const u32x4 w = *(const u32x4*)((const char*)p.q + ((b * p.hq + qh0 + h) * 128 + sub * 8) * 2);
-    unpack8<T>(w, qf[h]);
-#pragma unroll
-    for (int i = 0; i < 8; i++) qf[h][i] *= p.scale_log2;
-  }
+  for (int h = 0; h < GT; h++) qw[h] = *(const u32x4*)((const char*)p.q + ((b * p.hq + qh0 + h) * 128 + sub * 8) * 2);
 
   for (int64_t blk = blk_begin; blk < blk_end; blk++) {
     const int64_t t0 = blk * p.block_seq;
     int64_t t1 = t0 + p.block_seq;
     if (t1 > len) t1 = len;
+    const int64_t t_last = t1 - 1;
 
     float m[GT], l[GT], o[GT][8];
 #pragma unroll
@@ -85,69 +91,83 @@ __global__ __launch_bounds__(NW * 64) void decode_stage1_kernel(Stage1Params p) 
       for (int i = 0; i < 8; i++) o[h][i] = 0.f;
     }
 
-    // slot indices of the first batch of rows
+    // Slot indices of the first batch of rows.  A row position past the block repeats the block's
+    // last row (always a real slot): it is loaded like any other and dropped by the validity mask,
+    // so the loop body has no divergent control flow.
     int32_t slot[kTok];
 #pragma unroll
     for (int j = 0; j < kTok; j++) {
       const int64_t tok = t0 + j * 4 + grp;
-      slot[j] = tok < t1 ? table[tok] : -1;
+      slot[j] = table[tok < t1 ? tok : t_last];
     }
 
     for (int64_t it = t0; it < t1; it += 4 * kTok) {
       u32x4 kr[kTok], vr[kTok];
 #pragma unroll
-      for (int j = 0; j < kTok; j++) {
-        if (slot[j] >= 0) {
-          kr[j] = *(const u32x4*)(kbase + (int64_t)slot[j] * k_row_bytes);
-          vr[j] = *(const u32x4*)(vbase + (int64_t)slot[j] * v_row_bytes);
-        } else {
-          kr[j] = u32x4{0, 0, 0, 0};
-          vr[j] = u32x4{0, 0, 0, 0};
-        }
-      }
-      bool valid[kTok];
+      for (int j = 0; j < kTok; j++) kr[j] = *(const u32x4*)(kbase + (int64_t)slot[j] * k_row_bytes);
 #pragma unroll
-      for (int j = 0; j < kTok; j++) valid[j] = slot[j] >= 0;
-      // prefetch the slot indices of the next batch while the rows are in flight
+      for (int j = 0; j < kTok; j++) vr[j] = *(const u32x4*)(vbase + (int64_t)slot[j] * v_row_bytes);
+      // all 16 row loads are issued before anything else happens (the scheduler would otherwise sink
+      // each load next to its first use and expose its latency)
+      __builtin_amdgcn_sched_barrier(0);
+      // slot indices of the next batch while the rows are in flight
 #pragma unroll
       for (int j = 0; j < kTok; j++) {
         const int64_t tok = it + 4 * kTok + j * 4 + grp;
-        slot[j] = tok < t1 ? table[tok] : -1;
+        slot[j] = table[tok < t1 ? tok : t_last];
       }
+      __builtin_amdgcn_sched_barrier(0);
 
+      // raw dots (the softmax scale is folded into the exp2 argument); rows past the block only
+      // exist in its last batch and are masked there
+      const bool tail = it + 4 * kTok > t1;
       float s[kTok][GT];
 #pragma unroll
       for (int j = 0; j < kTok; j++) {
-        float kf[8];
-        unpack8<T>(kr[j], kf);
 #pragma unroll
         for (int h = 0; h < GT; h++) {
-          float d = 0.f;
+          float d = dot2acc<T>(qw[h][0], kr[j][0], 0.f);
+          d = dot2acc<T>(qw[h][1], kr[j][1], d);
+          d = dot2acc<T>(qw[h][2], kr[j][2], d);
+          d = dot2acc<T>(qw[h][3], kr[j][3], d);
+          s[j][h] = sum_row16(d);
+        }
+      }
+      if (tail) {
 #pragma unroll
-          for (int i = 0; i < 8; i++) d = __builtin_fmaf(qf[h][i], kf[i], d);
-          d = sum_row16(d);
-          s[j][h] = valid[j] ? d : -INFINITY;
+        for (int j = 0; j < kTok; j++) {
+          const bool valid = it + j * 4 + grp < t1;
+#pragma unroll
+          for (int h = 0; h < GT; h++) s[j][h] = valid ? s[j][h] : -INFINITY;
         }
       }
       float pj[kTok][GT];
+      float alpha[GT];
+      bool grow = false;
 #pragma unroll
       for (int h = 0; h < GT; h++) {
-        float mx = s[0][h];
+        float mx = fmaxf(s[0][h], s[1][h]);
 #pragma unroll
-        for (int j = 1; j < kTok; j++) mx = fmaxf(mx, s[j][h]);
-        const float m_new = fmaxf(m[h], mx);
+        for (int j = 2; j < kTok; j += 2) mx = fmaxf(mx, fmaxf(s[j][h], s[j + 1][h]));
+        const float m_new = fmaxf(m[h], mx * p.scale_log2);  // scale > 0
         const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
-        const float alpha = __builtin_amdgcn_exp2f(m[h] - m_safe);
+        alpha[h] = __builtin_amdgcn_exp2f(m[h] - m_safe);
+        grow |= m_new != m[h];
         float ps = 0.f;
 #pragma unroll
         for (int j = 0; j < kTok; j++) {
-          pj[j][h] = __builtin_amdgcn_exp2f(s[j][h] - m_safe);
+          pj[j][h] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[j][h], p.scale_log2, -m_safe));
           ps += pj[j][h];
         }
-        l[h] = l[h] * alpha + ps;
+        l[h] = l[h] * alpha[h] + ps;
         m[h] = m_new;
+      }
+      // the accumulators only need rescaling when some running max moved (rare once warmed up)
+      if (__builtin_amdgcn_ballot_w64(grow) != 0) {
 #pragma unroll
-        for (int i = 0; i < 8; i++) o[h][i] *= alpha;
+        for (int h = 0; h < GT; h++)
+#pragma unroll
+          for (int i = 0; i < 8; i++) o[h][i] *= alpha[h];
       }
 #pragma unroll
       for (int j = 0; j < kTok; j++) {
@@ -267,7 +287,10 @@ __global__ __launch_bounds__(256) void decode_stage2_kernel(Stage2Params p) {
 
 template <typename T, int GT>
 static int launch_stage1(const lsattn_decode_stage1_args* a, hipStream_t st) {
-  constexpr int NW = 8;
+#ifndef LSATTN_DECODE_NW
+#define LSATTN_DECODE_NW 4
+#endif
+  constexpr int NW = LSATTN_DECODE_NW;
   Stage1Params p;
   p.mid_o = a->mid_o;
   p.mid_lse = a->mid_o_logexpsum;
@@ -293,7 +316,10 @@ static int launch_stage1(const lsattn_decode_stage1_args* a, hipStream_t st) {
   p.tasks = (int)a->num_kv_heads * (group / GT);
   const int wgs_y = (p.tasks + NW - 1) / NW;
   // tokens per workgroup: at least ~1024, and few enough workgroups-per-launch to stay cheap
-  int64_t per_wg = (1024 + a->seq_block_size - 1) / a->seq_block_size;
+#ifndef LSATTN_DECODE_TOK_PER_WG
+#define LSATTN_DECODE_TOK_PER_WG 256
+#endif
+  int64_t per_wg = (LSATTN_DECODE_TOK_PER_WG + a->seq_block_size - 1) / a->seq_block_size;
   if (per_wg < 1) per_wg = 1;
   int64_t nblk = p.grid_blocks < a->num_blocks ? p.grid_blocks : a->num_blocks;
   if (nblk < 1) return LSATTN_OK;
