@@ -7,7 +7,7 @@ kernel launch per shard, then the fp32 partials are LSE-merged.  The same run al
 the token-indexed decode workload (config 3) and reports it next to the prefill number.
 Inputs are synthetic (seeded N(0,1)*0.5) and resident in HBM before the timed region.
 
-One JSON line goes to stdout; `--all` adds one (non-contract) line per other config.
+One JSON line goes to stdout; `--all` adds the other baseline configs under `other_configs`.
 """
 from __future__ import annotations
 
@@ -93,7 +93,7 @@ class RingPrefill:
             lsa.prefill_attention_step(self.q, c.k(self.Hkv), c.v(self.Hkv), self.qs, self.ql, self.qf, c.b_start_loc, c.b_seq_len,
                                        c.first_token_global_idx, 1, self.shard, ob, lb)
 
-    def cpu_baseline(self, heads=4, rows=2048):
+    def cpu_baseline(self, heads=8, rows=4096):
         """Oracle (PyTorch CPU fp32) on a slice: `heads` heads, the last `rows` query rows of the
         shard, against all four KV shards; scaled by algorithmic FLOPs."""
         from oracle import attn_oracle as orc
@@ -163,7 +163,7 @@ class TokenDecode:
         lsa.longserve_flash_decode_stage1(self.q, self.kv[:, :self.Hkv], self.kv[:, self.Hkv:], self.table, self.b_req, self.b_len,
                                           self.max_len, self.mid_o, self.mid_l, self.BS)
 
-    def cpu_baseline(self, nreq=8):
+    def cpu_baseline(self, nreq=64):
         from oracle import attn_oracle as orc
         torch.set_num_threads(os.cpu_count() or 1)
         idx = list(range(nreq))
@@ -192,10 +192,127 @@ class TokenDecode:
                           "(oracle/attn_oracle.py, PyTorch CPU fp32)" % (nreq, self.B, sum(lens), nbytes / 1e9, dt)}
 
 
+# --------------------------------------------------------------------------------------
+# config 4: long-context elastic decode, B=4 x 524288, MHA 32, 4 simulated instances
+# --------------------------------------------------------------------------------------
+class ElasticDecode:
+    def __init__(self, B=4, ctx=524288, H=32, D=128, n_inst=4, pool=2_200_000, dtype=torch.float16, seed=4000):
+        from loongserve_amd.simulate import DecodeInstance
+        g = torch.Generator().manual_seed(20244)
+        self.B, self.H, self.D, self.ctx, self.n_inst = B, H, D, ctx, n_inst
+        total = B * ctx
+        assert total <= pool
+        self.kv = _randn_half((pool, 2 * H, D), seed, dtype, chunk_rows=1 << 15)
+        self.q = _randn_half((B, H, D), seed + 1, dtype)
+        self.perm = torch.randperm(pool, generator=g)[:total].to(torch.int32).view(B, ctx)
+        part = ctx // n_inst
+        self.b_req = torch.arange(B, dtype=torch.int32, device=DEV)
+        self.instances = []
+        for r in range(n_inst):
+            table = self.perm[:, r * part:(r + 1) * part].contiguous().to(DEV)
+            self.instances.append(DecodeInstance(self.kv, table, self.b_req, _i32([part] * B), part))
+        self.full_table = self.perm.to(DEV)
+        self.ws = {}
+        self.out = torch.empty((B, H, D), dtype=dtype, device=DEV)
+        self.bytes = total * (2 * H * D * 2 + 4) + self.q.numel() * 2 + self.out.numel() * 2 + B * H * 4
+        self.tokens = total
+
+    def step(self):
+        from loongserve_amd.simulate import multi_instance_decode
+        return multi_instance_decode(self.q, self.instances, self.H, out=self.out, workspace=self.ws)
+
+
+# --------------------------------------------------------------------------------------
+# config 5: mixed varlen prefill, 24 sequences log-uniform in [1024, 200000], GQA 32/8, bf16,
+# K/V rows scattered to pool slots and registered during the pass
+# --------------------------------------------------------------------------------------
+class VarlenPrefill:
+    def __init__(self, n_seq=24, lo=1024, hi=200000, Hq=32, Hkv=8, D=128, dtype=torch.bfloat16, seed=5000, lens=None):
+        g = torch.Generator().manual_seed(20245)
+        if lens is None:
+            u = torch.rand(n_seq, generator=g, dtype=torch.float64)
+            lens = torch.round(torch.exp(math.log(lo) + u * (math.log(hi) - math.log(lo)))).to(torch.int64).tolist()
+        self.lens, self.Hq, self.Hkv, self.D = lens, Hq, Hkv, D
+        T = sum(lens)
+        self.T = T
+        self.q = _randn_half((T, Hq, D), seed, dtype, chunk_rows=1 << 16)
+        self.kv = _randn_half((T, 2 * Hkv, D), seed + 1, dtype)
+        self.o = torch.empty((T, Hq, D), dtype=dtype, device=DEV)
+        self.m = torch.empty((T, Hq), dtype=torch.float32, device=DEV)
+        self.l = torch.empty((T, Hq), dtype=torch.float32, device=DEV)
+        lens_t = torch.tensor(lens, dtype=torch.int64)
+        self.start = (torch.cumsum(lens_t, 0) - lens_t).to(torch.int32).to(DEV)
+        self.len = lens_t.to(torch.int32).to(DEV)
+        self.first = torch.zeros(n_seq if lens is None else len(lens), dtype=torch.int32, device=DEV)
+        self.max_len = max(lens)
+        pool_slots = T + 4096
+        self.pool = torch.zeros((pool_slots, 2 * Hkv, D), dtype=dtype, device=DEV)
+        self.mem_index = torch.randperm(pool_slots, generator=g)[:T].to(torch.int32).to(DEV)
+        self.b_req = torch.arange(len(lens), dtype=torch.int32, device=DEV)
+        self.req_to_token = torch.full((len(lens), self.max_len), 2147483647, dtype=torch.int32, device=DEV)
+        self.pairs = sum(n * (n + 1) // 2 for n in lens)
+        self.flops = 4 * D * Hq * self.pairs
+        self.scatter_bytes = T * 2 * Hkv * D * 2 * 2  # read + write of every K/V row
+
+    def attention(self):
+        import loongserve_amd as lsa
+        self.m.fill_(float("-inf"))
+        self.l.zero_()
+        lsa.context_attention_fwd(self.q, self.kv[:, :self.Hkv], self.kv[:, self.Hkv:], self.o, self.start, self.len, self.first,
+                                  self.start, self.len, self.first, 1, self.max_len, self.m, self.l)
+
+    def persist(self):
+        import loongserve_amd as lsa
+        lsa.kv_scatter(self.kv, self.mem_index, self.pool)
+        lsa.init_req_to_token_indexes(self.req_to_token, self.b_req, self.len, self.mem_index, self.start, self.max_len)
+
+    def step(self):
+        self.attention()
+        self.persist()
+
+
 def _stats(ms):
     s = sorted(ms)
     n = len(s)
     return {"median_ms": s[n // 2], "p10_ms": s[int(0.1 * (n - 1))], "p90_ms": s[int(math.ceil(0.9 * (n - 1)))], "mean_ms": sum(s) / n}
+
+
+def other_configs(steps):
+    """Configs 1, 4 and 5 of the baseline, timed the same way (not part of the one-line contract)."""
+    import loongserve_amd as lsa
+    out = {}
+    # config 1: single causal prefill, 2048 tokens, 32/32 heads
+    T, H, D = 2048, 32, 128
+    q, kv = _randn_half((T, H, D), 1001), _randn_half((T, 2 * H, D), 1002)
+    s0, ln, f0 = _i32([0]), _i32([T]), _i32([0])
+    ob = torch.empty((T, H, D), dtype=torch.float32, device=DEV)
+    lb = torch.empty((T, H), dtype=torch.float32, device=DEV)
+    ms = _time_events(lambda: lsa.prefill_attention_step(q, kv[:, :H], kv[:, H:], s0, ln, f0, s0, ln, f0, 1, T, ob, lb), 50, 10)
+    fl = 4 * D * H * (T * (T + 1) // 2)
+    st = _stats(ms)
+    out["config1"] = {"workload": "1 x 2048 causal, 32/32 heads, fp16", "median_ms": st["median_ms"], "tflops": fl / (st["median_ms"] * 1e-3) / 1e12,
+                      "pct_of_mfma_peak": 100 * fl / (st["median_ms"] * 1e-3) / 1e12 / PEAK_MFMA_TFLOPS}
+    del q, kv, ob, lb
+    # config 4
+    e = ElasticDecode()
+    ms = _time_events(e.step, steps, 2)
+    st = _stats(ms)
+    out["config4"] = {"workload": "decode 4 x 524288, MHA 32, 4 instances x (stage1+stage2) + merge", "median_ms": st["median_ms"],
+                      "gbs": e.bytes / (st["median_ms"] * 1e-3) / 1e9, "pct_of_hbm_peak": 100 * e.bytes / (st["median_ms"] * 1e-3) / 1e9 / PEAK_HBM_GBS}
+    del e
+    torch.cuda.empty_cache()
+    # config 5
+    v = VarlenPrefill()
+    ms_a = _time_events(v.attention, 3, 1)
+    ms_p = _time_events(v.persist, 5, 1)
+    sa, sp = _stats(ms_a), _stats(ms_p)
+    out["config5"] = {"workload": "24 packed sequences, %d tokens, GQA 32/8, bf16, causal + KV scatter/registration" % v.T,
+                      "attention_median_ms": sa["median_ms"], "tflops": v.flops / (sa["median_ms"] * 1e-3) / 1e12,
+                      "pct_of_mfma_peak": 100 * v.flops / (sa["median_ms"] * 1e-3) / 1e12 / PEAK_MFMA_TFLOPS,
+                      "scatter_median_ms": sp["median_ms"], "scatter_gbs": v.scatter_bytes / (sp["median_ms"] * 1e-3) / 1e9}
+    del v
+    torch.cuda.empty_cache()
+    return out
 
 
 def main():
@@ -205,6 +322,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     ap.add_argument("--only", choices=["prefill", "decode"], default=None, help="time one workload only (profiling aid)")
+    ap.add_argument("--calib-copy", action="store_true",
+                    help="only run three plain 1 GiB device-to-device copies (known traffic, for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE)")
+    ap.add_argument("--all", action="store_true", help="also time configs 1, 4 and 5 (reported under 'other_configs')")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU (no collectives, no second GPU); --gpus %d is not supported" % args.gpus,
@@ -215,6 +335,14 @@ def main():
         sys.exit(1)
     import loongserve_amd  # noqa: F401  (raises if liblsattn.so is missing)
     torch.cuda.set_device(0)
+    if args.calib_copy:
+        src = torch.ones(1 << 28, dtype=torch.float32, device=DEV)  # 1 GiB
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"calibration": "3 x copy of 1 GiB (reads 1048576 KiB, writes 1048576 KiB per copy)"}))
+        return
 
     line = {
         "metric": "prefill attn TFLOP/s + decode KV GB/s, as % of MI355X roofline (1 GPU)",
@@ -245,7 +373,10 @@ def main():
                                    "shards 3 (causal), 0, 1, 2 (full) + LSE merge; 32 heads MHA, head_dim 128, fp16",
                        "algorithmic_tflop_per_step": w.flops / 1e12, "launches_per_step": w.launches + 1, "step_stats": st},
             "roofline": {"kernel": "prefill_kernel<F16,0>", "bound": "mfma", "achieved": ach, "peak": PEAK_MFMA_TFLOPS, "unit": "TFLOP/s",
-                         "frac": ach / PEAK_MFMA_TFLOPS, "traffic": None,
+                         "frac": ach / PEAK_MFMA_TFLOPS,
+                         # HBM bytes per launch (read 772.8 MB + written 509.6 MB), rocprofv3 FETCH_SIZE / WRITE_SIZE scaled by a
+                         # plain copy: profiles/bench_default_hbm_traffic.txt
+                         "traffic": 1282.4e6,
                          "per_launch_ms": per_launch_ms, "algorithmic_tflop_per_launch": w.flops / w.launches / 1e12},
         })
         if not args.no_cpu:
@@ -269,7 +400,9 @@ def main():
                                    "2.5M-slot scattered pool; stage1 (split-K, block_seq %d) + stage2" % d.BS,
                        "tokens": d.tokens, "algorithmic_gb_per_step": d.bytes / 1e9, "step_stats": st},
             "roofline": {"kernel": "decode_stage1_kernel<F16,4,4>", "bound": "hbm", "achieved": ach, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                         "frac": ach / PEAK_HBM_GBS, "traffic": None, "per_launch_ms": s1},
+                         "frac": ach / PEAK_HBM_GBS,
+                         # HBM bytes per launch (read 5176.4 MB + written 81.9 MB), same source as above
+                         "traffic": 5258.3e6, "per_launch_ms": s1},
         }
         if not args.no_cpu:
             dec["cpu_baseline"] = d.cpu_baseline()
@@ -279,6 +412,8 @@ def main():
                 line["cpu_baseline"] = dec["cpu_baseline"]
         else:
             line["decode"] = dec
+    if args.all:
+        line["other_configs"] = other_configs(max(3, min(args.steps, 10)))
     print(json.dumps(line))
 
 

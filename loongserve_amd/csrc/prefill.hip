@@ -18,9 +18,6 @@
 //   * workgroup ids are mapped so that the workgroups sharing one KV head run on one XCD
 //     (ids are dealt round-robin to the 8 XCDs) and heavy (late) query tiles start first.
 #include <type_traits>
-#ifndef LSATTN_EXP
-#define LSATTN_EXP 0
-#endif
 
 #include "common.hip.h"
 
@@ -341,9 +338,6 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
   // to stay finite and in bounds; a tile index past the walk prefetches into a free buffer).
   auto load_tiles = [&](auto full_tag, int tk, int tv, int i_begin = 0, int i_end = 4, bool do_k = true, bool do_v = true) {
     constexpr bool FULL = decltype(full_tag)::value;
-#if LSATTN_EXP == 12
-    if (FULL) return;
-#endif
 #pragma unroll
     for (int i = i_begin; i < i_end; i++) {
       const int r = 16 * wave + 4 * i + st_row;
@@ -351,13 +345,8 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
       const char* vsrc;
       if (FULL) {
         // uniform (scalar) tile base + 32-bit per-lane offset
-#if LSATTN_EXP == 7
-        const char* kt = kg + (int64_t)(tk & 3) * BN * k_row_bytes;
-        const char* vt = vg + (int64_t)(tv & 3) * BN * v_row_bytes;
-#else
         const char* kt = kg + (int64_t)tk * BN * k_row_bytes;
         const char* vt = vg + (int64_t)tv * BN * v_row_bytes;
-#endif
         asm volatile("" : "+s"(kt), "+s"(vt));
         ksrc = kt + k_lane_off[i];
         vsrc = vt + v_lane_off[i];
@@ -566,15 +555,8 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
   // in front of the barrier only covers the loads issued up to iteration it-2 (each wave issues 8
   // per iteration and they complete in order), so one iteration's worth of loads stays in flight.
   auto iteration = [&](auto fast_tag, int it) {
-#if LSATTN_EXP == 6
-    if (!decltype(fast_tag)::value) {
-      wait_vmem<8>();
-      __syncthreads();
-    }
-#else
     if (DirectV<T>::value) wait_vmem<8>(); else wait_vmem<0>();
     __syncthreads();
-#endif
     // the general form issues the 8 tile loads here; the fast form spreads them over its four parts
     if (!decltype(fast_tag)::value) load_tiles(fast_tag, it + 3, it + 1);
     step(std::integral_constant<int, 1>{}, fast_tag, 2 * it - 1, it + 3, it + 1);
