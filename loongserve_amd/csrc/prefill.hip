@@ -96,10 +96,11 @@ constexpr int kTileBytes = BN * 256;
 constexpr int kRing = 4;  // tiles per ring
 constexpr int kLdsV = kRing * kTileBytes;
 constexpr int kLdsBytes = 2 * kRing * kTileBytes;
-// LDS moves 128 bytes per clock: eight lanes of a 16-byte read, sixteen lanes of an 8-byte read.  With
-// this XOR the eight K rows read together land in eight different 16-byte bank groups, and the four
-// V rows of a transposing read (32 contiguous bytes each) land in four different 32-byte groups.
-__device__ __forceinline__ int swz_bits(int row) { return ((row & 3) << 1) | ((row >> 2) & 1); }
+// LDS has 64 four-byte banks (256 bytes per clock): sixteen lanes of a 16-byte read, thirty-two lanes of
+// an 8-byte read are served together.  With this XOR the sixteen K rows read together land in sixteen
+// different 16-byte bank groups, and the four V rows of a transposing read (64 contiguous bytes each)
+// land in four different 64-byte groups; both patterns then run at the rate of a linear read.
+__device__ __forceinline__ int swz_bits(int row) { return ((row & 3) << 2) | ((row >> 2) & 3); }
 
 typedef __attribute__((address_space(3))) i16x4* lds_i16x4_ptr;
 typedef __attribute__((address_space(3))) void* lds_void_ptr;
@@ -665,6 +666,468 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
   }
 }
 
+// ------------------------------------------------------------------------------------------------
+// Eight-wave form: the same 256-row workgroup and the same three-sub-tile pipeline, but each wave owns
+// 32 query rows and two waves share a SIMD, so that one wave's vector work issues while the other
+// wave's MFMA holds the matrix pipe (a single wave cannot issue past its own MFMA for ~16 cycles).
+// Per wave: Q 32 + O^T 64 + S^T 2x16 accumulator registers, P^T 2x8.
+// ------------------------------------------------------------------------------------------------
+constexpr int NWAVE8 = 8;
+
+// a wave-uniform pointer, moved to scalar registers if the compiler held it in vector registers
+__device__ __forceinline__ const char* uniform_ptr(const char* ptr) {
+  const uint64_t u = (uint64_t)ptr;
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)u), hi = __builtin_amdgcn_readfirstlane((uint32_t)(u >> 32));
+  return (const char*)(((uint64_t)hi << 32) | lo);
+}
+
+template <bool MASK>
+__device__ __forceinline__ bool softmax32(f32x16& s, u32x4 (&pk)[2], float& m_run, float& l_run, float& alpha, float scale_log2, int g, int n0,
+                                          int kv_len, int kf, int P, int qpos) {
+  if (MASK) {
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+      const int n = n0 + (i >> 2) * 8 + 4 * g + (i & 3);
+      const bool vis = (n < kv_len) && (kf + n * P <= qpos);
+      s[i] = vis ? s[i] : -INFINITY;
+    }
+  }
+  float mx = fmaxf(s[0], s[1]);
+#pragma unroll
+  for (int i = 2; i < 16; i += 2) mx = fmaxf(mx, fmaxf(s[i], s[i + 1]));
+  mx = fmaxf(mx, other_half(mx, g)) * scale_log2;
+  const bool any = __builtin_amdgcn_ballot_w64(mx > m_run + kLazyRescale) != 0;
+  const float m_new = any ? fmaxf(m_run, mx) : m_run;
+  float m_use = m_new;
+  if (MASK) {
+    m_use = (m_new == -INFINITY) ? 0.f : m_new;
+    alpha = (m_run == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m_run - m_use);
+  } else {
+    alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+  }
+  m_run = m_new;
+  float ps0 = 0.f, ps1 = 0.f;
+#pragma unroll
+  for (int jj = 0; jj < 2; jj++) {
+    u32x4 w;
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[8 * jj + 2 * e], scale_log2, -m_use));
+      const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[8 * jj + 2 * e + 1], scale_log2, -m_use));
+      w[e] = pack2<F16>(p0, p1);
+      ps0 += p0;
+      ps1 += p1;
+    }
+    pk[jj] = w;
+  }
+  l_run = l_run * alpha + (ps0 + ps1);
+  return any;
+}
+
+template <typename T, int MODE>
+__global__ __launch_bounds__(NWAVE8 * 64, 1) void prefill_kernel8(PrefillParams p) {
+  __shared__ __attribute__((aligned(1024))) char lds[kLdsBytes];
+
+  const int group = p.hq / p.hkv;
+  int j = blockIdx.x >> 3;
+  const int xcd = blockIdx.x & 7;
+  const int gq = j % group;
+  j /= group;
+  const int zr = j % p.nz;
+  j /= p.nz;
+  const int slot = j % p.kv_slots;
+  const int b = j / p.kv_slots;
+  const int kvh = xcd + 8 * slot;
+  if (kvh >= p.hkv) return;
+  const int h = kvh * group + gq;
+  const int z = p.nz - 1 - zr;
+
+  const int q_len = p.q_len[b];
+  const int m_lo = z * BM;
+  if (m_lo >= q_len) return;
+  const int kv_len = p.kv_len[b];
+  const int64_t q_start = p.q_start[b], kv_start = p.kv_start[b];
+  const int qf = p.q_first[b], kf = p.kv_first[b];
+  const int P = p.peers;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int qc = lane & 31, g = lane >> 5;
+
+  auto visible_keys = [&](int qpos) -> int {
+    const int dq = qpos - kf;
+    const int n = dq >= 0 ? dq / P + 1 : 0;
+    return n > kv_len ? kv_len : n;
+  };
+  const int m_hi = (m_lo + BM < q_len ? m_lo + BM : q_len) - 1;
+  const int nt = (visible_keys(qf + m_hi * P) + BN - 1) / BN;
+
+  const int m_w0 = m_lo + wave * 32;
+  const bool wave_has_rows = m_w0 < q_len;
+  const int m_wlast = m_w0 + 31 > q_len - 1 ? q_len - 1 : m_w0 + 31;
+  const int ns_w = wave_has_rows ? (visible_keys(qf + m_wlast * P) + SUB - 1) / SUB : 0;
+  const int i_mask = wave_has_rows ? visible_keys(qf + m_w0 * P) / SUB : 0;
+
+  // Q as B operands: qreg[t] = Q[row qc][16t + 8g .. +7]
+  u32x4 qreg[8];
+  {
+    const int m = m_w0 + qc;
+    const bool ok = m < q_len;
+    const char* src = (const char*)p.q + ((q_start + (ok ? m : 0)) * p.q_st + (int64_t)h * p.q_sh + 8 * g) * 2;
+#pragma unroll
+    for (int t = 0; t < 8; t++) qreg[t] = ok ? *(const u32x4*)(src + t * 32) : u32x4{0, 0, 0, 0};
+  }
+
+  int koff0 = qc * 256 + ((g ^ swz_bits(qc)) << 4);
+  int voffa0, voffb0;
+  {
+    const int blk16 = lane >> 4, li = lane & 15;
+    const int row_a = 4 * (blk16 >> 1) + (li >> 2);
+    const int row_b = row_a + 8;
+    const int d_off = (blk16 & 1) * 16 + 4 * (li & 3);
+    voffa0 = row_a * 256 + (((d_off >> 3) ^ swz_bits(row_a)) << 4) + (d_off & 7) * 2;
+    voffb0 = row_b * 256 + (((d_off >> 3) ^ swz_bits(row_b)) << 4) + (d_off & 7) * 2;
+  }
+  const int lds_base = (int)(uintptr_t)(__attribute__((address_space(3))) char*)lds;
+
+  // staging: wave w owns rows [8w, 8w+8) of every tile, 4 rows per instruction
+  const char* kg = (const char*)p.k + (kv_start * p.k_st + (int64_t)kvh * p.k_sh) * 2;
+  const char* vg = (const char*)p.v + (kv_start * p.v_st + (int64_t)kvh * p.v_sh) * 2;
+  const int64_t k_row_bytes = p.k_st * 2, v_row_bytes = p.v_st * 2;
+  const int st_row = lane >> 4;
+  const int last_row = kv_len - 1;
+  uint32_t k_lane_off[2], v_lane_off[2];
+  int st_chunk[2];
+#pragma unroll
+  for (int i = 0; i < 2; i++) {
+    const int r = 8 * wave + 4 * i + st_row;
+    st_chunk[i] = ((lane & 15) ^ swz_bits(r)) << 4;
+    k_lane_off[i] = (uint32_t)(r * k_row_bytes) + st_chunk[i];
+    v_lane_off[i] = (uint32_t)(r * v_row_bytes) + st_chunk[i];
+  }
+  u32x4 vst[2];
+  auto load_tiles = [&](auto full_tag, int tk, int tv) __attribute__((always_inline)) {
+    constexpr bool FULL = decltype(full_tag)::value;
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+      const int r = 8 * wave + 4 * i + st_row;
+      const char* ksrc;
+      const char* vsrc;
+      if (FULL) {
+        const char* kt = kg + (int64_t)__builtin_amdgcn_readfirstlane(tk) * BN * k_row_bytes;
+        const char* vt = vg + (int64_t)__builtin_amdgcn_readfirstlane(tv) * BN * v_row_bytes;
+        kt = uniform_ptr(kt);
+        vt = uniform_ptr(vt);
+        ksrc = kt + k_lane_off[i];
+        vsrc = vt + v_lane_off[i];
+      } else {
+        int nk = tk * BN + r, nv = tv * BN + r;
+        nk = nk > last_row ? last_row : nk;
+        nv = nv > last_row ? last_row : nv;
+        nv = nv < 0 ? 0 : nv;
+        ksrc = kg + nk * k_row_bytes + st_chunk[i];
+        vsrc = vg + nv * v_row_bytes + st_chunk[i];
+      }
+      const int kdst = (tk & (kRing - 1)) * kTileBytes + (8 * wave + 4 * i) * 256;
+      const int vdst = kLdsV + (tv & (kRing - 1)) * kTileBytes + (8 * wave + 4 * i) * 256;
+      if (FULL) {
+        // issued from inline assembly: see the four-wave kernel
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_base + kdst), "v"(ksrc) : "m0");
+        if (DirectV<T>::value)
+          asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_base + vdst), "v"(vsrc) : "m0");
+        else
+          vst[i] = *(const u32x4*)vsrc;
+        continue;
+      }
+      __builtin_amdgcn_global_load_lds((global_void_ptr)ksrc, (lds_void_ptr)(lds + kdst), 16, 0, 0);
+      if (DirectV<T>::value) {
+        __builtin_amdgcn_global_load_lds((global_void_ptr)vsrc, (lds_void_ptr)(lds + vdst), 16, 0, 0);
+      } else {
+        vst[i] = *(const u32x4*)vsrc;
+      }
+    }
+  };
+  auto store_v_tile = [&](int tv) __attribute__((always_inline)) {
+    if (!DirectV<T>::value) {
+#pragma unroll
+      for (int i = 0; i < 2; i++)
+        *(u32x4*)(lds + kLdsV + (tv & (kRing - 1)) * kTileBytes + (8 * wave + 4 * i) * 256 + lane * 16) = to_pv_operand<T>(vst[i]);
+    }
+  };
+
+  f32x16 oacc[4];
+#pragma unroll
+  for (int db = 0; db < 4; db++)
+#pragma unroll
+    for (int i = 0; i < 16; i++) oacc[db][i] = 0.f;
+  float m_run = -INFINITY, l_run = 0.f, alpha = 1.f;
+  f32x16 s;
+  u32x4 pk[2];
+  u32x4 ka[8], va[2][4];
+  const int qpos = qf + (m_w0 + qc) * P;
+
+  // General step for sub-tile i: bounds-checked, masked, nothing carried over between steps.
+  auto step = [&](int i) __attribute__((always_inline)) {
+    if (i >= ns_w) return;  // no row of this wave sees a key of this sub-tile (wave-uniform)
+    const int ksub = lds_base + ((i >> 1) & (kRing - 1)) * kTileBytes + (i & 1) * (SUB * 256);
+    asm volatile("" : "+v"(koff0), "+v"(voffa0), "+v"(voffb0));
+    load_k_operands(ksub, koff0, ka);
+    load_v_operands(ksub + kLdsV, voffa0, voffb0, va);
+#pragma unroll
+    for (int i2 = 0; i2 < 16; i2++) s[i2] = 0.f;
+#pragma unroll
+    for (int t8 = 0; t8 < 8; t8++) s = Mfma<T>::run(ka[t8], qreg[t8], s);
+    const bool any = softmax32<true>(s, pk, m_run, l_run, alpha, p.scale_log2, g, i * SUB, kv_len, kf, P, qpos);
+    if (any) {
+      asm volatile("s_nop 15\n\ts_nop 7");  // inline assembly is outside the compiler's hazard bookkeeping
+#pragma unroll
+      for (int db = 0; db < 4; db++)
+#pragma unroll
+        for (int i2 = 0; i2 < 16; i2++) asm volatile("v_mul_f32 %0, %1, %0" : "+v"(oacc[db][i2]) : "v"(alpha));
+    }
+#pragma unroll
+    for (int jj = 0; jj < 2; jj++)
+#pragma unroll
+      for (int db = 0; db < 4; db++) oacc[db] = Mfma<F16>::run(va[jj][db], pk[jj], oacc[db]);
+  };
+  // Iteration `it` works on tile `it` (sub-tiles 2it, 2it+1) and issues the loads of K tile it+3 and
+  // V tile it+2.  The wait in the middle leaves only this iteration's loads in flight, so the previous
+  // iteration's are complete for every wave after the next barrier.
+  auto iteration = [&](int it) __attribute__((always_inline)) {
+    __syncthreads();
+    load_tiles(std::false_type{}, it + 3, it + 2);
+    step(2 * it);
+    if (DirectV<T>::value) wait_vmem<4>();
+    step(2 * it + 1);
+    store_v_tile(it + 2);
+  };
+
+  // Fast iterations: every key of the tile exists and is visible to every row of the workgroup, and the
+  // ring slot (it & 3 == R) is a compile-time constant, so every LDS read is a fixed register plus an
+  // immediate.  A step has an MFMA phase (S(i) = K(i) Q^T, then O += V(i-1) P(i-1), each operand register
+  // refilled for the next step right behind the MFMA that consumed it) and a softmax phase (P(i)).
+  // Running state in this form: neg_m = -m, thr_raw = (m + 2^kLazyRescale) / scale, l = l0 + l1.
+  int kaddr[8], vaddr_a[4], vaddr_b[4];
+  float neg_m = 0.f, thr_raw = 0.f, l0 = 0.f, l1 = 0.f;
+  const float scale = p.scale_log2, inv_scale = 1.f / p.scale_log2;
+  uint32_t ones = 0x3C003C00u;  // two fp16 ones
+  auto fphase_mfma = [&](auto par_tag, auto r_tag) __attribute__((always_inline)) {
+    constexpr int PAR = decltype(par_tag)::value;  // sub-tile i = 2it + PAR
+    constexpr int R = decltype(r_tag)::value;
+    constexpr int koff = (PAR ? ((R + 1) & 3) : R) * kTileBytes + (PAR ^ 1) * (SUB * 256);  // K sub-tile i+1
+    constexpr int voff = R * kTileBytes + PAR * (SUB * 256);                               // V sub-tile i
+#pragma unroll
+    for (int i2 = 0; i2 < 16; i2++) s[i2] = 0.f;
+#pragma unroll
+    for (int t8 = 0; t8 < 8; t8++) {
+      s = Mfma<T>::run(ka[t8], qreg[t8], s);
+      ka[t8] = *(const __attribute__((address_space(3))) u32x4*)(kaddr[t8] + koff);
+    }
+#pragma unroll
+    for (int jj = 0; jj < 2; jj++)
+#pragma unroll
+      for (int db = 0; db < 4; db++) {
+        oacc[db] = Mfma<F16>::run(va[jj][db], pk[jj], oacc[db]);
+        const i16x4 xa = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_ptr)(vaddr_a[db] + voff + jj * (16 * 256)));
+        const i16x4 xb = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_ptr)(vaddr_b[db] + voff + jj * (16 * 256)));
+        const u32x2 wa = __builtin_bit_cast(u32x2, xa), wb = __builtin_bit_cast(u32x2, xb);
+        va[jj][db] = u32x4{wa[0], wa[1], wb[0], wb[1]};
+      }
+#pragma unroll
+    for (int t8 = 0; t8 < 8; t8++) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    }
+#pragma unroll
+    for (int t8 = 0; t8 < 8; t8++) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  auto fphase_softmax = [&]() __attribute__((always_inline)) {
+    float ma = fmaxf(fmaxf(s[0], s[1]), s[2]), mb = fmaxf(fmaxf(s[8], s[9]), s[10]);
+    ma = fmaxf(fmaxf(ma, s[3]), s[4]);
+    mb = fmaxf(fmaxf(mb, s[11]), s[12]);
+    ma = fmaxf(fmaxf(ma, s[5]), s[6]);
+    mb = fmaxf(fmaxf(mb, s[13]), s[14]);
+    ma = fmaxf(fmaxf(ma, s[7]), s[15]);
+    float mx = fmaxf(ma, mb);
+    {
+      const unsigned u = __builtin_bit_cast(unsigned, mx);
+      auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+      mx = fmaxf(__builtin_bit_cast(float, r[0]), __builtin_bit_cast(float, r[1]));
+    }
+    if (__builtin_amdgcn_ballot_w64(mx > thr_raw) != 0) {
+      const float m_new = fminf(neg_m, -mx * scale);  // -max(m, mx*scale)
+      const float al = __builtin_amdgcn_exp2f(m_new - neg_m);
+      neg_m = m_new;
+      thr_raw = (kLazyRescale - m_new) * inv_scale;
+      // inline assembly is outside the compiler's hazard bookkeeping: the factor comes from a
+      // transcendental op and the accumulators from MFMAs that may still be in flight
+      asm volatile("s_nop 15\n\ts_nop 7");
+      asm volatile("v_mul_f32 %0, %1, %0" : "+v"(l0) : "v"(al));
+      asm volatile("v_mul_f32 %0, %1, %0" : "+v"(l1) : "v"(al));
+#pragma unroll
+      for (int db = 0; db < 4; db++)
+#pragma unroll
+        for (int i2 = 0; i2 < 16; i2++) asm volatile("v_mul_f32 %0, %1, %0" : "+v"(oacc[db][i2]) : "v"(al));
+    }
+#pragma unroll
+    for (int jj = 0; jj < 2; jj++) {
+      u32x4 w;
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[8 * jj + 2 * e], scale, neg_m));
+        const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[8 * jj + 2 * e + 1], scale, neg_m));
+        // the packed pair goes through a scalar: taking the dot product's operand from the vector
+        // element after the insertion makes this compiler read element 0 for every e
+        const uint32_t pp = pack2<F16>(p0, p1);
+        float& acc = (e & 1) ? l1 : l0;
+        acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, pp), __builtin_bit_cast(f16x2, ones), acc, false);
+        w[e] = pp;
+      }
+      pk[jj] = w;
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  // The two waves that share a SIMD (w and w + 4) run the fast loop half a step apart, one in its MFMA
+  // phase while the other is in its softmax phase; a workgroup barrier ends every phase.  With K loaded
+  // three tiles and V two tiles ahead, and the wait at the start of an iteration's second step, a tile is
+  // complete for both groups one barrier before its first read, and no read of the slot a load overwrites
+  // is still pending when the load is issued.
+  auto fast_iteration = [&](auto r_tag, int it) __attribute__((always_inline)) {
+    load_tiles(std::true_type{}, it + 3, it + 2);
+    __builtin_amdgcn_s_setprio(1);
+    fphase_mfma(std::integral_constant<int, 0>{}, r_tag);
+    __builtin_amdgcn_s_setprio(0);
+    __builtin_amdgcn_s_barrier();
+    fphase_softmax();
+    __builtin_amdgcn_s_barrier();
+    if (DirectV<T>::value) wait_vmem<4>();
+    __builtin_amdgcn_s_setprio(1);
+    fphase_mfma(std::integral_constant<int, 1>{}, r_tag);
+    __builtin_amdgcn_s_setprio(0);
+    __builtin_amdgcn_s_barrier();
+    fphase_softmax();
+    __builtin_amdgcn_s_barrier();
+    store_v_tile(it + 2);
+  };
+
+  if (nt > 0) {
+    load_tiles(std::false_type{}, 0, 0);
+    store_v_tile(0);
+    load_tiles(std::false_type{}, 1, 1);
+    store_v_tile(1);
+    load_tiles(std::false_type{}, 2, 1);
+    store_v_tile(1);
+    wait_vmem<0>();
+    // the fast loop's trip count is the same for every wave of the workgroup (it holds barriers):
+    // sub-tiles below i_mask_wg are visible to the first row of the workgroup, hence to all of them
+    const int i_mask_wg = visible_keys(qf + m_lo * P) / SUB;
+    int fast_end = i_mask_wg / 2;
+    if (fast_end > kv_len / BN - 3) fast_end = kv_len / BN - 3;
+    if (fast_end > nt) fast_end = nt;
+    int it = 0;
+    if (fast_end >= 4) {
+#pragma unroll
+      for (int t8 = 0; t8 < 8; t8++) {
+        kaddr[t8] = (lds_base + koff0) ^ (t8 << 5);
+        asm volatile("" : "+v"(kaddr[t8]));
+      }
+#pragma unroll
+      for (int db = 0; db < 4; db++) {
+        vaddr_a[db] = (lds_base + kLdsV + voffa0) ^ (db << 6);
+        vaddr_b[db] = (lds_base + kLdsV + voffb0) ^ (db << 6);
+        asm volatile("" : "+v"(vaddr_a[db]), "+v"(vaddr_b[db]));
+      }
+      neg_m = INFINITY;
+      thr_raw = -INFINITY;
+      asm volatile("" : "+v"(ones));
+      __syncthreads();
+      // operands of step 0; its "previous" product is V(tile 0) times a zero P
+      load_k_operands(lds_base, koff0, ka);
+      load_v_operands(lds_base + kLdsV, voffa0, voffb0, va);
+      pk[0] = u32x4{0, 0, 0, 0};
+      pk[1] = u32x4{0, 0, 0, 0};
+      if (wave >= 4) __builtin_amdgcn_s_barrier();
+      for (; it + 3 < fast_end; it += 4) {
+        fast_iteration(std::integral_constant<int, 0>{}, it);
+        fast_iteration(std::integral_constant<int, 1>{}, it + 1);
+        fast_iteration(std::integral_constant<int, 2>{}, it + 2);
+        fast_iteration(std::integral_constant<int, 3>{}, it + 3);
+      }
+      if (wave < 4) __builtin_amdgcn_s_barrier();
+      // the product of the last fast step is still owed
+#pragma unroll
+      for (int jj = 0; jj < 2; jj++)
+#pragma unroll
+        for (int db = 0; db < 4; db++) oacc[db] = Mfma<F16>::run(va[jj][db], pk[jj], oacc[db]);
+      m_run = -neg_m;
+      l_run = l0 + l1;
+    }
+    for (; it < nt; it++) iteration(it);
+  }
+
+  // ---- epilogue ----
+  {
+    const int m = m_w0 + qc;
+    const float l_tot = l_run + other_half(l_run, g);
+    if (m < q_len) {
+      const int64_t tok = q_start + m;
+      if (MODE == 0) {
+        const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+        float* orow = (float*)p.o + tok * p.o_st + (int64_t)h * p.o_sh;
+#pragma unroll
+        for (int db = 0; db < 4; db++)
+#pragma unroll
+          for (int i4 = 0; i4 < 4; i4++) {
+            const int d = db * 32 + i4 * 8 + 4 * g;
+            const f32x4 v = {oacc[db][i4 * 4 + 0] * inv, oacc[db][i4 * 4 + 1] * inv, oacc[db][i4 * 4 + 2] * inv, oacc[db][i4 * 4 + 3] * inv};
+            *(f32x4*)(orow + d) = v;
+          }
+        if (g == 0) p.lse[tok * p.hq + h] = l_tot > 0.f ? (m_run + __builtin_amdgcn_logf(l_tot)) * kLn2 : -INFINITY;
+      } else {
+        float* mp = p.m + tok * p.ml_st + (int64_t)h * p.ml_sh;
+        float* lp = p.l + tok * p.ml_st + (int64_t)h * p.ml_sh;
+        const float m_old = *mp, l_old = *lp;
+        const float M = fmaxf(m_run, m_old);
+        if (M != -INFINITY && l_tot > 0.f) {
+          const float w_old = l_old * exp2_diff(m_old, M);
+          const float w_new = exp2_diff(m_run, M);
+          const float L = w_old + l_tot * w_new;
+          const float inv = 1.f / L;
+          uint16_t* orow = (uint16_t*)p.o + tok * p.o_st + (int64_t)h * p.o_sh;
+#pragma unroll
+          for (int db = 0; db < 4; db++)
+#pragma unroll
+            for (int i4 = 0; i4 < 4; i4++) {
+              const int d = db * 32 + i4 * 8 + 4 * g;
+              u32x2* dst = (u32x2*)(orow + d);
+              float o0, o1, o2, o3;
+              if (w_old != 0.f) {
+                const u32x2 old = *dst;
+                unpack2<T>(old[0], o0, o1);
+                unpack2<T>(old[1], o2, o3);
+              } else {
+                o0 = o1 = o2 = o3 = 0.f;
+              }
+              const float r0 = (o0 * w_old + oacc[db][i4 * 4 + 0] * w_new) * inv;
+              const float r1 = (o1 * w_old + oacc[db][i4 * 4 + 1] * w_new) * inv;
+              const float r2 = (o2 * w_old + oacc[db][i4 * 4 + 2] * w_new) * inv;
+              const float r3 = (o3 * w_old + oacc[db][i4 * 4 + 3] * w_new) * inv;
+              *dst = u32x2{pack2<T>(r0, r1), pack2<T>(r2, r3)};
+            }
+          if (g == 0) {
+            *mp = M;
+            *lp = L;
+          }
+        }
+      }
+    }
+  }
+}
+
 template <typename T, int MODE> static int launch_prefill(const lsattn_prefill_args* a, hipStream_t st) {
   PrefillParams p;
   p.q = a->q;
@@ -700,7 +1163,13 @@ template <typename T, int MODE> static int launch_prefill(const lsattn_prefill_a
   const int group = a->num_q_heads / a->num_kv_heads;
   const int64_t wgs = (int64_t)8 * group * p.nz * p.kv_slots * a->batch;
   if (wgs > 0x7fffffff) return LSATTN_ERR_INVALID_ARG;
-  hipLaunchKernelGGL((prefill_kernel<T, MODE>), dim3((unsigned)wgs), dim3(NWAVE * 64), 0, st, p);
+#ifndef LSATTN_PREFILL_WAVES
+#define LSATTN_PREFILL_WAVES 8
+#endif
+  if (LSATTN_PREFILL_WAVES == 8)
+    hipLaunchKernelGGL((prefill_kernel8<T, MODE>), dim3((unsigned)wgs), dim3(NWAVE8 * 64), 0, st, p);
+  else
+    hipLaunchKernelGGL((prefill_kernel<T, MODE>), dim3((unsigned)wgs), dim3(NWAVE * 64), 0, st, p);
   return check_launch();
 }
 
