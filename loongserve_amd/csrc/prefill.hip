@@ -855,6 +855,26 @@ __global__ __launch_bounds__(NWAVE8 * 64, 1) void prefill_kernel8(PrefillParams 
     }
   };
 
+  // Full tiles in the fast loop: running scalar tile pointers, the lane's 32-bit offset and the LDS
+  // destination of a compile-time ring slot, issued from inline assembly (see the four-wave kernel).
+  const char* kt_run = kg;
+  const char* vt_run = vg;
+  const int st_lds = lds_base + 8 * wave * 256;
+  auto load_tiles_fast = [&](auto r_tag) __attribute__((always_inline)) {
+    constexpr int R = decltype(r_tag)::value;
+    constexpr int kslot = ((R + 3) & 3) * kTileBytes, vslot = kLdsV + ((R + 2) & 3) * kTileBytes;
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(st_lds + kslot + i * 1024), "v"(k_lane_off[i]), "s"(kt_run) : "m0", "memory");
+      if (DirectV<T>::value)
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(st_lds + vslot + i * 1024), "v"(v_lane_off[i]), "s"(vt_run) : "m0", "memory");
+      else
+        vst[i] = *(const u32x4*)(vt_run + v_lane_off[i]);
+    }
+    kt_run += BN * k_row_bytes;
+    vt_run += BN * v_row_bytes;
+  };
+
   f32x16 oacc[4];
 #pragma unroll
   for (int db = 0; db < 4; db++)
@@ -908,9 +928,8 @@ __global__ __launch_bounds__(NWAVE8 * 64, 1) void prefill_kernel8(PrefillParams 
   // refilled for the next step right behind the MFMA that consumed it) and a softmax phase (P(i)).
   // Running state in this form: neg_m = -m, thr_raw = (m + 2^kLazyRescale) / scale, l = l0 + l1.
   int kaddr[8], vaddr_a[4], vaddr_b[4];
-  float neg_m = 0.f, thr_raw = 0.f, l0 = 0.f, l1 = 0.f;
+  float neg_m = 0.f, thr_raw = 0.f, l0 = 0.f, l1 = 0.f, l2 = 0.f, l3 = 0.f;
   const float scale = p.scale_log2, inv_scale = 1.f / p.scale_log2;
-  uint32_t ones = 0x3C003C00u;  // two fp16 ones
   auto fphase_mfma = [&](auto par_tag, auto r_tag) __attribute__((always_inline)) {
     constexpr int PAR = decltype(par_tag)::value;  // sub-tile i = 2it + PAR
     constexpr int R = decltype(r_tag)::value;
@@ -945,20 +964,51 @@ __global__ __launch_bounds__(NWAVE8 * 64, 1) void prefill_kernel8(PrefillParams 
     }
     __builtin_amdgcn_sched_barrier(0);
   };
+  // P(i) = exp2(S(i) * scale - m) with the current m, the sub-tile's row sums in d[0..3] and the lane's
+  // largest score as the result.  Stage by stage, sixteen independent operations at a time, the levels of
+  // the maximum's tree spread between them, plain fp32 adds for the sums: this wave's vector work runs
+  // beside the other wave's MFMAs only without short dependent chains and without dot-product
+  // instructions (those queue behind the MFMAs).
+  auto compute_p = [&](float (&d)[4]) __attribute__((always_inline)) -> float {
+    float m6[6], t[16];
+    // maximum of the sixteen scores as a tree of three-input maxima: 5 + 2 + 1 operations
+#pragma unroll
+    for (int i = 0; i < 5; i++) m6[i] = fmaxf(fmaxf(s[3 * i], s[3 * i + 1]), s[3 * i + 2]);
+    m6[5] = s[15];
+#pragma unroll
+    for (int i = 0; i < 16; i++) t[i] = __builtin_fmaf(s[i], scale, neg_m);
+    __builtin_amdgcn_sched_barrier(0);
+    m6[0] = fmaxf(fmaxf(m6[0], m6[1]), m6[2]);
+    m6[3] = fmaxf(fmaxf(m6[3], m6[4]), m6[5]);
+#pragma unroll
+    for (int i = 0; i < 16; i++) t[i] = __builtin_amdgcn_exp2f(t[i]);
+    __builtin_amdgcn_sched_barrier(0);
+    const float mx = fmaxf(m6[0], m6[3]);
+#pragma unroll
+    for (int i = 0; i < 4; i++) d[i] = t[i] + t[i + 4];
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < 4; i++) d[i] += t[i + 8];
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < 4; i++) d[i] += t[i + 12];
+#pragma unroll
+    for (int jj = 0; jj < 2; jj++)
+#pragma unroll
+      for (int e = 0; e < 4; e++) pk[jj][e] = pack2<F16>(t[8 * jj + 2 * e], t[8 * jj + 2 * e + 1]);
+    __builtin_amdgcn_sched_barrier(0);
+    return mx;
+  };
   auto fphase_softmax = [&]() __attribute__((always_inline)) {
-    float ma = fmaxf(fmaxf(s[0], s[1]), s[2]), mb = fmaxf(fmaxf(s[8], s[9]), s[10]);
-    ma = fmaxf(fmaxf(ma, s[3]), s[4]);
-    mb = fmaxf(fmaxf(mb, s[11]), s[12]);
-    ma = fmaxf(fmaxf(ma, s[5]), s[6]);
-    mb = fmaxf(fmaxf(mb, s[13]), s[14]);
-    ma = fmaxf(fmaxf(ma, s[7]), s[15]);
-    float mx = fmaxf(ma, mb);
-    {
-      const unsigned u = __builtin_bit_cast(unsigned, mx);
-      auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
-      mx = fmaxf(__builtin_bit_cast(float, r[0]), __builtin_bit_cast(float, r[1]));
-    }
+    float d[4];
+    float mx = compute_p(d);
     if (__builtin_amdgcn_ballot_w64(mx > thr_raw) != 0) {
+      // rare: some score is above the lazy threshold; raise the running maximum and redo the sub-tile
+      {
+        const unsigned u = __builtin_bit_cast(unsigned, mx);
+        auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+        mx = fmaxf(__builtin_bit_cast(float, r[0]), __builtin_bit_cast(float, r[1]));
+      }
       const float m_new = fminf(neg_m, -mx * scale);  // -max(m, mx*scale)
       const float al = __builtin_amdgcn_exp2f(m_new - neg_m);
       neg_m = m_new;
@@ -968,50 +1018,42 @@ __global__ __launch_bounds__(NWAVE8 * 64, 1) void prefill_kernel8(PrefillParams 
       asm volatile("s_nop 15\n\ts_nop 7");
       asm volatile("v_mul_f32 %0, %1, %0" : "+v"(l0) : "v"(al));
       asm volatile("v_mul_f32 %0, %1, %0" : "+v"(l1) : "v"(al));
+      asm volatile("v_mul_f32 %0, %1, %0" : "+v"(l2) : "v"(al));
+      asm volatile("v_mul_f32 %0, %1, %0" : "+v"(l3) : "v"(al));
 #pragma unroll
       for (int db = 0; db < 4; db++)
 #pragma unroll
         for (int i2 = 0; i2 < 16; i2++) asm volatile("v_mul_f32 %0, %1, %0" : "+v"(oacc[db][i2]) : "v"(al));
+      compute_p(d);
     }
-#pragma unroll
-    for (int jj = 0; jj < 2; jj++) {
-      u32x4 w;
-#pragma unroll
-      for (int e = 0; e < 4; e++) {
-        const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[8 * jj + 2 * e], scale, neg_m));
-        const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[8 * jj + 2 * e + 1], scale, neg_m));
-        // the packed pair goes through a scalar: taking the dot product's operand from the vector
-        // element after the insertion makes this compiler read element 0 for every e
-        const uint32_t pp = pack2<F16>(p0, p1);
-        float& acc = (e & 1) ? l1 : l0;
-        acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, pp), __builtin_bit_cast(f16x2, ones), acc, false);
-        w[e] = pp;
-      }
-      pk[jj] = w;
-    }
+    l0 += d[0];
+    l1 += d[1];
+    l2 += d[2];
+    l3 += d[3];
     __builtin_amdgcn_sched_barrier(0);
   };
   // The two waves that share a SIMD (w and w + 4) run the fast loop half a step apart, one in its MFMA
-  // phase while the other is in its softmax phase; a workgroup barrier ends every phase.  With K loaded
-  // three tiles and V two tiles ahead, and the wait at the start of an iteration's second step, a tile is
-  // complete for both groups one barrier before its first read, and no read of the slot a load overwrites
-  // is still pending when the load is issued.
+  // phase while the other is in its softmax phase (at the higher priority, or the MFMA wave starves it);
+  // a workgroup barrier ends every phase.  The loads of K tile it+3 and V tile it+2 go out in the first
+  // softmax phase of iteration it; the wait before the iteration's second MFMA phase leaves only those
+  // in flight, so a tile is complete for both groups one barrier before its first read, and no read of
+  // the slot a load overwrites is still pending when the load is issued.
   auto fast_iteration = [&](auto r_tag, int it) __attribute__((always_inline)) {
-    load_tiles(std::true_type{}, it + 3, it + 2);
-    __builtin_amdgcn_s_setprio(1);
     fphase_mfma(std::integral_constant<int, 0>{}, r_tag);
-    __builtin_amdgcn_s_setprio(0);
     __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_s_setprio(3);
+    load_tiles_fast(r_tag);
     fphase_softmax();
+    __builtin_amdgcn_s_setprio(0);
     __builtin_amdgcn_s_barrier();
     if (DirectV<T>::value) wait_vmem<4>();
-    __builtin_amdgcn_s_setprio(1);
     fphase_mfma(std::integral_constant<int, 1>{}, r_tag);
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_s_setprio(3);
+    fphase_softmax();
+    store_v_tile(it + 2);
     __builtin_amdgcn_s_setprio(0);
     __builtin_amdgcn_s_barrier();
-    fphase_softmax();
-    __builtin_amdgcn_s_barrier();
-    store_v_tile(it + 2);
   };
 
   if (nt > 0) {
@@ -1043,13 +1085,14 @@ __global__ __launch_bounds__(NWAVE8 * 64, 1) void prefill_kernel8(PrefillParams 
       }
       neg_m = INFINITY;
       thr_raw = -INFINITY;
-      asm volatile("" : "+v"(ones));
       __syncthreads();
       // operands of step 0; its "previous" product is V(tile 0) times a zero P
       load_k_operands(lds_base, koff0, ka);
       load_v_operands(lds_base + kLdsV, voffa0, voffb0, va);
       pk[0] = u32x4{0, 0, 0, 0};
       pk[1] = u32x4{0, 0, 0, 0};
+      kt_run = uniform_ptr(kg + (int64_t)3 * BN * k_row_bytes);
+      vt_run = uniform_ptr(vg + (int64_t)2 * BN * v_row_bytes);
       if (wave >= 4) __builtin_amdgcn_s_barrier();
       for (; it + 3 < fast_end; it += 4) {
         fast_iteration(std::integral_constant<int, 0>{}, it);
@@ -1064,7 +1107,7 @@ __global__ __launch_bounds__(NWAVE8 * 64, 1) void prefill_kernel8(PrefillParams 
 #pragma unroll
         for (int db = 0; db < 4; db++) oacc[db] = Mfma<F16>::run(va[jj][db], pk[jj], oacc[db]);
       m_run = -neg_m;
-      l_run = l0 + l1;
+      l_run = (l0 + l1) + (l2 + l3);
     }
     for (; it < nt; it++) iteration(it);
   }
