@@ -868,8 +868,8 @@ __global__ __launch_bounds__(NWAVE8 * 64, 1) void prefill_kernel8(PrefillParams 
       asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(st_lds + kslot + i * 1024), "v"(k_lane_off[i]), "s"(kt_run) : "m0", "memory");
       if (DirectV<T>::value)
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(st_lds + vslot + i * 1024), "v"(v_lane_off[i]), "s"(vt_run) : "m0", "memory");
-      else
-        vst[i] = *(const u32x4*)(vt_run + v_lane_off[i]);
+      else  // the compiler does not see this load: fast_iteration waits for it before it stores the tile
+        asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(vst[i]) : "v"(v_lane_off[i]), "s"(vt_run) : "memory");
     }
     kt_run += BN * k_row_bytes;
     vt_run += BN * v_row_bytes;
@@ -1051,6 +1051,7 @@ __global__ __launch_bounds__(NWAVE8 * 64, 1) void prefill_kernel8(PrefillParams 
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_s_setprio(3);
     fphase_softmax();
+    if (!DirectV<T>::value) asm volatile("s_waitcnt vmcnt(0)" : "+v"(vst[0]), "+v"(vst[1]));
     store_v_tile(it + 2);
     __builtin_amdgcn_s_setprio(0);
     __builtin_amdgcn_s_barrier();
