@@ -4,17 +4,25 @@
 // (loongserve/models/llama/triton_kernel/ring_context_flashattention_nopad.py:13-284).
 //
 // Shape of the computation (head_dim 128):
-//   * a workgroup of 4 waves owns 256 consecutive local query rows of one (sequence, q head);
-//     each wave owns 64 of them and keeps their Q as MFMA B operands in registers;
-//   * K/V tiles of 64 keys are staged through LDS (double buffered, XOR-swizzled 16-byte
-//     chunks so that both the row-wise K reads and the transposing V reads are conflict free);
+//   * a workgroup of 8 waves owns 256 consecutive local query rows of one (sequence, q head);
+//     each wave owns 32 of them and keeps their Q as MFMA B operands in registers; waves w and
+//     w + 4 share a SIMD;
+//   * K/V tiles of 64 keys are staged through LDS (rings of four tiles, filled by global->LDS DMA,
+//     XOR-swizzled 16-byte chunks so that both the row-wise K reads and the transposing V reads
+//     use all 64 banks);
 //   * scores are computed transposed, S^T = K Q^T with v_mfma_f32_32x32x16, so every lane
 //     owns one query column: row max / row sum are in-lane reductions plus one
 //     half-wave swap, and the fp32 S^T accumulators convert in place into the B operand
-//     of O^T += V^T P^T without any cross-lane movement;
+//     of O^T += V^T P^T without any cross-lane movement (P and V always as fp16);
 //   * V^T operands come from LDS through ds_read_b64_tr_b16 (the tile is stored row-major);
-//   * causal work is skipped per wave (64 rows) and masks are applied only on tiles that
-//     straddle the diagonal or the end of the KV chunk;
+//   * on this hardware an MFMA holds its own wave until it is done, and vector work of the
+//     SIMD's other wave runs beside it only under conditions (higher wave priority, no short
+//     dependent chains, no dot-product instructions).  The fully visible part of the key range
+//     therefore runs as alternating phases: one wave of the SIMD issues the sixteen MFMAs of a
+//     32-key step while the other does the exponentials of its own step, a workgroup barrier
+//     ends each phase;
+//   * tiles that straddle the diagonal or the end of the KV chunk take a general, masked,
+//     bounds-checked step; causal work is skipped per wave;
 //   * workgroup ids are mapped so that the workgroups sharing one KV head run on one XCD
 //     (ids are dealt round-robin to the 8 XCDs) and heavy (late) query tiles start first.
 #include <type_traits>
@@ -44,10 +52,10 @@ struct PrefillParams {
   int64_t ml_st, ml_sh;
 };
 
-constexpr int BM = 256;   // query rows per workgroup (64 per wave)
+constexpr int BM = 256;   // query rows per workgroup (32 per wave)
 constexpr int BN = 64;    // keys per LDS tile
 constexpr int SUB = 32;   // keys per pipeline step (one 32x32 MFMA block row)
-constexpr int NWAVE = 4;
+constexpr int NWAVE = 8;  // two per SIMD
 constexpr float kLazyRescale = 8.f;  // log2 units the running max may lag before O is rescaled
 
 template <typename T> struct Mfma;
@@ -118,21 +126,6 @@ __device__ __forceinline__ void load_k_operands(int lds_k_sub, int koff0, u32x4 
 #pragma unroll
   for (int t8 = 0; t8 < 8; t8++) ka[t8] = *(const __attribute__((address_space(3))) u32x4*)(base ^ (t8 << 5));
 }
-// S^T block row of 32 keys x 64 queries: s[qb] = K[kb*32 .. +32) Q^T
-template <typename T>
-__device__ __forceinline__ void qk_stage(const u32x4 (&ka)[8], const u32x4 (&qreg)[2][8], f32x16 (&s)[2]) {
-#pragma unroll
-  for (int i = 0; i < 16; i++) {
-    s[0][i] = 0.f;
-    s[1][i] = 0.f;
-  }
-#pragma unroll
-  for (int t8 = 0; t8 < 8; t8++) {
-    s[0] = Mfma<T>::run(ka[t8], qreg[0][t8], s[0]);
-    s[1] = Mfma<T>::run(ka[t8], qreg[1][t8], s[1]);
-  }
-}
-
 // V^T A-operands of one 32-key sub-tile through transposing LDS reads
 // voffa0 / voffb0 are the lane's byte offsets for d-block 0 (keys base+4g'+r and +8); d-block db sits at
 // offset ^ (db << 6), the second group of 16 keys 4 KB further.
@@ -149,530 +142,6 @@ __device__ __forceinline__ void load_v_operands(int lds_v_sub, int voffa0, int v
     }
   }
 }
-// O^T += V^T[., 32 keys) P^T
-__device__ __forceinline__ void pv_stage(const u32x4 (&va)[2][4], const u32x4 (&pk)[2][2], f32x16 (&oacc)[4][2]) {
-#pragma unroll
-  for (int jj = 0; jj < 2; jj++) {
-#pragma unroll
-    for (int db = 0; db < 4; db++) {
-      oacc[db][0] = Mfma<F16>::run(va[jj][db], pk[0][jj], oacc[db][0]);
-      oacc[db][1] = Mfma<F16>::run(va[jj][db], pk[1][jj], oacc[db][1]);
-    }
-  }
-}
-
-// Online softmax of one 32-key block row for the two query columns of this lane.  The running
-// max only moves when some lane of the wave would otherwise exceed it by 2^kLazyRescale; the
-// factor the O accumulators then owe is returned in alpha (applied by the caller after the
-// P V products that still belong to the old max).
-struct MaskInfo {
-  int n0, kv_len, kf, P, qpos0, qpos1;  // sub-tile start, bounds and the two query positions
-};
-// Part 1 of the softmax: mask (if needed), row max of both query columns, the wave-uniform
-// decision whether the running max moves, and the factors that follow from it.
-template <bool MASK>
-__device__ __forceinline__ bool softmax_max(f32x16 (&s)[2], float (&m_run)[2], float (&m_use)[2], float (&alpha)[2], float scale_log2, int g,
-                                            const MaskInfo& mi) {
-  float scaled[2];
-#pragma unroll
-  for (int qb = 0; qb < 2; qb++) {
-    if (MASK) {
-      const int qpos = qb ? mi.qpos1 : mi.qpos0;
-#pragma unroll
-      for (int i = 0; i < 16; i++) {
-        const int n = mi.n0 + (i >> 2) * 8 + 4 * g + (i & 3);
-        const bool vis = (n < mi.kv_len) && (mi.kf + n * mi.P <= qpos);
-        s[qb][i] = vis ? s[qb][i] : -INFINITY;
-      }
-    }
-    float mx = fmaxf(s[qb][0], s[qb][1]);
-#pragma unroll
-    for (int i = 2; i < 16; i += 2) mx = fmaxf(mx, fmaxf(s[qb][i], s[qb][i + 1]));
-    mx = fmaxf(mx, other_half(mx, g));
-    scaled[qb] = mx * scale_log2;
-  }
-  const bool grow = (scaled[0] > m_run[0] + kLazyRescale) || (scaled[1] > m_run[1] + kLazyRescale);
-  const bool any = __builtin_amdgcn_ballot_w64(grow) != 0;
-#pragma unroll
-  for (int qb = 0; qb < 2; qb++) {
-    const float m_new = any ? fmaxf(m_run[qb], scaled[qb]) : m_run[qb];
-    m_use[qb] = m_new;
-    if (MASK) {
-      m_use[qb] = (m_new == -INFINITY) ? 0.f : m_new;
-      alpha[qb] = (m_run[qb] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m_run[qb] - m_use[qb]);
-    } else {
-      alpha[qb] = __builtin_amdgcn_exp2f(m_run[qb] - m_new);
-    }
-    m_run[qb] = m_new;
-  }
-  return any;
-}
-// Part 2, one query column: probabilities against m_use, packed to f16 as the B operand of the
-// P V product, and their fp32 row sum.
-__device__ __forceinline__ void softmax_exp(const f32x16& s, float m_use, float alpha, float& l_run, u32x4 (&pk)[2], float scale_log2) {
-  float ps0 = 0.f, ps1 = 0.f;
-#pragma unroll
-  for (int jj = 0; jj < 2; jj++) {
-    u32x4 w;
-#pragma unroll
-    for (int e = 0; e < 4; e++) {
-      const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[8 * jj + 2 * e], scale_log2, -m_use));
-      const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[8 * jj + 2 * e + 1], scale_log2, -m_use));
-      w[e] = pack2<F16>(p0, p1);
-      ps0 += p0;
-      ps1 += p1;
-    }
-    pk[jj] = w;
-  }
-  l_run = l_run * alpha + (ps0 + ps1);
-}
-
-__device__ __forceinline__ void rescale_o(f32x16 (&oacc)[4][2], const float (&alpha)[2]) {
-#pragma unroll
-  for (int db = 0; db < 4; db++)
-#pragma unroll
-    for (int qb = 0; qb < 2; qb++)
-#pragma unroll
-      for (int i = 0; i < 16; i++) {
-        // volatile asm: the multiply cannot be speculated, so the caller's branch around this
-        // (rarely needed) pass over the accumulators stays a branch
-        asm volatile("v_mul_f32 %0, %1, %0" : "+v"(oacc[db][qb][i]) : "v"(alpha[qb]));
-      }
-}
-
-template <typename T, int MODE>  // MODE 0: partial (o fp32, lse)   MODE 1: in-place (o, m, l) update
-__global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p) {
-  __shared__ __attribute__((aligned(1024))) char lds[kLdsBytes];
-
-  // ---- workgroup -> (sequence, q head, query tile) ----
-  const int group = p.hq / p.hkv;
-  int j = blockIdx.x >> 3;
-  const int xcd = blockIdx.x & 7;
-  const int gq = j % group;
-  j /= group;
-  const int zr = j % p.nz;
-  j /= p.nz;
-  const int slot = j % p.kv_slots;
-  const int b = j / p.kv_slots;
-  const int kvh = xcd + 8 * slot;
-  if (kvh >= p.hkv) return;
-  const int h = kvh * group + gq;
-  const int z = p.nz - 1 - zr;
-
-  // token counts and global positions are int32 in the interface; only byte offsets need 64 bits
-  const int q_len = p.q_len[b];
-  const int m_lo = z * BM;
-  if (m_lo >= q_len) return;
-  const int kv_len = p.kv_len[b];
-  const int64_t q_start = p.q_start[b], kv_start = p.kv_start[b];
-  const int qf = p.q_first[b], kf = p.kv_first[b];
-  const int P = p.peers;
-
-  const int tid = threadIdx.x;
-  const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int qc = lane & 31, g = lane >> 5;
-
-  // number of keys visible to global position qpos, clamped to the chunk
-  auto visible_keys = [&](int qpos) -> int {
-    const int dq = qpos - kf;
-    const int n = dq >= 0 ? dq / P + 1 : 0;
-    return n > kv_len ? kv_len : n;
-  };
-  const int m_hi = (m_lo + BM < q_len ? m_lo + BM : q_len) - 1;
-  const int nt = (visible_keys(qf + m_hi * P) + BN - 1) / BN;  // LDS tiles the workgroup walks
-
-  // ---- this wave's rows and its sub-tile range ----
-  const int m_w0 = m_lo + wave * 64;
-  const bool wave_has_rows = m_w0 < q_len;
-  const int m_wlast = m_w0 + 63 > q_len - 1 ? q_len - 1 : m_w0 + 63;
-  // sub-tiles [0, ns_w) hold a key some row of the wave sees; sub-tiles [0, i_mask) are seen
-  // entirely by every row of the wave (no mask needed)
-  const int ns_w = wave_has_rows ? (visible_keys(qf + m_wlast * P) + SUB - 1) / SUB : 0;
-  const int i_mask = wave_has_rows ? visible_keys(qf + m_w0 * P) / SUB : 0;
-
-  // Q as B operands: qreg[qb][t] = Q[row qb*32+qc][16t + 8g .. +7]
-  u32x4 qreg[2][8];
-#pragma unroll
-  for (int qb = 0; qb < 2; qb++) {
-    const int m = m_w0 + qb * 32 + qc;
-    const bool ok = m < q_len;
-    const char* src = (const char*)p.q + ((q_start + (ok ? m : 0)) * p.q_st + (int64_t)h * p.q_sh + 8 * g) * 2;
-#pragma unroll
-    for (int t = 0; t < 8; t++) qreg[qb][t] = ok ? *(const u32x4*)(src + t * 32) : u32x4{0, 0, 0, 0};
-  }
-
-  // ---- per-lane LDS byte offsets inside a tile ----
-  // K A-operand of k-step t8: row qc (+32 for the second half), logical chunk 2*t8+g
-  int koff0 = qc * 256 + ((g ^ swz_bits(qc)) << 4);
-  // V^T A-operand of d-block db via transposing reads: key rows base+4g'+(li>>2) (and +8), 4 consecutive
-  // elements starting at db*32 + (blk16&1)*16 + 4*(li&3)
-  int voffa0, voffb0;
-  {
-    const int blk16 = lane >> 4, li = lane & 15;
-    const int row_a = 4 * (blk16 >> 1) + (li >> 2);
-    const int row_b = row_a + 8;
-    const int d_off = (blk16 & 1) * 16 + 4 * (li & 3);
-    voffa0 = row_a * 256 + (((d_off >> 3) ^ swz_bits(row_a)) << 4) + (d_off & 7) * 2;
-    voffb0 = row_b * 256 + (((d_off >> 3) ^ swz_bits(row_b)) << 4) + (d_off & 7) * 2;
-  }
-  const int lds_base = (int)(uintptr_t)(__attribute__((address_space(3))) char*)lds;
-
-  // ---- global -> LDS staging: wave w owns rows [16w, 16w+16) of every tile, 4 rows per instruction.
-  // The lane that fills physical chunk slot (lane & 15) of row r fetches logical chunk slot ^ swz_bits(r).
-  const char* kg = (const char*)p.k + (kv_start * p.k_st + (int64_t)kvh * p.k_sh) * 2;
-  const char* vg = (const char*)p.v + (kv_start * p.v_st + (int64_t)kvh * p.v_sh) * 2;
-  const int64_t k_row_bytes = p.k_st * 2, v_row_bytes = p.v_st * 2;
-  const int st_row = lane >> 4;
-  const int last_row = kv_len - 1;
-  uint32_t k_lane_off[4], v_lane_off[4];  // byte offset of this lane's chunk inside a full tile
-  int st_chunk[4];
-#pragma unroll
-  for (int i = 0; i < 4; i++) {
-    const int r = 16 * wave + 4 * i + st_row;
-    st_chunk[i] = ((lane & 15) ^ swz_bits(r)) << 4;
-    k_lane_off[i] = (uint32_t)(r * k_row_bytes) + st_chunk[i];
-    v_lane_off[i] = (uint32_t)(r * v_row_bytes) + st_chunk[i];
-  }
-  u32x4 vst[4];  // V staging registers (element types whose V is converted on the way)
-  // FULL: every row of tile t exists, so the per-lane offsets are added to a uniform tile base.
-  // Otherwise the row index is clamped (rows past the chunk are masked later, the data only has
-  // to stay finite and in bounds; a tile index past the walk prefetches into a free buffer).
-  auto load_tiles = [&](auto full_tag, int tk, int tv, int i_begin = 0, int i_end = 4, bool do_k = true, bool do_v = true) {
-    constexpr bool FULL = decltype(full_tag)::value;
-#pragma unroll
-    for (int i = i_begin; i < i_end; i++) {
-      const int r = 16 * wave + 4 * i + st_row;
-      const char* ksrc;
-      const char* vsrc;
-      if (FULL) {
-        // uniform (scalar) tile base + 32-bit per-lane offset
-        const char* kt = kg + (int64_t)tk * BN * k_row_bytes;
-        const char* vt = vg + (int64_t)tv * BN * v_row_bytes;
-        asm volatile("" : "+s"(kt), "+s"(vt));
-        ksrc = kt + k_lane_off[i];
-        vsrc = vt + v_lane_off[i];
-      } else {
-        int nk = tk * BN + r, nv = tv * BN + r;
-        nk = nk > last_row ? last_row : nk;
-        nv = nv > last_row ? last_row : nv;
-        nv = nv < 0 ? 0 : nv;
-        ksrc = kg + nk * k_row_bytes + st_chunk[i];
-        vsrc = vg + nv * v_row_bytes + st_chunk[i];
-      }
-      const int kdst = (tk & (kRing - 1)) * kTileBytes + (16 * wave + 4 * i) * 256;
-      const int vdst = kLdsV + (tv & (kRing - 1)) * kTileBytes + (16 * wave + 4 * i) * 256;
-      if (FULL) {
-        // Issued from inline assembly on purpose: the compiler then does not know that LDS is written
-        // behind its back and does not put a full vector-memory wait in front of every later LDS read
-        // (it cannot tell the ring slots apart).  Completion is tracked by hand: wait_vmem<8>() plus
-        // the workgroup barrier at the top of the iteration in which a slot is first read.
-        if (do_k) asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_base + kdst), "v"(ksrc) : "m0");
-        if (do_v) {
-          if (DirectV<T>::value)
-            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_base + vdst), "v"(vsrc) : "m0");
-          else
-            vst[i] = *(const u32x4*)vsrc;
-        }
-        continue;
-      }
-      __builtin_amdgcn_global_load_lds((global_void_ptr)ksrc, (lds_void_ptr)(lds + kdst), 16, 0, 0);
-      if (DirectV<T>::value) {
-        __builtin_amdgcn_global_load_lds((global_void_ptr)vsrc, (lds_void_ptr)(lds + vdst), 16, 0, 0);
-      } else {
-        vst[i] = *(const u32x4*)vsrc;
-      }
-    }
-  };
-  auto store_v_tile = [&](int tv) {  // only for element types whose V goes through registers
-    if (!DirectV<T>::value) {
-#pragma unroll
-      for (int i = 0; i < 4; i++)
-        *(u32x4*)(lds + kLdsV + (tv & (kRing - 1)) * kTileBytes + (16 * wave + 4 * i) * 256 + lane * 16) = to_pv_operand<T>(vst[i]);
-    }
-  };
-
-  f32x16 oacc[4][2];
-#pragma unroll
-  for (int db = 0; db < 4; db++)
-#pragma unroll
-    for (int qb = 0; qb < 2; qb++)
-#pragma unroll
-      for (int i = 0; i < 16; i++) oacc[db][qb][i] = 0.f;
-  float m_run[2] = {-INFINITY, -INFINITY};
-  float l_run[2] = {0.f, 0.f};
-  f32x16 s0[2], s1[2];         // S^T of even / odd sub-tiles
-  u32x4 pk0[2][2], pk1[2][2];  // P^T of even / odd sub-tiles
-  u32x4 ka[8];                 // K operands of the sub-tile whose S^T product comes next
-  float alpha[2];
-  MaskInfo mi;
-  mi.kf = kf;
-  mi.P = P;
-  mi.qpos0 = qf + (m_w0 + qc) * P;
-  mi.qpos1 = qf + (m_w0 + 32 + qc) * P;
-
-  // One pipeline step on sub-tile i:  S(i+1) = K(i+1) Q^T,  P(i) = softmax(S(i)),  O += V(i-1) P(i-1).
-  // The three stages touch three different sub-tiles, so nothing in a step waits for a matrix
-  // product issued in the same step.  PAR is the parity of i: S/P of sub-tile i live in the PAR set,
-  // those of i+-1 in the other.  Part 1 issues the transposing V reads for sub-tile i-1 and the S^T
-  // products on K operands that were read during the previous step; part 2 issues the K reads for
-  // sub-tile i+2, the P V products and the softmax.  Scheduling fences between the parts keep the
-  // register live ranges as written.
-  // The FAST form assumes all three stages are live and sub-tile i needs no mask.  The general
-  // form runs the same stages unconditionally and folds "stage not live" into the mask: a dead
-  // softmax sees an empty key range (P = 0, state untouched), a dead S(i+1) is never read, and a
-  // dead P V product multiplies finite LDS contents by P = 0.
-  auto step = [&](auto par_tag, auto fast_tag, int i, int tk, int tv) {
-    constexpr int PAR = decltype(par_tag)::value;
-    constexpr bool FAST = decltype(fast_tag)::value;
-    f32x16(&s_cur)[2] = PAR ? s1 : s0;
-    f32x16(&s_nxt)[2] = PAR ? s0 : s1;
-    u32x4(&pk_cur)[2][2] = PAR ? pk1 : pk0;
-    u32x4(&pk_prv)[2][2] = PAR ? pk0 : pk1;
-    // sub-tile i-1 lives in V tile (i-1)/2, half !PAR; sub-tile i+2 in K tile (i+2)/2, half PAR
-    const int vsub = lds_base + kLdsV + (((i - 1) >> 1) & (kRing - 1)) * kTileBytes + (PAR ^ 1) * (SUB * 256);
-    const int ksub2 = lds_base + (((i + 2) >> 1) & (kRing - 1)) * kTileBytes + PAR * (SUB * 256);
-    // the per-lane offsets are made opaque here so that the XOR-derived addresses are formed where
-    // they are used instead of being hoisted into sixteen long-lived registers
-    asm volatile("" : "+v"(koff0), "+v"(voffa0), "+v"(voffb0));
-    if (!FAST) {
-      const bool live = i >= 0 && i < ns_w;
-      mi.n0 = live ? i * SUB : 0;
-      mi.kv_len = live ? kv_len : 0;
-    }
-    u32x4 va[2][4];
-    float m_use[2];
-    bool any;
-    if (!FAST) {
-      // part 1: transposing V reads for sub-tile i-1, S^T products, row maxima and the first query column
-      load_v_operands(vsub, voffa0, voffb0, va);
-      qk_stage<T>(ka, qreg, s_nxt);
-      any = softmax_max<true>(s_cur, m_run, m_use, alpha, p.scale_log2, g, mi);
-      softmax_exp(s_cur[0], m_use[0], alpha[0], l_run[0], pk_cur[0], p.scale_log2);
-      __builtin_amdgcn_sched_barrier(0);
-      // part 2: K reads for sub-tile i+2, P V products, the second query column
-      load_k_operands(ksub2, koff0, ka);
-      pv_stage(va, pk_prv, oacc);
-      softmax_exp(s_cur[1], m_use[1], alpha[1], l_run[1], pk_cur[1], p.scale_log2);
-      __builtin_amdgcn_sched_barrier(0);
-    } else {
-      // Hand-placed form: each part is cut into 8 chunks of two MFMAs that share an A operand, the LDS
-      // reads issued that far ahead of their use, and a share of the softmax; a scheduling fence after
-      // every chunk keeps the issue order as written, so that consecutive MFMAs never chain on one
-      // accumulator and the matrix pipe always has vector work to hide behind.
-      const float sc = p.scale_log2;
-      float sv0[16], sv1[16];
-      float mx0 = -INFINITY, mx1 = -INFINITY;
-      float ps0 = 0.f, ps1 = 0.f;
-      const int va_base_a = vsub + voffa0, va_base_b = vsub + voffb0;
-      const int ka_base = ksub2 + koff0;
-      // ---- part 1: S(i+1) = K(i+1) Q^T, V reads for sub-tile i-1, maxima of S(i), query column 0 ----
-      u32x2 vlo[2][4], vhi[2][4];
-      float pr0[16];
-#pragma unroll
-      for (int k = 0; k < 16; k++) {
-        const int c = k >> 1, qb = k & 1;
-        if (c == 0) {
-          const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-          s_nxt[qb] = Mfma<T>::run(ka[0], qreg[qb][0], zero);
-        } else {
-          s_nxt[qb] = Mfma<T>::run(ka[c], qreg[qb][c], s_nxt[qb]);
-        }
-        {
-          // one transposing read per chunk: the pair (keys +0..3, keys +8..11) of V operand c
-          const int jj = c >> 2, db = c & 3;
-          const int base = qb ? va_base_b : va_base_a;
-          const i16x4 x = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_ptr)((base ^ (db << 6)) + jj * (16 * 256)));
-          if (qb) vhi[jj][db] = __builtin_bit_cast(u32x2, x); else vlo[jj][db] = __builtin_bit_cast(u32x2, x);
-        }
-        if (k == 5 || k == 11) load_tiles(fast_tag, tk, tv, 2 * (PAR ^ 1), 2 * (PAR ^ 1) + 1, k == 5, k == 11);
-        if (k < 8) {
-          // S(i) leaves the accumulators, 4 values per chunk, and feeds the row maxima
-          const int e0 = 4 * (k >> 1);
-          if (qb == 0) {
-#pragma unroll
-            for (int e = e0; e < e0 + 4; e++) sv0[e] = s_cur[0][e];
-            mx0 = fmaxf(fmaxf(mx0, fmaxf(sv0[e0], sv0[e0 + 1])), fmaxf(sv0[e0 + 2], sv0[e0 + 3]));
-            asm volatile("" : "+v"(mx0));
-          } else {
-#pragma unroll
-            for (int e = e0; e < e0 + 4; e++) sv1[e] = s_cur[1][e];
-            mx1 = fmaxf(fmaxf(mx1, fmaxf(sv1[e0], sv1[e0 + 1])), fmaxf(sv1[e0 + 2], sv1[e0 + 3]));
-            asm volatile("" : "+v"(mx1));
-          }
-        } else {
-          if (k == 8) {
-            mx0 = fmaxf(mx0, other_half(mx0, g)) * sc;
-            mx1 = fmaxf(mx1, other_half(mx1, g)) * sc;
-            const bool grow = (mx0 > m_run[0] + kLazyRescale) || (mx1 > m_run[1] + kLazyRescale);
-            any = __builtin_amdgcn_ballot_w64(grow) != 0;
-            const float mn0 = any ? fmaxf(m_run[0], mx0) : m_run[0];
-            const float mn1 = any ? fmaxf(m_run[1], mx1) : m_run[1];
-            alpha[0] = __builtin_amdgcn_exp2f(m_run[0] - mn0);
-            alpha[1] = __builtin_amdgcn_exp2f(m_run[1] - mn1);
-            m_run[0] = m_use[0] = mn0;
-            m_run[1] = m_use[1] = mn1;
-          }
-          // query column 0: 2 probabilities per chunk -> 1 packed word
-          const int e0 = 2 * (k - 8);
-          const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sv0[e0], sc, -m_use[0]));
-          const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(sv0[e0 + 1], sc, -m_use[0]));
-          ps0 += p0 + p1;
-          pk_cur[0][(e0 >> 3)][(e0 >> 1) & 3] = pack2<F16>(p0, p1);
-          asm volatile("" : "+v"(ps0));
-        }
-        __builtin_amdgcn_sched_barrier(0);
-      }
-      l_run[0] = l_run[0] * alpha[0] + ps0;
-      // ---- part 2: O += V(i-1) P(i-1), K reads for sub-tile i+2, query column 1 ----
-#pragma unroll
-      for (int k = 0; k < 16; k++) {
-        const int c = k >> 1, qb = k & 1;
-        {
-          const int jj = c >> 2, db = c & 3;
-          const u32x4 a = {vlo[jj][db][0], vlo[jj][db][1], vhi[jj][db][0], vhi[jj][db][1]};
-          oacc[db][qb] = Mfma<F16>::run(a, pk_prv[qb][jj], oacc[db][qb]);
-        }
-        if (qb == 0) ka[c] = *(const __attribute__((address_space(3))) u32x4*)(ka_base ^ (c << 5));
-        if (k == 5 || k == 11) load_tiles(fast_tag, tk, tv, 2 * (PAR ^ 1) + 1, 2 * (PAR ^ 1) + 2, k == 5, k == 11);
-        {
-          // query column 1: 1 probability per chunk, packed every second chunk
-          const float pe = __builtin_amdgcn_exp2f(__builtin_fmaf(sv1[k], sc, -m_use[1]));
-          ps1 += pe;
-          if (qb == 0) {
-            pr0[c] = pe;
-          } else {
-            pk_cur[1][c >> 2][c & 3] = pack2<F16>(pr0[c], pe);
-          }
-          asm volatile("" : "+v"(ps1));
-        }
-        __builtin_amdgcn_sched_barrier(0);
-      }
-      l_run[1] = l_run[1] * alpha[1] + ps1;
-    }
-    if (any) rescale_o(oacc, alpha);
-  };
-  // Iteration `it` runs steps 2it-1 and 2it.  Tiles are requested two iterations before they are
-  // first read: the loads issued at the top of iteration `it` are K(it+3) and V(it+1), and the wait
-  // in front of the barrier only covers the loads issued up to iteration it-2 (each wave issues 8
-  // per iteration and they complete in order), so one iteration's worth of loads stays in flight.
-  auto iteration = [&](auto fast_tag, int it) {
-    if (DirectV<T>::value) wait_vmem<8>(); else wait_vmem<0>();
-    __syncthreads();
-    // the general form issues the 8 tile loads here; the fast form spreads them over its four parts
-    if (!decltype(fast_tag)::value) load_tiles(fast_tag, it + 3, it + 1);
-    step(std::integral_constant<int, 1>{}, fast_tag, 2 * it - 1, it + 3, it + 1);
-    step(std::integral_constant<int, 0>{}, fast_tag, 2 * it, it + 3, it + 1);
-    store_v_tile(it + 1);
-  };
-
-  if (nt > 0) {
-    // the V ring starts finite (zero): the general step may multiply it by P = 0 before real data arrives
-    for (int i = tid; i < kRing * kTileBytes / 16; i += NWAVE * 64) *(u32x4*)(lds + kLdsV + i * 16) = u32x4{0, 0, 0, 0};
-#pragma unroll
-    for (int qb = 0; qb < 2; qb++) {
-#pragma unroll
-      for (int jj = 0; jj < 2; jj++) {
-        pk0[qb][jj] = u32x4{0, 0, 0, 0};
-        pk1[qb][jj] = u32x4{0, 0, 0, 0};
-      }
-#pragma unroll
-      for (int i = 0; i < 16; i++) {
-        s0[qb][i] = 0.f;
-        s1[qb][i] = 0.f;
-      }
-    }
-    __syncthreads();
-    // K(0..2) and V(0); a V tile index of -1 is a clamped, harmless refill of a slot that is not read live
-    load_tiles(std::false_type{}, 0, -1);
-    store_v_tile(-1);
-    load_tiles(std::false_type{}, 1, -1);
-    store_v_tile(-1);
-    load_tiles(std::false_type{}, 2, 0);
-    store_v_tile(0);
-    wait_vmem<0>();
-    __syncthreads();
-    load_k_operands(lds_base, koff0, ka);
-    // iterations [1, fast_end) of this wave have all stages live and unmasked, and prefetch full tiles
-    int fast_end = ns_w / 2 < (i_mask + 1) / 2 ? ns_w / 2 : (i_mask + 1) / 2;
-    if (fast_end > kv_len / BN - 3) fast_end = kv_len / BN - 3;
-    if (fast_end < 1) fast_end = 1;
-    if (fast_end > nt + 1) fast_end = nt + 1;
-    iteration(std::false_type{}, 0);
-    // nothing the compiler tracks on the vector-memory counter may be pending when the fast loop is
-    // entered, or it protects the loop header with a full wait that would also drain the prefetch
-    wait_vmem<0>();
-    for (int it = 1; it < fast_end; it++) iteration(std::true_type{}, it);
-    for (int it = fast_end; it <= nt; it++) iteration(std::false_type{}, it);
-  }
-
-  // ---- epilogue ----
-#pragma unroll
-  for (int qb = 0; qb < 2; qb++) {
-    const int64_t m = m_w0 + qb * 32 + qc;
-    const float l_tot = l_run[qb] + other_half(l_run[qb], g);
-    if (m >= q_len) continue;
-    const int64_t tok = q_start + m;
-    if (MODE == 0) {
-      const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
-      float* orow = (float*)p.o + tok * p.o_st + (int64_t)h * p.o_sh;
-#pragma unroll
-      for (int db = 0; db < 4; db++)
-#pragma unroll
-        for (int i4 = 0; i4 < 4; i4++) {
-          const int d = db * 32 + i4 * 8 + 4 * g;
-          const f32x4 v = {oacc[db][qb][i4 * 4 + 0] * inv, oacc[db][qb][i4 * 4 + 1] * inv, oacc[db][qb][i4 * 4 + 2] * inv,
-                           oacc[db][qb][i4 * 4 + 3] * inv};
-          *(f32x4*)(orow + d) = v;
-        }
-      if (g == 0) p.lse[tok * p.hq + h] = l_tot > 0.f ? (m_run[qb] + __builtin_amdgcn_logf(l_tot)) * kLn2 : -INFINITY;
-    } else {
-      // RING:171-188: M = max(m_i, m_old); L = l_old 2^(m_old-M) + l_i 2^(m_i-M);
-      // o = (o_old l_old 2^(m_old-M) + acc 2^(m_i-M)) / L
-      float* mp = p.m + tok * p.ml_st + (int64_t)h * p.ml_sh;
-      float* lp = p.l + tok * p.ml_st + (int64_t)h * p.ml_sh;
-      const float m_old = *mp, l_old = *lp;
-      const float M = fmaxf(m_run[qb], m_old);
-      if (M == -INFINITY || l_tot <= 0.f) continue;  // nothing seen in this step: state unchanged
-      const float w_old = l_old * exp2_diff(m_old, M);
-      const float w_new = exp2_diff(m_run[qb], M);
-      const float L = w_old + l_tot * w_new;
-      const float inv = 1.f / L;
-      uint16_t* orow = (uint16_t*)p.o + tok * p.o_st + (int64_t)h * p.o_sh;
-#pragma unroll
-      for (int db = 0; db < 4; db++)
-#pragma unroll
-        for (int i4 = 0; i4 < 4; i4++) {
-          const int d = db * 32 + i4 * 8 + 4 * g;
-          u32x2* dst = (u32x2*)(orow + d);
-          float o0, o1, o2, o3;
-          if (w_old != 0.f) {
-            const u32x2 old = *dst;
-            unpack2<T>(old[0], o0, o1);
-            unpack2<T>(old[1], o2, o3);
-          } else {
-            o0 = o1 = o2 = o3 = 0.f;
-          }
-          const float r0 = (o0 * w_old + oacc[db][qb][i4 * 4 + 0] * w_new) * inv;
-          const float r1 = (o1 * w_old + oacc[db][qb][i4 * 4 + 1] * w_new) * inv;
-          const float r2 = (o2 * w_old + oacc[db][qb][i4 * 4 + 2] * w_new) * inv;
-          const float r3 = (o3 * w_old + oacc[db][qb][i4 * 4 + 3] * w_new) * inv;
-          *dst = u32x2{pack2<T>(r0, r1), pack2<T>(r2, r3)};
-        }
-      if (g == 0) {
-        *mp = M;
-        *lp = L;
-      }
-    }
-  }
-}
-
-// ------------------------------------------------------------------------------------------------
-// Eight-wave form: the same 256-row workgroup and the same three-sub-tile pipeline, but each wave owns
-// 32 query rows and two waves share a SIMD, so that one wave's vector work issues while the other
-// wave's MFMA holds the matrix pipe (a single wave cannot issue past its own MFMA for ~16 cycles).
-// Per wave: Q 32 + O^T 64 + S^T 2x16 accumulator registers, P^T 2x8.
-// ------------------------------------------------------------------------------------------------
-constexpr int NWAVE8 = 8;
 
 // a wave-uniform pointer, moved to scalar registers if the compiler held it in vector registers
 __device__ __forceinline__ const char* uniform_ptr(const char* ptr) {
@@ -725,7 +194,7 @@ __device__ __forceinline__ bool softmax32(f32x16& s, u32x4 (&pk)[2], float& m_ru
 }
 
 template <typename T, int MODE>
-__global__ __launch_bounds__(NWAVE8 * 64, 1) void prefill_kernel8(PrefillParams p) {
+__global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p) {
   __shared__ __attribute__((aligned(1024))) char lds[kLdsBytes];
 
   const int group = p.hq / p.hkv;
@@ -831,7 +300,9 @@ __global__ __launch_bounds__(NWAVE8 * 64, 1) void prefill_kernel8(PrefillParams 
       const int kdst = (tk & (kRing - 1)) * kTileBytes + (8 * wave + 4 * i) * 256;
       const int vdst = kLdsV + (tv & (kRing - 1)) * kTileBytes + (8 * wave + 4 * i) * 256;
       if (FULL) {
-        // issued from inline assembly: see the four-wave kernel
+        // issued from inline assembly: behind a load to LDS that the compiler sees, it waits for
+        // vmcnt(0) before every later LDS read (it cannot tell which LDS bytes the load writes);
+        // the waits for these loads are the explicit wait_vmem calls
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_base + kdst), "v"(ksrc) : "m0");
         if (DirectV<T>::value)
           asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_base + vdst), "v"(vsrc) : "m0");
@@ -856,7 +327,7 @@ __global__ __launch_bounds__(NWAVE8 * 64, 1) void prefill_kernel8(PrefillParams 
   };
 
   // Full tiles in the fast loop: running scalar tile pointers, the lane's 32-bit offset and the LDS
-  // destination of a compile-time ring slot, issued from inline assembly (see the four-wave kernel).
+  // destination of a compile-time ring slot, issued from inline assembly (as in load_tiles).
   const char* kt_run = kg;
   const char* vt_run = vg;
   const int st_lds = lds_base + 8 * wave * 256;
@@ -1207,13 +678,7 @@ template <typename T, int MODE> static int launch_prefill(const lsattn_prefill_a
   const int group = a->num_q_heads / a->num_kv_heads;
   const int64_t wgs = (int64_t)8 * group * p.nz * p.kv_slots * a->batch;
   if (wgs > 0x7fffffff) return LSATTN_ERR_INVALID_ARG;
-#ifndef LSATTN_PREFILL_WAVES
-#define LSATTN_PREFILL_WAVES 8
-#endif
-  if (LSATTN_PREFILL_WAVES == 8)
-    hipLaunchKernelGGL((prefill_kernel8<T, MODE>), dim3((unsigned)wgs), dim3(NWAVE8 * 64), 0, st, p);
-  else
-    hipLaunchKernelGGL((prefill_kernel<T, MODE>), dim3((unsigned)wgs), dim3(NWAVE * 64), 0, st, p);
+  hipLaunchKernelGGL((prefill_kernel<T, MODE>), dim3((unsigned)wgs), dim3(NWAVE * 64), 0, st, p);
   return check_launch();
 }
 
