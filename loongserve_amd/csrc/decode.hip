@@ -12,6 +12,8 @@
 //     result is deterministic;
 //   * a workgroup walks several consecutive blocks, so the launch is sized for the chip
 //     and not for block_seq.
+#include <type_traits>
+
 #include "common.hip.h"
 
 namespace lsattn {
@@ -34,6 +36,14 @@ struct Stage1Params {
 
 constexpr int kTok = 8;  // K/V rows in flight per 16-lane group
 
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N-1>): loop indices that must be constant expressions
+template <int N, typename F> __device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (N > 0) {
+    static_for<N - 1>(f);
+    f(std::integral_constant<int, N - 1>{});
+  }
+}
+
 // sum over two packed 16-bit products with fp32 accumulation (v_dot2c_f32_f16 / v_dot2c_f32_bf16)
 template <typename T> __device__ __forceinline__ float dot2acc(uint32_t a, uint32_t b, float c);
 template <> __device__ __forceinline__ float dot2acc<F16>(uint32_t a, uint32_t b, float c) {
@@ -42,6 +52,16 @@ template <> __device__ __forceinline__ float dot2acc<F16>(uint32_t a, uint32_t b
 template <> __device__ __forceinline__ float dot2acc<BF16>(uint32_t a, uint32_t b, float c) {
   return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a), __builtin_bit_cast(bf16x2, b), c, false);
 }
+// the same as volatile inline assembly, for sequences whose instruction order is fixed by hand
+template <typename T> struct Dot;
+template <> struct Dot<F16> {
+  static __device__ __forceinline__ void first(float& d, uint32_t a, uint32_t b) { asm volatile("v_dot2_f32_f16 %0, %1, %2, 0" : "=v"(d) : "v"(a), "v"(b)); }
+  static __device__ __forceinline__ void next(float& d, uint32_t a, uint32_t b) { asm volatile("v_dot2c_f32_f16 %0, %1, %2" : "+v"(d) : "v"(a), "v"(b)); }
+};
+template <> struct Dot<BF16> {
+  static __device__ __forceinline__ void first(float& d, uint32_t a, uint32_t b) { asm volatile("v_dot2_f32_bf16 %0, %1, %2, 0" : "=v"(d) : "v"(a), "v"(b)); }
+  static __device__ __forceinline__ void next(float& d, uint32_t a, uint32_t b) { asm volatile("v_dot2c_f32_bf16 %0, %1, %2" : "+v"(d) : "v"(a), "v"(b)); }
+};
 
 template <typename T, int GT, int NW>
 __global__ __launch_bounds__(NW * 64) void decode_stage1_kernel(Stage1Params p) {
@@ -49,6 +69,7 @@ __global__ __launch_bounds__(NW * 64) void decode_stage1_kernel(Stage1Params p) 
   const int wave = threadIdx.x >> 6;
   const int grp = lane >> 4;   // which of the 4 row slots of the wave
   const int sub = lane & 15;   // 16-byte column slot: elements sub*8 .. sub*8+7
+  const int jbase = (sub >> 2) * 2;  // first of the two rows whose scores this lane finishes (see the reduction)
   const int64_t b = blockIdx.z;
   const int task = blockIdx.y * NW + wave;
   if (task >= p.tasks) return;
@@ -57,8 +78,8 @@ __global__ __launch_bounds__(NW * 64) void decode_stage1_kernel(Stage1Params p) 
   const int kvh = task / sub_groups;
   const int qh0 = kvh * group + (task % sub_groups) * GT;
 
-  const int64_t len = p.b_seqlen[b];
-  int64_t nblk = len <= 0 ? 0 : (len + p.block_seq - 1) / p.block_seq;
+  const int len = p.b_seqlen[b];  // positions inside a request are 32-bit (max_seq_len is checked on the host)
+  int64_t nblk = len <= 0 ? 0 : ((int64_t)len + p.block_seq - 1) / p.block_seq;
   if (nblk > p.grid_blocks) nblk = p.grid_blocks;
   if (nblk > p.num_blocks) nblk = p.num_blocks;
   const int64_t blk_begin = (int64_t)blockIdx.x * p.blocks_per_wg;
@@ -77,10 +98,10 @@ __global__ __launch_bounds__(NW * 64) void decode_stage1_kernel(Stage1Params p) 
   for (int h = 0; h < GT; h++) qw[h] = *(const u32x4*)((const char*)p.q + ((b * p.hq + qh0 + h) * 128 + sub * 8) * 2);
 
   for (int64_t blk = blk_begin; blk < blk_end; blk++) {
-    const int64_t t0 = blk * p.block_seq;
-    int64_t t1 = t0 + p.block_seq;
-    if (t1 > len) t1 = len;
-    const int64_t t_last = t1 - 1;
+    const int t0 = (int)(blk * p.block_seq);
+    const int64_t t1_64 = (int64_t)t0 + p.block_seq;
+    const int t1 = t1_64 > len ? len : (int)t1_64;
+    const int t_last = t1 - 1;
 
     float m[GT], l[GT], o[GT][8];
 #pragma unroll
@@ -97,68 +118,107 @@ __global__ __launch_bounds__(NW * 64) void decode_stage1_kernel(Stage1Params p) 
     int32_t slot[kTok];
 #pragma unroll
     for (int j = 0; j < kTok; j++) {
-      const int64_t tok = t0 + j * 4 + grp;
+      const int tok = t0 + j * 4 + grp;
       slot[j] = table[tok < t1 ? tok : t_last];
     }
 
-    for (int64_t it = t0; it < t1; it += 4 * kTok) {
+    for (int it = t0; it < t1; it += 4 * kTok) {
       u32x4 kr[kTok], vr[kTok];
+      // (the empty statements keep each 64-bit address next to its load instead of sixteen of them live at once)
 #pragma unroll
-      for (int j = 0; j < kTok; j++) kr[j] = *(const u32x4*)(kbase + (int64_t)slot[j] * k_row_bytes);
+      for (int j = 0; j < kTok; j++) {
+        asm volatile("" : "+v"(slot[j]));
+        kr[j] = *(const u32x4*)(kbase + (int64_t)slot[j] * k_row_bytes);
+      }
 #pragma unroll
-      for (int j = 0; j < kTok; j++) vr[j] = *(const u32x4*)(vbase + (int64_t)slot[j] * v_row_bytes);
+      for (int j = 0; j < kTok; j++) {
+        asm volatile("" : "+v"(slot[j]));
+        vr[j] = *(const u32x4*)(vbase + (int64_t)slot[j] * v_row_bytes);
+      }
       // all 16 row loads are issued before anything else happens (the scheduler would otherwise sink
       // each load next to its first use and expose its latency)
       __builtin_amdgcn_sched_barrier(0);
       // slot indices of the next batch while the rows are in flight
 #pragma unroll
       for (int j = 0; j < kTok; j++) {
-        const int64_t tok = it + 4 * kTok + j * 4 + grp;
+        const int tok = it + 4 * kTok + j * 4 + grp;
         slot[j] = table[tok < t1 ? tok : t_last];
       }
       __builtin_amdgcn_sched_barrier(0);
 
-      // raw dots (the softmax scale is folded into the exp2 argument); rows past the block only
-      // exist in its last batch and are masked there
-      const bool tail = it + 4 * kTok > t1;
-      float s[kTok][GT];
+      // Partial dots over this lane's 8 elements for the 8 rows x GT heads of the group (value index
+      // v = GT*j + h), then a transposing reduction over the 16 lanes of the row group: two halving steps
+      // with bank-masked DPP adds (lanes with sub bits (3,2) = (B3,B2) keep values [NV/2*B3 + NV/4*B2, +NV/4))
+      // and a sum over the quad.  Every lane ends with the finished raw scores of two rows,
+      // jbase = 4*B3 + 2*B2 and jbase + 1, for all GT heads: w[GT*r + h].  The softmax scale is folded
+      // into the exp2 argument.
+      constexpr int NV = kTok * GT;
+      float u[NV / 2], w[NV / 4];
+      // Everything up to the quad sums is volatile inline assembly in a fixed order: a DPP read needs two
+      // wait states after the write of its source, the compiler's hazard recogniser does not look into inline
+      // assembly, and it would otherwise move the dots between the DPP adds.  The first halving step of a
+      // value pair (v, v + NV/2) follows the dots of the next pair, so only two partial dots are live at a time.
+      float lo_prev = 0.f, hi_prev = 0.f;
 #pragma unroll
-      for (int j = 0; j < kTok; j++) {
+      for (int i = 0; i < NV / 2; i++) {
+        const int j = i / GT, h = i % GT;
+        float lo, hi;
+        Dot<T>::first(lo, qw[h][0], kr[j][0]);
+        Dot<T>::first(hi, qw[h][0], kr[j + kTok / 2][0]);
 #pragma unroll
-        for (int h = 0; h < GT; h++) {
-          float d = dot2acc<T>(qw[h][0], kr[j][0], 0.f);
-          d = dot2acc<T>(qw[h][1], kr[j][1], d);
-          d = dot2acc<T>(qw[h][2], kr[j][2], d);
-          d = dot2acc<T>(qw[h][3], kr[j][3], d);
-          s[j][h] = sum_row16(d);
+        for (int c = 1; c < 4; c++) {
+          Dot<T>::next(lo, qw[h][c], kr[j][c]);
+          Dot<T>::next(hi, qw[h][c], kr[j + kTok / 2][c]);
         }
+        if (i > 0) {
+          asm volatile("v_add_f32_dpp %0, %1, %1 row_ror:8 row_mask:0xf bank_mask:0x3" : "=v"(u[i - 1]) : "v"(lo_prev));
+          asm volatile("v_add_f32_dpp %0, %1, %1 row_ror:8 row_mask:0xf bank_mask:0xc" : "+v"(u[i - 1]) : "v"(hi_prev));
+        }
+        lo_prev = lo;
+        hi_prev = hi;
       }
+      asm volatile("s_nop 1");
+      asm volatile("v_add_f32_dpp %0, %1, %1 row_ror:8 row_mask:0xf bank_mask:0x3" : "=v"(u[NV / 2 - 1]) : "v"(lo_prev));
+      asm volatile("v_add_f32_dpp %0, %1, %1 row_ror:8 row_mask:0xf bank_mask:0xc" : "+v"(u[NV / 2 - 1]) : "v"(hi_prev));
+      asm volatile("s_nop 1");
+#pragma unroll
+      for (int i = 0; i < NV / 4; i++) asm volatile("v_add_f32_dpp %0, %1, %1 row_ror:12 row_mask:0xf bank_mask:0x5" : "=v"(w[i]) : "v"(u[i]));
+      asm volatile("s_nop 1");
+#pragma unroll
+      for (int i = 0; i < NV / 4; i++) asm volatile("v_add_f32_dpp %0, %1, %1 row_ror:4 row_mask:0xf bank_mask:0xa" : "+v"(w[i]) : "v"(u[i + NV / 4]));
+      asm volatile("s_nop 1");
+#pragma unroll
+      for (int i = 0; i < NV / 4; i++) {
+        w[i] += dpp_mov<0xB1>(w[i]);  // quad_perm [1,0,3,2]
+        w[i] += dpp_mov<0x4E>(w[i]);  // quad_perm [2,3,0,1]
+      }
+      // rows past the block only exist in its last batch and are masked there
+      const bool tail = it + 4 * kTok > t1;
       if (tail) {
 #pragma unroll
-        for (int j = 0; j < kTok; j++) {
-          const bool valid = it + j * 4 + grp < t1;
+        for (int r = 0; r < 2; r++) {
+          const bool valid = it + (jbase + r) * 4 + grp < t1;
 #pragma unroll
-          for (int h = 0; h < GT; h++) s[j][h] = valid ? s[j][h] : -INFINITY;
+          for (int h = 0; h < GT; h++) w[GT * r + h] = valid ? w[GT * r + h] : -INFINITY;
         }
       }
-      float pj[kTok][GT];
+      float pw[2 * GT];
       float alpha[GT];
       bool grow = false;
 #pragma unroll
       for (int h = 0; h < GT; h++) {
-        float mx = fmaxf(s[0][h], s[1][h]);
-#pragma unroll
-        for (int j = 2; j < kTok; j += 2) mx = fmaxf(mx, fmaxf(s[j][h], s[j + 1][h]));
+        float mx = fmaxf(w[h], w[GT + h]);
+        mx = fmaxf(mx, dpp_mov<0x124>(mx));  // row_ror:4
+        mx = fmaxf(mx, dpp_mov<0x128>(mx));  // row_ror:8: now the maximum over the 8 rows, in every lane
         const float m_new = fmaxf(m[h], mx * p.scale_log2);  // scale > 0
         const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
         alpha[h] = __builtin_amdgcn_exp2f(m[h] - m_safe);
         grow |= m_new != m[h];
-        float ps = 0.f;
-#pragma unroll
-        for (int j = 0; j < kTok; j++) {
-          pj[j][h] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[j][h], p.scale_log2, -m_safe));
-          ps += pj[j][h];
-        }
+        pw[h] = __builtin_amdgcn_exp2f(__builtin_fmaf(w[h], p.scale_log2, -m_safe));
+        pw[GT + h] = __builtin_amdgcn_exp2f(__builtin_fmaf(w[GT + h], p.scale_log2, -m_safe));
+        float ps = pw[h] + pw[GT + h];
+        ps += dpp_mov<0x124>(ps);
+        ps += dpp_mov<0x128>(ps);
         l[h] = l[h] * alpha[h] + ps;
         m[h] = m_new;
       }
@@ -169,14 +229,41 @@ __global__ __launch_bounds__(NW * 64) void decode_stage1_kernel(Stage1Params p) 
 #pragma unroll
           for (int i = 0; i < 8; i++) o[h][i] *= alpha[h];
       }
+      if (std::is_same<T, F16>::value) {
+        // O += P V on pairs of rows: the owners pack (p[2q], p[2q+1]) to fp16 (p <= 1), row pair q is
+        // broadcast from lane 4q of the group, the two V rows are interleaved element by element
+        uint32_t pp[GT];
 #pragma unroll
-      for (int j = 0; j < kTok; j++) {
-        float vf[8];
-        unpack8<T>(vr[j], vf);
+        for (int h = 0; h < GT; h++) pp[h] = pack2<F16>(pw[h], pw[GT + h]);
+        static_for<kTok / 2>([&](auto q_tag) {
+          constexpr int q = decltype(q_tag)::value;
+          uint32_t bq[GT];
 #pragma unroll
-        for (int h = 0; h < GT; h++)
+          for (int h = 0; h < GT; h++) bq[h] = __builtin_bit_cast(uint32_t, dpp_mov<0x150 + 4 * q>(__builtin_bit_cast(float, pp[h])));  // row_newbcast
 #pragma unroll
-          for (int i = 0; i < 8; i++) o[h][i] = __builtin_fmaf(pj[j][h], vf[i], o[h][i]);
+          for (int w4 = 0; w4 < 4; w4++) {
+            const uint32_t lo = __builtin_amdgcn_perm(vr[2 * q + 1][w4], vr[2 * q][w4], 0x05040100u);
+            const uint32_t hi = __builtin_amdgcn_perm(vr[2 * q + 1][w4], vr[2 * q][w4], 0x07060302u);
+#pragma unroll
+            for (int h = 0; h < GT; h++) {
+              o[h][2 * w4] = dot2acc<F16>(bq[h], lo, o[h][2 * w4]);
+              o[h][2 * w4 + 1] = dot2acc<F16>(bq[h], hi, o[h][2 * w4 + 1]);
+            }
+          }
+        });
+      } else {
+        // bf16: a bf16 P would cost ~1e-3 relative error, so P stays fp32 and is broadcast row by row
+        static_for<kTok>([&](auto j_tag) {
+          constexpr int j = decltype(j_tag)::value;
+          float vf[8];
+          unpack8<T>(vr[j], vf);
+#pragma unroll
+          for (int h = 0; h < GT; h++) {
+            const float pb = dpp_mov<0x150 + 4 * (j >> 1)>(pw[GT * (j & 1) + h]);  // row_newbcast
+#pragma unroll
+            for (int i = 0; i < 8; i++) o[h][i] = __builtin_fmaf(pb, vf[i], o[h][i]);
+          }
+        });
       }
     }
 
@@ -333,7 +420,10 @@ static int launch_stage1(const lsattn_decode_stage1_args* a, hipStream_t st) {
 
 template <typename T> static int dispatch_stage1(const lsattn_decode_stage1_args* a, hipStream_t st) {
   const int group = (int)(a->num_q_heads / a->num_kv_heads);
-  if (group % 4 == 0) return launch_stage1<T, 4>(a, st);
+#ifndef LSATTN_DECODE_MAX_GT
+#define LSATTN_DECODE_MAX_GT 4
+#endif
+  if (group % 4 == 0 && LSATTN_DECODE_MAX_GT >= 4) return launch_stage1<T, 4>(a, st);
   if (group % 2 == 0) return launch_stage1<T, 2>(a, st);
   return launch_stage1<T, 1>(a, st);
 }
@@ -347,7 +437,7 @@ extern "C" int lsattn_decode_stage1(const lsattn_decode_stage1_args* a, void* st
       !a->b_seqlen)
     return LSATTN_ERR_INVALID_ARG;
   if (a->batch < 0 || a->num_q_heads <= 0 || a->num_kv_heads <= 0 || a->num_blocks < 0 || a->seq_block_size < 1 ||
-      a->max_len_in_batch < 0 || a->max_seq_len < 0)
+      a->max_len_in_batch < 0 || a->max_seq_len < 0 || a->max_seq_len > 0x7fffff00)  // 32-bit token positions in the kernel
     return LSATTN_ERR_INVALID_ARG;
   if (a->num_q_heads % a->num_kv_heads != 0) return LSATTN_ERR_INVALID_ARG;
   // 16-byte row loads: strides must keep every row 16-byte aligned
