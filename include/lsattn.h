@@ -183,6 +183,57 @@ int lsattn_register_tokens(int32_t* req_to_tokens, int64_t max_seq_len, const in
                            const int32_t* b_start_loc, const int32_t* b_seq_len, const int32_t* mem_index,
                            int64_t batch, int64_t max_len_in_batch, void* stream);
 
+/*
+ * Which locally held KV rows of each request belong to the cache-index window
+ * [kv_cache_index_begin, kv_cache_index_end) when local row n holds global token
+ * kv_first_token_global_idx + n * sp_peers:
+ *   kv_range_begin = ceil((kv_cache_index_begin - kv_first_token_global_idx) / sp_peers)
+ *   kv_range_end   = ceil((kv_cache_index_end   - kv_first_token_global_idx) / sp_peers)
+ *   new_kv_cache_len = kv_range_end - kv_range_begin
+ * (ceil as Python floor division of x + sp_peers - 1, the form the reference documents).
+ * Replaces pre_copy_and_register_kv
+ * (loongserve/models/llama/triton_kernel/copy_and_register_kv.py:6-62).
+ */
+int lsattn_kv_ranges(const int32_t* kv_cache_index_begin, const int32_t* kv_cache_index_end,
+                     const int32_t* kv_first_token_global_idx, int32_t sp_peers, int64_t batch,
+                     int32_t* kv_range_begin, int32_t* kv_range_end, int32_t* new_kv_cache_len, void* stream);
+
+/*
+ * Context migration during prefill: for every request b with new_kv_cache_len[b] > 0 and non-negative
+ * range bounds, and every n < min(new_kv_cache_len[b], row_limit):
+ *   slot = mem_index[num_used_mem_index + (b > 0 ? new_kv_cache_len_sum[b-1] : 0) + n]
+ *   pool[slot] = kv[kv_b_start_loc[b] + kv_range_begin[b] + n]                    (bit-exact row copy)
+ *   if should_register: req_to_tokens[b_req_idx[b], cur_kv_cache_index[b] + n] = slot
+ * row_limit is the reference's grid bound, max_len_in_batch rounded up to a multiple of 256.
+ * Replaces destindex_copy_and_register_kv
+ * (loongserve/models/llama/triton_kernel/copy_and_register_kv.py:64-170; called from
+ * longserve_transformer_layer_infer.py:199-215).
+ * Rows are row_bytes long (a multiple of 16, 16-byte aligned); strides are in bytes.
+ */
+typedef struct lsattn_kv_copy_register_args {
+  const void* kv;                      /* [tokens, row_bytes] source rows              */
+  int64_t kv_stride_bytes;
+  void* pool;                          /* [slots, row_bytes] KV pool of this layer     */
+  int64_t pool_stride_bytes;
+  int64_t row_bytes;
+  const int32_t* new_kv_cache_len;     /* [batch] */
+  const int32_t* kv_range_begin;       /* [batch] */
+  const int32_t* kv_range_end;         /* [batch] */
+  const int64_t* new_kv_cache_len_sum; /* [batch] inclusive prefix sum of new_kv_cache_len */
+  const int32_t* kv_b_start_loc;       /* [batch] */
+  const int32_t* cur_kv_cache_index;   /* [batch] (read only when should_register)     */
+  const int32_t* mem_index;            /* [>= num_used_mem_index + sum] pool slots      */
+  const int32_t* b_req_idx;            /* [batch] (read only when should_register)     */
+  int32_t* req_to_tokens;              /* [max_req, max_seq_len] (written only when should_register) */
+  int64_t max_seq_len;
+  int64_t batch;
+  int64_t num_used_mem_index;
+  int64_t max_len_in_batch;
+  int32_t should_register;
+  int32_t reserved;
+} lsattn_kv_copy_register_args;
+int lsattn_kv_copy_register(const lsattn_kv_copy_register_args* a, void* stream);
+
 const char* lsattn_strerror(int code);
 int lsattn_version(void);
 

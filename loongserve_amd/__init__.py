@@ -7,18 +7,25 @@ longserve_token_decode_attention_flash_decoding, and the extension-module stand-
 `longserve_cuda_kernels`.  All of them run hand-written gfx950 HIP kernels from
 liblsattn.so; importing this package fails if that library has not been built.
 """
+import sys as _sys
+
 from . import _lib
 
-_lib.load()  # fail loudly at import time if the HIP library is missing
+# `python -m loongserve_amd.build` imports this package on its way to the build recipe: the library it is
+# about to (re)build may be missing or lack a new entry point, so that one invocation skips the load.
+_building = len(getattr(_sys, "orig_argv", [])) >= 3 and _sys.orig_argv[1:3] == ["-m", "loongserve_amd.build"]
+if not _building:
+    _lib.load()  # fail loudly at import time if the HIP library is missing or stale
 
 from . import longserve_cuda_kernels  # noqa: E402
 from .decoding import (longserve_flash_decode_stage1, longserve_flash_decode_stage2,  # noqa: E402
                        longserve_token_decode_attention_flash_decoding)
-from .ops import (context_attention_fwd, init_req_to_token_indexes, kv_scatter, lse_merge,  # noqa: E402
-                  prefill_attention_step)
+from .ops import (context_attention_fwd, destindex_copy_and_register_kv, init_req_to_token_indexes,  # noqa: E402
+                  kv_scatter, lse_merge, pre_copy_and_register_kv, prefill_attention_step)
 
 __all__ = [
     "context_attention_fwd", "prefill_attention_step", "lse_merge", "kv_scatter", "init_req_to_token_indexes",
+    "pre_copy_and_register_kv", "destindex_copy_and_register_kv",
     "longserve_flash_decode_stage1", "longserve_flash_decode_stage2",
     "longserve_token_decode_attention_flash_decoding", "longserve_cuda_kernels",
 ]

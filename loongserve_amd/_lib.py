@@ -64,6 +64,16 @@ class DecodeStage2Args(C.Structure):
 
 
 # every symbol include/lsattn.h declares: name -> (restype, argtypes)
+class KvCopyRegisterArgs(C.Structure):  # mirrors lsattn_kv_copy_register_args
+    _fields_ = [("kv", C.c_void_p), ("kv_stride_bytes", C.c_int64), ("pool", C.c_void_p), ("pool_stride_bytes", C.c_int64),
+                ("row_bytes", C.c_int64), ("new_kv_cache_len", C.c_void_p), ("kv_range_begin", C.c_void_p),
+                ("kv_range_end", C.c_void_p), ("new_kv_cache_len_sum", C.c_void_p), ("kv_b_start_loc", C.c_void_p),
+                ("cur_kv_cache_index", C.c_void_p), ("mem_index", C.c_void_p), ("b_req_idx", C.c_void_p),
+                ("req_to_tokens", C.c_void_p), ("max_seq_len", C.c_int64), ("batch", C.c_int64),
+                ("num_used_mem_index", C.c_int64), ("max_len_in_batch", C.c_int64), ("should_register", C.c_int32),
+                ("reserved", C.c_int32)]
+
+
 EXPORTS = {
     "lsattn_prefill_step": (C.c_int, [C.POINTER(PrefillArgs), _vp]),
     "lsattn_prefill_step_merge": (C.c_int, [C.POINTER(PrefillArgs), _vp]),
@@ -72,6 +82,8 @@ EXPORTS = {
     "lsattn_decode_stage2": (C.c_int, [C.POINTER(DecodeStage2Args), _vp]),
     "lsattn_kv_scatter": (C.c_int, [_vp, _i64, _vp, _i64, _vp, _i64, _i64, _vp]),
     "lsattn_register_tokens": (C.c_int, [_vp, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _vp]),
+    "lsattn_kv_ranges": (C.c_int, [_vp, _vp, _vp, C.c_int32, _i64, _vp, _vp, _vp, _vp]),
+    "lsattn_kv_copy_register": (C.c_int, [C.POINTER(KvCopyRegisterArgs), _vp]),
     "lsattn_strerror": (C.c_char_p, [C.c_int]),
     "lsattn_version": (C.c_int, []),
 }

@@ -74,6 +74,69 @@ __global__ __launch_bounds__(256) void register_tokens_kernel(int32_t* __restric
   req_to_tokens[(int64_t)b_req_idx[b] * max_seq_len + j] = mem_index[(int64_t)b_start_loc[b] + j];
 }
 
+// ceil(x / p) for p > 0 as floor((x + p - 1) / p), also for negative x
+__device__ __forceinline__ int32_t ceil_div_floor(int32_t x, int32_t p) {
+  const int64_t a = (int64_t)x + p - 1;
+  int64_t q = a / p;
+  if ((a % p != 0) && (a < 0)) q -= 1;
+  return (int32_t)q;
+}
+
+__global__ __launch_bounds__(256) void kv_ranges_kernel(const int32_t* __restrict__ idx_begin, const int32_t* __restrict__ idx_end,
+                                                        const int32_t* __restrict__ first, int32_t peers, int64_t batch,
+                                                        int32_t* __restrict__ range_begin, int32_t* __restrict__ range_end,
+                                                        int32_t* __restrict__ new_len) {
+  const int64_t b = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (b >= batch) return;
+  const int32_t rb = ceil_div_floor(idx_begin[b] - first[b], peers);
+  const int32_t re = ceil_div_floor(idx_end[b] - first[b], peers);
+  range_begin[b] = rb;
+  range_end[b] = re;
+  new_len[b] = re - rb;
+}
+
+struct CopyRegisterParams {
+  const char* kv;
+  int64_t kv_stride;
+  char* pool;
+  int64_t pool_stride;
+  const int32_t* new_len;
+  const int32_t* range_begin;
+  const int32_t* range_end;
+  const int64_t* len_sum;
+  const int32_t* start_loc;
+  const int32_t* cur_index;
+  const int32_t* mem_index;
+  const int32_t* b_req_idx;
+  int32_t* req_to_tokens;
+  int64_t max_seq_len, num_used, row_limit;
+  int32_t chunks_per_row, should_register, rows_per_block;
+};
+
+// grid (groups of rows_per_block rows, batch); 16 bytes per lane and step, consecutive lanes cover one row.
+// A workgroup past the end of its request leaves at once: the grid is sized by the longest request.
+__global__ __launch_bounds__(256) void kv_copy_register_kernel(CopyRegisterParams p) {
+  const int64_t b = blockIdx.y;
+  int64_t n_new = p.new_len[b];
+  const int64_t begin = p.range_begin[b];
+  if (n_new <= 0 || begin < 0 || p.range_end[b] < 0) return;
+  if (n_new > p.row_limit) n_new = p.row_limit;
+  const int64_t row0 = (int64_t)blockIdx.x * p.rows_per_block;
+  if (row0 >= n_new) return;
+  const int64_t rows = n_new - row0 < p.rows_per_block ? n_new - row0 : p.rows_per_block;
+  const int64_t mi0 = p.num_used + (b > 0 ? p.len_sum[b - 1] : 0) + row0;
+  const char* src = p.kv + ((int64_t)p.start_loc[b] + begin + row0) * p.kv_stride;
+  const int64_t pieces = rows * p.chunks_per_row;
+  for (int64_t i = threadIdx.x; i < pieces; i += 256) {
+    const int64_t r = i / p.chunks_per_row;
+    const int c = (int)(i % p.chunks_per_row);
+    const int32_t slot = p.mem_index[mi0 + r];
+    const u32x4 w = *(const u32x4*)(src + r * p.kv_stride + (int64_t)c * 16);
+    *(u32x4*)(p.pool + (int64_t)slot * p.pool_stride + (int64_t)c * 16) = w;
+    if (p.should_register && c == 0) p.req_to_tokens[(int64_t)p.b_req_idx[b] * p.max_seq_len + p.cur_index[b] + row0 + r] = slot;
+  }
+}
+
 template <typename OT> static int launch_merge(const MergeParams& p, int D, hipStream_t st) {
   const int64_t threads = p.rows * (D / 4);
   const int64_t blocks = (threads + 255) / 256;
@@ -139,6 +202,61 @@ extern "C" int lsattn_register_tokens(int32_t* req_to_tokens, int64_t max_seq_le
   dim3 grid((unsigned)((max_len_in_batch + 255) / 256), (unsigned)batch);
   hipLaunchKernelGGL(register_tokens_kernel, grid, dim3(256), 0, (hipStream_t)stream, req_to_tokens, max_seq_len,
                      b_req_idx, b_start_loc, b_seq_len, mem_index);
+  return check_launch();
+}
+
+extern "C" int lsattn_kv_ranges(const int32_t* kv_cache_index_begin, const int32_t* kv_cache_index_end,
+                                const int32_t* kv_first_token_global_idx, int32_t sp_peers, int64_t batch,
+                                int32_t* kv_range_begin, int32_t* kv_range_end, int32_t* new_kv_cache_len, void* stream) {
+  if (!kv_cache_index_begin || !kv_cache_index_end || !kv_first_token_global_idx || !kv_range_begin || !kv_range_end ||
+      !new_kv_cache_len || sp_peers < 1 || batch < 0)
+    return LSATTN_ERR_INVALID_ARG;
+  if (batch == 0) return LSATTN_OK;
+  const int64_t blocks = (batch + 255) / 256;
+  if (blocks > 0x7fffffff) return LSATTN_ERR_INVALID_ARG;
+  hipLaunchKernelGGL(kv_ranges_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, kv_cache_index_begin,
+                     kv_cache_index_end, kv_first_token_global_idx, sp_peers, batch, kv_range_begin, kv_range_end,
+                     new_kv_cache_len);
+  return check_launch();
+}
+
+extern "C" int lsattn_kv_copy_register(const lsattn_kv_copy_register_args* a, void* stream) {
+  if (!a || !a->kv || !a->pool || !a->new_kv_cache_len || !a->kv_range_begin || !a->kv_range_end ||
+      !a->new_kv_cache_len_sum || !a->kv_b_start_loc || !a->mem_index || a->batch < 0 || a->row_bytes <= 0 ||
+      a->num_used_mem_index < 0 || a->max_len_in_batch < 0)
+    return LSATTN_ERR_INVALID_ARG;
+  if (a->should_register && (!a->cur_kv_cache_index || !a->b_req_idx || !a->req_to_tokens || a->max_seq_len <= 0))
+    return LSATTN_ERR_INVALID_ARG;
+  if (a->row_bytes % 16 || a->kv_stride_bytes % 16 || a->pool_stride_bytes % 16 ||
+      (((uintptr_t)a->kv | (uintptr_t)a->pool) & 15))
+    return LSATTN_ERR_INVALID_ARG;
+  if (a->batch == 0 || a->max_len_in_batch == 0) return LSATTN_OK;
+  if (a->batch > 65535) return LSATTN_ERR_INVALID_ARG;
+  CopyRegisterParams p;
+  p.kv = (const char*)a->kv;
+  p.kv_stride = a->kv_stride_bytes;
+  p.pool = (char*)a->pool;
+  p.pool_stride = a->pool_stride_bytes;
+  p.new_len = a->new_kv_cache_len;
+  p.range_begin = a->kv_range_begin;
+  p.range_end = a->kv_range_end;
+  p.len_sum = a->new_kv_cache_len_sum;
+  p.start_loc = a->kv_b_start_loc;
+  p.cur_index = a->cur_kv_cache_index;
+  p.mem_index = a->mem_index;
+  p.b_req_idx = a->b_req_idx;
+  p.req_to_tokens = a->req_to_tokens;
+  p.max_seq_len = a->max_seq_len;
+  p.num_used = a->num_used_mem_index;
+  p.row_limit = (a->max_len_in_batch + 255) / 256 * 256;  // the reference's grid: (batch, cdiv(max_len_in_batch, 256)) x 256 rows
+  const int64_t cpr = a->row_bytes / 16;
+  if (cpr > 0x7fffffff) return LSATTN_ERR_INVALID_ARG;
+  p.rows_per_block = cpr >= 4096 ? 1 : (int32_t)(4096 / cpr);  // about 64 KB per workgroup
+  const int64_t blocks = (p.row_limit + p.rows_per_block - 1) / p.rows_per_block;
+  if (blocks > 0x7fffffff) return LSATTN_ERR_INVALID_ARG;
+  p.chunks_per_row = (int32_t)cpr;
+  p.should_register = a->should_register;
+  hipLaunchKernelGGL(kv_copy_register_kernel, dim3((unsigned)blocks, (unsigned)a->batch), dim3(256), 0, (hipStream_t)stream, p);
   return check_launch();
 }
 

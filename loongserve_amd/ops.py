@@ -198,3 +198,66 @@ def init_req_to_token_indexes(req_to_token_indexs, b_req_idx, b_seq_len, alloc_m
                                             b_req_idx.data_ptr(), b_start_loc.data_ptr(), b_seq_len.data_ptr(),
                                             alloc_mem_index.data_ptr(), B, max_len_in_batch, _stream())
     _lib.check(rc, "lsattn_register_tokens")
+
+
+@torch.inference_mode()
+def pre_copy_and_register_kv(kv_cache_index_begin: torch.Tensor, kv_cache_index_end: torch.Tensor,
+                             kv_first_token_global_idx: torch.Tensor, num_logical_sp_peers: int):
+    """(kv_range_begin, kv_range_end, new_kv_cache_len): the locally held rows of each request that fall in
+    the cache-index window, with local row n holding global token first + n * peers.
+
+    Signature and results of pre_copy_and_register_kv
+    (loongserve/models/llama/triton_kernel/copy_and_register_kv.py:34-62)."""
+    B = kv_cache_index_begin.shape[0]
+    _i32vec(kv_cache_index_begin, "kv_cache_index_begin", B); _i32vec(kv_cache_index_end, "kv_cache_index_end", B)
+    _i32vec(kv_first_token_global_idx, "kv_first_token_global_idx", B)
+    rb, re, nl = (torch.empty_like(kv_cache_index_begin) for _ in range(3))
+    if B == 0:
+        return rb, re, nl
+    rc = _lib.load().lsattn_kv_ranges(kv_cache_index_begin.data_ptr(), kv_cache_index_end.data_ptr(),
+                                      kv_first_token_global_idx.data_ptr(), int(num_logical_sp_peers), B,
+                                      rb.data_ptr(), re.data_ptr(), nl.data_ptr(), _stream())
+    _lib.check(rc, "lsattn_kv_ranges")
+    return rb, re, nl
+
+
+@torch.inference_mode()
+def destindex_copy_and_register_kv(batch_size: int, new_kv_cache_len: torch.Tensor, kv_range_begin: torch.Tensor,
+                                   kv_range_end: torch.Tensor, new_kv_cache_len_sum: torch.Tensor, kv: torch.Tensor,
+                                   kv_b_start_loc: torch.Tensor, cur_kv_cache_index: torch.Tensor, mem_index: torch.Tensor,
+                                   total_kv_cache: torch.Tensor, req_to_token_indexs: torch.Tensor, b_req_idx: torch.Tensor,
+                                   num_used_mem_index: int, max_len_in_batch: int, should_register_kv: bool) -> None:
+    """Copy the migrating KV rows of every request into their pool slots and, on the first layer, register
+    the slots in the request table.
+
+    Signature and semantics of destindex_copy_and_register_kv
+    (loongserve/models/llama/triton_kernel/copy_and_register_kv.py:119-170)."""
+    B = int(batch_size)
+    if B == 0:
+        return
+    for t, name in ((new_kv_cache_len, "new_kv_cache_len"), (kv_range_begin, "kv_range_begin"), (kv_range_end, "kv_range_end"),
+                    (kv_b_start_loc, "kv_b_start_loc"), (cur_kv_cache_index, "cur_kv_cache_index"), (b_req_idx, "b_req_idx")):
+        _i32vec(t, name, B)
+    _i32vec(mem_index, "mem_index")
+    _dev(new_kv_cache_len_sum, "new_kv_cache_len_sum")
+    if new_kv_cache_len_sum.dtype != torch.int64 or new_kv_cache_len_sum.shape != (B,) or not new_kv_cache_len_sum.is_contiguous():
+        raise ValueError("new_kv_cache_len_sum must be a contiguous int64 vector of length batch_size")
+    _dev(kv, "kv"); _dev(total_kv_cache, "total_kv_cache"); _dev(req_to_token_indexs, "req_to_token_indexs")
+    if kv.dtype != total_kv_cache.dtype or kv.shape[1:] != total_kv_cache.shape[1:]:
+        raise ValueError("kv and total_kv_cache rows must match")
+    if not kv[0].is_contiguous() or not total_kv_cache[0].is_contiguous():
+        raise ValueError("rows must be contiguous")
+    if req_to_token_indexs.dtype != torch.int32 or not req_to_token_indexs.is_contiguous():
+        raise ValueError("req_to_token_indexs must be contiguous int32")
+    a = _lib.KvCopyRegisterArgs()
+    a.kv, a.kv_stride_bytes = kv.data_ptr(), kv.stride(0) * kv.element_size()
+    a.pool, a.pool_stride_bytes = total_kv_cache.data_ptr(), total_kv_cache.stride(0) * total_kv_cache.element_size()
+    a.row_bytes = kv[0].numel() * kv.element_size()
+    a.new_kv_cache_len, a.kv_range_begin, a.kv_range_end = new_kv_cache_len.data_ptr(), kv_range_begin.data_ptr(), kv_range_end.data_ptr()
+    a.new_kv_cache_len_sum, a.kv_b_start_loc = new_kv_cache_len_sum.data_ptr(), kv_b_start_loc.data_ptr()
+    a.cur_kv_cache_index, a.mem_index, a.b_req_idx = cur_kv_cache_index.data_ptr(), mem_index.data_ptr(), b_req_idx.data_ptr()
+    a.req_to_tokens, a.max_seq_len = req_to_token_indexs.data_ptr(), req_to_token_indexs.shape[1]
+    a.batch, a.num_used_mem_index, a.max_len_in_batch = B, int(num_used_mem_index), int(max_len_in_batch)
+    a.should_register = 1 if should_register_kv else 0
+    rc = _lib.load().lsattn_kv_copy_register(C.byref(a), _stream())
+    _lib.check(rc, "lsattn_kv_copy_register")

@@ -289,3 +289,32 @@ def register_tokens(req_to_tokens, b_req_idx, b_start_loc, b_seq_len, mem_index)
     for b in range(len(b_req_idx)):
         s, n = int(b_start_loc[b]), int(b_seq_len[b])
         req_to_tokens[int(b_req_idx[b]), 0:n] = mem_index[s:s + n].to(req_to_tokens.dtype)
+
+
+def kv_ranges(kv_cache_index_begin, kv_cache_index_end, kv_first_token_global_idx, peers: int):
+    """(kv_range_begin, kv_range_end, new_kv_cache_len) of pre_copy_and_register_kv
+    (loongserve/models/llama/triton_kernel/copy_and_register_kv.py:24-31, docstring :42-48):
+    ceil((index - first) / peers) written as Python floor division of x + peers - 1."""
+    rb = [(int(b) - int(f) + (peers - 1)) // peers for b, f in zip(kv_cache_index_begin, kv_first_token_global_idx)]
+    re = [(int(e) - int(f) + (peers - 1)) // peers for e, f in zip(kv_cache_index_end, kv_first_token_global_idx)]
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32)
+    return i32(rb), i32(re), i32([e - b for b, e in zip(rb, re)])
+
+
+def kv_copy_register(batch_size, new_kv_cache_len, kv_range_begin, kv_range_end, new_kv_cache_len_sum, kv, kv_b_start_loc,
+                     cur_kv_cache_index, mem_index, total_kv_cache, req_to_token_indexs, b_req_idx,
+                     num_used_mem_index: int, max_len_in_batch: int, should_register_kv: bool) -> None:
+    """destindex_copy_and_register_kv as plain loops
+    (loongserve/models/llama/triton_kernel/copy_and_register_kv.py:92-117: skip rule :96-97, slot list offset :99-100,
+    source row :106, row loop bounded by the grid :159 and BLOCK_N :157, registration :112-117)."""
+    row_limit = (max_len_in_batch + 255) // 256 * 256
+    for b in range(batch_size):
+        n_new, begin, end = int(new_kv_cache_len[b]), int(kv_range_begin[b]), int(kv_range_end[b])
+        if n_new <= 0 or begin < 0 or end < 0:
+            continue
+        start = (int(new_kv_cache_len_sum[b - 1]) if b > 0 else 0) + num_used_mem_index
+        for n in range(min(n_new, row_limit)):
+            slot = int(mem_index[start + n])
+            total_kv_cache[slot] = kv[int(kv_b_start_loc[b]) + begin + n]
+            if should_register_kv:
+                req_to_token_indexs[int(b_req_idx[b]), int(cur_kv_cache_index[b]) + n] = slot

@@ -39,10 +39,11 @@ def test_struct_layout_matches_header():
 #include <stddef.h>
 #include "lsattn.h"
 int main(void) {
-  printf("%zu %zu %zu %zu\n", sizeof(lsattn_prefill_args), sizeof(lsattn_merge_args),
-         sizeof(lsattn_decode_stage1_args), sizeof(lsattn_decode_stage2_args));
-  printf("%zu %zu %zu %zu\n", offsetof(lsattn_prefill_args, sm_scale), offsetof(lsattn_prefill_args, ml_stride_h),
-         offsetof(lsattn_decode_stage1_args, req_to_tokens), offsetof(lsattn_decode_stage2_args, block_seq));
+  printf("%zu %zu %zu %zu %zu\n", sizeof(lsattn_prefill_args), sizeof(lsattn_merge_args),
+         sizeof(lsattn_decode_stage1_args), sizeof(lsattn_decode_stage2_args), sizeof(lsattn_kv_copy_register_args));
+  printf("%zu %zu %zu %zu %zu %zu\n", offsetof(lsattn_prefill_args, sm_scale), offsetof(lsattn_prefill_args, ml_stride_h),
+         offsetof(lsattn_decode_stage1_args, req_to_tokens), offsetof(lsattn_decode_stage2_args, block_seq),
+         offsetof(lsattn_kv_copy_register_args, req_to_tokens), offsetof(lsattn_kv_copy_register_args, should_register));
   return 0;
 }'''
     with tempfile.TemporaryDirectory() as d:
@@ -51,12 +52,13 @@ int main(void) {
         exe = os.path.join(d, "t")
         subprocess.check_call(["gcc", "-std=c99", "-I", os.path.join(ROOT, "include"), c, "-o", exe])
         out = subprocess.check_output([exe]).decode().split()
-    sizes = [int(x) for x in out[:4]]
-    offs = [int(x) for x in out[4:]]
+    sizes = [int(x) for x in out[:5]]
+    offs = [int(x) for x in out[5:]]
     assert sizes == [C.sizeof(_lib.PrefillArgs), C.sizeof(_lib.MergeArgs), C.sizeof(_lib.DecodeStage1Args),
-                     C.sizeof(_lib.DecodeStage2Args)]
+                     C.sizeof(_lib.DecodeStage2Args), C.sizeof(_lib.KvCopyRegisterArgs)]
     assert offs == [_lib.PrefillArgs.sm_scale.offset, _lib.PrefillArgs.ml_stride_h.offset,
-                    _lib.DecodeStage1Args.req_to_tokens.offset, _lib.DecodeStage2Args.block_seq.offset]
+                    _lib.DecodeStage1Args.req_to_tokens.offset, _lib.DecodeStage2Args.block_seq.offset,
+                    _lib.KvCopyRegisterArgs.req_to_tokens.offset, _lib.KvCopyRegisterArgs.should_register.offset]
 
 
 def test_validation_rejects_bad_arguments_without_gpu():
@@ -67,6 +69,9 @@ def test_validation_rejects_bad_arguments_without_gpu():
     assert lib.lsattn_prefill_step(None, None) == -1
     d1 = _lib.DecodeStage1Args()
     assert lib.lsattn_decode_stage1(C.byref(d1), None) == -1
+    cr = _lib.KvCopyRegisterArgs()
+    assert lib.lsattn_kv_copy_register(C.byref(cr), None) == -1
+    assert lib.lsattn_kv_ranges(None, None, None, 1, 0, None, None, None, None) == -1
     d2 = _lib.DecodeStage2Args()
     assert lib.lsattn_decode_stage2(C.byref(d2), None) == -1
     m = _lib.MergeArgs()

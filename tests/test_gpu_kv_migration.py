@@ -1,0 +1,96 @@
+"""GPU parity of the context-migration KV copy + registration against the oracle (bit-exact, through the C ABI)."""
+import pytest
+import torch
+
+from oracle import attn_oracle as orc
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _i32(x):
+    return torch.tensor(x, dtype=torch.int32)
+
+
+def test_kv_ranges_match_oracle(lsa):
+    g = torch.Generator().manual_seed(3)
+    B = 700  # more than one 256-thread block
+    first = torch.randint(0, 9, (B,), generator=g, dtype=torch.int32)
+    begin = first + torch.randint(-5, 4000, (B,), generator=g, dtype=torch.int32)
+    end = begin + torch.randint(0, 5000, (B,), generator=g, dtype=torch.int32)
+    for P in (1, 2, 4, 7):
+        rb, re, nl = lsa.pre_copy_and_register_kv(begin.to(DEV), end.to(DEV), first.to(DEV), P)
+        rb_o, re_o, nl_o = orc.kv_ranges(begin.tolist(), end.tolist(), first.tolist(), P)
+        assert torch.equal(rb.cpu(), rb_o) and torch.equal(re.cpu(), re_o) and torch.equal(nl.cpu(), nl_o)
+    empty = torch.empty(0, dtype=torch.int32, device=DEV)
+    rb, re, nl = lsa.pre_copy_and_register_kv(empty, empty, empty, 4)
+    assert rb.numel() == 0
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("register", [True, False])
+def test_copy_and_register_matches_oracle(lsa, dtype, register):
+    g = torch.Generator().manual_seed(17)
+    B, Hkv, D = 6, 8, 128
+    lens = [300, 0, 1, 700, 257, 40]          # new_kv_cache_len per request (one empty)
+    begin = [0, 5, 3, 10, 0, 2]
+    begin[4] = -1                              # negative bound: the reference skips the request
+    start_loc, off = [], 0
+    for n, b0 in zip(lens, begin):
+        start_loc.append(off)
+        off += n + max(b0, 0) + 3
+    kv = torch.randn(off + 8, 2 * Hkv, D, generator=g).to(dtype)
+    pool_n = 4000
+    pool = torch.randn(pool_n, 2 * Hkv, D, generator=g).to(dtype)
+    table = torch.full((B + 2, 1200), orc.INT32_PAD, dtype=torch.int32)
+    new_len, rb = _i32(lens), _i32(begin)
+    re = rb + new_len
+    len_sum = torch.cumsum(new_len, 0, dtype=torch.int64)
+    cur = _i32([7, 0, 100, 0, 5, 1159])
+    b_req = _i32([3, 0, 7, 1, 5, 2])
+    used = 11
+    mem_index = torch.randperm(pool_n, generator=g)[:used + int(len_sum[-1])].to(torch.int32)
+    max_len = 600                               # rounds up to 768: request 3 (700 rows) is copied whole
+    pool_o, table_o = pool.clone(), table.clone()
+    orc.kv_copy_register(B, new_len, rb, re, len_sum, kv, _i32(start_loc), cur, mem_index, pool_o, table_o, b_req, used, max_len, register)
+    pool_d, table_d = pool.to(DEV), table.to(DEV)
+    lsa.destindex_copy_and_register_kv(B, new_len.to(DEV), rb.to(DEV), re.to(DEV), len_sum.to(DEV), kv.to(DEV), _i32(start_loc).to(DEV),
+                                       cur.to(DEV), mem_index.to(DEV), pool_d, table_d, b_req.to(DEV), used, max_len, register)
+    torch.cuda.synchronize()
+    assert torch.equal(pool_d.cpu().view(torch.int16), pool_o.view(torch.int16))
+    assert torch.equal(table_d.cpu(), table_o)
+    if not register:
+        assert torch.equal(table_o, table)
+    # the grid bound of the reference: with max_len_in_batch = 256 only the first 256 rows of a request are copied
+    pool_o2, table_o2 = pool.clone(), table.clone()
+    orc.kv_copy_register(B, new_len, rb, re, len_sum, kv, _i32(start_loc), cur, mem_index, pool_o2, table_o2, b_req, used, 256, register)
+    pool_d2, table_d2 = pool.to(DEV), table.to(DEV)
+    lsa.destindex_copy_and_register_kv(B, new_len.to(DEV), rb.to(DEV), re.to(DEV), len_sum.to(DEV), kv.to(DEV), _i32(start_loc).to(DEV),
+                                       cur.to(DEV), mem_index.to(DEV), pool_d2, table_d2, b_req.to(DEV), used, 256, register)
+    torch.cuda.synchronize()
+    assert torch.equal(pool_d2.cpu().view(torch.int16), pool_o2.view(torch.int16))
+    assert torch.equal(table_d2.cpu(), table_o2)
+    assert not torch.equal(pool_o2, pool_o)
+
+
+def test_migration_round_trip_feeds_decode(lsa):
+    """Rows copied by the migration kernel are found again by token-indexed decode through the registered table."""
+    g = torch.Generator().manual_seed(23)
+    Hq, Hkv, D, n = 8, 2, 128, 500
+    kv = (torch.randn(n, 2 * Hkv, D, generator=g) * 0.5).to(torch.float16)
+    q = (torch.randn(1, Hq, D, generator=g) * 0.5).to(torch.float16)
+    pool = torch.zeros(3000, 2 * Hkv, D, dtype=torch.float16, device=DEV)
+    table = torch.full((2, 600), orc.INT32_PAD, dtype=torch.int32, device=DEV)
+    mem_index = torch.randperm(3000, generator=g)[:n].to(torch.int32)
+    z = lambda v: _i32([v]).to(DEV)
+    lsa.destindex_copy_and_register_kv(1, z(n), z(0), z(n), torch.tensor([n], device=DEV), kv.to(DEV), z(0), z(0), mem_index.to(DEV),
+                                       pool, table, z(1), 0, n, True)
+    nblk = (n + 255) // 256
+    mo = torch.empty(nblk, 1, Hq, D, device=DEV)
+    ml = torch.empty(nblk, 1, Hq, device=DEV)
+    o, lse = lsa.longserve_token_decode_attention_flash_decoding(q.to(DEV), table, z(1), z(n), mo, ml, 1, n, Hq, D, pool[:, :Hkv], pool[:, Hkv:], 256)
+    torch.cuda.synchronize()
+    t_cpu = torch.arange(n, dtype=torch.int32)[None]
+    o_ref, l_ref = orc.decode_full(q, kv[:, :Hkv], kv[:, Hkv:], t_cpu, _i32([0]), _i32([n]))
+    assert (o.cpu() - o_ref).abs().max().item() <= 2e-3
+    assert torch.allclose(lse.cpu(), l_ref, rtol=1e-4, atol=1e-4)

@@ -293,3 +293,58 @@ def test_kv_scatter_and_register():
     assert table[2].tolist() == [7, 2, 9, 0, orc.INT32_PAD]
     assert table[0].tolist() == [4, 5] + [orc.INT32_PAD] * 3
     assert torch.all(table[[1, 3]] == orc.INT32_PAD)
+
+
+def test_kv_ranges_count_the_locally_held_tokens_of_the_window():
+    """Pin by brute force: local row n holds global token first + n * P, so [range_begin, range_end) must be exactly
+    the rows whose global index falls in [index_begin, index_end) (for windows that start at or after `first`)."""
+    import random
+    rnd = random.Random(5)
+    for _ in range(300):
+        P = rnd.randint(1, 6)
+        first = rnd.randint(0, 7)
+        n_rows = rnd.randint(0, 40)
+        begin = first + rnd.randint(0, 60)
+        end = begin + rnd.randint(0, 80)
+        rb, re, nl = orc.kv_ranges([begin], [end], [first], P)
+        rows = [n for n in range(0, 400) if begin <= first + n * P < end]
+        assert int(nl[0]) == len(rows)
+        if rows:
+            assert (int(rb[0]), int(re[0])) == (rows[0], rows[-1] + 1)
+    # a window that starts before the first held token: the Python floor form goes negative and the copy skips the request
+    rb, re, nl = orc.kv_ranges([0], [3], [9], 4)
+    assert int(rb[0]) == -2 and int(re[0]) == -1 and int(nl[0]) == 1
+
+
+def test_kv_copy_register_against_index_copy():
+    g = torch.Generator().manual_seed(11)
+    B, rows, pool_n, W = 4, 60, 200, 24
+    kv = torch.randn(rows, 3, 8, generator=g).to(torch.float16)
+    pool = torch.zeros(pool_n, 3, 8, dtype=torch.float16)
+    table = torch.full((6, 50), orc.INT32_PAD, dtype=torch.int32)
+    new_len = torch.tensor([5, 0, 7, 3], dtype=torch.int32)
+    begin = torch.tensor([2, 4, 0, 1], dtype=torch.int32)
+    end = begin + new_len
+    len_sum = torch.cumsum(new_len, 0, dtype=torch.int64)
+    start_loc = torch.tensor([0, 10, 20, 40], dtype=torch.int32)
+    cur = torch.tensor([3, 0, 9, 1], dtype=torch.int32)
+    b_req = torch.tensor([5, 1, 0, 2], dtype=torch.int32)
+    used = 4
+    mem_index = torch.randperm(pool_n, generator=g)[:used + int(len_sum[-1])].to(torch.int32)
+    orc.kv_copy_register(B, new_len, begin, end, len_sum, kv, start_loc, cur, mem_index, pool, table, b_req, used, 16, True)
+    # the same through index_copy_ on explicitly built row / slot lists
+    src_rows, slots = [], []
+    for b in range(B):
+        off = used + (int(len_sum[b - 1]) if b else 0)
+        for n in range(int(new_len[b])):
+            src_rows.append(int(start_loc[b]) + int(begin[b]) + n)
+            slots.append(int(mem_index[off + n]))
+            assert int(table[int(b_req[b]), int(cur[b]) + n]) == slots[-1]
+    want = torch.zeros_like(pool).index_copy_(0, torch.tensor(slots), kv[src_rows])
+    assert torch.equal(pool, want)
+    assert int((table != orc.INT32_PAD).sum()) == len(slots)
+    # negative bound: request skipped; row limit: rows past ceil(max_len/256)*256 are not copied
+    pool2 = torch.zeros_like(pool)
+    orc.kv_copy_register(1, torch.tensor([3], dtype=torch.int32), torch.tensor([-1], dtype=torch.int32), torch.tensor([2], dtype=torch.int32),
+                         torch.tensor([3]), kv, torch.tensor([5], dtype=torch.int32), cur, mem_index, pool2, table.clone(), b_req, 0, 16, False)
+    assert int(pool2.abs().sum()) == 0
