@@ -325,6 +325,26 @@ def other_configs(steps):
                       "migration_copy_register_gbs": v.scatter_bytes / (sm["median_ms"] * 1e-3) / 1e9}
     del v
     torch.cuda.empty_cache()
+    # the element-wise steps around attention at config 2's per-GPU shape (16384 tokens, hidden 4096, 32 heads, inter 11008)
+    from loongserve_amd import longserve_cuda_kernels as lk
+    T, H, I, NH, D = 16384, 4096, 11008, 32, 128
+    x = _randn_half((T, H), 7001, torch.float16)
+    w = _randn_half((H,), 7002, torch.float16)
+    io = _randn_half((T, 2 * I), 7003, torch.float16)
+    qkv = _randn_half((T, 3 * NH, D), 7004, torch.float16)
+    cs = _randn_half((T, D // 2), 7005, torch.float16)
+    sn = _randn_half((T, D // 2), 7006, torch.float16)
+    ew = {}
+    for name, fn, nbytes in (("rms_norm", lambda: lk.rms_norm(x, w, 1e-5), 2 * T * H * 2 + H * 2),
+                             ("silu_and_mul_inplace", lambda: lk.silu_and_mul_inplace(io), 3 * T * I * 2),
+                             ("rotary_emb", lambda: lk.rotary_emb(qkv[:, :NH], qkv[:, NH:2 * NH], cs, sn),
+                              2 * (2 * T * NH * D * 2) + 2 * 2 * T * (D // 2) * 2)):
+        st = _stats(_time_events(fn, steps, 3))
+        ew[name] = {"median_ms": st["median_ms"], "gbs": nbytes / (st["median_ms"] * 1e-3) / 1e9,
+                    "pct_of_hbm_peak": 100 * nbytes / (st["median_ms"] * 1e-3) / 1e9 / PEAK_HBM_GBS}
+    out["elementwise"] = {"workload": "%d tokens, hidden %d, inter %d, %d heads x %d, fp16" % (T, H, I, NH, D), **ew}
+    del x, w, io, qkv, cs, sn
+    torch.cuda.empty_cache()
     return out
 
 

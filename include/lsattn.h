@@ -234,6 +234,31 @@ typedef struct lsattn_kv_copy_register_args {
 } lsattn_kv_copy_register_args;
 int lsattn_kv_copy_register(const lsattn_kv_copy_register_args* a, void* stream);
 
+/*
+ * The element-wise fp16 steps before and after attention (the rest of the reference's extension module).
+ * All pointers are 16-byte aligned device pointers; sizes in elements.
+ *
+ * out[t, i] = half(float(in[t, i]) * float(weight[i]) * rsqrt(mean_i(in[t, i]^2) + eps)); hidden_size % 8 == 0.
+ * Replaces LongServe::rms_norm (longserve_cuda_kernels/src/rms_norm.cu:10-62; binding entrypoints.cpp:15-39).
+ */
+int lsattn_rms_norm(void* out, const void* in, const void* weight, int64_t num_tokens, int64_t hidden_size, float eps,
+                    void* stream);
+/*
+ * io is [num_tokens, 2 * ffn_inter_dim]: io[t, i] = half(silu(io[t, i])) * io[t, ffn_inter_dim + i] (half multiply) for
+ * i < ffn_inter_dim; the second half of every row is left as it is.  ffn_inter_dim % 8 == 0.
+ * Replaces LongServe::silu_and_mul_inplace (silu_and_mul.cu:12-49; binding entrypoints.cpp:41-52).
+ */
+int lsattn_silu_and_mul_inplace(void* io, int64_t num_tokens, int64_t ffn_inter_dim, void* stream);
+/*
+ * In-place rotary embedding of x[t, h, 0:head_dim] (last dimension contiguous, strides in elements, multiples of 8)
+ * with cos/sin [num_tokens, head_dim/2] contiguous: x1 = x[..., :D/2], x2 = x[..., D/2:],
+ *   x1' = fma(x1, cos, -(x2 * sin)),  x2' = fma(x1, sin, x2 * cos), every operation rounded to half once
+ * (bit-exact with the reference's half2 arithmetic).  head_dim % 16 == 0.
+ * Replaces LongServe::rotary_emb (rotary_emb.cu:10-55; binding entrypoints.cpp:54-89, called once for q and once for k).
+ */
+int lsattn_rotary_emb(void* x, const void* cos, const void* sin, int64_t x_stride_t, int64_t x_stride_h,
+                      int64_t num_tokens, int64_t num_heads, int64_t head_dim, void* stream);
+
 const char* lsattn_strerror(int code);
 int lsattn_version(void);
 

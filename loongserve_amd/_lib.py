@@ -84,6 +84,9 @@ EXPORTS = {
     "lsattn_register_tokens": (C.c_int, [_vp, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _vp]),
     "lsattn_kv_ranges": (C.c_int, [_vp, _vp, _vp, C.c_int32, _i64, _vp, _vp, _vp, _vp]),
     "lsattn_kv_copy_register": (C.c_int, [C.POINTER(KvCopyRegisterArgs), _vp]),
+    "lsattn_rms_norm": (C.c_int, [_vp, _vp, _vp, _i64, _i64, C.c_float, _vp]),
+    "lsattn_silu_and_mul_inplace": (C.c_int, [_vp, _i64, _i64, _vp]),
+    "lsattn_rotary_emb": (C.c_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp]),
     "lsattn_strerror": (C.c_char_p, [C.c_int]),
     "lsattn_version": (C.c_int, []),
 }

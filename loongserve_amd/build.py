@@ -14,7 +14,10 @@ PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(PKG_DIR)
 CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_PATH = os.path.join(PKG_DIR, "liblsattn.so")
-SOURCES = ["prefill.hip", "decode.hip", "merge_scatter.hip"]
+SOURCES = ["prefill.hip", "decode.hip", "merge_scatter.hip", "elementwise.hip"]
+# elementwise.hip reproduces the reference's half arithmetic operation by operation: no fused multiply-adds
+# other than the ones it writes
+FILE_FLAGS = {"elementwise.hip": ["-ffp-contract=off"]}
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
@@ -31,7 +34,7 @@ FLAGS = [
 
 def _compile(src: str, extra) -> str:
     obj = os.path.join(CSRC, os.path.splitext(src)[0] + ".o")
-    cmd = [HIPCC, *FLAGS, *extra, "-c", os.path.join(CSRC, src), "-o", obj]
+    cmd = [HIPCC, *FLAGS, *FILE_FLAGS.get(src, []), *extra, "-c", os.path.join(CSRC, src), "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError("hipcc failed for %s:\n%s\n%s" % (src, " ".join(cmd), r.stderr[-6000:]))

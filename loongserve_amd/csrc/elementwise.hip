@@ -1,0 +1,173 @@
+// The element-wise steps around attention in the reference's extension module, for gfx950:
+//   rms_norm              (longserve_cuda_kernels/src/rms_norm.cu:10-62)
+//   silu_and_mul_inplace  (longserve_cuda_kernels/src/silu_and_mul.cu:12-49)
+//   rotary_emb            (longserve_cuda_kernels/src/rotary_emb.cu:10-55)
+// All three are HBM-bound fp16 streams: 16 bytes per lane and access, every input byte read once.
+#include "common.hip.h"
+
+namespace lsattn {
+
+// ---------------------------------------------------------------------------------------------------
+// rms_norm: out[t, i] = half(float(x[t, i]) * float(w[i]) * inv_rms[t]),  inv_rms = rsqrt(sum x^2 / H + eps),
+// the product in the reference's order (rms_norm.cu:42-45).  One wave per token row; a row of up to
+// 64 * 8 * kRmsChunks elements stays in registers between the two passes, longer rows are read twice.
+// ---------------------------------------------------------------------------------------------------
+constexpr int kRmsChunks = 16;  // 16-byte pieces per lane held in registers: rows up to 8192 elements
+
+__device__ __forceinline__ float wave_sum(float v) {
+  v = sum_row16(v);
+  v += __shfl_xor(v, 16);
+  v += __shfl_xor(v, 32);
+  return v;
+}
+
+__global__ __launch_bounds__(256) void rms_norm_kernel(uint16_t* __restrict__ out, const uint16_t* __restrict__ in,
+                                                       const uint16_t* __restrict__ weight, int64_t num_tokens, int64_t hidden,
+                                                       float eps) {
+  const int lane = threadIdx.x & 63;
+  const int64_t t = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (t >= num_tokens) return;
+  const int64_t pieces = hidden / 8;  // 16-byte pieces in a row
+  const u32x4* row = (const u32x4*)(in + t * hidden);
+  const u32x4* wrow = (const u32x4*)weight;
+  u32x4* orow = (u32x4*)(out + t * hidden);
+  const bool cached = pieces <= 64 * kRmsChunks;
+  u32x4 keep[kRmsChunks];
+  float ss = 0.f;
+  if (cached) {
+#pragma unroll
+    for (int c = 0; c < kRmsChunks; c++) {
+      const int64_t i = lane + 64 * c;
+      keep[c] = i < pieces ? row[i] : u32x4{0, 0, 0, 0};
+    }
+#pragma unroll
+    for (int c = 0; c < kRmsChunks; c++) {
+      float f[8];
+      unpack8<F16>(keep[c], f);
+#pragma unroll
+      for (int e = 0; e < 8; e++) ss = __builtin_fmaf(f[e], f[e], ss);
+    }
+  } else {
+    for (int64_t i = lane; i < pieces; i += 64) {
+      float f[8];
+      unpack8<F16>(row[i], f);
+#pragma unroll
+      for (int e = 0; e < 8; e++) ss = __builtin_fmaf(f[e], f[e], ss);
+    }
+  }
+  ss = wave_sum(ss);
+  const float inv_rms = __builtin_amdgcn_rsqf(ss / (float)hidden + eps);
+  auto scale_piece = [&](const u32x4& x, const u32x4& w) {
+    float a[8], b[8];
+    unpack8<F16>(x, a);
+    unpack8<F16>(w, b);
+    u32x4 r;
+#pragma unroll
+    for (int e = 0; e < 4; e++) r[e] = pack2<F16>(a[2 * e] * b[2 * e] * inv_rms, a[2 * e + 1] * b[2 * e + 1] * inv_rms);
+    return r;
+  };
+  if (cached) {
+#pragma unroll
+    for (int c = 0; c < kRmsChunks; c++) {
+      const int64_t i = lane + 64 * c;
+      if (i < pieces) orow[i] = scale_piece(keep[c], wrow[i]);
+    }
+  } else {
+    for (int64_t i = lane; i < pieces; i += 64) orow[i] = scale_piece(row[i], wrow[i]);
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------
+// silu_and_mul_inplace: io[t, i] = half(silu(io[t, i])) * io[t, I + i] for i < I, the second half of the row untouched;
+// silu in fp32, rounded to half, then a half multiply (silu_and_mul.cu:14-17, :30-33).
+// ---------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void silu_and_mul_kernel(uint16_t* __restrict__ io, int64_t num_tokens, int64_t inter) {
+  const int64_t pieces_per_row = inter / 8;
+  const int64_t gid = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (gid >= num_tokens * pieces_per_row) return;
+  const int64_t t = gid / pieces_per_row, i = gid % pieces_per_row;
+  // (whole rows of eight halves: picking 32-bit words out of an integer vector and bit-casting them to half
+  // pairs made this compiler read word 0 every time)
+  f16x8* gate = (f16x8*)(io + t * 2 * inter) + i;
+  const f16x8 g = *gate;
+  const f16x8 u = *((const f16x8*)(io + t * 2 * inter + inter) + i);
+  f16x8 r;
+#pragma unroll
+  for (int e = 0; e < 8; e++) {
+    const float x = (float)g[e];
+    const _Float16 sl = (_Float16)(x / (1.f + __builtin_amdgcn_exp2f(-x * kLog2e)));
+    r[e] = sl * u[e];  // half multiply, round to nearest even
+  }
+  *gate = r;
+}
+
+// ---------------------------------------------------------------------------------------------------
+// rotary_emb, in place on x[t, h, :] (last dimension contiguous), in the reference's half arithmetic (rotary_emb.cu:30-33):
+//   new_x1 = fma(x1, cos, -(x2 * sin)),  new_x2 = fma(x1, sin, x2 * cos)   with x1 = x[..., :D/2], x2 = x[..., D/2:],
+// every product and fma rounded to half once.  A lane owns 8 elements of x1 and the matching 8 of x2.
+// ---------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void rotary_emb_kernel(uint16_t* __restrict__ x, const uint16_t* __restrict__ cos_t,
+                                                         const uint16_t* __restrict__ sin_t, int64_t stride_t, int64_t stride_h,
+                                                         int64_t num_tokens, int64_t num_heads, int64_t head_dim) {
+  const int64_t pieces = head_dim / 16;  // 16-byte pieces in half a head
+  const int64_t gid = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (gid >= num_tokens * num_heads * pieces) return;
+  const int64_t c = gid % pieces;
+  const int64_t h = (gid / pieces) % num_heads;
+  const int64_t t = gid / (pieces * num_heads);
+  uint16_t* base = x + t * stride_t + h * stride_h;
+  f16x8* p1 = (f16x8*)base + c;
+  f16x8* p2 = (f16x8*)(base + head_dim / 2) + c;
+  const f16x8 x1 = *p1, x2 = *p2;
+  const f16x8 co = *((const f16x8*)(cos_t + t * (head_dim / 2)) + c);
+  const f16x8 si = *((const f16x8*)(sin_t + t * (head_dim / 2)) + c);
+  const f16x8 t1 = x2 * si, t2 = x2 * co;  // rounded to half (this file is compiled without contraction)
+  f16x8 n1, n2;
+#pragma unroll
+  for (int e = 0; e < 8; e++) {
+    n1[e] = __builtin_fmaf16(x1[e], co[e], -t1[e]);
+    n2[e] = __builtin_fmaf16(x1[e], si[e], t2[e]);
+  }
+  *p1 = n1;
+  *p2 = n2;
+}
+
+}  // namespace lsattn
+
+using namespace lsattn;
+
+extern "C" int lsattn_rms_norm(void* out, const void* in, const void* weight, int64_t num_tokens, int64_t hidden_size,
+                               float eps, void* stream) {
+  if (!out || !in || !weight || num_tokens < 0 || hidden_size <= 0) return LSATTN_ERR_INVALID_ARG;
+  if (hidden_size % 8 || (((uintptr_t)out | (uintptr_t)in | (uintptr_t)weight) & 15)) return LSATTN_ERR_INVALID_ARG;
+  if (num_tokens == 0) return LSATTN_OK;
+  const int64_t blocks = (num_tokens + 3) / 4;
+  if (blocks > 0x7fffffff) return LSATTN_ERR_INVALID_ARG;
+  hipLaunchKernelGGL(rms_norm_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (uint16_t*)out,
+                     (const uint16_t*)in, (const uint16_t*)weight, num_tokens, hidden_size, eps);
+  return check_launch();
+}
+
+extern "C" int lsattn_silu_and_mul_inplace(void* io, int64_t num_tokens, int64_t ffn_inter_dim, void* stream) {
+  if (!io || num_tokens < 0 || ffn_inter_dim <= 0) return LSATTN_ERR_INVALID_ARG;
+  if (ffn_inter_dim % 8 || ((uintptr_t)io & 15)) return LSATTN_ERR_INVALID_ARG;
+  if (num_tokens == 0) return LSATTN_OK;
+  const int64_t blocks = (num_tokens * (ffn_inter_dim / 8) + 255) / 256;
+  if (blocks > 0x7fffffff) return LSATTN_ERR_INVALID_ARG;
+  hipLaunchKernelGGL(silu_and_mul_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (uint16_t*)io, num_tokens,
+                     ffn_inter_dim);
+  return check_launch();
+}
+
+extern "C" int lsattn_rotary_emb(void* x, const void* cos, const void* sin, int64_t x_stride_t, int64_t x_stride_h,
+                                 int64_t num_tokens, int64_t num_heads, int64_t head_dim, void* stream) {
+  if (!x || !cos || !sin || num_tokens < 0 || num_heads <= 0 || head_dim <= 0) return LSATTN_ERR_INVALID_ARG;
+  if (head_dim % 16 || x_stride_t % 8 || x_stride_h % 8 || (((uintptr_t)x | (uintptr_t)cos | (uintptr_t)sin) & 15))
+    return LSATTN_ERR_INVALID_ARG;
+  if (num_tokens == 0) return LSATTN_OK;
+  const int64_t blocks = (num_tokens * num_heads * (head_dim / 16) + 255) / 256;
+  if (blocks > 0x7fffffff) return LSATTN_ERR_INVALID_ARG;
+  hipLaunchKernelGGL(rotary_emb_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (uint16_t*)x,
+                     (const uint16_t*)cos, (const uint16_t*)sin, x_stride_t, x_stride_h, num_tokens, num_heads, head_dim);
+  return check_launch();
+}

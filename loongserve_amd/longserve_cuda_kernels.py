@@ -94,6 +94,63 @@ def flash_decoding_stage2(o, out_logexpsum, b_seqlen, mid_o, mid_o_logexpsum, bl
     _lib.check(_lib.load().lsattn_decode_stage2(C.byref(a), _stream()), "lsattn_decode_stage2")
 
 
+def _half2d(t: torch.Tensor, name: str, dim: int) -> None:
+    if not (t.is_cuda and t.dim() == dim and t.dtype == torch.float16 and t.is_contiguous()):
+        raise ValueError("%s must be a contiguous %d-d float16 CUDA tensor" % (name, dim))
+
+
+@torch.inference_mode()
+def rms_norm(input: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    """Argument order, checks and result of ENTRY:15-39 (a new [num_tokens, hidden] fp16 tensor)."""
+    _half2d(input, "input", 2); _half2d(weight, "weight", 1)
+    if input.size(1) != weight.size(0):
+        raise ValueError("input.size(1) must equal weight.size(0)")
+    out = torch.empty_like(input)
+    _lib.check(_lib.load().lsattn_rms_norm(out.data_ptr(), input.data_ptr(), weight.data_ptr(), input.size(0), input.size(1),
+                                           float(eps), _stream()), "lsattn_rms_norm")
+    return out
+
+
+@torch.inference_mode()
+def silu_and_mul_inplace(io: torch.Tensor) -> None:
+    """ENTRY:41-52: io is [num_tokens, 2 * inter]; the first half of every row becomes silu(gate) * up."""
+    _half2d(io, "io", 2)
+    if io.size(1) % 2:
+        raise ValueError("io.size(1) must be even")
+    _lib.check(_lib.load().lsattn_silu_and_mul_inplace(io.data_ptr(), io.size(0), io.size(1) // 2, _stream()),
+               "lsattn_silu_and_mul_inplace")
+
+
+def _rotary_single(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> None:
+    if not (x.is_cuda and x.dim() == 3 and x.dtype == torch.float16 and x.stride(2) == 1):
+        raise ValueError("x must be a 3-d float16 CUDA tensor with a contiguous last dimension")
+    T, H, D = x.shape
+    _half2d(cos, "cos", 2); _half2d(sin, "sin", 2)
+    if cos.shape != sin.shape or cos.size(0) != T or cos.size(1) != D // 2:
+        raise ValueError("cos and sin must be [num_tokens, head_dim/2]")
+    _lib.check(_lib.load().lsattn_rotary_emb(x.data_ptr(), cos.data_ptr(), sin.data_ptr(), x.stride(0), x.stride(1), T, H, D,
+                                             _stream()), "lsattn_rotary_emb")
+
+
+@torch.inference_mode()
+def rotary_emb(q: torch.Tensor, k: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> None:
+    """ENTRY:54-89: in-place rotary embedding of q and of k (strided views are fine)."""
+    _rotary_single(q, cos, sin)
+    _rotary_single(k, cos, sin)
+
+
+@torch.inference_mode()
+def ffn_block(input_embds: torch.Tensor, norm_weight: torch.Tensor, norm_eps: float, gate_up_proj: torch.Tensor,
+              down_proj: torch.Tensor) -> torch.Tensor:
+    """ENTRY:91-101: rms_norm -> mm -> silu_and_mul_inplace -> mm into the normed buffer, which is returned.
+    The two matrix products are plain library GEMMs (torch.mm), as in the reference."""
+    normed = rms_norm(input_embds, norm_weight, norm_eps)
+    up_gate = torch.mm(normed, gate_up_proj)
+    silu_and_mul_inplace(up_gate)
+    torch.mm(up_gate[:, :up_gate.size(-1) // 2], down_proj, out=normed)
+    return normed
+
+
 def hello_world() -> None:
     """Load check, as ENTRY:231-232."""
     print("Hello world from loongserve_amd.longserve_cuda_kernels (liblsattn v%d)!" % _lib.load().lsattn_version())

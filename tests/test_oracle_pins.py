@@ -348,3 +348,62 @@ def test_kv_copy_register_against_index_copy():
     orc.kv_copy_register(1, torch.tensor([3], dtype=torch.int32), torch.tensor([-1], dtype=torch.int32), torch.tensor([2], dtype=torch.int32),
                          torch.tensor([3]), kv, torch.tensor([5], dtype=torch.int32), cur, mem_index, pool2, table.clone(), b_req, 0, 16, False)
     assert int(pool2.abs().sum()) == 0
+
+
+def _ulp_diff_f16(a, b):
+    """Distance in fp16 representable steps between two float16 arrays (monotone integer mapping)."""
+    import numpy as np
+    def key(v):
+        i = v.view(np.int16).astype(np.int32)
+        return np.where(i < 0, -32768 - i, i)
+    return np.abs(key(a) - key(b))
+
+
+def test_elementwise_oracle_against_float64_formulas():
+    import numpy as np
+    from oracle import elementwise_oracle as ew
+    rng = np.random.default_rng(2)
+    x = (rng.standard_normal((7, 512)) * 2).astype(np.float16)
+    w = (1 + 0.1 * rng.standard_normal(512)).astype(np.float16)
+    want = torch.from_numpy(x.astype(np.float64)) * torch.from_numpy(w.astype(np.float64)) / torch.sqrt(
+        (torch.from_numpy(x.astype(np.float64)) ** 2).mean(dim=1, keepdim=True) + 1e-5)
+    got = ew.rms_norm(x, w, 1e-5)
+    assert _ulp_diff_f16(got, want.numpy().astype(np.float16)).max() <= 1  # fp32 product order vs float64
+    io = (rng.standard_normal((5, 256)) * 3).astype(np.float16)
+    ref = io.copy()
+    ew.silu_and_mul_inplace(io)
+    g, u = torch.from_numpy(ref[:, :128].astype(np.float64)), torch.from_numpy(ref[:, 128:].astype(np.float64))
+    want = (g * torch.sigmoid(g) * u).numpy()
+    assert np.array_equal(io[:, 128:], ref[:, 128:])                      # second half untouched
+    assert np.abs(io[:, :128].astype(np.float64) - want).max() <= 2 ** -10 * np.abs(want).max() * 2  # two half roundings
+    assert _ulp_diff_f16(io[:, :128], want.astype(np.float16)).max() <= 1
+
+
+def test_rotary_oracle_is_a_rotation_and_rounds_once():
+    import numpy as np
+    from fractions import Fraction
+    from oracle import elementwise_oracle as ew
+    rng = np.random.default_rng(4)
+    T, H, D = 6, 3, 32
+    x = rng.standard_normal((T, H, D)).astype(np.float16)
+    ang = rng.uniform(0, 6.28, (T, D // 2))
+    cos, sin = np.cos(ang).astype(np.float16), np.sin(ang).astype(np.float16)
+    y = x.copy()
+    ew.rotary_emb(y, cos, sin)
+    # complex multiplication (x1 + i x2)(cos + i sin) in float64, within the half roundings
+    z = (x[..., :D // 2].astype(np.float64) + 1j * x[..., D // 2:].astype(np.float64)) * (cos + 1j * sin.astype(np.float64))[:, None, :]
+    assert np.abs(y[..., :D // 2] - z.real).max() <= 4e-3 and np.abs(y[..., D // 2:] - z.imag).max() <= 4e-3
+    # norm preservation (cos^2 + sin^2 = 1 up to the rounding of the tables)
+    n0 = (x.astype(np.float64) ** 2).sum(-1); n1 = (y.astype(np.float64) ** 2).sum(-1)
+    assert np.abs(n1 / n0 - 1).max() < 5e-3
+    # exact rational arithmetic: t = round_half(x2*sin); x1' = round_half(x1*cos - t), each rounded exactly once
+    def rh(fr):  # nearest-even rounding of a Fraction to float16 through exact comparison
+        f = np.float16(float(fr))
+        cands = [f, np.nextafter(f, np.float16(np.inf)), np.nextafter(f, np.float16(-np.inf))]
+        best = min(cands, key=lambda c: (abs(Fraction(float(c)) - fr), int(np.float16(c).view(np.int16)) & 1))
+        return np.float16(best)
+    for (t, h, i) in [(0, 0, 0), (1, 2, 5), (5, 1, 15), (3, 0, 9)]:
+        x1, x2 = Fraction(float(x[t, h, i])), Fraction(float(x[t, h, D // 2 + i]))
+        c, s = Fraction(float(cos[t, i])), Fraction(float(sin[t, i]))
+        assert y[t, h, i] == rh(x1 * c - Fraction(float(rh(x2 * s))))
+        assert y[t, h, D // 2 + i] == rh(x1 * s + Fraction(float(rh(x2 * c))))
