@@ -342,6 +342,22 @@ def other_configs(steps):
         st = _stats(_time_events(fn, steps, 3))
         ew[name] = {"median_ms": st["median_ms"], "gbs": nbytes / (st["median_ms"] * 1e-3) / 1e9,
                     "pct_of_hbm_peak": 100 * nbytes / (st["median_ms"] * 1e-3) / 1e9 / PEAK_HBM_GBS}
+    # decoding-stage migration: the last 32768 tokens of 4 requests, 2 layers, MHA 32 (16 KB per token and layer)
+    import loongserve_amd as lsa
+    Lm, Bm, nm, pool_m = 2, 4, 32768, 300000
+    kvc = _randn_half((Lm, pool_m, 64, 128), 7101, torch.float16)
+    gm = torch.Generator().manual_seed(20249)
+    tab = torch.randperm(pool_m, generator=gm)[:Bm * 2 * nm].to(torch.int32).view(Bm, 2 * nm).to(DEV).contiguous()
+    sbuf = torch.empty((Lm, Bm * nm, 64, 128), dtype=torch.float16, device=DEV)
+    mstate = torch.ones(pool_m, dtype=torch.int32, device=DEV)
+    rid, ntok, blen = _i32(list(range(Bm))), _i32([nm] * Bm), _i32([2 * nm] * Bm)
+    st = _stats(_time_events(lambda: lsa.decoding_stage_migration_sender_kernel(sbuf, tab, mstate, kvc, rid, ntok, blen), steps, 2))
+    mig_bytes = 2 * Lm * Bm * nm * 64 * 128 * 2
+    out["decode_migration_send"] = {"workload": "%d requests x %d tokens, %d layers, 16 KB rows, scattered slots (includes the host read-back of max(num_tokens), as the reference)" % (Bm, nm, Lm),
+                                    "median_ms": st["median_ms"], "gbs": mig_bytes / (st["median_ms"] * 1e-3) / 1e9,
+                                    "pct_of_hbm_peak": 100 * mig_bytes / (st["median_ms"] * 1e-3) / 1e9 / PEAK_HBM_GBS}
+    del kvc, sbuf, tab, mstate
+    torch.cuda.empty_cache()
     out["elementwise"] = {"workload": "%d tokens, hidden %d, inter %d, %d heads x %d, fp16" % (T, H, I, NH, D), **ew}
     del x, w, io, qkv, cs, sn
     torch.cuda.empty_cache()

@@ -235,6 +235,42 @@ typedef struct lsattn_kv_copy_register_args {
 int lsattn_kv_copy_register(const lsattn_kv_copy_register_args* a, void* stream);
 
 /*
+ * Decoding-stage migration of the last num_tokens[b] tokens of every request b, all layers in one launch.
+ * kv_cache is [num_layers, kvcache_size, row_bytes], the staging buffer [num_layers, sum(num_tokens), row_bytes]
+ * (row strides and layer strides in bytes, rows a multiple of 16 bytes, 16-byte aligned); num_tokens_cumsum is the
+ * inclusive prefix sum of num_tokens (same integer type), max_num_tokens an upper bound of num_tokens[] for the launch.
+ *
+ * Sender, for j < num_tokens[b]:  slot = req_to_tokens[request_ids[b], b_seq_len[b] - num_tokens[b] + j];
+ *   mem_state[slot] = 0;  send_buf[:, cumsum[b-1] + j] = kv_cache[:, slot]      (bit-exact)
+ * Receiver, for j < num_tokens[b]:  slot = alloc_mem[cumsum[b-1] + j];
+ *   req_to_tokens[request_ids[b], b_seq_len[b] + j] = slot;  kv_cache[:, slot] = recv_buf[:, cumsum[b-1] + j]
+ * Replace _fwd_sender_kernel / _fwd_receiver_kernel
+ * (loongserve/models/llama/triton_kernel/decoding_stage_migration.py:6-68, :100-157; called longserve_model.py:600-619).
+ */
+typedef struct lsattn_decode_migration_args {
+  void* staging;                    /* send_buf (written) or recv_buf (read) */
+  int64_t staging_layer_stride_bytes;
+  int64_t staging_row_stride_bytes;
+  void* kv_cache;                   /* read by the sender, written by the receiver */
+  int64_t kv_layer_stride_bytes;
+  int64_t kv_row_stride_bytes;
+  int64_t row_bytes;
+  int64_t num_layers;
+  int32_t* req_to_tokens;           /* [max_req, max_seq_len] */
+  int64_t max_seq_len;
+  int32_t* mem_state;               /* sender only */
+  const int32_t* alloc_mem;         /* receiver only: [sum(num_tokens)] */
+  const int32_t* request_ids;       /* [batch] */
+  const int32_t* num_tokens;        /* [batch] */
+  const int32_t* num_tokens_cumsum; /* [batch] */
+  const int32_t* b_seq_len;         /* [batch] */
+  int64_t batch;
+  int64_t max_num_tokens;
+} lsattn_decode_migration_args;
+int lsattn_decode_migration_send(const lsattn_decode_migration_args* a, void* stream);
+int lsattn_decode_migration_recv(const lsattn_decode_migration_args* a, void* stream);
+
+/*
  * The element-wise fp16 steps before and after attention (the rest of the reference's extension module).
  * All pointers are 16-byte aligned device pointers; sizes in elements.
  *

@@ -74,6 +74,14 @@ class KvCopyRegisterArgs(C.Structure):  # mirrors lsattn_kv_copy_register_args
                 ("reserved", C.c_int32)]
 
 
+class DecodeMigrationArgs(C.Structure):  # mirrors lsattn_decode_migration_args
+    _fields_ = [("staging", C.c_void_p), ("staging_layer_stride_bytes", C.c_int64), ("staging_row_stride_bytes", C.c_int64),
+                ("kv_cache", C.c_void_p), ("kv_layer_stride_bytes", C.c_int64), ("kv_row_stride_bytes", C.c_int64),
+                ("row_bytes", C.c_int64), ("num_layers", C.c_int64), ("req_to_tokens", C.c_void_p), ("max_seq_len", C.c_int64),
+                ("mem_state", C.c_void_p), ("alloc_mem", C.c_void_p), ("request_ids", C.c_void_p), ("num_tokens", C.c_void_p),
+                ("num_tokens_cumsum", C.c_void_p), ("b_seq_len", C.c_void_p), ("batch", C.c_int64), ("max_num_tokens", C.c_int64)]
+
+
 EXPORTS = {
     "lsattn_prefill_step": (C.c_int, [C.POINTER(PrefillArgs), _vp]),
     "lsattn_prefill_step_merge": (C.c_int, [C.POINTER(PrefillArgs), _vp]),
@@ -84,6 +92,8 @@ EXPORTS = {
     "lsattn_register_tokens": (C.c_int, [_vp, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _vp]),
     "lsattn_kv_ranges": (C.c_int, [_vp, _vp, _vp, C.c_int32, _i64, _vp, _vp, _vp, _vp]),
     "lsattn_kv_copy_register": (C.c_int, [C.POINTER(KvCopyRegisterArgs), _vp]),
+    "lsattn_decode_migration_send": (C.c_int, [C.POINTER(DecodeMigrationArgs), _vp]),
+    "lsattn_decode_migration_recv": (C.c_int, [C.POINTER(DecodeMigrationArgs), _vp]),
     "lsattn_rms_norm": (C.c_int, [_vp, _vp, _vp, _i64, _i64, C.c_float, _vp]),
     "lsattn_silu_and_mul_inplace": (C.c_int, [_vp, _i64, _i64, _vp]),
     "lsattn_rotary_emb": (C.c_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp]),

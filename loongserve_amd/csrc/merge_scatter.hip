@@ -137,6 +137,91 @@ __global__ __launch_bounds__(256) void kv_copy_register_kernel(CopyRegisterParam
   }
 }
 
+struct MigrationParams {
+  char* staging;
+  int64_t staging_layer, staging_row;
+  char* kv;
+  int64_t kv_layer, kv_row;
+  int64_t layers, max_seq_len;
+  int32_t* req_to_tokens;
+  int32_t* mem_state;
+  const int32_t* alloc_mem;
+  const int32_t* request_ids;
+  const int32_t* num_tokens;
+  const int32_t* cumsum;
+  const int32_t* b_seq_len;
+  int32_t chunks_per_row, rows_per_block;
+};
+
+// grid (groups of migrating tokens, batch); a workgroup moves rows_per_block tokens of one request through every layer,
+// 16 bytes per lane and step
+template <bool SEND> __global__ __launch_bounds__(256) void decode_migration_kernel(MigrationParams p) {
+  const int64_t b = blockIdx.y;
+  const int64_t n = p.num_tokens[b];
+  const int64_t j0 = (int64_t)blockIdx.x * p.rows_per_block;
+  if (j0 >= n) return;
+  const int64_t rows = n - j0 < p.rows_per_block ? n - j0 : p.rows_per_block;
+  const int64_t buf0 = (b > 0 ? p.cumsum[b - 1] : 0) + j0;
+  int32_t* table = p.req_to_tokens + (int64_t)p.request_ids[b] * p.max_seq_len;
+  const int64_t pos0 = SEND ? p.b_seq_len[b] - n + j0 : p.b_seq_len[b] + j0;
+  const int64_t pieces = rows * p.chunks_per_row;
+  for (int64_t i = threadIdx.x; i < pieces; i += 256) {
+    const int64_t r = i / p.chunks_per_row;
+    const int64_t c = i % p.chunks_per_row;
+    int32_t slot;
+    if (SEND) {
+      slot = table[pos0 + r];
+      if (c == 0) p.mem_state[slot] = 0;
+    } else {
+      slot = p.alloc_mem[buf0 + r];
+      if (c == 0) table[pos0 + r] = slot;
+    }
+    char* kvp = p.kv + (int64_t)slot * p.kv_row + c * 16;
+    char* bp = p.staging + (buf0 + r) * p.staging_row + c * 16;
+    for (int64_t layer = 0; layer < p.layers; layer++) {
+      if (SEND) *(u32x4*)(bp + layer * p.staging_layer) = *(const u32x4*)(kvp + layer * p.kv_layer);
+      else *(u32x4*)(kvp + layer * p.kv_layer) = *(const u32x4*)(bp + layer * p.staging_layer);
+    }
+  }
+}
+
+template <bool SEND> static int launch_migration(const lsattn_decode_migration_args* a, hipStream_t st) {
+  if (!a || !a->staging || !a->kv_cache || !a->req_to_tokens || !a->request_ids || !a->num_tokens || !a->num_tokens_cumsum ||
+      !a->b_seq_len || (SEND ? !a->mem_state : !a->alloc_mem))
+    return LSATTN_ERR_INVALID_ARG;
+  if (a->batch < 0 || a->max_num_tokens < 0 || a->num_layers <= 0 || a->row_bytes <= 0 || a->max_seq_len <= 0)
+    return LSATTN_ERR_INVALID_ARG;
+  if (a->row_bytes % 16 || a->staging_row_stride_bytes % 16 || a->staging_layer_stride_bytes % 16 || a->kv_row_stride_bytes % 16 ||
+      a->kv_layer_stride_bytes % 16 || (((uintptr_t)a->staging | (uintptr_t)a->kv_cache) & 15))
+    return LSATTN_ERR_INVALID_ARG;
+  if (a->batch == 0 || a->max_num_tokens == 0) return LSATTN_OK;
+  if (a->batch > 65535) return LSATTN_ERR_INVALID_ARG;
+  MigrationParams p;
+  p.staging = (char*)a->staging;
+  p.staging_layer = a->staging_layer_stride_bytes;
+  p.staging_row = a->staging_row_stride_bytes;
+  p.kv = (char*)a->kv_cache;
+  p.kv_layer = a->kv_layer_stride_bytes;
+  p.kv_row = a->kv_row_stride_bytes;
+  p.layers = a->num_layers;
+  p.max_seq_len = a->max_seq_len;
+  p.req_to_tokens = a->req_to_tokens;
+  p.mem_state = a->mem_state;
+  p.alloc_mem = a->alloc_mem;
+  p.request_ids = a->request_ids;
+  p.num_tokens = a->num_tokens;
+  p.cumsum = a->num_tokens_cumsum;
+  p.b_seq_len = a->b_seq_len;
+  const int64_t cpr = a->row_bytes / 16;
+  if (cpr > 0x7fffffff) return LSATTN_ERR_INVALID_ARG;
+  p.chunks_per_row = (int32_t)cpr;
+  p.rows_per_block = cpr >= 256 ? 1 : (int32_t)(256 / cpr);  // one 16-byte piece per lane and layer
+  const int64_t blocks = (a->max_num_tokens + p.rows_per_block - 1) / p.rows_per_block;
+  if (blocks > 0x7fffffff) return LSATTN_ERR_INVALID_ARG;
+  hipLaunchKernelGGL((decode_migration_kernel<SEND>), dim3((unsigned)blocks, (unsigned)a->batch), dim3(256), 0, st, p);
+  return check_launch();
+}
+
 template <typename OT> static int launch_merge(const MergeParams& p, int D, hipStream_t st) {
   const int64_t threads = p.rows * (D / 4);
   const int64_t blocks = (threads + 255) / 256;
@@ -258,6 +343,13 @@ extern "C" int lsattn_kv_copy_register(const lsattn_kv_copy_register_args* a, vo
   p.should_register = a->should_register;
   hipLaunchKernelGGL(kv_copy_register_kernel, dim3((unsigned)blocks, (unsigned)a->batch), dim3(256), 0, (hipStream_t)stream, p);
   return check_launch();
+}
+
+extern "C" int lsattn_decode_migration_send(const lsattn_decode_migration_args* a, void* stream) {
+  return launch_migration<true>(a, (hipStream_t)stream);
+}
+extern "C" int lsattn_decode_migration_recv(const lsattn_decode_migration_args* a, void* stream) {
+  return launch_migration<false>(a, (hipStream_t)stream);
 }
 
 extern "C" const char* lsattn_strerror(int code) {

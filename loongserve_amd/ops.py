@@ -261,3 +261,55 @@ def destindex_copy_and_register_kv(batch_size: int, new_kv_cache_len: torch.Tens
     a.should_register = 1 if should_register_kv else 0
     rc = _lib.load().lsattn_kv_copy_register(C.byref(a), _stream())
     _lib.check(rc, "lsattn_kv_copy_register")
+
+
+def _migration_args(buf, req_to_token_indexes, kv_cache, request_ids, num_tokens, b_seq_len):
+    B = request_ids.shape[0]
+    for t, name in ((request_ids, "request_ids"), (num_tokens, "num_tokens"), (b_seq_len, "b_seq_len")):
+        _i32vec(t, name, B)
+    _dev(buf, "buffer"); _dev(kv_cache, "kv_cache"); _dev(req_to_token_indexes, "req_to_token_indexes")
+    if kv_cache.dim() != 4 or buf.dim() != 4 or buf.dtype != kv_cache.dtype or buf.shape[0] != kv_cache.shape[0] or \
+            buf.shape[2:] != kv_cache.shape[2:]:
+        raise ValueError("buffer [layers, tokens, 2*heads, head_dim] and kv_cache [layers, slots, 2*heads, head_dim] must match")
+    if not buf[0, 0].is_contiguous() or not kv_cache[0, 0].is_contiguous():
+        raise ValueError("rows must be contiguous")
+    if req_to_token_indexes.dtype != torch.int32 or not req_to_token_indexes.is_contiguous():
+        raise ValueError("req_to_token_indexes must be contiguous int32")
+    a = _lib.DecodeMigrationArgs()
+    es = kv_cache.element_size()
+    a.staging, a.staging_layer_stride_bytes, a.staging_row_stride_bytes = buf.data_ptr(), buf.stride(0) * es, buf.stride(1) * es
+    a.kv_cache, a.kv_layer_stride_bytes, a.kv_row_stride_bytes = kv_cache.data_ptr(), kv_cache.stride(0) * es, kv_cache.stride(1) * es
+    a.row_bytes, a.num_layers = kv_cache[0, 0].numel() * es, kv_cache.shape[0]
+    a.req_to_tokens, a.max_seq_len = req_to_token_indexes.data_ptr(), req_to_token_indexes.shape[1]
+    cumsum = torch.cumsum(num_tokens, dim=0, dtype=torch.int32)
+    a.request_ids, a.num_tokens, a.num_tokens_cumsum, a.b_seq_len = request_ids.data_ptr(), num_tokens.data_ptr(), cumsum.data_ptr(), b_seq_len.data_ptr()
+    a.batch = B
+    # the launch is sized by the longest migration, read back like the reference's torch.max(num_tokens) grid dimension
+    a.max_num_tokens = int(num_tokens.max().item()) if B > 0 else 0
+    return a, cumsum
+
+
+@torch.inference_mode()
+def decoding_stage_migration_sender_kernel(send_buf, req_to_token_indexes, mem_state, kv_cache, request_ids, num_tokens, b_seq_len) -> None:
+    """Gather the last num_tokens[b] tokens of every request from every layer of kv_cache into send_buf and mark their
+    slots free.  Signature of decoding_stage_migration_sender_kernel
+    (loongserve/models/llama/triton_kernel/decoding_stage_migration.py:70-98)."""
+    if request_ids.shape[0] == 0:
+        return
+    _i32vec(mem_state, "mem_state")
+    a, keep = _migration_args(send_buf, req_to_token_indexes, kv_cache, request_ids, num_tokens, b_seq_len)
+    a.mem_state = mem_state.data_ptr()
+    _lib.check(_lib.load().lsattn_decode_migration_send(C.byref(a), _stream()), "lsattn_decode_migration_send")
+
+
+@torch.inference_mode()
+def decoding_stage_migration_receiver_kernel(recv_buf, req_to_token_indexes, kv_cache, alloc_mem, request_ids, num_tokens, b_seq_len) -> None:
+    """Store recv_buf into the freshly allocated slots of every layer of kv_cache and append the slots to the request
+    table.  Signature of decoding_stage_migration_receiver_kernel
+    (loongserve/models/llama/triton_kernel/decoding_stage_migration.py:159-183)."""
+    if request_ids.shape[0] == 0:
+        return
+    _i32vec(alloc_mem, "alloc_mem")
+    a, keep = _migration_args(recv_buf, req_to_token_indexes, kv_cache, request_ids, num_tokens, b_seq_len)
+    a.alloc_mem = alloc_mem.data_ptr()
+    _lib.check(_lib.load().lsattn_decode_migration_recv(C.byref(a), _stream()), "lsattn_decode_migration_recv")

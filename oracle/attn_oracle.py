@@ -318,3 +318,27 @@ def kv_copy_register(batch_size, new_kv_cache_len, kv_range_begin, kv_range_end,
             total_kv_cache[slot] = kv[int(kv_b_start_loc[b]) + begin + n]
             if should_register_kv:
                 req_to_token_indexs[int(b_req_idx[b]), int(cur_kv_cache_index[b]) + n] = slot
+
+
+def decoding_stage_migration_sender(send_buf, req_to_token_indexes, mem_state, kv_cache, request_ids, num_tokens, b_seq_len) -> None:
+    """_fwd_sender_kernel as loops (loongserve/models/llama/triton_kernel/decoding_stage_migration.py:44-68)."""
+    off = 0
+    for b in range(len(request_ids)):
+        n, req = int(num_tokens[b]), int(request_ids[b])
+        for j in range(n):
+            slot = int(req_to_token_indexes[req, int(b_seq_len[b]) - n + j])
+            mem_state[slot] = 0
+            send_buf[:, off + j] = kv_cache[:, slot]
+        off += n
+
+
+def decoding_stage_migration_receiver(recv_buf, req_to_token_indexes, kv_cache, alloc_mem, request_ids, num_tokens, b_seq_len) -> None:
+    """_fwd_receiver_kernel as loops (decoding_stage_migration.py:133-157)."""
+    off = 0
+    for b in range(len(request_ids)):
+        n, req = int(num_tokens[b]), int(request_ids[b])
+        for j in range(n):
+            slot = int(alloc_mem[off + j])
+            req_to_token_indexes[req, int(b_seq_len[b]) + j] = slot
+            kv_cache[:, slot] = recv_buf[:, off + j]
+        off += n

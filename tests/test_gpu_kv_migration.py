@@ -94,3 +94,41 @@ def test_migration_round_trip_feeds_decode(lsa):
     o_ref, l_ref = orc.decode_full(q, kv[:, :Hkv], kv[:, Hkv:], t_cpu, _i32([0]), _i32([n]))
     assert (o.cpu() - o_ref).abs().max().item() <= 2e-3
     assert torch.allclose(lse.cpu(), l_ref, rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_decoding_stage_migration_matches_oracle(lsa, dtype):
+    g = torch.Generator().manual_seed(41)
+    L, slots, Hkv, D, B = 4, 3000, 4, 128, 5
+    kv = torch.randn(L, slots, 2 * Hkv, D, generator=g).to(dtype)
+    table = torch.full((8, 1400), orc.INT32_PAD, dtype=torch.int32)
+    lens = [1300, 40, 600, 1, 257]
+    req = _i32([3, 7, 0, 5, 1])
+    perm = torch.randperm(slots, generator=g).to(torch.int32)
+    off = 0
+    for b, n in enumerate(lens):
+        table[int(req[b]), :n] = perm[off:off + n]
+        off += n
+    num = _i32([700, 0, 600, 1, 33])
+    b_len = _i32(lens)
+    total = int(num.sum())
+    mem_state = torch.ones(slots, dtype=torch.int32)
+    # sender
+    buf_o, ms_o = torch.zeros(L, total, 2 * Hkv, D, dtype=dtype), mem_state.clone()
+    orc.decoding_stage_migration_sender(buf_o, table, ms_o, kv, req, num, b_len)
+    buf_d, ms_d = torch.zeros(L, total, 2 * Hkv, D, dtype=dtype, device=DEV), mem_state.to(DEV)
+    lsa.decoding_stage_migration_sender_kernel(buf_d, table.to(DEV), ms_d, kv.to(DEV), req.to(DEV), num.to(DEV), b_len.to(DEV))
+    torch.cuda.synchronize()
+    assert torch.equal(buf_d.cpu().view(torch.int16), buf_o.view(torch.int16))
+    assert torch.equal(ms_d.cpu(), ms_o)
+    # receiver (another instance: holds len - num tokens of each request, kv_cache is a strided view with spare slots)
+    pool_o = torch.randn(L, 2500, 2 * Hkv, D, generator=g).to(dtype)
+    table_o = torch.full((8, 1400), orc.INT32_PAD, dtype=torch.int32)
+    alloc = torch.randperm(2500, generator=g)[:total].to(torch.int32)
+    held = b_len - num
+    pool_d, table_d = pool_o.to(DEV), table_o.to(DEV)
+    orc.decoding_stage_migration_receiver(buf_o, table_o, pool_o, alloc, req, num, held)
+    lsa.decoding_stage_migration_receiver_kernel(buf_d, table_d, pool_d, alloc.to(DEV), req.to(DEV), num.to(DEV), held.to(DEV))
+    torch.cuda.synchronize()
+    assert torch.equal(pool_d.cpu().view(torch.int16), pool_o.view(torch.int16))
+    assert torch.equal(table_d.cpu(), table_o)

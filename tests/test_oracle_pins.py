@@ -407,3 +407,42 @@ def test_rotary_oracle_is_a_rotation_and_rounds_once():
         c, s = Fraction(float(cos[t, i])), Fraction(float(sin[t, i]))
         assert y[t, h, i] == rh(x1 * c - Fraction(float(rh(x2 * s))))
         assert y[t, h, D // 2 + i] == rh(x1 * s + Fraction(float(rh(x2 * c))))
+
+
+def test_decoding_stage_migration_oracle_round_trip():
+    """Pin by invariant: send then receive on another instance reproduces, slot for slot, the tail of every request
+    (torch.index_select is the independent routine), the sender frees exactly those slots and the receiver's table is
+    extended by exactly the new slots."""
+    g = torch.Generator().manual_seed(8)
+    L, slots, W, B = 3, 90, 6, 4
+    kv_a = torch.randn(L, slots, 2, W, generator=g).to(torch.float16)
+    table_a = torch.full((6, 40), orc.INT32_PAD, dtype=torch.int32)
+    lens = [20, 7, 33, 1]
+    req = torch.tensor([4, 0, 2, 5], dtype=torch.int32)
+    perm = torch.randperm(slots, generator=g).to(torch.int32)
+    off = 0
+    for b, n in enumerate(lens):
+        table_a[int(req[b]), :n] = perm[off:off + n]
+        off += n
+    mem_state = torch.ones(slots, dtype=torch.int32)
+    num = torch.tensor([5, 0, 33, 1], dtype=torch.int32)
+    b_len = torch.tensor(lens, dtype=torch.int32)
+    buf = torch.zeros(L, int(num.sum()), 2, W, dtype=torch.float16)
+    orc.decoding_stage_migration_sender(buf, table_a, mem_state, kv_a, req, num, b_len)
+    want_slots = torch.cat([table_a[int(req[b]), lens[b] - int(num[b]):lens[b]] for b in range(B)]).long()
+    assert torch.equal(buf, kv_a.index_select(1, want_slots))
+    freed = torch.zeros(slots, dtype=torch.bool); freed[want_slots] = True
+    assert torch.equal(mem_state == 0, freed)
+    # receiver on an instance that holds the first (len - num) tokens of each request
+    kv_b = torch.zeros(L, 70, 2, W, dtype=torch.float16)
+    table_b = torch.full((6, 40), orc.INT32_PAD, dtype=torch.int32)
+    alloc = torch.randperm(70, generator=g)[:int(num.sum())].to(torch.int32)
+    held = b_len - num
+    orc.decoding_stage_migration_receiver(buf, table_b, kv_b, alloc, req, num, held)
+    assert torch.equal(kv_b.index_select(1, alloc.long()), buf)
+    o = 0
+    for b in range(B):
+        n = int(num[b])
+        assert torch.equal(table_b[int(req[b]), int(held[b]):int(held[b]) + n], alloc[o:o + n])
+        o += n
+    assert int((table_b != orc.INT32_PAD).sum()) == int(num.sum())
