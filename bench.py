@@ -359,9 +359,63 @@ def other_configs(steps):
     del kvc, sbuf, tab, mstate
     torch.cuda.empty_cache()
     out["elementwise"] = {"workload": "%d tokens, hidden %d, inter %d, %d heads x %d, fp16" % (T, H, I, NH, D), **ew}
+    out["kv_pool_allocator"] = _bench_pool_allocator(steps)
     del x, w, io, qkv, cs, sn
     torch.cuda.empty_cache()
     return out
+
+
+def _bench_pool_allocator(steps):
+    """Slot searches of config 3's pool (2.5 M slots, about half in use, scattered): a decode step's 64 new slots.
+    Wall clock per call, host work and read-backs included.  `torch_nonzero_*` times the same searches written as
+    the reference writes them (nonzero over the whole pool, then slices), on the same device, for scale."""
+    import loongserve_amd as lsa
+    size, need = 2_500_000, 64
+    mm = lsa.LongServeMemoryManager(size, torch.float16, 1, 8, 1)
+    g = torch.Generator().manual_seed(20243)
+    mm.add_refs(torch.randperm(size, generator=g)[:size // 2].to(DEV))
+
+    def wall_us(fn, undo):
+        for _ in range(3):
+            undo(fn())
+        torch.cuda.synchronize()
+        t = []
+        for _ in range(max(steps, 10)):
+            t0 = time.perf_counter()
+            r = fn()
+            torch.cuda.synchronize()
+            t.append((time.perf_counter() - t0) * 1e6)
+            undo(r)
+            torch.cuda.synchronize()
+        return sorted(t)[len(t) // 2]
+
+    def ref_alloc():
+        can_use = torch.nonzero(mm.mem_state == 0).view(-1)
+        sel = can_use[0:need]
+        used = torch.count_nonzero(mm.mem_state[sel]).item()
+        mm.mem_state[sel] += 1
+        return sel
+
+    def ref_contig():
+        can_use = torch.nonzero(mm.mem_state == 0).view(-1)
+        n = len(can_use)
+        hit = can_use[0:n - 8 + 1][(can_use[8 - 1:] - can_use[0:n - 8 + 1]) == 8 - 1]
+        return int(hit[0].item()) if hit.shape[0] else -1
+
+    def undo_ref(sel):
+        mm.mem_state[sel] -= 1
+
+    res = {"workload": "pool of %d slots, half in use (scattered); alloc(%d) and the first run of 8 free slots" % (size, need),
+           "alloc_us": wall_us(lambda: mm.alloc(need), mm.free),
+           "find_contiguous_us": wall_us(lambda: mm._slots.first_fit(8), lambda r: None),
+           "torch_nonzero_alloc_us": wall_us(ref_alloc, undo_ref),
+           "torch_nonzero_find_contiguous_us": wall_us(ref_contig, lambda r: None)}
+    ev = _stats(_time_events(lambda: mm._slots.first_fit(8), max(steps, 10), 3))
+    res["find_contiguous_device_ms"] = ev["median_ms"]
+    res["state_bytes_scanned"] = 2 * size * 4
+    del mm
+    torch.cuda.empty_cache()
+    return res
 
 
 def main():

@@ -29,6 +29,7 @@ extern "C" {
 #define LSATTN_ERR_INVALID_ARG (-1) /* null pointer, negative size, bad stride            */
 #define LSATTN_ERR_UNSUPPORTED (-2) /* head_dim / dtype / head ratio the kernels lack     */
 #define LSATTN_ERR_LAUNCH (-3)      /* hipGetLastError() after the launch was not success */
+#define LSATTN_ERR_WORKSPACE (-4)   /* the workspace passed in is smaller than required    */
 
 /* element types of q/k/v and of `o` outputs */
 #define LSATTN_F16 0
@@ -294,6 +295,39 @@ int lsattn_silu_and_mul_inplace(void* io, int64_t num_tokens, int64_t ffn_inter_
  */
 int lsattn_rotary_emb(void* x, const void* cos, const void* sin, int64_t x_stride_t, int64_t x_stride_h,
                       int64_t num_tokens, int64_t num_heads, int64_t head_dim, void* stream);
+
+/*
+ * Slot allocator of the KV pool.  mem_state is int32 [pool_size] on the device (16-byte aligned), 0 = free slot,
+ * otherwise the slot's reference count.  The searches need a device workspace of
+ * lsattn_pool_search_workspace_bytes(pool_size) bytes (16-byte aligned); nothing is allocated or kept by the library
+ * and no call waits for the device.
+ *
+ * lsattn_pool_alloc: out_index[0:need] = the first `need` free slots in ascending order, each marked in use
+ * (0 -> 1).  If fewer are free, the rest of out_index is -1; the caller compares `need` with its own count of
+ * free slots first, as the reference does.  Replaces torch.nonzero(mem_state == 0)[0:need] + add_refs in
+ * LongServeMemoryManager.alloc (loongserve/common/longserve_mem_manager.py:32-40).
+ */
+size_t lsattn_pool_search_workspace_bytes(int64_t pool_size);
+int lsattn_pool_alloc(int32_t* mem_state, int64_t pool_size, int64_t need, int64_t* out_index, void* workspace,
+                      size_t workspace_bytes, void* stream);
+/*
+ * *out_start (device) = the lowest s such that slots s .. s+need-1 are all free, or -1 if there is no such run.
+ * mem_state is not changed.  Replaces the nonzero / shifted-difference search of
+ * LongServeMemoryManager.alloc_contiguous (longserve_mem_manager.py:50-55); need >= 1.
+ */
+int lsattn_pool_find_contiguous(const int32_t* mem_state, int64_t pool_size, int64_t need, int64_t* out_start,
+                                void* workspace, size_t workspace_bytes, void* stream);
+/*
+ * mem_state[index[i]] = old value + delta (delta = +1 or -1) for i < n; a slot listed several times still changes
+ * by delta once, as `mem_state[index] += delta` does in torch.  counted (device, int64[2]):
+ *   counted[0] = entries whose slot is non-zero before the update (delta = +1) or after it (delta = -1): the
+ *                has_used_tokens / used_tokens of add_refs and decrease_refs (longserve_mem_manager.py:73-88);
+ *   counted[1] = entries outside [-pool_size, pool_size), which are skipped (negative entries wrap once).
+ * workspace: lsattn_pool_refs_workspace_bytes(n) bytes, 16-byte aligned.
+ */
+size_t lsattn_pool_refs_workspace_bytes(int64_t n);
+int lsattn_pool_update_refs(int32_t* mem_state, int64_t pool_size, const int64_t* index, int64_t n, int delta,
+                            int64_t* counted, void* workspace, size_t workspace_bytes, void* stream);
 
 const char* lsattn_strerror(int code);
 int lsattn_version(void);

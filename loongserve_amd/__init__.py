@@ -18,6 +18,7 @@ if not _building:
     _lib.load()  # fail loudly at import time if the HIP library is missing or stale
 
 from . import longserve_cuda_kernels  # noqa: E402
+from .kv_pool import LongServeMemoryManager, LongServeReqManager  # noqa: E402
 from .decoding import (longserve_flash_decode_stage1, longserve_flash_decode_stage2,  # noqa: E402
                        longserve_token_decode_attention_flash_decoding)
 from .ops import (context_attention_fwd, decoding_stage_migration_receiver_kernel,  # noqa: E402
@@ -30,4 +31,5 @@ __all__ = [
     "decoding_stage_migration_sender_kernel", "decoding_stage_migration_receiver_kernel",
     "longserve_flash_decode_stage1", "longserve_flash_decode_stage2",
     "longserve_token_decode_attention_flash_decoding", "longserve_cuda_kernels",
+    "LongServeMemoryManager", "LongServeReqManager",
 ]

@@ -97,6 +97,11 @@ EXPORTS = {
     "lsattn_rms_norm": (C.c_int, [_vp, _vp, _vp, _i64, _i64, C.c_float, _vp]),
     "lsattn_silu_and_mul_inplace": (C.c_int, [_vp, _i64, _i64, _vp]),
     "lsattn_rotary_emb": (C.c_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp]),
+    "lsattn_pool_search_workspace_bytes": (C.c_size_t, [_i64]),
+    "lsattn_pool_alloc": (C.c_int, [_vp, _i64, _i64, _vp, _vp, C.c_size_t, _vp]),
+    "lsattn_pool_find_contiguous": (C.c_int, [_vp, _i64, _i64, _vp, _vp, C.c_size_t, _vp]),
+    "lsattn_pool_refs_workspace_bytes": (C.c_size_t, [_i64]),
+    "lsattn_pool_update_refs": (C.c_int, [_vp, _i64, _vp, _i64, C.c_int, _vp, _vp, C.c_size_t, _vp]),
     "lsattn_strerror": (C.c_char_p, [C.c_int]),
     "lsattn_version": (C.c_int, []),
 }

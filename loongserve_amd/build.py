@@ -14,7 +14,7 @@ PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(PKG_DIR)
 CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_PATH = os.path.join(PKG_DIR, "liblsattn.so")
-SOURCES = ["prefill.hip", "decode.hip", "merge_scatter.hip", "elementwise.hip"]
+SOURCES = ["prefill.hip", "decode.hip", "merge_scatter.hip", "elementwise.hip", "pool.hip"]
 # elementwise.hip reproduces the reference's half arithmetic operation by operation: no fused multiply-adds
 # other than the ones it writes
 FILE_FLAGS = {"elementwise.hip": ["-ffp-contract=off"]}

@@ -358,6 +358,7 @@ extern "C" const char* lsattn_strerror(int code) {
     case LSATTN_ERR_INVALID_ARG: return "invalid argument (null pointer, bad size, stride or alignment)";
     case LSATTN_ERR_UNSUPPORTED: return "unsupported head_dim, dtype or head ratio";
     case LSATTN_ERR_LAUNCH: return "kernel launch failed";
+    case LSATTN_ERR_WORKSPACE: return "workspace too small";
     default: return "unknown error";
   }
 }

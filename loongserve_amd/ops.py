@@ -41,6 +41,16 @@ def _i32vec(t: torch.Tensor, name: str, n: Optional[int] = None) -> None:
         raise ValueError("%s must have %d entries" % (name, n))
 
 
+def _slots(t: torch.Tensor, name: str, n: Optional[int] = None) -> torch.Tensor:
+    """A vector of pool slot numbers.  The reference's allocator hands these out as int64 (torch.nonzero /
+    arange, loongserve/common/longserve_mem_manager.py:21, :37) while the kernels read int32: an int64 vector is
+    narrowed on the device first (pools have fewer than 2**31 slots)."""
+    if t.dtype == torch.int64:
+        t = t.to(torch.int32)
+    _i32vec(t, name, n)
+    return t
+
+
 def _prefill_args(q, k, v, o, q_b_start_loc, q_b_seq_len, q_first, kv_b_start_loc, kv_b_seq_len, kv_first,
                   peers: int, max_q_len: int, sm_scale: Optional[float]) -> _lib.PrefillArgs:
     for t, n in ((q, "q"), (k, "k"), (v, "v"), (o, "o")):
@@ -165,7 +175,8 @@ def kv_scatter(src: torch.Tensor, dest_index: torch.Tensor, pool: torch.Tensor) 
     Semantics of destindex_copy_kv
     (loongserve/common/basemodel/triton_kernel/destindex_copy_kv.py:31-51).
     """
-    _dev(src, "src"); _dev(pool, "pool"); _i32vec(dest_index, "dest_index", src.shape[0])
+    _dev(src, "src"); _dev(pool, "pool")
+    dest_index = _slots(dest_index, "dest_index", src.shape[0])
     if src.dtype != pool.dtype or src.shape[1:] != pool.shape[1:]:
         raise ValueError("src and pool rows must match")
     if not src[0].is_contiguous() or not pool[0].is_contiguous():
@@ -188,7 +199,8 @@ def init_req_to_token_indexes(req_to_token_indexs, b_req_idx, b_seq_len, alloc_m
     if req_to_token_indexs.dtype != torch.int32 or not req_to_token_indexs.is_contiguous():
         raise ValueError("req_to_token_indexs must be contiguous int32")
     B = b_req_idx.shape[0]
-    _i32vec(b_req_idx, "b_req_idx", B); _i32vec(b_seq_len, "b_seq_len", B); _i32vec(alloc_mem_index, "alloc_mem_index")
+    _i32vec(b_req_idx, "b_req_idx", B); _i32vec(b_seq_len, "b_seq_len", B)
+    alloc_mem_index = _slots(alloc_mem_index, "alloc_mem_index")
     if b_start_loc is None:
         b_start_loc = (torch.cumsum(b_seq_len, 0, dtype=torch.int32) - b_seq_len).to(torch.int32)
     if max_len_in_batch is None:
@@ -238,7 +250,7 @@ def destindex_copy_and_register_kv(batch_size: int, new_kv_cache_len: torch.Tens
     for t, name in ((new_kv_cache_len, "new_kv_cache_len"), (kv_range_begin, "kv_range_begin"), (kv_range_end, "kv_range_end"),
                     (kv_b_start_loc, "kv_b_start_loc"), (cur_kv_cache_index, "cur_kv_cache_index"), (b_req_idx, "b_req_idx")):
         _i32vec(t, name, B)
-    _i32vec(mem_index, "mem_index")
+    mem_index = _slots(mem_index, "mem_index")
     _dev(new_kv_cache_len_sum, "new_kv_cache_len_sum")
     if new_kv_cache_len_sum.dtype != torch.int64 or new_kv_cache_len_sum.shape != (B,) or not new_kv_cache_len_sum.is_contiguous():
         raise ValueError("new_kv_cache_len_sum must be a contiguous int64 vector of length batch_size")
@@ -309,7 +321,7 @@ def decoding_stage_migration_receiver_kernel(recv_buf, req_to_token_indexes, kv_
     (loongserve/models/llama/triton_kernel/decoding_stage_migration.py:159-183)."""
     if request_ids.shape[0] == 0:
         return
-    _i32vec(alloc_mem, "alloc_mem")
+    alloc_mem = _slots(alloc_mem, "alloc_mem")
     a, keep = _migration_args(recv_buf, req_to_token_indexes, kv_cache, request_ids, num_tokens, b_seq_len)
     a.alloc_mem = alloc_mem.data_ptr()
     _lib.check(_lib.load().lsattn_decode_migration_recv(C.byref(a), _stream()), "lsattn_decode_migration_recv")

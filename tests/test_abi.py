@@ -83,6 +83,19 @@ def test_validation_rejects_bad_arguments_without_gpu():
     m = _lib.MergeArgs()
     assert lib.lsattn_lse_merge(C.byref(m), None) == -1
     assert lib.lsattn_kv_scatter(None, 0, None, 0, None, 0, 0, None) == -1
+    # slot allocator: sizes of the workspaces are host arithmetic, argument checks come before any launch
+    assert lib.lsattn_pool_search_workspace_bytes(0) == 0
+    assert lib.lsattn_pool_search_workspace_bytes(4096) == 16 + 28 + 4          # one workgroup of slots, padded to 16
+    assert lib.lsattn_pool_search_workspace_bytes(2_500_000) >= 16 + 611 * 28
+    assert lib.lsattn_pool_refs_workspace_bytes(0) == 0
+    assert lib.lsattn_pool_refs_workspace_bytes(257) == 2 * 16 + 1040
+    assert lib.lsattn_pool_alloc(None, 8, 1, None, None, 0, None) == -1
+    assert lib.lsattn_pool_alloc(0x1000, 8192, 1, 0x2000, 0x3000, 16, None) == -4  # workspace too small
+    assert lib.lsattn_pool_find_contiguous(0x1000, 8192, 0, 0x2000, 0x3000, 1 << 20, None) == -1  # need >= 1
+    assert lib.lsattn_pool_find_contiguous(0x1004, 8192, 1, 0x2000, 0x3000, 1 << 20, None) == -1  # misaligned state
+    assert lib.lsattn_pool_update_refs(0x1000, 8, 0x2000, 4, 2, 0x3000, 0x4000, 1 << 20, None) == -1  # delta must be +-1
+    assert lib.lsattn_pool_update_refs(0x1000, 8, 0x2000, 4, 1, 0x3000, 0x4000, 8, None) == -4
+    assert b"workspace" in lib.lsattn_strerror(-4)
     # unsupported head_dim is reported as such (pointers are fake but never dereferenced)
     fake = 0x1000
     for f in ("q", "k", "v", "o", "lse", "q_b_start_loc", "q_b_seq_len", "q_first_token_global_idx", "kv_b_start_loc",

@@ -446,3 +446,88 @@ def test_decoding_stage_migration_oracle_round_trip():
         assert torch.equal(table_b[int(req[b]), int(held[b]):int(held[b]) + n], alloc[o:o + n])
         o += n
     assert int((table_b != orc.INT32_PAD).sum()) == int(num.sum())
+
+
+# --------------------------------------------------------------------------------------------------------------
+# KV-pool slot allocator oracle: pinned by slot-by-slot scans written without nonzero / slicing
+# --------------------------------------------------------------------------------------------------------------
+def _scan_first_free(state, need):
+    out = []
+    for p, s in enumerate(state):
+        if len(out) == need:
+            break
+        if s == 0:
+            out.append(p)
+    return out
+
+
+def _scan_first_fit(state, need):
+    run = 0
+    for p, s in enumerate(state):
+        run = run + 1 if s == 0 else 0
+        if run == need:
+            return p - need + 1
+    return None
+
+
+def test_pool_oracle_searches_against_slot_scans():
+    import numpy as np
+    from oracle.pool_oracle import MemoryManagerOracle
+    rng = np.random.default_rng(5)
+    for trial in range(60):
+        size = int(rng.integers(1, 300))
+        m = MemoryManagerOracle(size)
+        busy = rng.random(size) < rng.choice([0.05, 0.3, 0.7])
+        m.add_refs(np.nonzero(busy)[0])
+        assert m.can_use_mem_size == int((m.mem_state == 0).sum())
+        before = m.mem_state.copy()
+        need = int(rng.integers(1, 12))
+        want = _scan_first_fit(before, need)
+        got = m.alloc_contiguous(need)
+        if want is None:
+            assert got is None and (m.mem_state == before).all()
+        else:
+            idx, start, end = got
+            assert (start, end) == (want, want + need) and idx.tolist() == list(range(want, want + need))
+            assert (m.mem_state[start:end] == 1).all()
+        assert m.can_use_mem_size == int((m.mem_state == 0).sum())
+        before = m.mem_state.copy()
+        need = int(rng.integers(0, m.can_use_mem_size + 1))
+        got = m.alloc(need)
+        assert got.tolist() == _scan_first_free(before, need)
+        assert (m.mem_state[got] == 1).all() and m.can_use_mem_size == int((m.mem_state == 0).sum())
+    # a run that ends exactly at the last slot, and one slot short of fitting
+    m = MemoryManagerOracle(10)
+    m.add_refs(np.array([0, 1, 2, 3, 4, 5]))
+    assert m.alloc_contiguous(5) is None
+    assert m.alloc_contiguous(4)[1:] == (6, 10)
+    with pytest.raises(AssertionError):
+        MemoryManagerOracle(4).alloc(5)
+
+
+def test_pool_oracle_reference_counts_and_duplicates():
+    import numpy as np
+    from oracle.pool_oracle import MemoryManagerOracle
+    m = MemoryManagerOracle(8)
+    m.add_refs(np.array([1, 1, 3]))           # slot 1 listed twice: gains one reference, but both entries count as new
+    assert m.mem_state.tolist() == [0, 1, 0, 1, 0, 0, 0, 0] and m.can_use_mem_size == 8 - 3
+    m.add_refs(np.array([1, 2]))              # slot 1 is shared now
+    assert m.mem_state.tolist() == [0, 2, 1, 1, 0, 0, 0, 0] and m.can_use_mem_size == 8 - 3 - 1
+    m.free(np.array([1, 2], dtype=np.int32))  # slot 1 keeps one reference, slot 2 becomes free
+    assert m.mem_state.tolist() == [0, 1, 0, 1, 0, 0, 0, 0] and m.can_use_mem_size == 8 - 3
+    m.free_all()
+    assert m.can_use_mem_size == 8 and not m.mem_state.any()
+    # a random trace without duplicates keeps the conservation law
+    rng = np.random.default_rng(11)
+    m = MemoryManagerOracle(200)
+    held = []
+    for step in range(200):
+        if held and rng.random() < 0.45:
+            m.free(held.pop(int(rng.integers(len(held)))))
+        else:
+            need = int(rng.integers(1, 20))
+            if need <= m.can_use_mem_size:
+                got = m.alloc_contiguous(need) if rng.random() < 0.5 else None
+                held.append(got[0].copy() if got is not None else m.alloc(need).copy())
+        assert m.can_use_mem_size == int((m.mem_state == 0).sum())
+        assert sum(len(h) for h in held) == int(m.mem_state.sum())
