@@ -10,15 +10,17 @@
 //   * K/V tiles of 64 keys are staged through LDS (rings of four tiles, filled by global->LDS DMA,
 //     XOR-swizzled 16-byte chunks so that both the row-wise K reads and the transposing V reads
 //     use all 64 banks);
-//   * scores are computed transposed, S^T = K Q^T with v_mfma_f32_32x32x16, so every lane
-//     owns one query column: row max / row sum are in-lane reductions plus one
-//     half-wave swap, and the fp32 S^T accumulators convert in place into the B operand
-//     of O^T += V^T P^T without any cross-lane movement (P and V always as fp16);
+//   * scores are computed transposed, S^T = K Q^T with v_mfma_f32_16x16x32 (under this kernel's load the
+//     chip is power-limited, and this shape sustains a clearly higher clock than 32x32x16 at the same
+//     operand traffic), so every lane owns one query column of each of the wave's two 16-row blocks:
+//     row max / row sum are in-lane reductions plus an exchange between the four lanes of a column,
+//     and the fp32 S^T accumulators convert in place into the B operand of O^T += V^T P^T without
+//     any cross-lane movement (P and V always as fp16);
 //   * V^T operands come from LDS through ds_read_b64_tr_b16 (the tile is stored row-major);
 //   * on this hardware an MFMA holds its own wave until it is done, and vector work of the
 //     SIMD's other wave runs beside it only under conditions (higher wave priority, no short
 //     dependent chains, no dot-product instructions).  The fully visible part of the key range
-//     therefore runs as alternating phases: one wave of the SIMD issues the sixteen MFMAs of a
+//     therefore runs as alternating phases: one wave of the SIMD issues the thirty-two MFMAs of a
 //     32-key step while the other does the exponentials of its own step, a workgroup barrier
 //     ends each phase;
 //   * tiles that straddle the diagonal or the end of the KV chunk take a general, masked,
@@ -54,19 +56,42 @@ struct PrefillParams {
 
 constexpr int BM = 256;   // query rows per workgroup (32 per wave)
 constexpr int BN = 64;    // keys per LDS tile
-constexpr int SUB = 32;   // keys per pipeline step (one 32x32 MFMA block row)
+constexpr int SUB = 32;   // keys per pipeline step (the contraction length of one P V MFMA)
 constexpr int NWAVE = 8;  // two per SIMD
 constexpr float kLazyRescale = 8.f;  // log2 units the running max may lag before O is rescaled
 
 template <typename T> struct Mfma;
 template <> struct Mfma<F16> {
-  static __device__ __forceinline__ f32x16 run(const u32x4& a, const u32x4& b, const f32x16& c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  static __device__ __forceinline__ f32x4 run(const u32x4& a, const u32x4& b, const f32x4& c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
   }
 };
 template <> struct Mfma<BF16> {
-  static __device__ __forceinline__ f32x16 run(const u32x4& a, const u32x4& b, const f32x16& c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  static __device__ __forceinline__ f32x4 run(const u32x4& a, const u32x4& b, const f32x4& c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  }
+};
+
+// The same MFMAs issued from inline assembly with the accumulator tied to the destination.  Left to itself the register
+// allocator gives every 16x16 result a fresh register tuple (this shape allows any overlap of destination and
+// accumulator), the accumulators then wander through the register file over the unrolled loop and the kernel spills.
+// The compiler's hazard bookkeeping does not cover these: each use below is far enough from the producers and
+// consumers of its operands (see the fast loop).
+template <typename T> struct MfmaAsm;
+template <> struct MfmaAsm<F16> {
+  static __device__ __forceinline__ void acc(f32x4& c, const u32x4& a, const u32x4& b) {
+    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
+  }
+  static __device__ __forceinline__ void first(f32x4& c, const u32x4& a, const u32x4& b) {
+    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "v"(b));
+  }
+};
+template <> struct MfmaAsm<BF16> {
+  static __device__ __forceinline__ void acc(f32x4& c, const u32x4& a, const u32x4& b) {
+    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
+  }
+  static __device__ __forceinline__ void first(f32x4& c, const u32x4& a, const u32x4& b) {
+    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "v"(b));
   }
 };
 
@@ -91,11 +116,27 @@ template <> __device__ __forceinline__ u32x4 to_pv_operand<BF16>(const u32x4& w)
 template <typename T> struct DirectV { static constexpr bool value = true; };
 template <> struct DirectV<BF16> { static constexpr bool value = false; };
 
-// value of the same register in the other half of the wave (lane ^ 32)
-__device__ __forceinline__ float other_half(float v, int upper) {
-  const unsigned u = __builtin_bit_cast(unsigned, v);
-  auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
-  return __builtin_bit_cast(float, upper ? r[0] : r[1]);
+// Maxima on values that come out of inline-assembly MFMAs: through the fmaxf builtin the compiler first quiets
+// possible signalling NaNs (one more instruction per input), which these accumulators never hold.
+__device__ __forceinline__ float max3_raw(float a, float b, float c) {
+  float r;
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+}
+__device__ __forceinline__ float max_raw(float a, float b) {
+  float r;
+  asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+  return r;
+}
+
+// A query column of a 16x16 block lives in the four lanes c, c + 16, c + 32, c + 48: maximum / sum over them
+__device__ __forceinline__ float column_max(float v) {
+  v = fmaxf(v, __shfl_xor(v, 16));
+  return fmaxf(v, __shfl_xor(v, 32));
+}
+__device__ __forceinline__ float column_sum(float v) {
+  v += __shfl_xor(v, 16);
+  return v + __shfl_xor(v, 32);
 }
 
 // LDS: a ring of four K tiles at [0, 64K) and a ring of four V tiles at [64K, 128K); a tile is [64 rows][16 chunks of 16 bytes]
@@ -106,9 +147,10 @@ constexpr int kLdsV = kRing * kTileBytes;
 constexpr int kLdsBytes = 2 * kRing * kTileBytes;
 // LDS has 64 four-byte banks (256 bytes per clock): sixteen lanes of a 16-byte read, thirty-two lanes of
 // an 8-byte read are served together.  With this XOR the sixteen K rows read together land in sixteen
-// different 16-byte bank groups, and the four V rows of a transposing read (64 contiguous bytes each)
-// land in four different 64-byte groups; both patterns then run at the rate of a linear read.
-__device__ __forceinline__ int swz_bits(int row) { return ((row & 3) << 2) | ((row >> 2) & 3); }
+// different 16-byte bank groups, and the eight V rows of half a transposing read (32 contiguous bytes each)
+// land in eight different 32-byte groups; both patterns then run at the rate of a linear read.  Only the
+// low four bits of the row count, so rows 16 apart share their XOR.
+__device__ __forceinline__ int swz_bits(int row) { return ((row & 7) << 1) | ((row >> 3) & 1); }
 
 typedef __attribute__((address_space(3))) i16x4* lds_i16x4_ptr;
 typedef __attribute__((address_space(3))) void* lds_void_ptr;
@@ -117,29 +159,29 @@ typedef const __attribute__((address_space(1))) void* global_void_ptr;
 // s_waitcnt on the vector-memory counter only (expcnt / lgkmcnt fields left at their maximum)
 template <int N> __device__ __forceinline__ void wait_vmem() { __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14)); }
 
-// K A-operands of one 32-key sub-tile: 8 x 16 bytes per lane
-// koff0 is the lane's byte offset for k-step 0; the swizzle is an XOR on the chunk index, so k-step t8
-// sits at koff0 ^ (t8 << 5).  lds_k_sub is the LDS byte address of the sub-tile (a multiple of 8 KB,
-// so adding the offset never carries into the XORed bits).
-__device__ __forceinline__ void load_k_operands(int lds_k_sub, int koff0, u32x4 (&ka)[8]) {
+// K A-operands of one 32-key sub-tile, ka[kb][ks] = K[16 kb + lane % 16][32 ks + 8 (lane / 16) .. + 7]: 8 x 16 bytes per lane.
+// koff0 is the lane's byte offset for key block 0 and k-step 0; the swizzle is an XOR on the chunk index, so k-step ks
+// sits at koff0 ^ (ks << 6), key block 1 sixteen rows (4 KB) further.  lds_k_sub is the LDS byte address of the
+// sub-tile (a multiple of 8 KB, so adding the offset never carries into the XORed bits).
+__device__ __forceinline__ void load_k_operands(int lds_k_sub, int koff0, u32x4 (&ka)[2][4]) {
   const int base = lds_k_sub + koff0;
 #pragma unroll
-  for (int t8 = 0; t8 < 8; t8++) ka[t8] = *(const __attribute__((address_space(3))) u32x4*)(base ^ (t8 << 5));
+  for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++) ka[kb][ks] = *(const __attribute__((address_space(3))) u32x4*)((base ^ (ks << 6)) + kb * (16 * 256));
 }
-// V^T A-operands of one 32-key sub-tile through transposing LDS reads
-// voffa0 / voffb0 are the lane's byte offsets for d-block 0 (keys base+4g'+r and +8); d-block db sits at
-// offset ^ (db << 6), the second group of 16 keys 4 KB further.
-__device__ __forceinline__ void load_v_operands(int lds_v_sub, int voffa0, int voffb0, u32x4 (&va)[2][4]) {
-  const int base_a = lds_v_sub + voffa0, base_b = lds_v_sub + voffb0;
+// V^T A-operands of one 32-key sub-tile through transposing LDS reads: va[db] = V^T[16 db + lane % 16][the lane group's
+// eight keys], which are keys 4g .. 4g+3 and 16+4g .. 16+4g+3 of the sub-tile (g = lane / 16): the keys whose scores
+// the lane group holds after S^T = K Q^T.  voff0 is the lane's byte offset for d-block 0 and the first four keys;
+// d-block db sits at voff0 ^ (db << 5), the second four keys sixteen rows (4 KB) further.
+__device__ __forceinline__ void load_v_operands(int lds_v_sub, int voff0, u32x4 (&va)[8]) {
+  const int base = lds_v_sub + voff0;
 #pragma unroll
-  for (int jj = 0; jj < 2; jj++) {
-#pragma unroll
-    for (int db = 0; db < 4; db++) {
-      const i16x4 xa = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_ptr)((base_a ^ (db << 6)) + jj * (16 * 256)));
-      const i16x4 xb = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_ptr)((base_b ^ (db << 6)) + jj * (16 * 256)));
-      const u32x2 wa = __builtin_bit_cast(u32x2, xa), wb = __builtin_bit_cast(u32x2, xb);
-      va[jj][db] = u32x4{wa[0], wa[1], wb[0], wb[1]};
-    }
+  for (int db = 0; db < 8; db++) {
+    const i16x4 xa = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_ptr)(base ^ (db << 5)));
+    const i16x4 xb = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_ptr)((base ^ (db << 5)) + 16 * 256));
+    const u32x2 wa = __builtin_bit_cast(u32x2, xa), wb = __builtin_bit_cast(u32x2, xb);
+    va[db] = u32x4{wa[0], wa[1], wb[0], wb[1]};
   }
 }
 
@@ -150,46 +192,54 @@ __device__ __forceinline__ const char* uniform_ptr(const char* ptr) {
   return (const char*)(((uint64_t)hi << 32) | lo);
 }
 
+// Online-softmax update for one 32-key sub-tile in the general path.  s[kb][qb][r] is the score of key
+// n0 + 16 kb + 4 g + r for the lane's query row of block qb; on return pk[qb] holds that row's eight P values as
+// the B operand of the P V MFMA, in the key order the V^T operands use.  The running maximum only moves when some
+// row of the wave exceeds it by more than kLazyRescale (then every row takes its true maximum).
 template <bool MASK>
-__device__ __forceinline__ bool softmax32(f32x16& s, u32x4 (&pk)[2], float& m_run, float& l_run, float& alpha, float scale_log2, int g, int n0,
-                                          int kv_len, int kf, int P, int qpos) {
-  if (MASK) {
+__device__ __forceinline__ bool softmax32(f32x4 (&s)[2][2], u32x4 (&pk)[2], float (&m_run)[2], float (&l_run)[2], float (&alpha)[2],
+                                          float scale_log2, int g, int n0, int kv_len, int kf, int P, const int (&qpos)[2]) {
+  float mx[2];
+  bool over = false;
 #pragma unroll
-    for (int i = 0; i < 16; i++) {
-      const int n = n0 + (i >> 2) * 8 + 4 * g + (i & 3);
-      const bool vis = (n < kv_len) && (kf + n * P <= qpos);
-      s[i] = vis ? s[i] : -INFINITY;
+  for (int qb = 0; qb < 2; qb++) {
+    if (MASK) {
+#pragma unroll
+      for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+          const int n = n0 + 16 * kb + 4 * g + r;
+          const bool vis = (n < kv_len) && (kf + n * P <= qpos[qb]);
+          s[kb][qb][r] = vis ? s[kb][qb][r] : -INFINITY;
+        }
     }
+    float m8 = fmaxf(fmaxf(s[0][qb][0], s[0][qb][1]), fmaxf(s[0][qb][2], s[0][qb][3]));
+    m8 = fmaxf(m8, fmaxf(fmaxf(s[1][qb][0], s[1][qb][1]), fmaxf(s[1][qb][2], s[1][qb][3])));
+    mx[qb] = column_max(m8) * scale_log2;
+    over = over || (mx[qb] > m_run[qb] + kLazyRescale);
   }
-  float mx = fmaxf(s[0], s[1]);
+  const bool any = __builtin_amdgcn_ballot_w64(over) != 0;
 #pragma unroll
-  for (int i = 2; i < 16; i += 2) mx = fmaxf(mx, fmaxf(s[i], s[i + 1]));
-  mx = fmaxf(mx, other_half(mx, g)) * scale_log2;
-  const bool any = __builtin_amdgcn_ballot_w64(mx > m_run + kLazyRescale) != 0;
-  const float m_new = any ? fmaxf(m_run, mx) : m_run;
-  float m_use = m_new;
-  if (MASK) {
-    m_use = (m_new == -INFINITY) ? 0.f : m_new;
-    alpha = (m_run == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m_run - m_use);
-  } else {
-    alpha = __builtin_amdgcn_exp2f(m_run - m_new);
-  }
-  m_run = m_new;
-  float ps0 = 0.f, ps1 = 0.f;
-#pragma unroll
-  for (int jj = 0; jj < 2; jj++) {
+  for (int qb = 0; qb < 2; qb++) {
+    const float m_new = any ? fmaxf(m_run[qb], mx[qb]) : m_run[qb];
+    const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+    alpha[qb] = (m_run[qb] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m_run[qb] - m_use);
+    m_run[qb] = m_new;
+    float ps0 = 0.f, ps1 = 0.f;
     u32x4 w;
 #pragma unroll
-    for (int e = 0; e < 4; e++) {
-      const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[8 * jj + 2 * e], scale_log2, -m_use));
-      const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[8 * jj + 2 * e + 1], scale_log2, -m_use));
-      w[e] = pack2<F16>(p0, p1);
-      ps0 += p0;
-      ps1 += p1;
-    }
-    pk[jj] = w;
+    for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+      for (int e = 0; e < 2; e++) {
+        const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kb][qb][2 * e], scale_log2, -m_use));
+        const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kb][qb][2 * e + 1], scale_log2, -m_use));
+        w[2 * kb + e] = pack2<F16>(p0, p1);
+        ps0 += p0;
+        ps1 += p1;
+      }
+    pk[qb] = w;
+    l_run[qb] = l_run[qb] * alpha[qb] + (ps0 + ps1);
   }
-  l_run = l_run * alpha + (ps0 + ps1);
   return any;
 }
 
@@ -221,7 +271,7 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int qc = lane & 31, g = lane >> 5;
+  const int qc = lane & 15, g = lane >> 4;  // query column within a 16-row block, lane group
 
   auto visible_keys = [&](int qpos) -> int {
     const int dq = qpos - kf;
@@ -237,25 +287,25 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
   const int ns_w = wave_has_rows ? (visible_keys(qf + m_wlast * P) + SUB - 1) / SUB : 0;
   const int i_mask = wave_has_rows ? visible_keys(qf + m_w0 * P) / SUB : 0;
 
-  // Q as B operands: qreg[t] = Q[row qc][16t + 8g .. +7]
-  u32x4 qreg[8];
-  {
-    const int m = m_w0 + qc;
+  // Q as B operands: qreg[qb][ks] = Q[row 16 qb + qc][32 ks + 8g .. +7]
+  u32x4 qreg[2][4];
+#pragma unroll
+  for (int qb = 0; qb < 2; qb++) {
+    const int m = m_w0 + 16 * qb + qc;
     const bool ok = m < q_len;
     const char* src = (const char*)p.q + ((q_start + (ok ? m : 0)) * p.q_st + (int64_t)h * p.q_sh + 8 * g) * 2;
 #pragma unroll
-    for (int t = 0; t < 8; t++) qreg[t] = ok ? *(const u32x4*)(src + t * 32) : u32x4{0, 0, 0, 0};
+    for (int ks = 0; ks < 4; ks++) qreg[qb][ks] = ok ? *(const u32x4*)(src + ks * 64) : u32x4{0, 0, 0, 0};
   }
 
   int koff0 = qc * 256 + ((g ^ swz_bits(qc)) << 4);
-  int voffa0, voffb0;
+  int voff0;
   {
-    const int blk16 = lane >> 4, li = lane & 15;
-    const int row_a = 4 * (blk16 >> 1) + (li >> 2);
-    const int row_b = row_a + 8;
-    const int d_off = (blk16 & 1) * 16 + 4 * (li & 3);
-    voffa0 = row_a * 256 + (((d_off >> 3) ^ swz_bits(row_a)) << 4) + (d_off & 7) * 2;
-    voffb0 = row_b * 256 + (((d_off >> 3) ^ swz_bits(row_b)) << 4) + (d_off & 7) * 2;
+    // a transposing read hands lane c of a 16-lane group column d0 + c of the 4 x 16 block its lanes point at:
+    // lane c points at row (c >> 2), columns d0 + 4 (c & 3) .. + 3
+    const int row = 4 * g + (qc >> 2);
+    const int d_off = 4 * (qc & 3);
+    voff0 = row * 256 + (((d_off >> 3) ^ swz_bits(row)) << 4) + (d_off & 7) * 2;
   }
   const int lds_base = (int)(uintptr_t)(__attribute__((address_space(3))) char*)lds;
 
@@ -346,40 +396,46 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
     vt_run += BN * v_row_bytes;
   };
 
-  f32x16 oacc[4];
+  // O^T accumulators: oacc[db][qb][r] = O[row 16 qb + qc][16 db + 4g + r]
+  f32x4 oacc[8][2];
 #pragma unroll
-  for (int db = 0; db < 4; db++)
+  for (int db = 0; db < 8; db++)
 #pragma unroll
-    for (int i = 0; i < 16; i++) oacc[db][i] = 0.f;
-  float m_run = -INFINITY, l_run = 0.f, alpha = 1.f;
-  f32x16 s;
+    for (int qb = 0; qb < 2; qb++) oacc[db][qb] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m_run[2] = {-INFINITY, -INFINITY}, l_run[2] = {0.f, 0.f}, alpha[2] = {1.f, 1.f};
+  f32x4 s[2][2];  // s[kb][qb][r] = S[row 16 qb + qc][key 16 kb + 4g + r of the sub-tile]
   u32x4 pk[2];
-  u32x4 ka[8], va[2][4];
-  const int qpos = qf + (m_w0 + qc) * P;
+  u32x4 ka[2][4], va[8];
+  const int qpos[2] = {qf + (m_w0 + qc) * P, qf + (m_w0 + 16 + qc) * P};
 
   // General step for sub-tile i: bounds-checked, masked, nothing carried over between steps.
   auto step = [&](int i) __attribute__((always_inline)) {
     if (i >= ns_w) return;  // no row of this wave sees a key of this sub-tile (wave-uniform)
     const int ksub = lds_base + ((i >> 1) & (kRing - 1)) * kTileBytes + (i & 1) * (SUB * 256);
-    asm volatile("" : "+v"(koff0), "+v"(voffa0), "+v"(voffb0));
+    asm volatile("" : "+v"(koff0), "+v"(voff0));
     load_k_operands(ksub, koff0, ka);
-    load_v_operands(ksub + kLdsV, voffa0, voffb0, va);
+    load_v_operands(ksub + kLdsV, voff0, va);
 #pragma unroll
-    for (int i2 = 0; i2 < 16; i2++) s[i2] = 0.f;
+    for (int kb = 0; kb < 2; kb++)
 #pragma unroll
-    for (int t8 = 0; t8 < 8; t8++) s = Mfma<T>::run(ka[t8], qreg[t8], s);
+      for (int qb = 0; qb < 2; qb++) s[kb][qb] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++)
+#pragma unroll
+      for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+        for (int qb = 0; qb < 2; qb++) s[kb][qb] = Mfma<T>::run(ka[kb][ks], qreg[qb][ks], s[kb][qb]);
     const bool any = softmax32<true>(s, pk, m_run, l_run, alpha, p.scale_log2, g, i * SUB, kv_len, kf, P, qpos);
     if (any) {
-      asm volatile("s_nop 15\n\ts_nop 7");  // inline assembly is outside the compiler's hazard bookkeeping
 #pragma unroll
-      for (int db = 0; db < 4; db++)
+      for (int db = 0; db < 8; db++)
 #pragma unroll
-        for (int i2 = 0; i2 < 16; i2++) asm volatile("v_mul_f32 %0, %1, %0" : "+v"(oacc[db][i2]) : "v"(alpha));
+        for (int qb = 0; qb < 2; qb++) oacc[db][qb] *= alpha[qb];
     }
 #pragma unroll
-    for (int jj = 0; jj < 2; jj++)
+    for (int db = 0; db < 8; db++)
 #pragma unroll
-      for (int db = 0; db < 4; db++) oacc[db] = Mfma<F16>::run(va[jj][db], pk[jj], oacc[db]);
+      for (int qb = 0; qb < 2; qb++) oacc[db][qb] = Mfma<F16>::run(va[db], pk[qb], oacc[db][qb]);
   };
   // Iteration `it` works on tile `it` (sub-tiles 2it, 2it+1) and issues the loads of K tile it+3 and
   // V tile it+2.  The wait in the middle leaves only this iteration's loads in flight, so the previous
@@ -397,9 +453,17 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
   // ring slot (it & 3 == R) is a compile-time constant, so every LDS read is a fixed register plus an
   // immediate.  A step has an MFMA phase (S(i) = K(i) Q^T, then O += V(i-1) P(i-1), each operand register
   // refilled for the next step right behind the MFMA that consumed it) and a softmax phase (P(i)).
-  // Running state in this form: neg_m = -m, thr_raw = (m + 2^kLazyRescale) / scale, l = l0 + l1.
-  int kaddr[8], vaddr_a[4], vaddr_b[4];
-  float neg_m = 0.f, thr_raw = 0.f, l0 = 0.f, l1 = 0.f, l2 = 0.f, l3 = 0.f;
+  // Running state in this form, per 16-row block qb: neg_m = -m, thr_raw = (m + 2^kLazyRescale) / scale,
+  // l = lacc[qb] (any element).
+  int kaddr[4], vaddr[8];
+  float neg_m[2] = {0.f, 0.f}, thr_raw[2] = {0.f, 0.f};
+  // row sums of P on the matrix pipe: lacc[qb] += ones(16 x 32) P^T, every element of a lane's lacc[qb] is the sum of
+  // its query column over all keys so far (of the fp16 P values, the ones that multiply V)
+  f32x4 lacc[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};
+  // (held in registers as an opaque value: rebuilt from constants next to the inline-assembly MFMAs it would be
+  // written by vector moves the compiler cannot order against them)
+  u32x4 ones = u32x4{0x3C003C00u, 0x3C003C00u, 0x3C003C00u, 0x3C003C00u};
+  asm volatile("" : "+v"(ones));
   const float scale = p.scale_log2, inv_scale = 1.f / p.scale_log2;
   auto fphase_mfma = [&](auto par_tag, auto r_tag) __attribute__((always_inline)) {
     constexpr int PAR = decltype(par_tag)::value;  // sub-tile i = 2it + PAR
@@ -407,100 +471,85 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
     constexpr int koff = (PAR ? ((R + 1) & 3) : R) * kTileBytes + (PAR ^ 1) * (SUB * 256);  // K sub-tile i+1
     constexpr int voff = R * kTileBytes + PAR * (SUB * 256);                               // V sub-tile i
 #pragma unroll
-    for (int i2 = 0; i2 < 16; i2++) s[i2] = 0.f;
+    for (int ks = 0; ks < 4; ks++)
 #pragma unroll
-    for (int t8 = 0; t8 < 8; t8++) {
-      s = Mfma<T>::run(ka[t8], qreg[t8], s);
-      ka[t8] = *(const __attribute__((address_space(3))) u32x4*)(kaddr[t8] + koff);
-    }
-#pragma unroll
-    for (int jj = 0; jj < 2; jj++)
-#pragma unroll
-      for (int db = 0; db < 4; db++) {
-        oacc[db] = Mfma<F16>::run(va[jj][db], pk[jj], oacc[db]);
-        const i16x4 xa = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_ptr)(vaddr_a[db] + voff + jj * (16 * 256)));
-        const i16x4 xb = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_ptr)(vaddr_b[db] + voff + jj * (16 * 256)));
-        const u32x2 wa = __builtin_bit_cast(u32x2, xa), wb = __builtin_bit_cast(u32x2, xb);
-        va[jj][db] = u32x4{wa[0], wa[1], wb[0], wb[1]};
+      for (int kb = 0; kb < 2; kb++) {
+        if (ks == 0) {
+          MfmaAsm<T>::first(s[kb][0], ka[kb][ks], qreg[0][ks]);
+          MfmaAsm<T>::first(s[kb][1], ka[kb][ks], qreg[1][ks]);
+        } else {
+          MfmaAsm<T>::acc(s[kb][0], ka[kb][ks], qreg[0][ks]);
+          MfmaAsm<T>::acc(s[kb][1], ka[kb][ks], qreg[1][ks]);
+        }
+        ka[kb][ks] = *(const __attribute__((address_space(3))) u32x4*)(kaddr[ks] + koff + kb * (16 * 256));
+        __builtin_amdgcn_sched_barrier(0);
       }
 #pragma unroll
-    for (int t8 = 0; t8 < 8; t8++) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    for (int db = 0; db < 8; db++) {
+      MfmaAsm<F16>::acc(oacc[db][0], va[db], pk[0]);
+      MfmaAsm<F16>::acc(oacc[db][1], va[db], pk[1]);
+      const i16x4 xa = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_ptr)(vaddr[db] + voff));
+      const i16x4 xb = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_ptr)(vaddr[db] + voff + 16 * 256));
+      const u32x2 wa = __builtin_bit_cast(u32x2, xa), wb = __builtin_bit_cast(u32x2, xb);
+      va[db] = u32x4{wa[0], wa[1], wb[0], wb[1]};
+      __builtin_amdgcn_sched_barrier(0);
     }
-#pragma unroll
-    for (int t8 = 0; t8 < 8; t8++) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-    }
+    MfmaAsm<F16>::acc(lacc[0], ones, pk[0]);
+    MfmaAsm<F16>::acc(lacc[1], ones, pk[1]);
     __builtin_amdgcn_sched_barrier(0);
   };
-  // P(i) = exp2(S(i) * scale - m) with the current m, the sub-tile's row sums in d[0..3] and the lane's
-  // largest score as the result.  Stage by stage, sixteen independent operations at a time, the levels of
-  // the maximum's tree spread between them, plain fp32 adds for the sums: this wave's vector work runs
-  // beside the other wave's MFMAs only without short dependent chains and without dot-product
-  // instructions (those queue behind the MFMAs).
-  auto compute_p = [&](float (&d)[4]) __attribute__((always_inline)) -> float {
-    float m6[6], t[16];
-    // maximum of the sixteen scores as a tree of three-input maxima: 5 + 2 + 1 operations
+  // P(i) = exp2(S(i) * scale - m) with the current m, and the lane's largest score of each block in mx[qb].  Sixteen
+  // independent operations at a time, the levels of the maxima's trees spread between them: this wave's vector work
+  // runs beside the other wave's MFMAs only without short dependent chains and without dot-product instructions
+  // (those queue behind the MFMAs).
+  auto compute_p = [&](float (&mx)[2]) __attribute__((always_inline)) {
+    float ma[2], mb[2], t[2][8];
 #pragma unroll
-    for (int i = 0; i < 5; i++) m6[i] = fmaxf(fmaxf(s[3 * i], s[3 * i + 1]), s[3 * i + 2]);
-    m6[5] = s[15];
+    for (int qb = 0; qb < 2; qb++) {
+      ma[qb] = max3_raw(s[0][qb][0], s[0][qb][1], s[0][qb][2]);
+      mb[qb] = max3_raw(s[0][qb][3], s[1][qb][0], s[1][qb][1]);
+    }
 #pragma unroll
-    for (int i = 0; i < 16; i++) t[i] = __builtin_fmaf(s[i], scale, neg_m);
-    __builtin_amdgcn_sched_barrier(0);
-    m6[0] = fmaxf(fmaxf(m6[0], m6[1]), m6[2]);
-    m6[3] = fmaxf(fmaxf(m6[3], m6[4]), m6[5]);
+    for (int qb = 0; qb < 2; qb++)
 #pragma unroll
-    for (int i = 0; i < 16; i++) t[i] = __builtin_amdgcn_exp2f(t[i]);
-    __builtin_amdgcn_sched_barrier(0);
-    const float mx = fmaxf(m6[0], m6[3]);
+      for (int kb = 0; kb < 2; kb++)
 #pragma unroll
-    for (int i = 0; i < 4; i++) d[i] = t[i] + t[i + 4];
+        for (int r = 0; r < 4; r++) t[qb][4 * kb + r] = __builtin_fmaf(s[kb][qb][r], scale, neg_m[qb]);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int i = 0; i < 4; i++) d[i] += t[i + 8];
+    for (int qb = 0; qb < 2; qb++) ma[qb] = max3_raw(ma[qb], s[1][qb][2], s[1][qb][3]);
+#pragma unroll
+    for (int qb = 0; qb < 2; qb++)
+#pragma unroll
+      for (int i = 0; i < 8; i++) t[qb][i] = __builtin_amdgcn_exp2f(t[qb][i]);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int i = 0; i < 4; i++) d[i] += t[i + 12];
+    for (int qb = 0; qb < 2; qb++) mx[qb] = max_raw(ma[qb], mb[qb]);
 #pragma unroll
-    for (int jj = 0; jj < 2; jj++)
+    for (int qb = 0; qb < 2; qb++)
 #pragma unroll
-      for (int e = 0; e < 4; e++) pk[jj][e] = pack2<F16>(t[8 * jj + 2 * e], t[8 * jj + 2 * e + 1]);
+      for (int e = 0; e < 4; e++) pk[qb][e] = pack2<F16>(t[qb][2 * e], t[qb][2 * e + 1]);
     __builtin_amdgcn_sched_barrier(0);
-    return mx;
   };
   auto fphase_softmax = [&]() __attribute__((always_inline)) {
-    float d[4];
-    float mx = compute_p(d);
-    if (__builtin_amdgcn_ballot_w64(mx > thr_raw) != 0) {
-      // rare: some score is above the lazy threshold; raise the running maximum and redo the sub-tile
-      {
-        const unsigned u = __builtin_bit_cast(unsigned, mx);
-        auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
-        mx = fmaxf(__builtin_bit_cast(float, r[0]), __builtin_bit_cast(float, r[1]));
+    float mx[2];
+    compute_p(mx);
+    if (__builtin_amdgcn_ballot_w64((mx[0] > thr_raw[0]) | (mx[1] > thr_raw[1])) != 0) {
+      // rare: some score is above the lazy threshold; raise the running maxima and redo the sub-tile
+      // (the accumulators' last MFMAs were issued before this phase's barrier and the whole of compute_p lies
+      // between them and these multiplies)
+#pragma unroll
+      for (int qb = 0; qb < 2; qb++) {
+        const float m_new = fminf(neg_m[qb], -column_max(mx[qb]) * scale);  // -max(m, mx*scale)
+        const float al = __builtin_amdgcn_exp2f(m_new - neg_m[qb]);
+        neg_m[qb] = m_new;
+        thr_raw[qb] = (kLazyRescale - m_new) * inv_scale;
+        lacc[qb] *= al;
+#pragma unroll
+        for (int db = 0; db < 8; db++) oacc[db][qb] *= al;
       }
-      const float m_new = fminf(neg_m, -mx * scale);  // -max(m, mx*scale)
-      const float al = __builtin_amdgcn_exp2f(m_new - neg_m);
-      neg_m = m_new;
-      thr_raw = (kLazyRescale - m_new) * inv_scale;
-      // inline assembly is outside the compiler's hazard bookkeeping: the factor comes from a
-      // transcendental op and the accumulators from MFMAs that may still be in flight
-      asm volatile("s_nop 15\n\ts_nop 7");
-      asm volatile("v_mul_f32 %0, %1, %0" : "+v"(l0) : "v"(al));
-      asm volatile("v_mul_f32 %0, %1, %0" : "+v"(l1) : "v"(al));
-      asm volatile("v_mul_f32 %0, %1, %0" : "+v"(l2) : "v"(al));
-      asm volatile("v_mul_f32 %0, %1, %0" : "+v"(l3) : "v"(al));
-#pragma unroll
-      for (int db = 0; db < 4; db++)
-#pragma unroll
-        for (int i2 = 0; i2 < 16; i2++) asm volatile("v_mul_f32 %0, %1, %0" : "+v"(oacc[db][i2]) : "v"(al));
-      compute_p(d);
+      compute_p(mx);
     }
-    l0 += d[0];
-    l1 += d[1];
-    l2 += d[2];
-    l3 += d[3];
     __builtin_amdgcn_sched_barrier(0);
   };
   // The two waves that share a SIMD (w and w + 4) run the fast loop half a step apart, one in its MFMA
@@ -545,22 +594,21 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
     int it = 0;
     if (fast_end >= 4) {
 #pragma unroll
-      for (int t8 = 0; t8 < 8; t8++) {
-        kaddr[t8] = (lds_base + koff0) ^ (t8 << 5);
-        asm volatile("" : "+v"(kaddr[t8]));
+      for (int ks = 0; ks < 4; ks++) {
+        kaddr[ks] = (lds_base + koff0) ^ (ks << 6);
+        asm volatile("" : "+v"(kaddr[ks]));
       }
 #pragma unroll
-      for (int db = 0; db < 4; db++) {
-        vaddr_a[db] = (lds_base + kLdsV + voffa0) ^ (db << 6);
-        vaddr_b[db] = (lds_base + kLdsV + voffb0) ^ (db << 6);
-        asm volatile("" : "+v"(vaddr_a[db]), "+v"(vaddr_b[db]));
+      for (int db = 0; db < 8; db++) {
+        vaddr[db] = (lds_base + kLdsV + voff0) ^ (db << 5);
+        asm volatile("" : "+v"(vaddr[db]));
       }
-      neg_m = INFINITY;
-      thr_raw = -INFINITY;
+      neg_m[0] = neg_m[1] = INFINITY;
+      thr_raw[0] = thr_raw[1] = -INFINITY;
       __syncthreads();
       // operands of step 0; its "previous" product is V(tile 0) times a zero P
       load_k_operands(lds_base, koff0, ka);
-      load_v_operands(lds_base + kLdsV, voffa0, voffb0, va);
+      load_v_operands(lds_base + kLdsV, voff0, va);
       pk[0] = u32x4{0, 0, 0, 0};
       pk[1] = u32x4{0, 0, 0, 0};
       kt_run = uniform_ptr(kg + (int64_t)3 * BN * k_row_bytes);
@@ -575,65 +623,61 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
       if (wave < 4) __builtin_amdgcn_s_barrier();
       // the product of the last fast step is still owed
 #pragma unroll
-      for (int jj = 0; jj < 2; jj++)
+      for (int db = 0; db < 8; db++)
 #pragma unroll
-        for (int db = 0; db < 4; db++) oacc[db] = Mfma<F16>::run(va[jj][db], pk[jj], oacc[db]);
-      m_run = -neg_m;
-      l_run = (l0 + l1) + (l2 + l3);
+        for (int qb = 0; qb < 2; qb++) oacc[db][qb] = Mfma<F16>::run(va[db], pk[qb], oacc[db][qb]);
+#pragma unroll
+      for (int qb = 0; qb < 2; qb++) {
+        lacc[qb] = Mfma<F16>::run(ones, pk[qb], lacc[qb]);
+        m_run[qb] = -neg_m[qb];
+        l_run[qb] = g == 0 ? lacc[qb][0] : 0.f;  // the general steps keep per-lane partial sums, added up over the column at the end
+      }
     }
     for (; it < nt; it++) iteration(it);
   }
 
   // ---- epilogue ----
-  {
-    const int m = m_w0 + qc;
-    const float l_tot = l_run + other_half(l_run, g);
+#pragma unroll
+  for (int qb = 0; qb < 2; qb++) {
+    const int m = m_w0 + 16 * qb + qc;
+    const float l_tot = column_sum(l_run[qb]);
     if (m < q_len) {
       const int64_t tok = q_start + m;
       if (MODE == 0) {
         const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
         float* orow = (float*)p.o + tok * p.o_st + (int64_t)h * p.o_sh;
 #pragma unroll
-        for (int db = 0; db < 4; db++)
-#pragma unroll
-          for (int i4 = 0; i4 < 4; i4++) {
-            const int d = db * 32 + i4 * 8 + 4 * g;
-            const f32x4 v = {oacc[db][i4 * 4 + 0] * inv, oacc[db][i4 * 4 + 1] * inv, oacc[db][i4 * 4 + 2] * inv, oacc[db][i4 * 4 + 3] * inv};
-            *(f32x4*)(orow + d) = v;
-          }
-        if (g == 0) p.lse[tok * p.hq + h] = l_tot > 0.f ? (m_run + __builtin_amdgcn_logf(l_tot)) * kLn2 : -INFINITY;
+        for (int db = 0; db < 8; db++) *(f32x4*)(orow + db * 16 + 4 * g) = oacc[db][qb] * inv;
+        if (g == 0) p.lse[tok * p.hq + h] = l_tot > 0.f ? (m_run[qb] + __builtin_amdgcn_logf(l_tot)) * kLn2 : -INFINITY;
       } else {
         float* mp = p.m + tok * p.ml_st + (int64_t)h * p.ml_sh;
         float* lp = p.l + tok * p.ml_st + (int64_t)h * p.ml_sh;
         const float m_old = *mp, l_old = *lp;
-        const float M = fmaxf(m_run, m_old);
+        const float M = fmaxf(m_run[qb], m_old);
         if (M != -INFINITY && l_tot > 0.f) {
           const float w_old = l_old * exp2_diff(m_old, M);
-          const float w_new = exp2_diff(m_run, M);
+          const float w_new = exp2_diff(m_run[qb], M);
           const float L = w_old + l_tot * w_new;
           const float inv = 1.f / L;
           uint16_t* orow = (uint16_t*)p.o + tok * p.o_st + (int64_t)h * p.o_sh;
 #pragma unroll
-          for (int db = 0; db < 4; db++)
-#pragma unroll
-            for (int i4 = 0; i4 < 4; i4++) {
-              const int d = db * 32 + i4 * 8 + 4 * g;
-              u32x2* dst = (u32x2*)(orow + d);
-              float o0, o1, o2, o3;
-              if (w_old != 0.f) {
-                const u32x2 old = *dst;
-                unpack2<T>(old[0], o0, o1);
-                unpack2<T>(old[1], o2, o3);
-              } else {
-                o0 = o1 = o2 = o3 = 0.f;
-              }
-              const float r0 = (o0 * w_old + oacc[db][i4 * 4 + 0] * w_new) * inv;
-              const float r1 = (o1 * w_old + oacc[db][i4 * 4 + 1] * w_new) * inv;
-              const float r2 = (o2 * w_old + oacc[db][i4 * 4 + 2] * w_new) * inv;
-              const float r3 = (o3 * w_old + oacc[db][i4 * 4 + 3] * w_new) * inv;
-              *dst = u32x2{pack2<T>(r0, r1), pack2<T>(r2, r3)};
+          for (int db = 0; db < 8; db++) {
+            u32x2* dst = (u32x2*)(orow + db * 16 + 4 * g);
+            float o0, o1, o2, o3;
+            if (w_old != 0.f) {
+              const u32x2 old = *dst;
+              unpack2<T>(old[0], o0, o1);
+              unpack2<T>(old[1], o2, o3);
+            } else {
+              o0 = o1 = o2 = o3 = 0.f;
             }
-          if (g == 0) {
+            const float r0 = (o0 * w_old + oacc[db][qb][0] * w_new) * inv;
+            const float r1 = (o1 * w_old + oacc[db][qb][1] * w_new) * inv;
+            const float r2 = (o2 * w_old + oacc[db][qb][2] * w_new) * inv;
+            const float r3 = (o3 * w_old + oacc[db][qb][3] * w_new) * inv;
+            *dst = u32x2{pack2<T>(r0, r1), pack2<T>(r2, r3)};
+          }
+          if (g == 0) {  // M and L depend on the old state every lane of the column has loaded by now
             *mp = M;
             *lp = L;
           }
