@@ -102,14 +102,14 @@ template <> struct MfmaAsm<BF16> {
 template <typename T> __device__ __forceinline__ u32x4 to_pv_operand(const u32x4& w);
 template <> __device__ __forceinline__ u32x4 to_pv_operand<F16>(const u32x4& w) { return w; }
 template <> __device__ __forceinline__ u32x4 to_pv_operand<BF16>(const u32x4& w) {
+  // round-toward-zero conversion: exact for every bfloat16 in fp16's normal range, and a magnitude above 65504
+  // becomes +-65504 without a separate clamp
   u32x4 r;
 #pragma unroll
   for (int i = 0; i < 4; i++) {
     float lo, hi;
     unpack2<BF16>(w[i], lo, hi);
-    lo = __builtin_amdgcn_fmed3f(lo, -65504.f, 65504.f);
-    hi = __builtin_amdgcn_fmed3f(hi, -65504.f, 65504.f);
-    r[i] = pack2<F16>(lo, hi);
+    r[i] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(lo, hi));
   }
   return r;
 }
@@ -389,10 +389,17 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
       asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(st_lds + kslot + i * 1024), "v"(k_lane_off[i]), "s"(kt_run) : "m0", "memory");
       if (DirectV<T>::value)
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(st_lds + vslot + i * 1024), "v"(v_lane_off[i]), "s"(vt_run) : "m0", "memory");
-      else  // the compiler does not see this load: fast_iteration waits for it before it stores the tile
-        asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(vst[i]) : "v"(v_lane_off[i]), "s"(vt_run) : "memory");
     }
     kt_run += BN * k_row_bytes;
+    if (DirectV<T>::value) vt_run += BN * v_row_bytes;
+  };
+  // A V tile that has to be converted on its way into LDS goes through registers: loaded one iteration before it is
+  // stored (three tiles ahead of its use), so the wait in front of the store is for loads a whole iteration old.
+  // The compiler does not see these loads: fast_iteration waits for them before it stores the tile.
+  auto load_v_regs_fast = [&]() __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+      asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(vst[i]) : "v"(v_lane_off[i]), "s"(vt_run) : "memory");
     vt_run += BN * v_row_bytes;
   };
 
@@ -571,8 +578,13 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_s_setprio(3);
     fphase_softmax();
-    if (!DirectV<T>::value) asm volatile("s_waitcnt vmcnt(0)" : "+v"(vst[0]), "+v"(vst[1]));
-    store_v_tile(it + 2);
+    if (!DirectV<T>::value) {
+      // everything but this iteration's two K loads has arrived: the registers hold V tile it+2, and K tile it+2
+      // (loaded one iteration ago) is complete as well
+      asm volatile("s_waitcnt vmcnt(2)" : "+v"(vst[0]), "+v"(vst[1]));
+      store_v_tile(it + 2);
+      load_v_regs_fast();  // V tile it+3
+    }
     __builtin_amdgcn_s_setprio(0);
     __builtin_amdgcn_s_barrier();
   };
@@ -613,6 +625,7 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
       pk[1] = u32x4{0, 0, 0, 0};
       kt_run = uniform_ptr(kg + (int64_t)3 * BN * k_row_bytes);
       vt_run = uniform_ptr(vg + (int64_t)2 * BN * v_row_bytes);
+      if (!DirectV<T>::value) load_v_regs_fast();  // V tile 2
       if (wave >= 4) __builtin_amdgcn_s_barrier();
       for (; it + 3 < fast_end; it += 4) {
         fast_iteration(std::integral_constant<int, 0>{}, it);
@@ -621,6 +634,9 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
         fast_iteration(std::integral_constant<int, 3>{}, it + 3);
       }
       if (wave < 4) __builtin_amdgcn_s_barrier();
+      // (a V tile loaded ahead is dropped: the general steps load what they need themselves; its loads must have
+      // landed before the registers are used for anything else)
+      if (!DirectV<T>::value) asm volatile("s_waitcnt vmcnt(0)" : "+v"(vst[0]), "+v"(vst[1]));
       // the product of the last fast step is still owed
 #pragma unroll
       for (int db = 0; db < 8; db++)
