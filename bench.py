@@ -479,7 +479,7 @@ def main():
                          "frac": ach / PEAK_MFMA_TFLOPS,
                          # HBM bytes per launch (read 772.8 MB + written 509.6 MB), rocprofv3 FETCH_SIZE / WRITE_SIZE scaled by a
                          # plain copy: profiles/bench_default_hbm_traffic.txt
-                         "traffic": 1064.4e6,
+                         "traffic": 1107.8e6,
                          "per_launch_ms": per_launch_ms, "algorithmic_tflop_per_launch": w.flops / w.launches / 1e12},
         })
         if not args.no_cpu:
