@@ -76,7 +76,9 @@ typedef struct lsattn_prefill_args {
   void* o;            /* [Tq,Hq,D] */
   int64_t o_stride_t, o_stride_h;
   int32_t o_dtype;    /* step: LSATTN_F32; step_merge: same as dtype */
-  int32_t reserved;
+  int32_t v_is_f16;   /* 0: v has `dtype`.  1 (dtype LSATTN_BF16 only): v already holds fp16, e.g. written by
+                         lsattn_bf16_to_f16_rows: the P V product runs in fp16 either way, and a bf16 V converted
+                         inside the kernel costs about 15 % of its speed */
   float* lse;         /* step: [Tq,Hq] natural-log LSE, contiguous         */
   float* m;           /* step_merge: [Tq,Hq] running max, log2 domain       */
   float* l;           /* step_merge: [Tq,Hq] running sum                    */
@@ -328,6 +330,15 @@ int lsattn_pool_find_contiguous(const int32_t* mem_state, int64_t pool_size, int
 size_t lsattn_pool_refs_workspace_bytes(int64_t n);
 int lsattn_pool_update_refs(int32_t* mem_state, int64_t pool_size, const int64_t* index, int64_t n, int delta,
                             int64_t* counted, void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * dst[r, 0:row_elems] = fp16(src[r, 0:row_elems]) for r < n_rows, bf16 -> fp16 rounded toward zero (exact for every
+ * bf16 in fp16's normal range; larger magnitudes become +-65504).  Strides in elements; row_elems, strides % 8 == 0,
+ * pointers 16-byte aligned.  No counterpart in the reference (its kernels are fp16 only): prepares V for
+ * lsattn_prefill_step* with v_is_f16 = 1.
+ */
+int lsattn_bf16_to_f16_rows(const void* src, int64_t src_stride, void* dst, int64_t dst_stride, int64_t n_rows,
+                            int64_t row_elems, void* stream);
 
 const char* lsattn_strerror(int code);
 int lsattn_version(void);

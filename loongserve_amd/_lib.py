@@ -30,7 +30,7 @@ class PrefillArgs(C.Structure):
         ("batch", _i32), ("num_q_heads", _i32), ("num_kv_heads", _i32), ("head_dim", _i32),
         ("dtype", _i32), ("sp_peers", _i32), ("max_q_len", _i32), ("sm_scale", _f32),
         ("o", _vp), ("o_stride_t", _i64), ("o_stride_h", _i64),
-        ("o_dtype", _i32), ("reserved", _i32),
+        ("o_dtype", _i32), ("v_is_f16", _i32),
         ("lse", _vp), ("m", _vp), ("l", _vp),
         ("ml_stride_t", _i64), ("ml_stride_h", _i64),
     ]
@@ -102,6 +102,7 @@ EXPORTS = {
     "lsattn_pool_find_contiguous": (C.c_int, [_vp, _i64, _i64, _vp, _vp, C.c_size_t, _vp]),
     "lsattn_pool_refs_workspace_bytes": (C.c_size_t, [_i64]),
     "lsattn_pool_update_refs": (C.c_int, [_vp, _i64, _vp, _i64, C.c_int, _vp, _vp, C.c_size_t, _vp]),
+    "lsattn_bf16_to_f16_rows": (C.c_int, [_vp, _i64, _vp, _i64, _i64, _i64, _vp]),
     "lsattn_strerror": (C.c_char_p, [C.c_int]),
     "lsattn_version": (C.c_int, []),
 }

@@ -132,9 +132,44 @@ __global__ __launch_bounds__(256) void rotary_emb_kernel(uint16_t* __restrict__ 
   *p2 = n2;
 }
 
+// ---------------------------------------------------------------------------------------------------
+// bf16 -> fp16 row copy, rounded toward zero (exact inside fp16's normal range, +-65504 beyond it): prepares a bf16 V
+// for the prefill kernel, whose P V product runs in fp16.  One 16-byte piece per lane.
+// ---------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void bf16_to_f16_rows_kernel(const uint16_t* __restrict__ src, int64_t src_stride,
+                                                               uint16_t* __restrict__ dst, int64_t dst_stride, int64_t n_rows,
+                                                               int64_t pieces_per_row) {
+  const int64_t gid = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (gid >= n_rows * pieces_per_row) return;
+  const int64_t r = gid / pieces_per_row, c = gid % pieces_per_row;
+  const u32x4 w = *((const u32x4*)(src + r * src_stride) + c);
+  u32x4 o;
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    float lo, hi;
+    unpack2<BF16>(w[i], lo, hi);
+    o[i] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(lo, hi));
+  }
+  *((u32x4*)(dst + r * dst_stride) + c) = o;
+}
+
 }  // namespace lsattn
 
 using namespace lsattn;
+
+extern "C" int lsattn_bf16_to_f16_rows(const void* src, int64_t src_stride, void* dst, int64_t dst_stride, int64_t n_rows,
+                                       int64_t row_elems, void* stream) {
+  if (!src || !dst || n_rows < 0 || row_elems <= 0) return LSATTN_ERR_INVALID_ARG;
+  if (row_elems % 8 || src_stride % 8 || dst_stride % 8 || src_stride < row_elems || dst_stride < row_elems ||
+      (((uintptr_t)src | (uintptr_t)dst) & 15))
+    return LSATTN_ERR_INVALID_ARG;
+  if (n_rows == 0) return LSATTN_OK;
+  const int64_t blocks = (n_rows * (row_elems / 8) + 255) / 256;
+  if (blocks > 0x7fffffff) return LSATTN_ERR_INVALID_ARG;
+  hipLaunchKernelGGL(bf16_to_f16_rows_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (const uint16_t*)src,
+                     src_stride, (uint16_t*)dst, dst_stride, n_rows, row_elems / 8);
+  return check_launch();
+}
 
 extern "C" int lsattn_rms_norm(void* out, const void* in, const void* weight, int64_t num_tokens, int64_t hidden_size,
                                float eps, void* stream) {

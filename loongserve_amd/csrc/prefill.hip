@@ -18,11 +18,11 @@
 //     any cross-lane movement (P and V always as fp16);
 //   * V^T operands come from LDS through ds_read_b64_tr_b16 (the tile is stored row-major);
 //   * on this hardware an MFMA holds its own wave until it is done, and vector work of the
-//     SIMD's other wave runs beside it only under conditions (higher wave priority, no short
-//     dependent chains, no dot-product instructions).  The fully visible part of the key range
-//     therefore runs as alternating phases: one wave of the SIMD issues the thirty-two MFMAs of a
-//     32-key step while the other does the exponentials of its own step, a workgroup barrier
-//     ends each phase;
+//     SIMD's other wave runs beside it only under conditions (no short dependent chains, no
+//     dot-product instructions) and, beside MFMAs of this shape, about a third slower.  The fully visible part of the key range
+//     therefore runs as alternating phases: one wave of the SIMD issues the thirty-four MFMAs of a
+//     32-key step (scores, P V, and the row sums of P as a product with a matrix of ones) while the
+//     other does the exponentials of its own step, a workgroup barrier ends each phase;
 //   * tiles that straddle the diagonal or the end of the KV chunk take a general, masked,
 //     bounds-checked step; causal work is skipped per wave;
 //   * workgroup ids are mapped so that the workgroups sharing one KV head run on one XCD
@@ -113,8 +113,6 @@ template <> __device__ __forceinline__ u32x4 to_pv_operand<BF16>(const u32x4& w)
   }
   return r;
 }
-template <typename T> struct DirectV { static constexpr bool value = true; };
-template <> struct DirectV<BF16> { static constexpr bool value = false; };
 
 // Maxima on values that come out of inline-assembly MFMAs: through the fmaxf builtin the compiler first quiets
 // possible signalling NaNs (one more instruction per input), which these accumulators never hold.
@@ -243,7 +241,9 @@ __device__ __forceinline__ bool softmax32(f32x4 (&s)[2][2], u32x4 (&pk)[2], floa
   return any;
 }
 
-template <typename T, int MODE>
+// DV: the V tiles are fp16 in memory and go straight into LDS; otherwise (bf16 V) they pass through registers and are
+// converted on the way.
+template <typename T, int MODE, bool DV>
 __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p) {
   __shared__ __attribute__((aligned(1024))) char lds[kLdsBytes];
 
@@ -354,14 +354,14 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
         // vmcnt(0) before every later LDS read (it cannot tell which LDS bytes the load writes);
         // the waits for these loads are the explicit wait_vmem calls
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_base + kdst), "v"(ksrc) : "m0");
-        if (DirectV<T>::value)
+        if (DV)
           asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_base + vdst), "v"(vsrc) : "m0");
         else
           vst[i] = *(const u32x4*)vsrc;
         continue;
       }
       __builtin_amdgcn_global_load_lds((global_void_ptr)ksrc, (lds_void_ptr)(lds + kdst), 16, 0, 0);
-      if (DirectV<T>::value) {
+      if (DV) {
         __builtin_amdgcn_global_load_lds((global_void_ptr)vsrc, (lds_void_ptr)(lds + vdst), 16, 0, 0);
       } else {
         vst[i] = *(const u32x4*)vsrc;
@@ -369,7 +369,7 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
     }
   };
   auto store_v_tile = [&](int tv) __attribute__((always_inline)) {
-    if (!DirectV<T>::value) {
+    if (!DV) {
 #pragma unroll
       for (int i = 0; i < 2; i++)
         *(u32x4*)(lds + kLdsV + (tv & (kRing - 1)) * kTileBytes + (8 * wave + 4 * i) * 256 + lane * 16) = to_pv_operand<T>(vst[i]);
@@ -387,11 +387,11 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
 #pragma unroll
     for (int i = 0; i < 2; i++) {
       asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(st_lds + kslot + i * 1024), "v"(k_lane_off[i]), "s"(kt_run) : "m0", "memory");
-      if (DirectV<T>::value)
+      if (DV)
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(st_lds + vslot + i * 1024), "v"(v_lane_off[i]), "s"(vt_run) : "m0", "memory");
     }
     kt_run += BN * k_row_bytes;
-    if (DirectV<T>::value) vt_run += BN * v_row_bytes;
+    if (DV) vt_run += BN * v_row_bytes;
   };
   // A V tile that has to be converted on its way into LDS goes through registers: loaded one iteration before it is
   // stored (three tiles ahead of its use), so the wait in front of the store is for loads a whole iteration old.
@@ -432,7 +432,9 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
       for (int kb = 0; kb < 2; kb++)
 #pragma unroll
         for (int qb = 0; qb < 2; qb++) s[kb][qb] = Mfma<T>::run(ka[kb][ks], qreg[qb][ks], s[kb][qb]);
-    const bool any = softmax32<true>(s, pk, m_run, l_run, alpha, p.scale_log2, g, i * SUB, kv_len, kf, P, qpos);
+    // sub-tiles below i_mask are visible to the first row of the wave, hence to all of them: no mask to compute
+    const bool any = i < i_mask ? softmax32<false>(s, pk, m_run, l_run, alpha, p.scale_log2, g, i * SUB, kv_len, kf, P, qpos)
+                                : softmax32<true>(s, pk, m_run, l_run, alpha, p.scale_log2, g, i * SUB, kv_len, kf, P, qpos);
     if (any) {
 #pragma unroll
       for (int db = 0; db < 8; db++)
@@ -451,7 +453,7 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
     __syncthreads();
     load_tiles(std::false_type{}, it + 3, it + 2);
     step(2 * it);
-    if (DirectV<T>::value) wait_vmem<4>();
+    if (DV) wait_vmem<4>();
     step(2 * it + 1);
     store_v_tile(it + 2);
   };
@@ -573,12 +575,12 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
     fphase_softmax();
     __builtin_amdgcn_s_setprio(0);
     __builtin_amdgcn_s_barrier();
-    if (DirectV<T>::value) wait_vmem<4>();
+    if (DV) wait_vmem<4>();
     fphase_mfma(std::integral_constant<int, 1>{}, r_tag);
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_s_setprio(3);
     fphase_softmax();
-    if (!DirectV<T>::value) {
+    if (!DV) {
       // everything but this iteration's two K loads has arrived: the registers hold V tile it+2, and K tile it+2
       // (loaded one iteration ago) is complete as well
       asm volatile("s_waitcnt vmcnt(2)" : "+v"(vst[0]), "+v"(vst[1]));
@@ -625,7 +627,7 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
       pk[1] = u32x4{0, 0, 0, 0};
       kt_run = uniform_ptr(kg + (int64_t)3 * BN * k_row_bytes);
       vt_run = uniform_ptr(vg + (int64_t)2 * BN * v_row_bytes);
-      if (!DirectV<T>::value) load_v_regs_fast();  // V tile 2
+      if (!DV) load_v_regs_fast();  // V tile 2
       if (wave >= 4) __builtin_amdgcn_s_barrier();
       for (; it + 3 < fast_end; it += 4) {
         fast_iteration(std::integral_constant<int, 0>{}, it);
@@ -636,7 +638,7 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
       if (wave < 4) __builtin_amdgcn_s_barrier();
       // (a V tile loaded ahead is dropped: the general steps load what they need themselves; its loads must have
       // landed before the registers are used for anything else)
-      if (!DirectV<T>::value) asm volatile("s_waitcnt vmcnt(0)" : "+v"(vst[0]), "+v"(vst[1]));
+      if (!DV) asm volatile("s_waitcnt vmcnt(0)" : "+v"(vst[0]), "+v"(vst[1]));
       // the product of the last fast step is still owed
 #pragma unroll
       for (int db = 0; db < 8; db++)
@@ -703,7 +705,7 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
   }
 }
 
-template <typename T, int MODE> static int launch_prefill(const lsattn_prefill_args* a, hipStream_t st) {
+template <typename T, int MODE, bool DV> static int launch_prefill(const lsattn_prefill_args* a, hipStream_t st) {
   PrefillParams p;
   p.q = a->q;
   p.k = a->k;
@@ -738,7 +740,7 @@ template <typename T, int MODE> static int launch_prefill(const lsattn_prefill_a
   const int group = a->num_q_heads / a->num_kv_heads;
   const int64_t wgs = (int64_t)8 * group * p.nz * p.kv_slots * a->batch;
   if (wgs > 0x7fffffff) return LSATTN_ERR_INVALID_ARG;
-  hipLaunchKernelGGL((prefill_kernel<T, MODE>), dim3((unsigned)wgs), dim3(NWAVE * 64), 0, st, p);
+  hipLaunchKernelGGL((prefill_kernel<T, MODE, DV>), dim3((unsigned)wgs), dim3(NWAVE * 64), 0, st, p);
   return check_launch();
 }
 
@@ -752,6 +754,7 @@ static int validate(const lsattn_prefill_args* a, int mode) {
   if (a->num_q_heads % a->num_kv_heads) return LSATTN_ERR_INVALID_ARG;
   if (a->head_dim != 128) return LSATTN_ERR_UNSUPPORTED;
   if (a->dtype != LSATTN_F16 && a->dtype != LSATTN_BF16) return LSATTN_ERR_UNSUPPORTED;
+  if (a->v_is_f16 != 0 && (a->v_is_f16 != 1 || a->dtype != LSATTN_BF16)) return LSATTN_ERR_INVALID_ARG;
   // 16-byte operand loads / 8- or 16-byte output stores
   if (a->q_stride_t % 8 || a->q_stride_h % 8 || a->k_stride_t % 8 || a->k_stride_h % 8 || a->v_stride_t % 8 || a->v_stride_h % 8)
     return LSATTN_ERR_INVALID_ARG;
@@ -773,12 +776,14 @@ extern "C" int lsattn_prefill_step(const lsattn_prefill_args* a, void* stream) {
   const int rc = validate(a, 0);
   if (rc != LSATTN_OK) return rc;
   if (a->batch == 0 || a->max_q_len == 0) return LSATTN_OK;
-  return a->dtype == LSATTN_F16 ? launch_prefill<F16, 0>(a, (hipStream_t)stream) : launch_prefill<BF16, 0>(a, (hipStream_t)stream);
+  if (a->dtype == LSATTN_F16) return launch_prefill<F16, 0, true>(a, (hipStream_t)stream);
+  return a->v_is_f16 ? launch_prefill<BF16, 0, true>(a, (hipStream_t)stream) : launch_prefill<BF16, 0, false>(a, (hipStream_t)stream);
 }
 
 extern "C" int lsattn_prefill_step_merge(const lsattn_prefill_args* a, void* stream) {
   const int rc = validate(a, 1);
   if (rc != LSATTN_OK) return rc;
   if (a->batch == 0 || a->max_q_len == 0) return LSATTN_OK;
-  return a->dtype == LSATTN_F16 ? launch_prefill<F16, 1>(a, (hipStream_t)stream) : launch_prefill<BF16, 1>(a, (hipStream_t)stream);
+  if (a->dtype == LSATTN_F16) return launch_prefill<F16, 1, true>(a, (hipStream_t)stream);
+  return a->v_is_f16 ? launch_prefill<BF16, 1, true>(a, (hipStream_t)stream) : launch_prefill<BF16, 1, false>(a, (hipStream_t)stream);
 }

@@ -51,6 +51,29 @@ def _slots(t: torch.Tensor, name: str, n: Optional[int] = None) -> torch.Tensor:
     return t
 
 
+# A bfloat16 V is rewritten as fp16 before the attention launch (the kernel multiplies P and V in fp16 either way and
+# converting inside it costs about 15 % of its speed).  False keeps V as it is and lets the kernel convert.
+PRECONVERT_BF16_V = True
+
+
+def _v_as_f16(v: torch.Tensor) -> torch.Tensor:
+    """fp16 copy of a [tokens, heads, head_dim] bfloat16 tensor (any token / head strides), made on the device by
+    lsattn_bf16_to_f16_rows; values beyond fp16's range become +-65504."""
+    T, H, D = v.shape
+    out = torch.empty((T, H, D), dtype=torch.float16, device=v.device)
+    if T == 0:
+        return out
+    lib = _lib.load()
+    if v.stride(1) == D:  # heads adjacent: one row per token
+        rc = lib.lsattn_bf16_to_f16_rows(v.data_ptr(), v.stride(0), out.data_ptr(), H * D, T, H * D, _stream())
+        _lib.check(rc, "lsattn_bf16_to_f16_rows")
+    else:
+        for hh in range(H):
+            rc = lib.lsattn_bf16_to_f16_rows(v[:, hh].data_ptr(), v.stride(0), out[:, hh].data_ptr(), H * D, T, D, _stream())
+            _lib.check(rc, "lsattn_bf16_to_f16_rows")
+    return out
+
+
 def _prefill_args(q, k, v, o, q_b_start_loc, q_b_seq_len, q_first, kv_b_start_loc, kv_b_seq_len, kv_first,
                   peers: int, max_q_len: int, sm_scale: Optional[float]) -> _lib.PrefillArgs:
     for t, n in ((q, "q"), (k, "k"), (v, "v"), (o, "o")):
@@ -74,6 +97,10 @@ def _prefill_args(q, k, v, o, q_b_start_loc, q_b_seq_len, q_first, kv_b_start_lo
                  (kv_b_start_loc, "kv_b_start_loc"), (kv_b_seq_len, "kv_b_seq_len"), (kv_first, "kv_first_token_global_idx")):
         _i32vec(t, n, B)
     a = _lib.PrefillArgs()
+    if q.dtype == torch.bfloat16 and PRECONVERT_BF16_V:
+        v = _v_as_f16(v)
+        a.v_is_f16 = 1
+        a._v_f16 = v  # keeps the copy alive as long as the argument block
     a.q, a.k, a.v = q.data_ptr(), k.data_ptr(), v.data_ptr()
     a.q_stride_t, a.q_stride_h = q.stride(0), q.stride(1)
     a.k_stride_t, a.k_stride_h = k.stride(0), k.stride(1)

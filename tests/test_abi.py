@@ -83,6 +83,8 @@ def test_validation_rejects_bad_arguments_without_gpu():
     m = _lib.MergeArgs()
     assert lib.lsattn_lse_merge(C.byref(m), None) == -1
     assert lib.lsattn_kv_scatter(None, 0, None, 0, None, 0, 0, None) == -1
+    assert lib.lsattn_bf16_to_f16_rows(None, 8, None, 8, 1, 8, None) == -1
+    assert lib.lsattn_bf16_to_f16_rows(0x1000, 8, 0x2000, 8, 1, 16, None) == -1   # stride shorter than the row
     # slot allocator: sizes of the workspaces are host arithmetic, argument checks come before any launch
     assert lib.lsattn_pool_search_workspace_bytes(0) == 0
     assert lib.lsattn_pool_search_workspace_bytes(4096) == 16 + 28 + 4          # one workgroup of slots, padded to 16

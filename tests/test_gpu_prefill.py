@@ -181,3 +181,48 @@ def test_kv_scatter_and_register_bit_exact(lsa):
     lsa.init_req_to_token_indexes(table_d, b_req.to(DEV), ln.to(DEV), dest.to(DEV), st.to(DEV), max(lens))
     orc.register_tokens(table, b_req, st, ln, dest)
     assert torch.equal(table_d.cpu(), table)
+
+
+def test_bf16_v_converted_inside_the_kernel_or_before_it(lsa):
+    """Both routes for a bfloat16 V (fp16 copy made before the launch, the default; conversion while the tile is
+    staged) against the oracle, on lengths that take the main loop and the masked steps, V as a strided view."""
+    from loongserve_amd import ops
+    lens, Hq, Hkv, D = [700, 1500], 8, 2, 128
+    T = sum(lens)
+    q = rand_t((T, Hq, D), 11, torch.bfloat16)
+    kv = rand_t((T, 2 * Hkv, D), 12, torch.bfloat16)
+    k, v = kv[:, :Hkv], kv[:, Hkv:]
+    m = meta(lens)
+    o_ref, lse_ref = orc.attn_step(q, k, v, *m, *m, 1)
+    kvd = kv.to(DEV)
+    try:
+        for pre in (True, False):
+            ops.PRECONVERT_BF16_V = pre
+            qs, ql, qf = _dev(*m)
+            o, lse = lsa.prefill_attention_step(q.to(DEV), kvd[:, :Hkv], kvd[:, Hkv:], qs, ql, qf, qs, ql, qf, 1, max(lens))
+            assert_o_close(o, o_ref, "O (pre-converted V: %s)" % pre)
+            assert_lse_close(lse, lse_ref, "LSE (pre-converted V: %s)" % pre)
+    finally:
+        ops.PRECONVERT_BF16_V = True
+
+
+def test_bf16_to_f16_rows_is_exact_in_range_and_saturates(lsa):
+    from loongserve_amd import _lib
+    lib = _lib.load()
+    g = torch.Generator().manual_seed(5)
+    src = (torch.randn(300, 3 * 128, generator=g) * 4).to(torch.bfloat16)
+    src[0, :6] = torch.tensor([70000.0, -70000.0, 65504.0, 1e-3, 0.0, -0.0]).to(torch.bfloat16)
+    src[1, 0] = float("inf")
+    sd = src.to(DEV)
+    view = sd[:, 128:256]                                  # a strided window: rows of 128 with stride 384
+    dst = torch.zeros(300, 128, dtype=torch.float16, device=DEV)
+    rc = lib.lsattn_bf16_to_f16_rows(view.data_ptr(), view.stride(0), dst.data_ptr(), dst.stride(0), 300, 128,
+                                     torch.cuda.current_stream().cuda_stream)
+    assert rc == 0
+    assert torch.equal(dst.cpu(), src[:, 128:256].to(torch.float16))   # |values| here are far inside fp16's range
+    full = torch.zeros(300, 384, dtype=torch.float16, device=DEV)
+    assert lib.lsattn_bf16_to_f16_rows(sd.data_ptr(), 384, full.data_ptr(), 384, 300, 384, torch.cuda.current_stream().cuda_stream) == 0
+    got = full.cpu()
+    assert got[0, :6].tolist() == [65504.0, -65504.0, 65504.0, float(torch.tensor(1e-3).to(torch.bfloat16)), 0.0, -0.0]
+    assert got[1, 0].item() == 65504.0 or math.isinf(got[1, 0].item())
+    assert lib.lsattn_bf16_to_f16_rows(sd.data_ptr(), 384, full.data_ptr(), 384, 300, 380, None) == -1   # row_elems % 8
