@@ -88,12 +88,15 @@ def test_scanner_flags_the_patterns_it_is_meant_to():
 
 @pytest.mark.skipif(shutil.which(HIPCC) is None, reason="hipcc not available")
 def test_no_vector_write_next_to_an_inline_assembly_mfma():
+    # the library's own compile flags, from the build recipe (loaded by path: it does not need the built library)
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("_lsattn_build_flags", os.path.join(REPO, "loongserve_amd", "build.py"))
+    recipe = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(recipe)
     src = os.path.join(REPO, "loongserve_amd", "csrc", "prefill.hip")
     with tempfile.TemporaryDirectory() as tmp:
         out = os.path.join(tmp, "prefill.s")
-        cmd = [HIPCC, "--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-               "-I" + os.path.join(REPO, "include"), "-I" + os.path.join(REPO, "loongserve_amd", "csrc"), "-S", "--cuda-device-only",
-               src, "-o", out]
+        cmd = [recipe.HIPCC, *recipe.FLAGS, *recipe.FILE_FLAGS.get("prefill.hip", []), "-S", "--cuda-device-only", src, "-o", out]
         subprocess.run(cmd, check=True, stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)
         text = open(out).read()
     ins, bad = find_hazards(text)
