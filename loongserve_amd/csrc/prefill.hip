@@ -138,17 +138,18 @@ __device__ __forceinline__ float column_sum(float v) {
 }
 
 // LDS: a ring of four K tiles at [0, 64K) and a ring of four V tiles at [64K, 128K); a tile is [64 rows][16 chunks of 16 bytes]
-// and the chunk index is XORed with swz_bits(row).
+// and the chunk index is XORed with swz_k(row) / swz_v(row).
 constexpr int kTileBytes = BN * 256;
 constexpr int kRing = 4;  // tiles per ring
 constexpr int kLdsV = kRing * kTileBytes;
 constexpr int kLdsBytes = 2 * kRing * kTileBytes;
-// LDS has 64 four-byte banks (256 bytes per clock): sixteen lanes of a 16-byte read, thirty-two lanes of
-// an 8-byte read are served together.  With this XOR the sixteen K rows read together land in sixteen
-// different 16-byte bank groups, and the eight V rows of half a transposing read (32 contiguous bytes each)
-// land in eight different 32-byte groups; both patterns then run at the rate of a linear read.  Only the
-// low four bits of the row count, so rows 16 apart share their XOR.
-__device__ __forceinline__ int swz_bits(int row) { return ((row & 7) << 1) | ((row >> 3) & 1); }
+// The XOR on the 16-byte chunk index differs between the two rings, each chosen by measurement on the read pattern of
+// its operand (LDS has 64 four-byte banks; which lanes of a wide read are served together is not documented):
+// sixteen K rows read with ds_read_b128 run at the rate of a linear read with row & 15 (and at half of it with the V
+// ring's XOR); the transposing V reads, 32 contiguous bytes from each of eight rows per half wave, do so with the XOR
+// below (and not with row & 15).  Only the low four bits of the row count, so rows 16 apart share their XOR.
+__device__ __forceinline__ int swz_k(int row) { return row & 15; }
+__device__ __forceinline__ int swz_v(int row) { return ((row & 7) << 1) | ((row >> 3) & 1); }
 
 typedef __attribute__((address_space(3))) i16x4* lds_i16x4_ptr;
 typedef __attribute__((address_space(3))) void* lds_void_ptr;
@@ -298,14 +299,14 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
     for (int ks = 0; ks < 4; ks++) qreg[qb][ks] = ok ? *(const u32x4*)(src + ks * 64) : u32x4{0, 0, 0, 0};
   }
 
-  int koff0 = qc * 256 + ((g ^ swz_bits(qc)) << 4);
+  int koff0 = qc * 256 + ((g ^ swz_k(qc)) << 4);
   int voff0;
   {
     // a transposing read hands lane c of a 16-lane group column d0 + c of the 4 x 16 block its lanes point at:
     // lane c points at row (c >> 2), columns d0 + 4 (c & 3) .. + 3
     const int row = 4 * g + (qc >> 2);
     const int d_off = 4 * (qc & 3);
-    voff0 = row * 256 + (((d_off >> 3) ^ swz_bits(row)) << 4) + (d_off & 7) * 2;
+    voff0 = row * 256 + (((d_off >> 3) ^ swz_v(row)) << 4) + (d_off & 7) * 2;
   }
   const int lds_base = (int)(uintptr_t)(__attribute__((address_space(3))) char*)lds;
 
@@ -316,13 +317,14 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
   const int st_row = lane >> 4;
   const int last_row = kv_len - 1;
   uint32_t k_lane_off[2], v_lane_off[2];
-  int st_chunk[2];
+  int st_chunk_k[2], st_chunk_v[2];
 #pragma unroll
   for (int i = 0; i < 2; i++) {
     const int r = 8 * wave + 4 * i + st_row;
-    st_chunk[i] = ((lane & 15) ^ swz_bits(r)) << 4;
-    k_lane_off[i] = (uint32_t)(r * k_row_bytes) + st_chunk[i];
-    v_lane_off[i] = (uint32_t)(r * v_row_bytes) + st_chunk[i];
+    st_chunk_k[i] = ((lane & 15) ^ swz_k(r)) << 4;
+    st_chunk_v[i] = ((lane & 15) ^ swz_v(r)) << 4;
+    k_lane_off[i] = (uint32_t)(r * k_row_bytes) + st_chunk_k[i];
+    v_lane_off[i] = (uint32_t)(r * v_row_bytes) + st_chunk_v[i];
   }
   u32x4 vst[2];
   auto load_tiles = [&](auto full_tag, int tk, int tv) __attribute__((always_inline)) {
@@ -344,8 +346,8 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
         nk = nk > last_row ? last_row : nk;
         nv = nv > last_row ? last_row : nv;
         nv = nv < 0 ? 0 : nv;
-        ksrc = kg + nk * k_row_bytes + st_chunk[i];
-        vsrc = vg + nv * v_row_bytes + st_chunk[i];
+        ksrc = kg + nk * k_row_bytes + st_chunk_k[i];
+        vsrc = vg + nv * v_row_bytes + st_chunk_v[i];
       }
       const int kdst = (tk & (kRing - 1)) * kTileBytes + (8 * wave + 4 * i) * 256;
       const int vdst = kLdsV + (tv & (kRing - 1)) * kTileBytes + (8 * wave + 4 * i) * 256;
