@@ -475,11 +475,11 @@ def main():
             "config": {"workload": "config 2: ring prefill on one GPU, queries of shard 3 (16384 rows) of a 131072-token sequence vs KV "
                                    "shards 3 (causal), 0, 1, 2 (full) + LSE merge; 32 heads MHA, head_dim 128, fp16",
                        "algorithmic_tflop_per_step": w.flops / 1e12, "launches_per_step": w.launches + 1, "step_stats": st},
-            "roofline": {"kernel": "prefill_kernel<F16,0>", "bound": "mfma", "achieved": ach, "peak": PEAK_MFMA_TFLOPS, "unit": "TFLOP/s",
+            "roofline": {"kernel": "prefill_kernel<F16,0,true>", "bound": "mfma", "achieved": ach, "peak": PEAK_MFMA_TFLOPS, "unit": "TFLOP/s",
                          "frac": ach / PEAK_MFMA_TFLOPS,
                          # HBM bytes per launch (read 772.8 MB + written 509.6 MB), rocprofv3 FETCH_SIZE / WRITE_SIZE scaled by a
                          # plain copy: profiles/bench_default_hbm_traffic.txt
-                         "traffic": 1107.8e6,
+                         "traffic": 1130.6e6,
                          "per_launch_ms": per_launch_ms, "algorithmic_tflop_per_launch": w.flops / w.launches / 1e12},
         })
         if not args.no_cpu:
