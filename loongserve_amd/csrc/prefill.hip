@@ -127,14 +127,24 @@ __device__ __forceinline__ float max_raw(float a, float b) {
   return r;
 }
 
-// A query column of a 16x16 block lives in the four lanes c, c + 16, c + 32, c + 48: maximum / sum over them
+// A query column of a 16x16 block lives in the four lanes c, c + 16, c + 32, c + 48: maximum / sum over them.
+// ds_swizzle in bit mode (lane ^ 16 inside each half of the wave) and v_permlane32_swap (the other half) need no address
+// register, so nothing of this is computed ahead of the rare branch that uses it.
+__device__ __forceinline__ float lane_xor16(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x401F));  // and 0x1f, or 0, xor 0x10
+}
+__device__ __forceinline__ float lane_xor32(float v) {
+  const unsigned u = __builtin_bit_cast(unsigned, v);
+  auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);  // r[0] = (lower, lower), r[1] = (upper, upper)
+  return __builtin_bit_cast(float, (threadIdx.x & 32) ? r[0] : r[1]);
+}
 __device__ __forceinline__ float column_max(float v) {
-  v = fmaxf(v, __shfl_xor(v, 16));
-  return fmaxf(v, __shfl_xor(v, 32));
+  v = fmaxf(v, lane_xor16(v));
+  return fmaxf(v, lane_xor32(v));
 }
 __device__ __forceinline__ float column_sum(float v) {
-  v += __shfl_xor(v, 16);
-  return v + __shfl_xor(v, 32);
+  v += lane_xor16(v);
+  return v + lane_xor32(v);
 }
 
 // LDS: a ring of four K tiles at [0, 64K) and a ring of four V tiles at [64K, 128K); a tile is [64 rows][16 chunks of 16 bytes]
@@ -386,11 +396,23 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
   auto load_tiles_fast = [&](auto r_tag) __attribute__((always_inline)) {
     constexpr int R = decltype(r_tag)::value;
     constexpr int kslot = ((R + 3) & 3) * kTileBytes, vslot = kLdsV + ((R + 2) & 3) * kTileBytes;
-#pragma unroll
-    for (int i = 0; i < 2; i++) {
-      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(st_lds + kslot + i * 1024), "v"(k_lane_off[i]), "s"(kt_run) : "m0", "memory");
-      if (DV)
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(st_lds + vslot + i * 1024), "v"(v_lane_off[i]), "s"(vt_run) : "m0", "memory");
+    // one block, so that nothing is put between the loads (a wave issues an instruction every five cycles or so,
+    // whatever it is); the s_nop is the wait state a write of m0 needs before an LDS-DMA load reads it
+    if (DV) {
+      asm volatile(
+          "s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %4, %8\n\t"
+          "s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %5, %8\n\t"
+          "s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %6, %9\n\t"
+          "s_mov_b32 m0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %7, %9" ::"s"(st_lds + kslot),
+          "s"(st_lds + kslot + 1024), "s"(st_lds + vslot), "s"(st_lds + vslot + 1024), "v"(k_lane_off[0]), "v"(k_lane_off[1]),
+          "v"(v_lane_off[0]), "v"(v_lane_off[1]), "s"(kt_run), "s"(vt_run)
+          : "m0", "memory");
+    } else {
+      asm volatile(
+          "s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %4\n\t"
+          "s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %3, %4" ::"s"(st_lds + kslot),
+          "s"(st_lds + kslot + 1024), "v"(k_lane_off[0]), "v"(k_lane_off[1]), "s"(kt_run)
+          : "m0", "memory");
     }
     kt_run += BN * k_row_bytes;
     if (DV) vt_run += BN * v_row_bytes;
@@ -564,7 +586,7 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
     __builtin_amdgcn_sched_barrier(0);
   };
   // The two waves that share a SIMD (w and w + 4) run the fast loop half a step apart, one in its MFMA
-  // phase while the other is in its softmax phase (at the higher priority, or the MFMA wave starves it);
+  // phase while the other is in its softmax phase (wave priorities make no measurable difference with this MFMA shape);
   // a workgroup barrier ends every phase.  The loads of K tile it+3 and V tile it+2 go out in the first
   // softmax phase of iteration it; the wait before the iteration's second MFMA phase leaves only those
   // in flight, so a tile is complete for both groups one barrier before its first read, and no read of
@@ -572,15 +594,12 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
   auto fast_iteration = [&](auto r_tag, int it) __attribute__((always_inline)) {
     fphase_mfma(std::integral_constant<int, 0>{}, r_tag);
     __builtin_amdgcn_s_barrier();
-    __builtin_amdgcn_s_setprio(3);
     load_tiles_fast(r_tag);
     fphase_softmax();
-    __builtin_amdgcn_s_setprio(0);
     __builtin_amdgcn_s_barrier();
     if (DV) wait_vmem<4>();
     fphase_mfma(std::integral_constant<int, 1>{}, r_tag);
     __builtin_amdgcn_s_barrier();
-    __builtin_amdgcn_s_setprio(3);
     fphase_softmax();
     if (!DV) {
       // everything but this iteration's two K loads has arrived: the registers hold V tile it+2, and K tile it+2
@@ -589,7 +608,6 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
       store_v_tile(it + 2);
       load_v_regs_fast();  // V tile it+3
     }
-    __builtin_amdgcn_s_setprio(0);
     __builtin_amdgcn_s_barrier();
   };
 
