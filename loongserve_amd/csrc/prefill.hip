@@ -114,19 +114,6 @@ template <> __device__ __forceinline__ u32x4 to_pv_operand<BF16>(const u32x4& w)
   return r;
 }
 
-// Maxima on values that come out of inline-assembly MFMAs: through the fmaxf builtin the compiler first quiets
-// possible signalling NaNs (one more instruction per input), which these accumulators never hold.
-__device__ __forceinline__ float max3_raw(float a, float b, float c) {
-  float r;
-  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
-  return r;
-}
-__device__ __forceinline__ float max_raw(float a, float b) {
-  float r;
-  asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
-  return r;
-}
-
 // A query column of a 16x16 block lives in the four lanes c, c + 16, c + 32, c + 48: maximum / sum over them.
 // ds_swizzle in bit mode (lane ^ 16 inside each half of the wave) and v_permlane32_swap (the other half) need no address
 // register, so nothing of this is computed ahead of the rare branch that uses it.
@@ -539,8 +526,8 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
     float ma[2], mb[2], t[2][8];
 #pragma unroll
     for (int qb = 0; qb < 2; qb++) {
-      ma[qb] = max3_raw(s[0][qb][0], s[0][qb][1], s[0][qb][2]);
-      mb[qb] = max3_raw(s[0][qb][3], s[1][qb][0], s[1][qb][1]);
+      ma[qb] = fmaxf(fmaxf(s[0][qb][0], s[0][qb][1]), s[0][qb][2]);
+      mb[qb] = fmaxf(fmaxf(s[0][qb][3], s[1][qb][0]), s[1][qb][1]);
     }
 #pragma unroll
     for (int qb = 0; qb < 2; qb++)
@@ -550,14 +537,14 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
         for (int r = 0; r < 4; r++) t[qb][4 * kb + r] = __builtin_fmaf(s[kb][qb][r], scale, neg_m[qb]);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int qb = 0; qb < 2; qb++) ma[qb] = max3_raw(ma[qb], s[1][qb][2], s[1][qb][3]);
+    for (int qb = 0; qb < 2; qb++) ma[qb] = fmaxf(fmaxf(ma[qb], s[1][qb][2]), s[1][qb][3]);
 #pragma unroll
     for (int qb = 0; qb < 2; qb++)
 #pragma unroll
       for (int i = 0; i < 8; i++) t[qb][i] = __builtin_amdgcn_exp2f(t[qb][i]);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int qb = 0; qb < 2; qb++) mx[qb] = max_raw(ma[qb], mb[qb]);
+    for (int qb = 0; qb < 2; qb++) mx[qb] = fmaxf(ma[qb], mb[qb]);
 #pragma unroll
     for (int qb = 0; qb < 2; qb++)
 #pragma unroll
