@@ -128,13 +128,15 @@ __global__ __launch_bounds__(NW * 64) void decode_stage1_kernel(Stage1Params p) 
 #pragma unroll
       for (int j = 0; j < kTok; j++) {
         asm volatile("" : "+v"(slot[j]));
-        kr[j] = *(const u32x4*)(kbase + (int64_t)slot[j] * k_row_bytes);
+        kr[j] = __builtin_nontemporal_load((const u32x4*)(kbase + (int64_t)slot[j] * k_row_bytes));
       }
 #pragma unroll
       for (int j = 0; j < kTok; j++) {
         asm volatile("" : "+v"(slot[j]));
-        vr[j] = *(const u32x4*)(vbase + (int64_t)slot[j] * v_row_bytes);
+        vr[j] = __builtin_nontemporal_load((const u32x4*)(vbase + (int64_t)slot[j] * v_row_bytes));
       }
+      // The rows are read once: non-temporal loads.  As ordinary loads they push the block partials (which stage 2
+      // reads back) out of the caches early, and the trickle of write-backs between the reads costs the gather 5 %.
       // all 16 row loads are issued before anything else happens (the scheduler would otherwise sink
       // each load next to its first use and expose its latency)
       __builtin_amdgcn_sched_barrier(0);
