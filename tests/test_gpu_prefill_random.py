@@ -1,0 +1,40 @@
+"""Seeded random sweep of the prefill step against the oracle: ragged batches, GQA groups, striped and offset steps,
+empty KV chunks, lengths on both sides of every tile boundary, both dtypes (through the C ABI)."""
+import random
+
+import pytest
+import torch
+
+from oracle import attn_oracle as orc
+from tests.helpers import assert_lse_close, assert_o_close, meta, rand_t
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.mark.parametrize("seed", [1, 7, 23])
+def test_random_steps_match_the_oracle(lsa, seed):
+    rng = random.Random(seed)
+    for case in range(16):
+        dtype = rng.choice([torch.float16, torch.bfloat16])
+        Hkv = rng.choice([1, 2, 3])
+        Hq = Hkv * rng.choice([1, 2, 4])
+        B = rng.choice([1, 2, 3])
+        P = rng.choice([1, 1, 2, 3, 4])
+        qlens = [rng.choice([1, 17, 255, 256, 257, 300, 511, 600, 900, 1400, 2100]) for _ in range(B)]
+        klens = [rng.choice([0, 1, 63, 64, 200, 256, 448, 511, 512, 700, 1300, 2500]) for _ in range(B)]
+        qf = [rng.choice([0, 1, 5, 300, 1000, 4000]) for _ in range(B)]
+        kf = [rng.choice([0, 1, 2, 3, 100, 700]) for _ in range(B)]
+        print("case", seed, case, dtype, Hq, Hkv, P, qlens, qf, klens, kf, flush=True)
+        Tq, Tk = sum(qlens), max(sum(klens), 1)
+        q = rand_t((Tq, Hq, 128), 1000 * seed + case, dtype)
+        k = rand_t((Tk, Hkv, 128), 1000 * seed + 100 + case, dtype)
+        v = rand_t((Tk, Hkv, 128), 1000 * seed + 200 + case, dtype)
+        qm, km = meta(qlens, qf), meta(klens, kf)
+        o_ref, lse_ref = orc.attn_step(q, k, v, *qm, *km, P)
+        o, lse = lsa.prefill_attention_step(q.to(DEV), k.to(DEV), v.to(DEV), *[t.to(DEV) for t in qm], *[t.to(DEV) for t in km],
+                                            P, max(qlens))
+        torch.cuda.synchronize()
+        what = "seed %d case %d" % (seed, case)
+        assert_o_close(o, o_ref, "O, " + what)
+        assert_lse_close(lse, lse_ref, "LSE, " + what)
