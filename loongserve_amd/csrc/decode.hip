@@ -32,6 +32,7 @@ struct Stage1Params {
   int64_t batch, hq, hkv, num_blocks, max_seq_len, block_seq, grid_blocks;
   int32_t blocks_per_wg;  // consecutive blocks walked by one workgroup
   int32_t tasks;          // hkv * (group / GT) wave tasks
+  int32_t tasks_on_x;     // grid = (task groups, chunks, batch) instead of (chunks, task groups, batch)
 };
 
 constexpr int kTok = 8;  // K/V rows in flight per 16-lane group
@@ -71,7 +72,10 @@ __global__ __launch_bounds__(NW * 64) void decode_stage1_kernel(Stage1Params p) 
   const int sub = lane & 15;   // 16-byte column slot: elements sub*8 .. sub*8+7
   const int jbase = (sub >> 2) * 2;  // first of the two rows whose scores this lane finishes (see the reduction)
   const int64_t b = blockIdx.z;
-  const int task = blockIdx.y * NW + wave;
+  // The workgroups that read the other KV heads of the same tokens are next to this one in dispatch order when the
+  // task index is the fastest grid dimension: the pieces of a token's K (and V) span are then fetched close together in
+  // time (measured 2 % faster on GQA 32/8, two task groups per chunk).
+  const int task = (p.tasks_on_x ? blockIdx.x : blockIdx.y) * NW + wave;
   if (task >= p.tasks) return;
   const int group = (int)(p.hq / p.hkv);
   const int sub_groups = group / GT;
@@ -82,7 +86,7 @@ __global__ __launch_bounds__(NW * 64) void decode_stage1_kernel(Stage1Params p) 
   int64_t nblk = len <= 0 ? 0 : ((int64_t)len + p.block_seq - 1) / p.block_seq;
   if (nblk > p.grid_blocks) nblk = p.grid_blocks;
   if (nblk > p.num_blocks) nblk = p.num_blocks;
-  const int64_t blk_begin = (int64_t)blockIdx.x * p.blocks_per_wg;
+  const int64_t blk_begin = (int64_t)(p.tasks_on_x ? blockIdx.y : blockIdx.x) * p.blocks_per_wg;
   int64_t blk_end = blk_begin + p.blocks_per_wg;
   if (blk_end > nblk) blk_end = nblk;
   if (blk_begin >= blk_end) return;
@@ -415,7 +419,9 @@ static int launch_stage1(const lsattn_decode_stage1_args* a, hipStream_t st) {
   p.blocks_per_wg = (int32_t)per_wg;
   const int64_t chunks = (nblk + per_wg - 1) / per_wg;
   if (chunks > 0x7fffffff || a->batch > 65535 || wgs_y > 65535) return LSATTN_ERR_INVALID_ARG;
-  dim3 grid((unsigned)chunks, (unsigned)wgs_y, (unsigned)a->batch);
+  p.tasks_on_x = wgs_y <= 2 && chunks <= 65535;  // with more task groups per chunk (MHA, 32 KV heads) it measured 2 % slower
+  dim3 grid = p.tasks_on_x ? dim3((unsigned)wgs_y, (unsigned)chunks, (unsigned)a->batch)
+                           : dim3((unsigned)chunks, (unsigned)wgs_y, (unsigned)a->batch);
   hipLaunchKernelGGL((decode_stage1_kernel<T, GT, NW>), grid, dim3(NW * 64), 0, st, p);
   return check_launch();
 }
