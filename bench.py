@@ -143,6 +143,9 @@ class TokenDecode:
         self.b_len = _i32(self.lens)
         from loongserve_amd.simulate import decode_block_seq
         self.BS = decode_block_seq(self.max_len) if block_seq is None else block_seq
+        # the fused call splits the context more coarsely than BLOCK_SEQ between its two stages (mid_o is scratch there)
+        from loongserve_amd.decoding import _fused_block_seq
+        self.split = _fused_block_seq(self.BS, B, self.max_len, Hkv)
         nblk = (self.max_len + self.BS - 1) // self.BS
         self.mid_o = torch.empty((nblk, B, Hq, D), dtype=torch.float32, device=DEV)
         self.mid_l = torch.empty((nblk, B, Hq), dtype=torch.float32, device=DEV)
@@ -161,7 +164,7 @@ class TokenDecode:
     def stage1_only(self):
         import loongserve_amd as lsa
         lsa.longserve_flash_decode_stage1(self.q, self.kv[:, :self.Hkv], self.kv[:, self.Hkv:], self.table, self.b_req, self.b_len,
-                                          self.max_len, self.mid_o, self.mid_l, self.BS)
+                                          self.max_len, self.mid_o, self.mid_l, self.split)
 
     def cpu_baseline(self, nreq=64):
         from oracle import attn_oracle as orc
@@ -500,7 +503,8 @@ def main():
         dec = {
             "value": gbs, "unit": "GB/s", "ms_per_step": st["mean_ms"], "pct_of_hbm_peak": 100.0 * gbs / PEAK_HBM_GBS,
             "config": {"workload": "config 3: token-indexed decode, batch 64, ctx U[4096,32768], GQA 32/8, head_dim 128, fp16, "
-                                   "2.5M-slot scattered pool; stage1 (split-K, block_seq %d) + stage2" % d.BS,
+                                   "2.5M-slot scattered pool; fused stage1 + stage2 call with BLOCK_SEQ %d (mid_o is scratch there: "
+                                   "split-K at %d tokens between the stages)" % (d.BS, d.split),
                        "tokens": d.tokens, "algorithmic_gb_per_step": d.bytes / 1e9, "step_stats": st},
             "roofline": {"kernel": "decode_stage1_kernel<F16,4,4>", "bound": "hbm", "achieved": ach, "peak": PEAK_HBM_GBS, "unit": "GB/s",
                          "frac": ach / PEAK_HBM_GBS,

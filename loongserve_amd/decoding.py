@@ -20,6 +20,26 @@ def longserve_flash_decode_stage2(mid_out, mid_out_logexpsum, B_Seqlen, O, out_l
     return
 
 
+# Split size between the two stages of the fused call.  There mid_o / mid_o_logexpsum are scratch (FDPY:12-27 never hands
+# them out, the callers at longserve_transformer_layer_infer.py:293-308 only use the returned pair), so the context may be
+# cut more coarsely than BLOCK_SEQ: fewer fp32 block partials are written while the gather saturates the memory system
+# (every MB of them costs about as much as 8 MB of reads).  The result is the same softmax, merged from fewer pieces.
+# longserve_flash_decode_stage1 / _stage2 called on their own always split at the block_seq they are given.
+FUSED_SPLIT_TOKENS = 1024
+FUSED_MIN_WORKGROUPS = 2048  # do not coarsen below this many (upper-bound estimate of) stage-1 workgroups
+
+
+def _fused_block_seq(block_seq: int, batch_size: int, max_len_in_batch: int, num_kv_heads: int) -> int:
+    bs = int(block_seq)
+    task_groups = (int(num_kv_heads) + 3) // 4
+    while bs * 2 <= FUSED_SPLIT_TOKENS and bs < int(max_len_in_batch):
+        blocks = (int(max_len_in_batch) + 2 * bs - 1) // (2 * bs)
+        if int(batch_size) * blocks * task_groups < FUSED_MIN_WORKGROUPS:
+            break
+        bs *= 2
+    return bs
+
+
 def longserve_token_decode_attention_flash_decoding(q, req_to_token_indexs, b_req_idx, b_seq_len, mid_o,
                                                     mid_o_logexpsum, batch_size, max_len_in_batch, q_head_num,
                                                     head_dim, cache_k, cache_v, BLOCK_SEQ, out=None,
@@ -29,8 +49,9 @@ def longserve_token_decode_attention_flash_decoding(q, req_to_token_indexs, b_re
     o_tensor = torch.empty_like(q, dtype=torch.float32) if out is None else out
     out_logexpsum = (torch.empty([batch_size, q_head_num], dtype=torch.float32, device=q.device)
                      if o_logexpsum is None else o_logexpsum)
+    split = _fused_block_seq(BLOCK_SEQ, batch_size, max_len_in_batch, cache_k.shape[1])
     longserve_flash_decode_stage1(q.view(calcu_shape1), cache_k, cache_v, req_to_token_indexs, b_req_idx, b_seq_len,
-                                  max_len_in_batch, mid_o, mid_o_logexpsum, BLOCK_SEQ)
+                                  max_len_in_batch, mid_o, mid_o_logexpsum, split)
     longserve_flash_decode_stage2(mid_o, mid_o_logexpsum, b_seq_len, o_tensor.view(calcu_shape1), out_logexpsum,
-                                  BLOCK_SEQ)
+                                  split)
     return o_tensor, out_logexpsum

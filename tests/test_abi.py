@@ -120,3 +120,18 @@ def test_python_wrappers_reject_cpu_tensors():
     with pytest.raises(ValueError):
         lsa.longserve_cuda_kernels.flash_decoding_stage1(torch.zeros(1, 1, 2, 128), torch.zeros(1, 1, 2), q[:1], q, q,
                                                          torch.zeros(1, 4, dtype=torch.int32), i, i, 4, 4)
+
+
+def test_fused_decode_split_rule():
+    """The fused decode call may split the context more coarsely than BLOCK_SEQ, but only while the launch keeps enough
+    workgroups; the stage functions called on their own never change the block size they are given."""
+    from loongserve_amd.decoding import FUSED_SPLIT_TOKENS, _fused_block_seq
+    assert _fused_block_seq(256, 64, 32768, 8) == 1024           # config 3: 64 x 32 blocks x 2 task groups
+    assert _fused_block_seq(256, 4, 131072, 32) == 1024          # one instance of config 4
+    assert _fused_block_seq(256, 1, 4096, 8) == 256              # a single short request: nothing to spare
+    assert _fused_block_seq(256, 16, 8192, 8) == 256
+    assert _fused_block_seq(2048, 64, 32768, 8) == 2048          # never below what the caller asked for
+    assert _fused_block_seq(16, 4096, 16, 8) == 16
+    for bs in (1, 16, 64, 256):
+        got = _fused_block_seq(bs, 1 << 14, 1 << 20, 32)
+        assert got % bs == 0 and got <= max(FUSED_SPLIT_TOKENS, bs)
