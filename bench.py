@@ -482,7 +482,7 @@ def main():
                          "frac": ach / PEAK_MFMA_TFLOPS,
                          # HBM bytes per launch (read 772.8 MB + written 509.6 MB), rocprofv3 FETCH_SIZE / WRITE_SIZE scaled by a
                          # plain copy: profiles/bench_default_hbm_traffic.txt
-                         "traffic": 1104.3e6,
+                         "traffic": 1104.5e6,
                          "per_launch_ms": per_launch_ms, "algorithmic_tflop_per_launch": w.flops / w.launches / 1e12},
         })
         if not args.no_cpu:
@@ -508,8 +508,8 @@ def main():
                        "tokens": d.tokens, "algorithmic_gb_per_step": d.bytes / 1e9, "step_stats": st},
             "roofline": {"kernel": "decode_stage1_kernel<F16,4,4>", "bound": "hbm", "achieved": ach, "peak": PEAK_HBM_GBS, "unit": "GB/s",
                          "frac": ach / PEAK_HBM_GBS,
-                         # HBM bytes per launch (read 5176.4 MB + written 81.9 MB), same source as above
-                         "traffic": 5253.7e6, "per_launch_ms": s1},
+                         # HBM bytes per launch (read 5174.6 MB + written 20.8 MB), same source as above
+                         "traffic": 5195.4e6, "per_launch_ms": s1},
         }
         if not args.no_cpu:
             dec["cpu_baseline"] = d.cpu_baseline()
