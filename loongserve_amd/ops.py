@@ -74,6 +74,17 @@ def _v_as_f16(v: torch.Tensor) -> torch.Tensor:
     return out
 
 
+KERNEL_HEAD_DIM = 128
+
+
+def _pad_head_dim(t: torch.Tensor) -> torch.Tensor:
+    """[tokens, heads, D] with D < 128 -> a new [tokens, heads, 128] tensor, zeros beyond D.  Zero columns leave q.k
+    unchanged and give zero output columns, so the 128-wide kernel computes the D-wide attention exactly."""
+    out = t.new_zeros((t.shape[0], t.shape[1], KERNEL_HEAD_DIM))
+    out[..., :t.shape[-1]] = t
+    return out
+
+
 def _prefill_args(q, k, v, o, q_b_start_loc, q_b_seq_len, q_first, kv_b_start_loc, kv_b_seq_len, kv_first,
                   peers: int, max_q_len: int, sm_scale: Optional[float]) -> _lib.PrefillArgs:
     for t, n in ((q, "q"), (k, "k"), (v, "v"), (o, "o")):
@@ -128,10 +139,18 @@ def context_attention_fwd(q, k, v, o, q_b_start_loc, q_b_seq_len, q_first_token_
     Start from m = -inf, l = 0 (o need not be zeroed).  After k calls o is the
     normalised attention output over all keys seen and ln2*(m + log2 l) their LSE.
     """
-    a = _prefill_args(q, k, v, o, q_b_start_loc, q_b_seq_len, q_first_token_global_idx, kv_b_start_loc,
-                      kv_b_seq_len, kv_first_token_global_idx, logical_sp_peers_num, max_q_b_seq_len, None)
     if o.dtype != q.dtype:
         raise ValueError("o must have the dtype of q")
+    D = q.shape[-1]
+    o_user = None
+    if q.dim() == 3 and D in (16, 32, 64) and k.shape[-1] == D and v.shape[-1] == D and o.shape == q.shape:
+        # head sizes below 128 (RING:250 admits them): run the 128-wide kernel on zero-padded copies, old o included
+        # (the step folds into it), and copy the first D columns back
+        o_user, o = o, _pad_head_dim(o)
+        q, k, v = _pad_head_dim(q), _pad_head_dim(k), _pad_head_dim(v)
+    a = _prefill_args(q, k, v, o, q_b_start_loc, q_b_seq_len, q_first_token_global_idx, kv_b_start_loc,
+                      kv_b_seq_len, kv_first_token_global_idx, logical_sp_peers_num, max_q_b_seq_len,
+                      1.0 / (D ** 0.5))
     for t, n in ((m, "m"), (l, "l")):
         _dev(t, n)
         if t.dtype != torch.float32 or t.dim() != 2 or tuple(t.shape) != (q.shape[0], q.shape[1]):
@@ -141,6 +160,8 @@ def context_attention_fwd(q, k, v, o, q_b_start_loc, q_b_seq_len, q_first_token_
     a.m, a.l = m.data_ptr(), l.data_ptr()
     a.ml_stride_t, a.ml_stride_h = m.stride(0), m.stride(1)
     _lib.check(_lib.load().lsattn_prefill_step_merge(C.byref(a), _stream()), "lsattn_prefill_step_merge")
+    if o_user is not None:
+        o_user.copy_(o[..., :D])
 
 
 @torch.inference_mode()
@@ -153,16 +174,26 @@ def prefill_attention_step(q, k, v, q_b_start_loc, q_b_seq_len, q_first_token_gl
 
     Same inputs as context_attention_fwd; rows that see no key get O = 0, LSE = -inf.
     """
+    D = q.shape[-1]
     if out is None:
         out = torch.empty(q.shape, dtype=torch.float32, device=q.device)
     if lse is None:
         lse = torch.empty(q.shape[:2], dtype=torch.float32, device=q.device)
     if out.dtype != torch.float32 or lse.dtype != torch.float32 or not lse.is_contiguous():
         raise ValueError("out and lse must be float32, lse contiguous")
+    out_user = None
+    if q.dim() == 3 and D in (16, 32, 64) and k.shape[-1] == D and v.shape[-1] == D and out.shape == q.shape:
+        out_user, out = out, torch.empty(q.shape[:2] + (KERNEL_HEAD_DIM,), dtype=torch.float32, device=q.device)
+        q, k, v = _pad_head_dim(q), _pad_head_dim(k), _pad_head_dim(v)
+        if sm_scale is None:
+            sm_scale = 1.0 / (D ** 0.5)
     a = _prefill_args(q, k, v, out, q_b_start_loc, q_b_seq_len, q_first_token_global_idx, kv_b_start_loc,
                       kv_b_seq_len, kv_first_token_global_idx, logical_sp_peers_num, max_q_b_seq_len, sm_scale)
     a.lse = lse.data_ptr()
     _lib.check(_lib.load().lsattn_prefill_step(C.byref(a), _stream()), "lsattn_prefill_step")
+    if out_user is not None:
+        out_user.copy_(out[..., :D])
+        out = out_user
     return out, lse
 
 

@@ -226,3 +226,34 @@ def test_bf16_to_f16_rows_is_exact_in_range_and_saturates(lsa):
     assert got[0, :6].tolist() == [65504.0, -65504.0, 65504.0, float(torch.tensor(1e-3).to(torch.bfloat16)), 0.0, -0.0]
     assert got[1, 0].item() == 65504.0 or math.isinf(got[1, 0].item())
     assert lib.lsattn_bf16_to_f16_rows(sd.data_ptr(), 384, full.data_ptr(), 384, 300, 380, None) == -1   # row_elems % 8
+
+
+@pytest.mark.parametrize("D", [16, 32, 64])
+def test_head_sizes_below_128(lsa, D):
+    """RING:250 admits head sizes 16, 32 and 64; the operators run them through the 128-wide kernel on zero-padded
+    copies.  One partial step, and two in-place steps whose second one folds into the first one's o."""
+    print("case D", D, flush=True)
+    lens, Hq, Hkv = [300, 77], 4, 2
+    T = sum(lens)
+    q, k, v = rand_t((T, Hq, D), 41), rand_t((T, Hkv, D), 42), rand_t((T, Hkv, D), 43)
+    m = meta(lens)
+    o, lse = _run_step(lsa, q, k, v, m, m, 1, max(lens))
+    assert o.shape == (T, Hq, D)
+    o_ref, lse_ref = orc.attn_step(q, k, v, *m, *m, 1)
+    assert_o_close(o, o_ref, "O")
+    assert_lse_close(lse, lse_ref, "LSE")
+    # an earlier chunk of 150 / 40 keys per request (positions before the queries': visible to all), then the causal one
+    klens = [150, 40]
+    k0, v0 = rand_t((sum(klens), Hkv, D), 44), rand_t((sum(klens), Hkv, D), 45)
+    qm = meta(lens, [150, 40])
+    km0 = meta(klens)
+    od = torch.empty(T, Hq, D, dtype=torch.float16, device=DEV)
+    md = torch.full((T, Hq), float("-inf"), device=DEV)
+    ld = torch.zeros(T, Hq, device=DEV)
+    oc, mc, lc = torch.zeros(T, Hq, D, dtype=torch.float16), torch.full((T, Hq), float("-inf")), torch.zeros(T, Hq)
+    for kk, vv, km in ((k, v, qm), (k0, v0, km0)):
+        lsa.context_attention_fwd(q.to(DEV), kk.to(DEV), vv.to(DEV), od, *_dev(*qm), *_dev(*km), 1, max(lens), md, ld)
+        orc.context_attention_fwd(q, kk, vv, oc, *qm, *km, 1, max(lens), mc, lc)
+    torch.cuda.synchronize()
+    assert_o_close(od, oc.float(), "in-place o")
+    assert_lse_close(orc.state_lse(md.cpu(), ld.cpu()).float(), orc.state_lse(mc, lc).float(), "state")
