@@ -766,6 +766,8 @@ static int validate(const lsattn_prefill_args* a, int mode) {
   if (a->q_stride_t % 8 || a->q_stride_h % 8 || a->k_stride_t % 8 || a->k_stride_h % 8 || a->v_stride_t % 8 || a->v_stride_h % 8)
     return LSATTN_ERR_INVALID_ARG;
   if (a->o_stride_t % 4 || a->o_stride_h % 4) return LSATTN_ERR_INVALID_ARG;
+  // a lane addresses the 64 rows of a K/V tile with a 32-bit byte offset from the tile's first row
+  if (a->k_stride_t <= 0 || a->v_stride_t <= 0 || a->k_stride_t > (1 << 24) || a->v_stride_t > (1 << 24)) return LSATTN_ERR_INVALID_ARG;
   if (((uintptr_t)a->q | (uintptr_t)a->k | (uintptr_t)a->v | (uintptr_t)a->o) & 15) return LSATTN_ERR_INVALID_ARG;
   if (mode == 0) {
     if (!a->lse || a->o_dtype != LSATTN_F32) return LSATTN_ERR_INVALID_ARG;

@@ -108,6 +108,14 @@ def test_validation_rejects_bad_arguments_without_gpu():
     assert lib.lsattn_prefill_step(C.byref(a), None) == -2
     a.head_dim, a.num_kv_heads = 128, 3
     assert lib.lsattn_prefill_step(C.byref(a), None) == -1
+    # K/V token strides must be positive and keep a 64-row tile within a 32-bit byte offset
+    a.num_kv_heads = 2
+    for f in ("q_stride_t", "q_stride_h", "k_stride_h", "v_stride_h", "o_stride_t", "o_stride_h"):
+        setattr(a, f, 128)
+    a.dtype = _lib.LSATTN_F16
+    for ks, vs in ((0, 256), (256, -256), ((1 << 24) + 8, 256), (256, 1 << 25)):
+        a.k_stride_t, a.v_stride_t = ks, vs
+        assert lib.lsattn_prefill_step(C.byref(a), None) == -1, (ks, vs)
 
 
 def test_python_wrappers_reject_cpu_tensors():
