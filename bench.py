@@ -24,6 +24,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
+PREFILL_TRAFFIC_BYTES = 1364.6e6  # per launch, averaged over a ring step: profiles/bench_default_hbm_traffic.txt
 PEAK_MFMA_TFLOPS = 2500.0  # dense fp16/bf16 MFMA, MI355X
 PEAK_HBM_GBS = 8000.0
 DEV = "cuda:0"
@@ -73,8 +74,7 @@ class RingPrefill:
         for j in self.order:
             kv = _randn_half((shard, 2 * kv_heads, D), seed + 1 + j, dtype)
             self.chunks.append(KVChunk(kv, _i32([0]), _i32([shard]), _i32([j * shard])))
-        self.bufs = [(torch.empty((shard, heads, D), dtype=torch.float32, device=DEV),
-                      torch.empty((shard, heads), dtype=torch.float32, device=DEV)) for _ in self.order]
+        self.bufs = None  # per-step partial buffers, only for the separate-merge route
         self.out = torch.empty((shard, heads, D), dtype=torch.float32, device=DEV)
         self.lse = torch.empty((shard, heads), dtype=torch.float32, device=DEV)
         n = shard
@@ -83,15 +83,18 @@ class RingPrefill:
         self.launches = len(self.order)
 
     def step(self):
-        from loongserve_amd.simulate import ring_prefill_partials
-        ring_prefill_partials(self.q, self.chunks, self.qs, self.ql, self.qf, 1, self.shard, self.Hkv, self.bufs, self.out, self.lse)
+        """Four launches in ring order; the first writes the fp32 partial (O, LSE) of the diagonal step, each later one
+        LSE-merges its own partial into it in its epilogue."""
+        from loongserve_amd.simulate import ring_prefill_accumulate
+        ring_prefill_accumulate(self.q, self.chunks, self.qs, self.ql, self.qf, 1, self.shard, self.Hkv, self.out, self.lse)
 
-    def kernel_only(self):
-        """The four attention launches without the merge (for the per-launch roofline figure)."""
-        import loongserve_amd as lsa
-        for c, (ob, lb) in zip(self.chunks, self.bufs):
-            lsa.prefill_attention_step(self.q, c.k(self.Hkv), c.v(self.Hkv), self.qs, self.ql, self.qf, c.b_start_loc, c.b_seq_len,
-                                       c.first_token_global_idx, 1, self.shard, ob, lb)
+    def step_separate_merge(self):
+        """The same four steps as four separate fp32 partials and one lsattn_lse_merge pass over them."""
+        from loongserve_amd.simulate import ring_prefill_partials
+        if self.bufs is None:
+            self.bufs = [(torch.empty((self.shard, self.H, self.D), dtype=torch.float32, device=DEV),
+                          torch.empty((self.shard, self.H), dtype=torch.float32, device=DEV)) for _ in self.order]
+        ring_prefill_partials(self.q, self.chunks, self.qs, self.ql, self.qf, 1, self.shard, self.Hkv, self.bufs, self.out, self.lse)
 
     def cpu_baseline(self, heads=8, rows=4096):
         """Oracle (PyTorch CPU fp32) on a slice: `heads` heads, the last `rows` query rows of the
@@ -467,22 +470,28 @@ def main():
             w.step()
         torch.cuda.synchronize()
         wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
-        kern_ms = _time_events(w.kernel_only, args.steps, 1)
         st = _stats(step_ms)
         tflops = w.flops / (wall_ms * 1e-3) / 1e12
-        per_launch_ms = (sum(kern_ms) / len(kern_ms)) / w.launches
+        # a step is nothing but its four launches: the average launch duration is the step's HIP-event time / 4
+        per_launch_ms = st["mean_ms"] / w.launches
         ach = (w.flops / w.launches) / (per_launch_ms * 1e-3) / 1e12
+        sep = _stats(_time_events(w.step_separate_merge, max(5, args.steps // 2), 2))
         line.update({
             "value": tflops, "unit": "TFLOP/s", "ms_per_step": wall_ms,
             "pct_of_mfma_peak": 100.0 * tflops / PEAK_MFMA_TFLOPS,
             "config": {"workload": "config 2: ring prefill on one GPU, queries of shard 3 (16384 rows) of a 131072-token sequence vs KV "
-                                   "shards 3 (causal), 0, 1, 2 (full) + LSE merge; 32 heads MHA, head_dim 128, fp16",
-                       "algorithmic_tflop_per_step": w.flops / 1e12, "launches_per_step": w.launches + 1, "step_stats": st},
-            "roofline": {"kernel": "prefill_kernel<F16,0,true>", "bound": "mfma", "achieved": ach, "peak": PEAK_MFMA_TFLOPS, "unit": "TFLOP/s",
+                                   "shards 3 (causal), 0, 1, 2 (full), in that order; 32 heads MHA, head_dim 128, fp16; fp32 partial "
+                                   "(O, LSE) per step, LSE-merged into the running result in the epilogue of the launch that produces it",
+                       "algorithmic_tflop_per_step": w.flops / 1e12, "launches_per_step": w.launches, "step_stats": st,
+                       "separate_merge": {"what": "the same steps as four separate fp32 partials + one lsattn_lse_merge pass",
+                                          "ms_per_step": sep["mean_ms"], "value": w.flops / (sep["mean_ms"] * 1e-3) / 1e12,
+                                          "launches_per_step": w.launches + 1}},
+            "roofline": {"kernel": "prefill_kernel<F16,0,true> (diagonal launch) + prefill_kernel<F16,2,true> (three full launches)",
+                         "bound": "mfma", "achieved": ach, "peak": PEAK_MFMA_TFLOPS, "unit": "TFLOP/s",
                          "frac": ach / PEAK_MFMA_TFLOPS,
-                         # HBM bytes per launch (read 772.8 MB + written 509.6 MB), rocprofv3 FETCH_SIZE / WRITE_SIZE scaled by a
-                         # plain copy: profiles/bench_default_hbm_traffic.txt
-                         "traffic": 1104.5e6,
+                         # HBM bytes per launch, averaged over the step's four launches: rocprofv3 FETCH_SIZE / WRITE_SIZE scaled
+                         # by a plain copy, profiles/bench_default_hbm_traffic.txt
+                         "traffic": PREFILL_TRAFFIC_BYTES,
                          "per_launch_ms": per_launch_ms, "algorithmic_tflop_per_launch": w.flops / w.launches / 1e12},
         })
         if not args.no_cpu:

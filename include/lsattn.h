@@ -75,11 +75,11 @@ typedef struct lsattn_prefill_args {
   /* outputs */
   void* o;            /* [Tq,Hq,D] */
   int64_t o_stride_t, o_stride_h;
-  int32_t o_dtype;    /* step: LSATTN_F32; step_merge: same as dtype */
+  int32_t o_dtype;    /* step, step_accumulate: LSATTN_F32; step_merge: same as dtype */
   int32_t v_is_f16;   /* 0: v has `dtype`.  1 (dtype LSATTN_BF16 only): v already holds fp16, e.g. written by
                          lsattn_bf16_to_f16_rows: the P V product runs in fp16 either way, and a bf16 V converted
                          inside the kernel costs about 15 % of its speed */
-  float* lse;         /* step: [Tq,Hq] natural-log LSE, contiguous         */
+  float* lse;         /* step, step_accumulate: [Tq,Hq] natural-log LSE, contiguous */
   float* m;           /* step_merge: [Tq,Hq] running max, log2 domain       */
   float* l;           /* step_merge: [Tq,Hq] running sum                    */
   int64_t ml_stride_t, ml_stride_h; /* strides of m and l (RING:274-275)     */
@@ -94,6 +94,14 @@ int lsattn_prefill_step(const lsattn_prefill_args* a, void* stream);
  * l = 0; after any number of calls ln2*(m + log2 l) is the natural LSE over all keys
  * seen and o is the normalised output in o_dtype.  Uses o (dtype of q), m, l. */
 int lsattn_prefill_step_merge(const lsattn_prefill_args* a, void* stream);
+
+/* The step of lsattn_prefill_step folded into a running fp32 partial instead of written from the empty state:
+ * (o, lse) <- LSE-merge of (o, lse) with this step's (O_i, LSE_i), in the kernel's epilogue.  It is the update of
+ * RING:171-188 with the state kept as (fp32 O, natural LSE), the form the decode path and lsattn_lse_merge exchange,
+ * and it saves a ring the separate merge pass over P partials.  A row with lse = -inf counts as empty, whatever its o
+ * holds; a row that sees no key in this step is left untouched.  First step of a ring: lsattn_prefill_step (or start
+ * from lse = -inf everywhere).  Uses o (F32), lse. */
+int lsattn_prefill_step_accumulate(const lsattn_prefill_args* a, void* stream);
 
 /*
  * Merge n normalised partials (O_i fp32 [rows,D] contiguous, LSE_i [rows]) over disjoint key

@@ -85,6 +85,7 @@ class DecodeMigrationArgs(C.Structure):  # mirrors lsattn_decode_migration_args
 EXPORTS = {
     "lsattn_prefill_step": (C.c_int, [C.POINTER(PrefillArgs), _vp]),
     "lsattn_prefill_step_merge": (C.c_int, [C.POINTER(PrefillArgs), _vp]),
+    "lsattn_prefill_step_accumulate": (C.c_int, [C.POINTER(PrefillArgs), _vp]),
     "lsattn_lse_merge": (C.c_int, [C.POINTER(MergeArgs), _vp]),
     "lsattn_decode_stage1": (C.c_int, [C.POINTER(DecodeStage1Args), _vp]),
     "lsattn_decode_stage2": (C.c_int, [C.POINTER(DecodeStage2Args), _vp]),

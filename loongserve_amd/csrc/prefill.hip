@@ -674,6 +674,8 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
 #pragma unroll
         for (int db = 0; db < 8; db++) *(f32x4*)(orow + db * 16 + 4 * g) = oacc[db][qb] * inv;
         if (g == 0) p.lse[tok * p.hq + h] = l_tot > 0.f ? (m_run[qb] + __builtin_amdgcn_logf(l_tot)) * kLn2 : -INFINITY;
+      } else if (MODE == 2) {
+        // handled after this loop: both row blocks at once, so that all reads of the old state are in flight together
       } else {
         float* mp = p.m + tok * p.ml_st + (int64_t)h * p.ml_sh;
         float* lp = p.l + tok * p.ml_st + (int64_t)h * p.ml_sh;
@@ -708,6 +710,55 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
           }
         }
       }
+    }
+  }
+  if (MODE == 2) {
+    // fold this step's partial into the running fp32 (O, LSE) of each row; a row that saw no key stays as it is.
+    // NB row blocks at a time: all reads of their old state are in flight together
+    auto fold = [&](auto nb_tag, int qb0) __attribute__((always_inline)) {
+      constexpr int NB = decltype(nb_tag)::value;
+      float l_tot[NB], a_old[NB];
+      f32x4 old[NB][8];
+      bool live[NB];
+#pragma unroll
+      for (int i = 0; i < NB; i++) {
+        const int qb = qb0 + i;
+        const int m = m_w0 + 16 * qb + qc;
+        l_tot[i] = column_sum(l_run[qb]);
+        live[i] = m < q_len && l_tot[i] > 0.f;
+        const int64_t tok = q_start + (m < q_len ? m : 0);
+        a_old[i] = p.lse[tok * p.hq + h] * kLog2e;
+        const float* orow = (const float*)p.o + tok * p.o_st + (int64_t)h * p.o_sh;
+#pragma unroll
+        for (int db = 0; db < 8; db++) old[i][db] = *(const f32x4*)(orow + db * 16 + 4 * g);
+      }
+#pragma unroll
+      for (int i = 0; i < NB; i++) {
+        if (!live[i]) continue;
+        const int qb = qb0 + i;
+        const int64_t tok = q_start + m_w0 + 16 * qb + qc;
+        const float a_new = m_run[qb] + __builtin_amdgcn_logf(l_tot[i]);
+        const float top = fmaxf(a_old[i], a_new);
+        const float w_old = exp2_diff(a_old[i], top);
+        const float w_new = __builtin_amdgcn_exp2f(a_new - top);
+        const float W = w_old + w_new;
+        const float c_old = w_old / W, c_new = w_new / (W * l_tot[i]);
+        float* orow = (float*)p.o + tok * p.o_st + (int64_t)h * p.o_sh;
+#pragma unroll
+        for (int db = 0; db < 8; db++) {
+          // an empty row (lse = -inf) may hold anything: its old values are dropped, not multiplied by zero
+          const f32x4 keep = w_old != 0.f ? old[i][db] : f32x4{0.f, 0.f, 0.f, 0.f};
+          *(f32x4*)(orow + db * 16 + 4 * g) = keep * c_old + oacc[db][qb] * c_new;
+        }
+        if (g == 0) p.lse[tok * p.hq + h] = (top + __builtin_amdgcn_logf(W)) * kLn2;  // the column's lanes read the old value above
+      }
+    };
+    if (DV) {
+      fold(std::integral_constant<int, 2>{}, 0);
+    } else {
+      // the variant that converts V in registers has none to spare: one block at a time
+      fold(std::integral_constant<int, 1>{}, 0);
+      fold(std::integral_constant<int, 1>{}, 1);
     }
   }
 }
@@ -769,7 +820,7 @@ static int validate(const lsattn_prefill_args* a, int mode) {
   // a lane addresses the 64 rows of a K/V tile with a 32-bit byte offset from the tile's first row
   if (a->k_stride_t <= 0 || a->v_stride_t <= 0 || a->k_stride_t > (1 << 24) || a->v_stride_t > (1 << 24)) return LSATTN_ERR_INVALID_ARG;
   if (((uintptr_t)a->q | (uintptr_t)a->k | (uintptr_t)a->v | (uintptr_t)a->o) & 15) return LSATTN_ERR_INVALID_ARG;
-  if (mode == 0) {
+  if (mode == 0 || mode == 2) {
     if (!a->lse || a->o_dtype != LSATTN_F32) return LSATTN_ERR_INVALID_ARG;
   } else {
     if (!a->m || !a->l || a->o_dtype != a->dtype) return LSATTN_ERR_INVALID_ARG;
@@ -795,4 +846,12 @@ extern "C" int lsattn_prefill_step_merge(const lsattn_prefill_args* a, void* str
   if (a->batch == 0 || a->max_q_len == 0) return LSATTN_OK;
   if (a->dtype == LSATTN_F16) return launch_prefill<F16, 1, true>(a, (hipStream_t)stream);
   return a->v_is_f16 ? launch_prefill<BF16, 1, true>(a, (hipStream_t)stream) : launch_prefill<BF16, 1, false>(a, (hipStream_t)stream);
+}
+
+extern "C" int lsattn_prefill_step_accumulate(const lsattn_prefill_args* a, void* stream) {
+  const int rc = validate(a, 2);
+  if (rc != LSATTN_OK) return rc;
+  if (a->batch == 0 || a->max_q_len == 0) return LSATTN_OK;
+  if (a->dtype == LSATTN_F16) return launch_prefill<F16, 2, true>(a, (hipStream_t)stream);
+  return a->v_is_f16 ? launch_prefill<BF16, 2, true>(a, (hipStream_t)stream) : launch_prefill<BF16, 2, false>(a, (hipStream_t)stream);
 }

@@ -169,11 +169,16 @@ def prefill_attention_step(q, k, v, q_b_start_loc, q_b_seq_len, q_first_token_gl
                            kv_b_start_loc, kv_b_seq_len, kv_first_token_global_idx,
                            logical_sp_peers_num: int, max_q_b_seq_len: int,
                            out: Optional[torch.Tensor] = None, lse: Optional[torch.Tensor] = None,
-                           sm_scale: Optional[float] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+                           sm_scale: Optional[float] = None, accumulate: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
     """One step as a mergeable partial: (O fp32 [Tq,Hq,D] normalised, LSE fp32 [Tq,Hq]).
 
     Same inputs as context_attention_fwd; rows that see no key get O = 0, LSE = -inf.
+    With accumulate=True the step is LSE-merged into the (out, lse) passed in (a running partial of earlier steps over
+    other keys; lse = -inf marks an empty row) in the kernel's epilogue, instead of being written from the empty state;
+    rows that see no key in this step keep what they hold.
     """
+    if accumulate and (out is None or lse is None):
+        raise ValueError("accumulate=True needs the running out and lse")
     D = q.shape[-1]
     if out is None:
         out = torch.empty(q.shape, dtype=torch.float32, device=q.device)
@@ -183,14 +188,18 @@ def prefill_attention_step(q, k, v, q_b_start_loc, q_b_seq_len, q_first_token_gl
         raise ValueError("out and lse must be float32, lse contiguous")
     out_user = None
     if q.dim() == 3 and D in (16, 32, 64) and k.shape[-1] == D and v.shape[-1] == D and out.shape == q.shape:
-        out_user, out = out, torch.empty(q.shape[:2] + (KERNEL_HEAD_DIM,), dtype=torch.float32, device=q.device)
+        out_user, out = out, (_pad_head_dim(out) if accumulate else
+                              torch.empty(q.shape[:2] + (KERNEL_HEAD_DIM,), dtype=torch.float32, device=q.device))
         q, k, v = _pad_head_dim(q), _pad_head_dim(k), _pad_head_dim(v)
         if sm_scale is None:
             sm_scale = 1.0 / (D ** 0.5)
     a = _prefill_args(q, k, v, out, q_b_start_loc, q_b_seq_len, q_first_token_global_idx, kv_b_start_loc,
                       kv_b_seq_len, kv_first_token_global_idx, logical_sp_peers_num, max_q_b_seq_len, sm_scale)
     a.lse = lse.data_ptr()
-    _lib.check(_lib.load().lsattn_prefill_step(C.byref(a), _stream()), "lsattn_prefill_step")
+    if accumulate:
+        _lib.check(_lib.load().lsattn_prefill_step_accumulate(C.byref(a), _stream()), "lsattn_prefill_step_accumulate")
+    else:
+        _lib.check(_lib.load().lsattn_prefill_step(C.byref(a), _stream()), "lsattn_prefill_step")
     if out_user is not None:
         out_user.copy_(out[..., :D])
         out = out_user

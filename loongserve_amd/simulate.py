@@ -71,6 +71,18 @@ def ring_prefill_partials(q, chunks: Sequence[KVChunk], q_b_start_loc, q_b_seq_l
     return lse_merge(parts, out, lse)
 
 
+def ring_prefill_accumulate(q, chunks: Sequence[KVChunk], q_b_start_loc, q_b_seq_len, q_first_token_global_idx,
+                            logical_sp_peers_num: int, max_q_len: int, num_kv_heads: int,
+                            out: Optional[torch.Tensor] = None, lse: Optional[torch.Tensor] = None):
+    """The first step writes the fp32 partial (O, LSE); every later step LSE-merges its partial into it in the
+    kernel's epilogue: no per-step buffers and no separate merge pass.  Returns (O, LSE)."""
+    for i, c in enumerate(chunks):
+        out, lse = prefill_attention_step(q, c.k(num_kv_heads), c.v(num_kv_heads), q_b_start_loc, q_b_seq_len,
+                                          q_first_token_global_idx, c.b_start_loc, c.b_seq_len, c.first_token_global_idx,
+                                          logical_sp_peers_num, max_q_len, out, lse, accumulate=i > 0)
+    return out, lse
+
+
 def next_power_of_2(n: int) -> int:
     return 1 if n <= 1 else 1 << (n - 1).bit_length()
 

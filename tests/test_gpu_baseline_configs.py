@@ -44,6 +44,12 @@ def test_config2_ring_prefill_full_size(lsa):
     o_ref, lse_ref = orc.lse_merge(parts)
     assert_o_close(w.out[rows][:, heads], o_ref, "cfg2 O (sampled rows)")
     assert_lse_close(w.lse[rows][:, heads], lse_ref, "cfg2 LSE (sampled rows)")
+    # the route with four separate partials and one merge pass agrees with the merge in the epilogues everywhere
+    o_acc, lse_acc = w.out.clone(), w.lse.clone()
+    w.step_separate_merge()
+    torch.cuda.synchronize()
+    assert (o_acc - w.out).abs().max().item() <= 1e-6 and torch.allclose(lse_acc, w.lse, rtol=0, atol=1e-5)
+    w.bufs = None
     # property: the in-place (o, m, l) ring state equals the merged fp32 partials everywhere
     o, m, l = ring_prefill(w.q, w.chunks, w.qs, w.ql, w.qf, 1, n, w.Hkv)
     torch.cuda.synchronize()

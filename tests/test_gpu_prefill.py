@@ -202,6 +202,20 @@ def test_bf16_v_converted_inside_the_kernel_or_before_it(lsa):
             o, lse = lsa.prefill_attention_step(q.to(DEV), kvd[:, :Hkv], kvd[:, Hkv:], qs, ql, qf, qs, ql, qf, 1, max(lens))
             assert_o_close(o, o_ref, "O (pre-converted V: %s)" % pre)
             assert_lse_close(lse, lse_ref, "LSE (pre-converted V: %s)" % pre)
+            # the same in two steps, the second folded into the first in the epilogue: keys [0, 400) of each request,
+            # then the rest (rows before position 400 see nothing of the second chunk and must keep their values)
+            cut = 400
+            idx = torch.cat([torch.arange(int(s0), int(s0) + n) for s0, n in zip(m[0], lens)])
+            first = torch.cat([torch.arange(int(s0), int(s0) + cut) for s0 in m[0]])
+            rest = torch.cat([torch.arange(int(s0) + cut, int(s0) + n) for s0, n in zip(m[0], lens)])
+            assert len(first) + len(rest) == len(idx)
+            out = lse = None
+            for rows, km in ((first, meta([cut] * len(lens))), (rest, meta([n - cut for n in lens], [cut] * len(lens)))):
+                part = kvd[rows.to(DEV)]
+                out, lse = lsa.prefill_attention_step(q.to(DEV), part[:, :Hkv], part[:, Hkv:], qs, ql, qf, *_dev(*km), 1,
+                                                      max(lens), out, lse, accumulate=out is not None)
+            assert_o_close(out, o_ref, "accumulated O (pre-converted V: %s)" % pre)
+            assert_lse_close(lse, lse_ref, "accumulated LSE (pre-converted V: %s)" % pre)
     finally:
         ops.PRECONVERT_BF16_V = True
 
@@ -257,3 +271,60 @@ def test_head_sizes_below_128(lsa, D):
     torch.cuda.synchronize()
     assert_o_close(od, oc.float(), "in-place o")
     assert_lse_close(orc.state_lse(md.cpu(), ld.cpu()).float(), orc.state_lse(mc, lc).float(), "state")
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_ring_accumulated_in_the_epilogue_matches_monolithic(lsa, dtype):
+    """Steps folded into a running fp32 (O, LSE) by the kernel's epilogue: same bars as the separate merge, from a
+    chunk order in which early steps leave some rows without any key (they must stay empty until a later step fills
+    them), and the same again for a striped ring."""
+    from loongserve_amd.simulate import KVChunk, ring_prefill_accumulate
+    g = torch.Generator().manual_seed(1)
+    lens = [int(x) for x in torch.randint(200, 1500, (3,), generator=g)]
+    T, Hq, Hkv, D = sum(lens), 8, 2, 128
+    q, k, v = rand_t((T, Hq, D), 91, dtype), rand_t((T, Hkv, D), 92, dtype), rand_t((T, Hkv, D), 93, dtype)
+    m = meta(lens)
+    o_ref, lse_ref = orc.attn_step(q, k, v, *m, *m, 1)
+    qs, ql, qf = _dev(*m)
+    for nshard, order in ((4, [3, 1, 0, 2]), (2, [1, 0]), (1, [0])):
+        print("case", dtype, nshard, flush=True)
+        _, chunks = _ring_chunks(k, v, lens, nshard, 6, Hkv)
+        # the running partial starts as garbage: the first step writes every row
+        out = torch.full((T, Hq, D), float("nan"), device=DEV)
+        lse = torch.full((T, Hq), float("nan"), device=DEV)
+        o, l = ring_prefill_accumulate(q.to(DEV), [chunks[i] for i in order], qs, ql, qf, 1, max(lens), Hkv, out, lse)
+        torch.cuda.synchronize()
+        assert o.data_ptr() == out.data_ptr() and l.data_ptr() == lse.data_ptr()
+        assert_o_close(o, o_ref, "accumulated O")
+        assert_lse_close(l, lse_ref, "accumulated LSE")
+    # from the empty state (lse = -inf, o anything) every step may accumulate
+    _, chunks = _ring_chunks(k, v, lens, 3, 7, Hkv)
+    out = torch.full((T, Hq, D), float("nan"), device=DEV)
+    lse = torch.full((T, Hq), float("-inf"), device=DEV)
+    for c in (chunks[2], chunks[0], chunks[1]):
+        lsa.prefill_attention_step(q.to(DEV), c.k(Hkv), c.v(Hkv), qs, ql, qf, c.b_start_loc, c.b_seq_len,
+                                   c.first_token_global_idx, 1, max(lens), out, lse, accumulate=True)
+    torch.cuda.synchronize()
+    assert_o_close(out, o_ref, "accumulated from empty O")
+    assert_lse_close(lse, lse_ref, "accumulated from empty LSE")
+    with pytest.raises(ValueError):
+        lsa.prefill_attention_step(q.to(DEV), c.k(Hkv), c.v(Hkv), qs, ql, qf, c.b_start_loc, c.b_seq_len,
+                                   c.first_token_global_idx, 1, max(lens), accumulate=True)
+    # striped ring, P = 3: rank r holds tokens r, r + P, ...
+    P, T1 = 3, 1000
+    q1, k1, v1 = q[:T1], k[:T1], v[:T1]
+    m1 = meta([T1])
+    o1_ref, lse1_ref = orc.attn_step(q1, k1, v1, *m1, *m1, 1)
+    chunks = []
+    for j in range(P):
+        kj = torch.cat([k1[j::P], v1[j::P]], 1)
+        st, ln, fr = meta([kj.shape[0]], [j])
+        chunks.append(KVChunk(kj.to(DEV), st.to(DEV), ln.to(DEV), fr.to(DEV)))
+    for r in range(P):
+        qi = q1[r::P].contiguous()
+        qs1, ql1, qf1 = _dev(*meta([qi.shape[0]], [r]))
+        order = [(r - i) % P for i in range(P)]
+        o, l = ring_prefill_accumulate(qi.to(DEV), [chunks[i] for i in order], qs1, ql1, qf1, P, qi.shape[0], Hkv)
+        torch.cuda.synchronize()
+        assert_o_close(o, o1_ref[r::P], "striped accumulated O rank %d" % r)
+        assert_lse_close(l, lse1_ref[r::P], "striped accumulated LSE rank %d" % r)
