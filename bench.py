@@ -75,6 +75,7 @@ class RingPrefill:
             kv = _randn_half((shard, 2 * kv_heads, D), seed + 1 + j, dtype)
             self.chunks.append(KVChunk(kv, _i32([0]), _i32([shard]), _i32([j * shard])))
         self.bufs = None  # per-step partial buffers, only for the separate-merge route
+        self.state = None  # (o, m, l) of the in-place route
         self.out = torch.empty((shard, heads, D), dtype=torch.float32, device=DEV)
         self.lse = torch.empty((shard, heads), dtype=torch.float32, device=DEV)
         n = shard
@@ -87,6 +88,14 @@ class RingPrefill:
         LSE-merges its own partial into it in its epilogue."""
         from loongserve_amd.simulate import ring_prefill_accumulate
         ring_prefill_accumulate(self.q, self.chunks, self.qs, self.ql, self.qf, 1, self.shard, self.Hkv, self.out, self.lse)
+
+    def step_in_place(self):
+        """The same four steps through context_attention_fwd, the reference's operator: (o fp16, m, l) updated in place."""
+        from loongserve_amd.simulate import ring_prefill
+        if self.state is None:
+            self.state = (torch.empty_like(self.q), torch.empty((self.shard, self.H), dtype=torch.float32, device=DEV),
+                          torch.empty((self.shard, self.H), dtype=torch.float32, device=DEV))
+        ring_prefill(self.q, self.chunks, self.qs, self.ql, self.qf, 1, self.shard, self.Hkv, *self.state)
 
     def step_separate_merge(self):
         """The same four steps as four separate fp32 partials and one lsattn_lse_merge pass over them."""
@@ -476,6 +485,7 @@ def main():
         per_launch_ms = st["mean_ms"] / w.launches
         ach = (w.flops / w.launches) / (per_launch_ms * 1e-3) / 1e12
         sep = _stats(_time_events(w.step_separate_merge, max(5, args.steps // 2), 2))
+        inp = _stats(_time_events(w.step_in_place, max(5, args.steps // 2), 2))
         line.update({
             "value": tflops, "unit": "TFLOP/s", "ms_per_step": wall_ms,
             "pct_of_mfma_peak": 100.0 * tflops / PEAK_MFMA_TFLOPS,
@@ -485,7 +495,9 @@ def main():
                        "algorithmic_tflop_per_step": w.flops / 1e12, "launches_per_step": w.launches, "step_stats": st,
                        "separate_merge": {"what": "the same steps as four separate fp32 partials + one lsattn_lse_merge pass",
                                           "ms_per_step": sep["mean_ms"], "value": w.flops / (sep["mean_ms"] * 1e-3) / 1e12,
-                                          "launches_per_step": w.launches + 1}},
+                                          "launches_per_step": w.launches + 1},
+                       "in_place": {"what": "the same steps through context_attention_fwd: (o fp16, m, l) reset and updated in place",
+                                    "ms_per_step": inp["mean_ms"], "value": w.flops / (inp["mean_ms"] * 1e-3) / 1e12}},
             "roofline": {"kernel": "prefill_kernel<F16,0,true> (diagonal launch) + prefill_kernel<F16,2,true> (three full launches)",
                          "bound": "mfma", "achieved": ach, "peak": PEAK_MFMA_TFLOPS, "unit": "TFLOP/s",
                          "frac": ach / PEAK_MFMA_TFLOPS,
