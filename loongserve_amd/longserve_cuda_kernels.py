@@ -37,8 +37,9 @@ def flash_decoding_stage1(mid_o, mid_o_logexpsum, q, k, v, req_to_tokens, b_req_
     # ENTRY:124-131
     for t, d, n in ((mid_o, 4, "mid_o"), (mid_o_logexpsum, 3, "mid_o_logexpsum"), (q, 3, "q"), (k, 3, "k"), (v, 3, "v"),
                     (req_to_tokens, 2, "req_to_tokens"), (b_req_idx, 1, "b_req_idx"), (b_seqlen, 1, "b_seqlen")):
-        _req(t.dim() == d, "%s.dim() == %d" % (n, d))
-        _req(t.is_cuda, "%s on the GPU" % n)
+        if t.dim() != d or not t.is_cuda:  # (the message is only built on failure: this runs once per decode step)
+            _req(t.dim() == d, "%s.dim() == %d" % (n, d))
+            _req(t.is_cuda, "%s on the GPU" % n)
     # ENTRY:133-140 (bfloat16 accepted in addition to half)
     _req(mid_o.dtype == torch.float32, "mid_o float32")
     _req(mid_o_logexpsum.dtype == torch.float32, "mid_o_logexpsum float32")
@@ -73,9 +74,10 @@ def flash_decoding_stage2(o, out_logexpsum, b_seqlen, mid_o, mid_o_logexpsum, bl
     # ENTRY:174-190
     for t, d, n in ((o, 3, "o"), (out_logexpsum, 2, "out_logexpsum"), (b_seqlen, 1, "b_seqlen"), (mid_o, 4, "mid_o"),
                     (mid_o_logexpsum, 3, "mid_o_logexpsum")):
-        _req(t.is_contiguous(), "%s.is_contiguous()" % n)
-        _req(t.dim() == d, "%s.dim() == %d" % (n, d))
-        _req(t.is_cuda, "%s on the GPU" % n)
+        if not t.is_contiguous() or t.dim() != d or not t.is_cuda:
+            _req(t.is_contiguous(), "%s.is_contiguous()" % n)
+            _req(t.dim() == d, "%s.dim() == %d" % (n, d))
+            _req(t.is_cuda, "%s on the GPU" % n)
     _req(o.dtype in (torch.float16, torch.float32, torch.bfloat16), "o half, bfloat16 or float")
     _req(out_logexpsum.dtype == torch.float32, "out_logexpsum float32")
     _req(b_seqlen.dtype == torch.int32, "b_seqlen int32")

@@ -24,7 +24,15 @@ from ._lib import LSATTN_BF16, LSATTN_F16, LSATTN_F32
 _DT = {torch.float16: LSATTN_F16, torch.bfloat16: LSATTN_BF16, torch.float32: LSATTN_F32}
 
 
+# torch.cuda.current_stream() builds a Stream object through several Python layers (about 8 us a call, more than a small
+# decode kernel runs); the raw handle of the same stream comes from one C call where this torch has it
+_raw_current_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream() -> int:
+    """Handle of the current PyTorch stream of the current device: the launches go there."""
+    if _raw_current_stream is not None:
+        return _raw_current_stream(torch.cuda.current_device())
     return torch.cuda.current_stream().cuda_stream
 
 
