@@ -326,10 +326,11 @@ template <> __device__ __forceinline__ void store4<BF16>(void* base, int64_t ele
   *(u32x2*)((uint16_t*)base + elem) = u32x2{pack2<BF16>(v[0], v[1]), pack2<BF16>(v[2], v[3])};
 }
 
-template <typename OT, int D>
-__global__ __launch_bounds__(256) void decode_stage2_kernel(Stage2Params p) {
+template <typename OT, int D, int NT>
+__global__ __launch_bounds__(NT) void decode_stage2_kernel(Stage2Params p) {
   constexpr int LPR = D / 4;      // lanes per row (float4 each)
-  constexpr int SL = 256 / LPR;   // slices walking the block axis
+  constexpr int SL = NT / LPR;    // slices walking the block axis
+  constexpr int U = 4;            // rows a slice has in flight
   const int64_t b = blockIdx.x, h = blockIdx.y;
   const int slice = threadIdx.x / LPR, c = threadIdx.x % LPR;
   const int64_t len = p.b_seqlen[b];
@@ -340,17 +341,31 @@ __global__ __launch_bounds__(256) void decode_stage2_kernel(Stage2Params p) {
 
   float M = -INFINITY, L = 0.f;
   f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-  for (int64_t i = slice; i < n; i += SL) {
-    const int64_t row = i * row_stride + row0;
-    const float lse = p.mid_lse[row];
-    const f32x4 tv = *(const f32x4*)(p.mid_o + row * D + c * 4);
-    if (lse == -INFINITY) continue;  // an empty partial contributes nothing
+  auto fold = [&](float lse, const f32x4& tv) {
+    if (lse == -INFINITY) return;  // an empty partial contributes nothing
     const float Mn = fmaxf(M, lse);
     const float so = exp2_diff(M * kLog2e, Mn * kLog2e);
     const float sn = __builtin_amdgcn_exp2f((lse - Mn) * kLog2e);
     acc = acc * so + tv * sn;
     L = L * so + sn;
     M = Mn;
+  };
+  int64_t i = slice;
+  for (; i + (U - 1) * SL < n; i += U * SL) {
+    float lse[U];
+    f32x4 tv[U];
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+      const int64_t row = (i + u * SL) * row_stride + row0;
+      lse[u] = p.mid_lse[row];
+      tv[u] = *(const f32x4*)(p.mid_o + row * D + c * 4);
+    }
+#pragma unroll
+    for (int u = 0; u < U; u++) fold(lse[u], tv[u]);
+  }
+  for (; i < n; i += SL) {
+    const int64_t row = i * row_stride + row0;
+    fold(p.mid_lse[row], *(const f32x4*)(p.mid_o + row * D + c * 4));
   }
   __shared__ float sM[SL], sL[SL];
   __shared__ f32x4 sAcc[SL][LPR];
@@ -460,10 +475,16 @@ extern "C" int lsattn_decode_stage1(const lsattn_decode_stage1_args* a, void* st
 }
 
 template <typename OT> static int dispatch_stage2(const Stage2Params& p, int64_t D, dim3 grid, hipStream_t st) {
+  // few (batch, head) pairs with many partials each (long contexts at small batch): 1024 threads walk the block axis in 32
+  // slices instead of 8, or the merge takes a fifth of the time of the gather it follows
+  const bool wide = D == 128 && p.num_seq_blocks >= 64 && (int64_t)grid.x * grid.y < 2048;
   switch (D) {
-    case 32: hipLaunchKernelGGL((decode_stage2_kernel<OT, 32>), grid, dim3(256), 0, st, p); break;
-    case 64: hipLaunchKernelGGL((decode_stage2_kernel<OT, 64>), grid, dim3(256), 0, st, p); break;
-    case 128: hipLaunchKernelGGL((decode_stage2_kernel<OT, 128>), grid, dim3(256), 0, st, p); break;
+    case 32: hipLaunchKernelGGL((decode_stage2_kernel<OT, 32, 256>), grid, dim3(256), 0, st, p); break;
+    case 64: hipLaunchKernelGGL((decode_stage2_kernel<OT, 64, 256>), grid, dim3(256), 0, st, p); break;
+    case 128:
+      if (wide) hipLaunchKernelGGL((decode_stage2_kernel<OT, 128, 1024>), grid, dim3(1024), 0, st, p);
+      else hipLaunchKernelGGL((decode_stage2_kernel<OT, 128, 256>), grid, dim3(256), 0, st, p);
+      break;
     default: return LSATTN_ERR_UNSUPPORTED;
   }
   return check_launch();

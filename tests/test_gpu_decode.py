@@ -113,3 +113,34 @@ def test_stage2_empty_request_defined(lsa):
     o_ref, l_ref = orc.lse_merge([(mo[i, 1].cpu(), ml[i, 1].cpu()) for i in range(3)])
     assert_o_close(o[1], o_ref, "o", max_abs=1e-5, rel=1e-5)
     assert_lse_close(l[1], l_ref, "lse", rel=1e-5)
+
+
+@pytest.mark.parametrize("nblk", [1, 7, 31, 64, 65, 300, 1029])
+def test_stage2_alone_over_few_and_many_partials(lsa, nblk):
+    """The merge on its own, on random partials: every count of blocks around the points where the kernel changes its
+    walk (rows in flight per slice, the wide launch for many partials of few rows), empty partials in between, requests
+    that use fewer blocks than the buffer has, fp32 and fp16 outputs."""
+    print("case nblk", nblk, flush=True)
+    B, H, D, BS = 3, 5, 128, 16
+    g = torch.Generator().manual_seed(nblk)
+    mo = torch.randn(nblk, B, H, D, generator=g)
+    ml = torch.randn(nblk, B, H, generator=g) * 6
+    ml[torch.rand(nblk, B, H, generator=g) < 0.15] = float("-inf")
+    lens = torch.tensor([nblk * BS, max(1, (nblk * BS) // 3 + 1), 0], dtype=torch.int32)
+    o_ref = torch.empty(B, H, D)
+    l_ref = torch.empty(B, H)
+    orc.decode_stage2(mo, ml, lens, o_ref, l_ref, BS)
+    for odt in (torch.float32, torch.float16):
+        o = torch.full((B, H, D), 9.0, dtype=odt, device=DEV)
+        l = torch.full((B, H), 9.0, device=DEV)
+        lsa.longserve_flash_decode_stage2(mo.to(DEV), ml.to(DEV), lens.to(DEV), o, l, BS)
+        torch.cuda.synchronize()
+        # a (b, h) whose partials are all empty merges to (0, -inf), like a request without tokens
+        dead = torch.isinf(l_ref) & (l_ref < 0)
+        assert torch.equal(torch.isinf(l.cpu()) & (l.cpu() < 0), dead)
+        assert torch.all(o.cpu()[dead] == 0)
+        if odt == torch.float32:
+            assert_o_close(o, torch.where(dead[..., None], torch.zeros(()), o_ref), "o", max_abs=2e-5, rel=1e-5)
+        else:
+            assert_o_close(o, torch.where(dead[..., None], torch.zeros(()), o_ref), "o fp16", max_abs=4e-3, rel=1e-3)
+        assert_lse_close(l, l_ref, "lse", rel=1e-5)
