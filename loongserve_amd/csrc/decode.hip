@@ -64,7 +64,10 @@ template <> struct Dot<BF16> {
   static __device__ __forceinline__ void next(float& d, uint32_t a, uint32_t b) { asm volatile("v_dot2c_f32_bf16 %0, %1, %2" : "+v"(d) : "v"(a), "v"(b)); }
 };
 
-template <typename T, int GT, int NW>
+// SPLIT: the NW waves of a workgroup share one task and take every NW-th batch of 32 tokens of a block; their partials
+// meet in LDS.  For launches too small to fill the chip otherwise (short contexts at small batch): NW times as many rows
+// in flight.
+template <typename T, int GT, int NW, bool SPLIT>
 __global__ __launch_bounds__(NW * 64) void decode_stage1_kernel(Stage1Params p) {
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -75,8 +78,8 @@ __global__ __launch_bounds__(NW * 64) void decode_stage1_kernel(Stage1Params p) 
   // The workgroups that read the other KV heads of the same tokens are next to this one in dispatch order when the
   // task index is the fastest grid dimension: the pieces of a token's K (and V) span are then fetched close together in
   // time (measured 2 % faster on GQA 32/8, two task groups per chunk).
-  const int task = (p.tasks_on_x ? blockIdx.x : blockIdx.y) * NW + wave;
-  if (task >= p.tasks) return;
+  const int task = SPLIT ? (int)(p.tasks_on_x ? blockIdx.x : blockIdx.y) : (int)(p.tasks_on_x ? blockIdx.x : blockIdx.y) * NW + wave;
+  if (task >= p.tasks) return;  // (SPLIT: the same for every wave of the workgroup, like the block range below)
   const int group = (int)(p.hq / p.hkv);
   const int sub_groups = group / GT;
   const int kvh = task / sub_groups;
@@ -119,14 +122,16 @@ __global__ __launch_bounds__(NW * 64) void decode_stage1_kernel(Stage1Params p) 
     // Slot indices of the first batch of rows.  A row position past the block repeats the block's
     // last row (always a real slot): it is loaded like any other and dropped by the validity mask,
     // so the loop body has no divergent control flow.
+    constexpr int kStep = 4 * kTok * (SPLIT ? NW : 1);
+    const int it0 = t0 + (SPLIT ? wave * 4 * kTok : 0);
     int32_t slot[kTok];
 #pragma unroll
     for (int j = 0; j < kTok; j++) {
-      const int tok = t0 + j * 4 + grp;
+      const int tok = it0 + j * 4 + grp;
       slot[j] = table[tok < t1 ? tok : t_last];
     }
 
-    for (int it = t0; it < t1; it += 4 * kTok) {
+    for (int it = it0; it < t1; it += kStep) {
       u32x4 kr[kTok], vr[kTok];
       // (the empty statements keep each 64-bit address next to its load instead of sixteen of them live at once)
 #pragma unroll
@@ -147,7 +152,7 @@ __global__ __launch_bounds__(NW * 64) void decode_stage1_kernel(Stage1Params p) 
       // slot indices of the next batch while the rows are in flight
 #pragma unroll
       for (int j = 0; j < kTok; j++) {
-        const int tok = it + 4 * kTok + j * 4 + grp;
+        const int tok = it + kStep + j * 4 + grp;
         slot[j] = table[tok < t1 ? tok : t_last];
       }
       __builtin_amdgcn_sched_barrier(0);
@@ -273,12 +278,21 @@ __global__ __launch_bounds__(NW * 64) void decode_stage1_kernel(Stage1Params p) 
       }
     }
 
-    // merge the four lane groups and write the block's partial
+    // merge the four lane groups (and, SPLIT, the waves) and write the block's partial
+    __shared__ float xw[SPLIT ? NW : 1][GT][16][10];  // per wave, head and column slot: 8 sums, running max, row sum
+    auto write_partial = [&](int h, float M, float L, const float (&ov)[8]) {
+      const float inv = 1.f / L;
+      const int64_t row = (blk * p.batch + b) * p.hq + qh0 + h;
+      f32x4* dst = (f32x4*)(p.mid_o + row * 128 + sub * 8);
+      dst[0] = f32x4{ov[0] * inv, ov[1] * inv, ov[2] * inv, ov[3] * inv};
+      dst[1] = f32x4{ov[4] * inv, ov[5] * inv, ov[6] * inv, ov[7] * inv};
+      if (sub == 0) p.mid_lse[row] = (M + __builtin_amdgcn_logf(L)) * kLn2;
+    };
 #pragma unroll
     for (int h = 0; h < GT; h++) {
       float M = fmaxf(m[h], __shfl_xor(m[h], 16));
       M = fmaxf(M, __shfl_xor(M, 32));
-      const float w = exp2_diff(m[h], M);  // the block holds >= 1 row, so M is finite
+      const float w = exp2_diff(m[h], M);  // 0 for a group (or, SPLIT, a whole wave) that saw no row
       float L = l[h] * w;
       L += __shfl_xor(L, 16);
       L += __shfl_xor(L, 32);
@@ -291,13 +305,38 @@ __global__ __launch_bounds__(NW * 64) void decode_stage1_kernel(Stage1Params p) 
         ov[i] = x;
       }
       if (grp == 0) {
-        const float inv = 1.f / L;
-        const int64_t row = (blk * p.batch + b) * p.hq + qh0 + h;
-        f32x4* dst = (f32x4*)(p.mid_o + row * 128 + sub * 8);
-        dst[0] = f32x4{ov[0] * inv, ov[1] * inv, ov[2] * inv, ov[3] * inv};
-        dst[1] = f32x4{ov[4] * inv, ov[5] * inv, ov[6] * inv, ov[7] * inv};
-        if (sub == 0) p.mid_lse[row] = (M + __builtin_amdgcn_logf(L)) * kLn2;
+        if (SPLIT) {
+          float* dst = xw[wave][h][sub];
+#pragma unroll
+          for (int i = 0; i < 8; i++) dst[i] = ov[i];
+          dst[8] = M;
+          dst[9] = L;
+        } else {
+          write_partial(h, M, L, ov);  // the block holds >= 1 row, so M is finite and L > 0
+        }
       }
+    }
+    if (SPLIT) {
+      __syncthreads();
+      if (wave == 0 && grp == 0) {
+#pragma unroll
+        for (int h = 0; h < GT; h++) {
+          float M = xw[0][h][sub][8];
+#pragma unroll
+          for (int w = 1; w < NW; w++) M = fmaxf(M, xw[w][h][sub][8]);
+          float L = 0.f, ov[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int w = 0; w < NW; w++) {
+            const float* src = xw[w][h][sub];
+            const float f = exp2_diff(src[8], M);
+            L += src[9] * f;
+#pragma unroll
+            for (int i = 0; i < 8; i++) ov[i] += src[i] * f;
+          }
+          write_partial(h, M, L, ov);
+        }
+      }
+      __syncthreads();  // the next block of this workgroup writes the same LDS
     }
   }
 }
@@ -434,10 +473,21 @@ static int launch_stage1(const lsattn_decode_stage1_args* a, hipStream_t st) {
   p.blocks_per_wg = (int32_t)per_wg;
   const int64_t chunks = (nblk + per_wg - 1) / per_wg;
   if (chunks > 0x7fffffff || a->batch > 65535 || wgs_y > 65535) return LSATTN_ERR_INVALID_ARG;
+  // A launch of less than one workgroup per CU leaves most of the chip's load slots empty: the waves of a workgroup then
+  // share one task and split each block's tokens (measured: 64 workgroups, one request of 8192 tokens with 8 KV heads,
+  // 19.9 -> 10.0 us; from 256 workgroups on it gains nothing; blocks shorter than 32 tokens per wave cannot use it).
+  const bool split = chunks * wgs_y * a->batch < 256 && a->seq_block_size >= 32 * NW && p.tasks <= 65535;
+  if (split) {
+    p.tasks_on_x = chunks <= 65535;
+    dim3 grid = p.tasks_on_x ? dim3((unsigned)p.tasks, (unsigned)chunks, (unsigned)a->batch)
+                             : dim3((unsigned)chunks, (unsigned)p.tasks, (unsigned)a->batch);
+    hipLaunchKernelGGL((decode_stage1_kernel<T, GT, NW, true>), grid, dim3(NW * 64), 0, st, p);
+    return check_launch();
+  }
   p.tasks_on_x = wgs_y <= 2 && chunks <= 65535;  // with more task groups per chunk (MHA, 32 KV heads) it measured 2 % slower
   dim3 grid = p.tasks_on_x ? dim3((unsigned)wgs_y, (unsigned)chunks, (unsigned)a->batch)
                            : dim3((unsigned)chunks, (unsigned)wgs_y, (unsigned)a->batch);
-  hipLaunchKernelGGL((decode_stage1_kernel<T, GT, NW>), grid, dim3(NW * 64), 0, st, p);
+  hipLaunchKernelGGL((decode_stage1_kernel<T, GT, NW, false>), grid, dim3(NW * 64), 0, st, p);
   return check_launch();
 }
 
