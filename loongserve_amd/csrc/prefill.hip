@@ -662,54 +662,78 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
   }
 
   // ---- epilogue ----
+  if (MODE == 0) {
+    // the step's partial from the empty state
 #pragma unroll
-  for (int qb = 0; qb < 2; qb++) {
-    const int m = m_w0 + 16 * qb + qc;
-    const float l_tot = column_sum(l_run[qb]);
-    if (m < q_len) {
-      const int64_t tok = q_start + m;
-      if (MODE == 0) {
+    for (int qb = 0; qb < 2; qb++) {
+      const int m = m_w0 + 16 * qb + qc;
+      const float l_tot = column_sum(l_run[qb]);
+      if (m < q_len) {
+        const int64_t tok = q_start + m;
         const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
         float* orow = (float*)p.o + tok * p.o_st + (int64_t)h * p.o_sh;
 #pragma unroll
         for (int db = 0; db < 8; db++) *(f32x4*)(orow + db * 16 + 4 * g) = oacc[db][qb] * inv;
         if (g == 0) p.lse[tok * p.hq + h] = l_tot > 0.f ? (m_run[qb] + __builtin_amdgcn_logf(l_tot)) * kLn2 : -INFINITY;
-      } else if (MODE == 2) {
-        // handled after this loop: both row blocks at once, so that all reads of the old state are in flight together
-      } else {
-        float* mp = p.m + tok * p.ml_st + (int64_t)h * p.ml_sh;
-        float* lp = p.l + tok * p.ml_st + (int64_t)h * p.ml_sh;
-        const float m_old = *mp, l_old = *lp;
-        const float M = fmaxf(m_run[qb], m_old);
-        if (M != -INFINITY && l_tot > 0.f) {
-          const float w_old = l_old * exp2_diff(m_old, M);
-          const float w_new = exp2_diff(m_run[qb], M);
-          const float L = w_old + l_tot * w_new;
-          const float inv = 1.f / L;
-          uint16_t* orow = (uint16_t*)p.o + tok * p.o_st + (int64_t)h * p.o_sh;
+      }
+    }
+  }
+  if (MODE == 1) {
+    // the reference's update of (o, m, l) (RING:171-188).  NB row blocks at a time: all reads of their old state are in
+    // flight together
+    auto fold_state = [&](auto nb_tag, int qb0) __attribute__((always_inline)) {
+      constexpr int NB = decltype(nb_tag)::value;
+      float l_tot[NB], m_old[NB], l_old[NB];
+      u32x2 old[NB][8];
+      bool in_range[NB];
 #pragma unroll
-          for (int db = 0; db < 8; db++) {
-            u32x2* dst = (u32x2*)(orow + db * 16 + 4 * g);
-            float o0, o1, o2, o3;
-            if (w_old != 0.f) {
-              const u32x2 old = *dst;
-              unpack2<T>(old[0], o0, o1);
-              unpack2<T>(old[1], o2, o3);
-            } else {
-              o0 = o1 = o2 = o3 = 0.f;
-            }
-            const float r0 = (o0 * w_old + oacc[db][qb][0] * w_new) * inv;
-            const float r1 = (o1 * w_old + oacc[db][qb][1] * w_new) * inv;
-            const float r2 = (o2 * w_old + oacc[db][qb][2] * w_new) * inv;
-            const float r3 = (o3 * w_old + oacc[db][qb][3] * w_new) * inv;
-            *dst = u32x2{pack2<T>(r0, r1), pack2<T>(r2, r3)};
+      for (int i = 0; i < NB; i++) {
+        const int qb = qb0 + i;
+        const int m = m_w0 + 16 * qb + qc;
+        l_tot[i] = column_sum(l_run[qb]);
+        in_range[i] = m < q_len;
+        const int64_t tok = q_start + (in_range[i] ? m : 0);
+        m_old[i] = p.m[tok * p.ml_st + (int64_t)h * p.ml_sh];
+        l_old[i] = p.l[tok * p.ml_st + (int64_t)h * p.ml_sh];
+        const uint16_t* orow = (const uint16_t*)p.o + tok * p.o_st + (int64_t)h * p.o_sh;
+#pragma unroll
+        for (int db = 0; db < 8; db++) old[i][db] = *(const u32x2*)(orow + db * 16 + 4 * g);
+      }
+#pragma unroll
+      for (int i = 0; i < NB; i++) {
+        const int qb = qb0 + i;
+        const float M = fmaxf(m_run[qb], m_old[i]);
+        if (!in_range[i] || M == -INFINITY || !(l_tot[i] > 0.f)) continue;
+        const int64_t tok = q_start + m_w0 + 16 * qb + qc;
+        const float w_old = l_old[i] * exp2_diff(m_old[i], M);
+        const float w_new = exp2_diff(m_run[qb], M);
+        const float L = w_old + l_tot[i] * w_new;
+        const float inv = 1.f / L;
+        uint16_t* orow = (uint16_t*)p.o + tok * p.o_st + (int64_t)h * p.o_sh;
+#pragma unroll
+        for (int db = 0; db < 8; db++) {
+          float o0 = 0.f, o1 = 0.f, o2 = 0.f, o3 = 0.f;
+          if (w_old != 0.f) {  // a row in its start state (m = -inf, l = 0) may hold anything in o
+            unpack2<T>(old[i][db][0], o0, o1);
+            unpack2<T>(old[i][db][1], o2, o3);
           }
-          if (g == 0) {  // M and L depend on the old state every lane of the column has loaded by now
-            *mp = M;
-            *lp = L;
-          }
+          const float r0 = (o0 * w_old + oacc[db][qb][0] * w_new) * inv;
+          const float r1 = (o1 * w_old + oacc[db][qb][1] * w_new) * inv;
+          const float r2 = (o2 * w_old + oacc[db][qb][2] * w_new) * inv;
+          const float r3 = (o3 * w_old + oacc[db][qb][3] * w_new) * inv;
+          *(u32x2*)(orow + db * 16 + 4 * g) = u32x2{pack2<T>(r0, r1), pack2<T>(r2, r3)};
+        }
+        if (g == 0) {  // every lane of the column has read the old state above
+          p.m[tok * p.ml_st + (int64_t)h * p.ml_sh] = M;
+          p.l[tok * p.ml_st + (int64_t)h * p.ml_sh] = L;
         }
       }
+    };
+    if (DV) {
+      fold_state(std::integral_constant<int, 2>{}, 0);
+    } else {
+      fold_state(std::integral_constant<int, 1>{}, 0);
+      fold_state(std::integral_constant<int, 1>{}, 1);
     }
   }
   if (MODE == 2) {
