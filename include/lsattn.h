@@ -176,6 +176,14 @@ typedef struct lsattn_decode_stage2_args {
 int lsattn_decode_stage2(const lsattn_decode_stage2_args* a, void* stream);
 
 /*
+ * Stage 1 and stage 2 over the same partials from one call: the two launches of
+ * longserve_token_decode_attention_flash_decoding (FDPY:12-27) back to back on `stream`.  Both argument blocks must name
+ * the same mid_o, mid_o_logexpsum, b_seqlen, batch, heads, block count, head_dim and block size (else
+ * LSATTN_ERR_INVALID_ARG); everything else as in the two calls it stands for.
+ */
+int lsattn_decode_attention(const lsattn_decode_stage1_args* s1, const lsattn_decode_stage2_args* s2, void* stream);
+
+/*
  * Row scatter into the KV pool: dst[dest_index[i]] = src[i] for i < n_rows, bit-exact.
  * Replaces _fwd_kernel_destindex_copy_kv
  * (loongserve/common/basemodel/triton_kernel/destindex_copy_kv.py:7-51).

@@ -558,3 +558,15 @@ extern "C" int lsattn_decode_stage2(const lsattn_decode_stage2_args* a, void* st
     default: return LSATTN_ERR_UNSUPPORTED;
   }
 }
+
+extern "C" int lsattn_decode_attention(const lsattn_decode_stage1_args* s1, const lsattn_decode_stage2_args* s2, void* stream) {
+  if (!s1 || !s2) return LSATTN_ERR_INVALID_ARG;
+  // the two stages must describe the same partials
+  if (s1->mid_o != s2->mid_o || s1->mid_o_logexpsum != s2->mid_o_logexpsum || s1->b_seqlen != s2->b_seqlen ||
+      s1->batch != s2->batch || s1->num_q_heads != s2->num_heads || s1->num_blocks != s2->num_seq_blocks ||
+      s1->head_dim != s2->head_dim || s1->seq_block_size != s2->block_seq)
+    return LSATTN_ERR_INVALID_ARG;
+  const int rc = lsattn_decode_stage1(s1, stream);
+  if (rc != LSATTN_OK) return rc;
+  return lsattn_decode_stage2(s2, stream);
+}

@@ -50,8 +50,7 @@ def longserve_token_decode_attention_flash_decoding(q, req_to_token_indexs, b_re
     out_logexpsum = (torch.empty([batch_size, q_head_num], dtype=torch.float32, device=q.device)
                      if o_logexpsum is None else o_logexpsum)
     split = _fused_block_seq(BLOCK_SEQ, batch_size, max_len_in_batch, cache_k.shape[1])
-    longserve_flash_decode_stage1(q.view(calcu_shape1), cache_k, cache_v, req_to_token_indexs, b_req_idx, b_seq_len,
-                                  max_len_in_batch, mid_o, mid_o_logexpsum, split)
-    longserve_flash_decode_stage2(mid_o, mid_o_logexpsum, b_seq_len, o_tensor.view(calcu_shape1), out_logexpsum,
-                                  split)
+    longserve_cuda_kernels.flash_decoding(mid_o, mid_o_logexpsum, q.view(calcu_shape1), cache_k, cache_v, req_to_token_indexs,
+                                          b_req_idx, b_seq_len, max_len_in_batch, o_tensor.view(calcu_shape1), out_logexpsum,
+                                          split)
     return o_tensor, out_logexpsum

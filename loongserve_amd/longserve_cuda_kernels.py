@@ -22,9 +22,9 @@ def _req(cond: bool, what: str) -> None:
         raise ValueError("longserve_cuda_kernels: check failed: " + what)
 
 
-@torch.inference_mode()
-def flash_decoding_stage1(mid_o, mid_o_logexpsum, q, k, v, req_to_tokens, b_req_idx, b_seqlen,
-                          max_len_in_batch: int, seq_block_size: int) -> None:
+def _stage1_args(mid_o, mid_o_logexpsum, q, k, v, req_to_tokens, b_req_idx, b_seqlen,
+                 max_len_in_batch: int, seq_block_size: int) -> _lib.DecodeStage1Args:
+    """The checks of ENTRY:115-160 and the argument block of lsattn_decode_stage1."""
     # ENTRY:115-122
     _req(mid_o.is_contiguous(), "mid_o.is_contiguous()")
     _req(mid_o_logexpsum.is_contiguous(), "mid_o_logexpsum.is_contiguous()")
@@ -66,11 +66,19 @@ def flash_decoding_stage1(mid_o, mid_o_logexpsum, q, k, v, req_to_tokens, b_req_
     a.batch, a.num_q_heads, a.num_kv_heads = B, Hq, k.size(1)
     a.num_blocks, a.head_dim, a.max_seq_len = mid_o.size(0), D, req_to_tokens.size(1)
     a.seq_block_size, a.max_len_in_batch = int(seq_block_size), int(max_len_in_batch)
-    _lib.check(_lib.load().lsattn_decode_stage1(C.byref(a), _stream()), "lsattn_decode_stage1")
+    return a
 
 
 @torch.inference_mode()
-def flash_decoding_stage2(o, out_logexpsum, b_seqlen, mid_o, mid_o_logexpsum, block_seq: int) -> None:
+def flash_decoding_stage1(mid_o, mid_o_logexpsum, q, k, v, req_to_tokens, b_req_idx, b_seqlen,
+                          max_len_in_batch: int, seq_block_size: int) -> None:
+    """ENTRY:103-164, same argument order."""
+    a = _stage1_args(mid_o, mid_o_logexpsum, q, k, v, req_to_tokens, b_req_idx, b_seqlen, max_len_in_batch, seq_block_size)
+    _lib.check(_lib.load().lsattn_decode_stage1(C.byref(a), _stream()), "lsattn_decode_stage1")
+
+
+def _stage2_args(o, out_logexpsum, b_seqlen, mid_o, mid_o_logexpsum, block_seq: int) -> _lib.DecodeStage2Args:
+    """The checks of ENTRY:174-190 and the argument block of lsattn_decode_stage2."""
     # ENTRY:174-190
     for t, d, n in ((o, 3, "o"), (out_logexpsum, 2, "out_logexpsum"), (b_seqlen, 1, "b_seqlen"), (mid_o, 4, "mid_o"),
                     (mid_o_logexpsum, 3, "mid_o_logexpsum")):
@@ -93,7 +101,24 @@ def flash_decoding_stage2(o, out_logexpsum, b_seqlen, mid_o, mid_o_logexpsum, bl
     a.o, a.o_dtype, a.out_logexpsum, a.b_seqlen = o.data_ptr(), _DT[o.dtype], out_logexpsum.data_ptr(), b_seqlen.data_ptr()
     a.mid_o, a.mid_o_logexpsum = mid_o.data_ptr(), mid_o_logexpsum.data_ptr()
     a.batch, a.num_heads, a.num_seq_blocks, a.head_dim, a.block_seq = B, H, mid_o.size(0), D, int(block_seq)
+    return a
+
+
+@torch.inference_mode()
+def flash_decoding_stage2(o, out_logexpsum, b_seqlen, mid_o, mid_o_logexpsum, block_seq: int) -> None:
+    """ENTRY:166-221, same argument order."""
+    a = _stage2_args(o, out_logexpsum, b_seqlen, mid_o, mid_o_logexpsum, block_seq)
     _lib.check(_lib.load().lsattn_decode_stage2(C.byref(a), _stream()), "lsattn_decode_stage2")
+
+
+@torch.inference_mode()
+def flash_decoding(mid_o, mid_o_logexpsum, q, k, v, req_to_tokens, b_req_idx, b_seqlen, max_len_in_batch: int,
+                   o, out_logexpsum, block_seq: int) -> None:
+    """Stage 1 and stage 2 with the same block size from one library call (what FDPY:12-27 does with two): the checks of
+    both, one argument pass, the two launches back to back."""
+    a1 = _stage1_args(mid_o, mid_o_logexpsum, q, k, v, req_to_tokens, b_req_idx, b_seqlen, max_len_in_batch, block_seq)
+    a2 = _stage2_args(o, out_logexpsum, b_seqlen, mid_o, mid_o_logexpsum, block_seq)
+    _lib.check(_lib.load().lsattn_decode_attention(C.byref(a1), C.byref(a2), _stream()), "lsattn_decode_attention")
 
 
 def _half2d(t: torch.Tensor, name: str, dim: int) -> None:

@@ -116,6 +116,14 @@ def test_validation_rejects_bad_arguments_without_gpu():
     for ks, vs in ((0, 256), (256, -256), ((1 << 24) + 8, 256), (256, 1 << 25)):
         a.k_stride_t, a.v_stride_t = ks, vs
         assert lib.lsattn_prefill_step(C.byref(a), None) == -1, (ks, vs)
+    # the fused decode call refuses argument blocks that do not describe the same partials
+    s1, s2 = _lib.DecodeStage1Args(), _lib.DecodeStage2Args()
+    assert lib.lsattn_decode_attention(None, C.byref(s2), None) == -1
+    s1.mid_o, s2.mid_o = 0x1000, 0x2000
+    assert lib.lsattn_decode_attention(C.byref(s1), C.byref(s2), None) == -1
+    s2.mid_o = 0x1000
+    s1.seq_block_size, s2.block_seq = 256, 128
+    assert lib.lsattn_decode_attention(C.byref(s1), C.byref(s2), None) == -1
 
 
 def test_python_wrappers_reject_cpu_tensors():
