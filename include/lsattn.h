@@ -203,6 +203,17 @@ int lsattn_register_tokens(int32_t* req_to_tokens, int64_t max_seq_len, const in
                            int64_t batch, int64_t max_len_in_batch, void* stream);
 
 /*
+ * Decode registration of one new slot per request:
+ *   req_to_tokens[b_req_idx[i], b_seq_len[i] - 1] = mem_index[i]   for i < batch.
+ * Replaces copy_kv_index_to_req (loongserve/common/basemodel/triton_kernel/copy_kv_index_to_req.py:7-40, called
+ * loongserve/models/llama/longserve_model.py:491, :497).  mem_index is int32, or int64 as the allocator hands it out
+ * (mem_index_is_i64 = 1).  An entry whose position falls outside the row is skipped (the reference would write there).
+ */
+int lsattn_register_decode_tokens(int32_t* req_to_tokens, int64_t max_seq_len, const int32_t* b_req_idx,
+                                  const int32_t* b_seq_len, const void* mem_index, int32_t mem_index_is_i64,
+                                  int64_t batch, void* stream);
+
+/*
  * Which locally held KV rows of each request belong to the cache-index window
  * [kv_cache_index_begin, kv_cache_index_end) when local row n holds global token
  * kv_first_token_global_idx + n * sp_peers:

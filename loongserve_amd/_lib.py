@@ -92,6 +92,7 @@ EXPORTS = {
     "lsattn_decode_attention": (C.c_int, [C.POINTER(DecodeStage1Args), C.POINTER(DecodeStage2Args), _vp]),
     "lsattn_kv_scatter": (C.c_int, [_vp, _i64, _vp, _i64, _vp, _i64, _i64, _vp]),
     "lsattn_register_tokens": (C.c_int, [_vp, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _vp]),
+    "lsattn_register_decode_tokens": (C.c_int, [_vp, _i64, _vp, _vp, _vp, C.c_int32, _i64, _vp]),
     "lsattn_kv_ranges": (C.c_int, [_vp, _vp, _vp, C.c_int32, _i64, _vp, _vp, _vp, _vp]),
     "lsattn_kv_copy_register": (C.c_int, [C.POINTER(KvCopyRegisterArgs), _vp]),
     "lsattn_decode_migration_send": (C.c_int, [C.POINTER(DecodeMigrationArgs), _vp]),

@@ -74,6 +74,19 @@ __global__ __launch_bounds__(256) void register_tokens_kernel(int32_t* __restric
   req_to_tokens[(int64_t)b_req_idx[b] * max_seq_len + j] = mem_index[(int64_t)b_start_loc[b] + j];
 }
 
+// one new token per request: req_to_tokens[b_req_idx[i], b_seq_len[i] - 1] = mem_index[i]
+template <typename IT>
+__global__ __launch_bounds__(256) void register_decode_tokens_kernel(int32_t* __restrict__ req_to_tokens, int64_t max_seq_len,
+                                                                     const int32_t* __restrict__ b_req_idx,
+                                                                     const int32_t* __restrict__ b_seq_len,
+                                                                     const IT* __restrict__ mem_index, int64_t batch) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= batch) return;
+  const int64_t pos = (int64_t)b_seq_len[i] - 1;
+  if (pos < 0 || pos >= max_seq_len) return;  // (the reference would write outside the row)
+  req_to_tokens[(int64_t)b_req_idx[i] * max_seq_len + pos] = (int32_t)mem_index[i];
+}
+
 // ceil(x / p) for p > 0 as floor((x + p - 1) / p), also for negative x
 __device__ __forceinline__ int32_t ceil_div_floor(int32_t x, int32_t p) {
   const int64_t a = (int64_t)x + p - 1;
@@ -287,6 +300,24 @@ extern "C" int lsattn_register_tokens(int32_t* req_to_tokens, int64_t max_seq_le
   dim3 grid((unsigned)((max_len_in_batch + 255) / 256), (unsigned)batch);
   hipLaunchKernelGGL(register_tokens_kernel, grid, dim3(256), 0, (hipStream_t)stream, req_to_tokens, max_seq_len,
                      b_req_idx, b_start_loc, b_seq_len, mem_index);
+  return check_launch();
+}
+
+extern "C" int lsattn_register_decode_tokens(int32_t* req_to_tokens, int64_t max_seq_len, const int32_t* b_req_idx,
+                                             const int32_t* b_seq_len, const void* mem_index, int32_t mem_index_is_i64,
+                                             int64_t batch, void* stream) {
+  if (!req_to_tokens || !b_req_idx || !b_seq_len || !mem_index || batch < 0 || max_seq_len <= 0 ||
+      (mem_index_is_i64 != 0 && mem_index_is_i64 != 1))
+    return LSATTN_ERR_INVALID_ARG;
+  if (batch == 0) return LSATTN_OK;
+  const int64_t blocks = (batch + 255) / 256;
+  if (blocks > 0x7fffffff) return LSATTN_ERR_INVALID_ARG;
+  if (mem_index_is_i64)
+    hipLaunchKernelGGL(register_decode_tokens_kernel<int64_t>, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+                       req_to_tokens, max_seq_len, b_req_idx, b_seq_len, (const int64_t*)mem_index, batch);
+  else
+    hipLaunchKernelGGL(register_decode_tokens_kernel<int32_t>, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+                       req_to_tokens, max_seq_len, b_req_idx, b_seq_len, (const int32_t*)mem_index, batch);
   return check_launch();
 }
 

@@ -1,10 +1,12 @@
-"""Stand-in for the `longserve_cuda_kernels` extension module (decode entry points only).
+"""Stand-in for the `longserve_cuda_kernels` extension module.
 
 Exports flash_decoding_stage1 / flash_decoding_stage2 with the argument order and the
-tensor checks of longserve_cuda_kernels/src/entrypoints.cpp:103-221 (exported at
-:237-238).  A failed check raises ValueError instead of aborting the process
-(the reference calls __assert_fail, longserve_cuda_kernels/src/common.h:29-32).
-Beyond the reference: q/k/v may be bfloat16, and stage-2 `o` may be bfloat16.
+tensor checks of longserve_cuda_kernels/src/entrypoints.cpp:103-221, and rms_norm,
+silu_and_mul_inplace, rotary_emb, ffn_block, hello_world (:15-101, :228-241).  A failed
+check raises ValueError instead of aborting the process (the reference calls
+__assert_fail, longserve_cuda_kernels/src/common.h:29-32).
+Beyond the reference: q/k/v may be bfloat16, stage-2 `o` may be bfloat16, and
+flash_decoding runs both decode stages from one library call.
 """
 from __future__ import annotations
 

@@ -263,6 +263,44 @@ def kv_scatter(src: torch.Tensor, dest_index: torch.Tensor, pool: torch.Tensor) 
     _lib.check(rc, "lsattn_kv_scatter")
 
 
+def rmsnorm_forward(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    """Name and signature of the Triton operator behind the final norm
+    (loongserve/models/llama/triton_kernel/rmsnorm.py:41-63, called
+    loongserve/models/llama/layer_infer/longserve_post_layer_infer.py:35): a new tensor y = x / rms(x) * weight over the
+    last dimension.  Runs the same kernel as longserve_cuda_kernels.rms_norm."""
+    from .longserve_cuda_kernels import rms_norm
+    if not x.is_contiguous():
+        raise ValueError("x must be contiguous")
+    return rms_norm(x.view(-1, x.shape[-1]), weight, eps).view(x.shape)
+
+
+def destindex_copy_kv(K: torch.Tensor, DestLoc: torch.Tensor, Out: torch.Tensor) -> None:
+    """Out[DestLoc[i]] = K[i]: name and argument order of the operator the layer calls to persist a step's K/V rows
+    (loongserve/common/basemodel/triton_kernel/destindex_copy_kv.py:32, called
+    loongserve/models/llama/layer_infer/longserve_transformer_layer_infer.py:377)."""
+    kv_scatter(K, DestLoc, Out)
+
+
+@torch.inference_mode()
+def copy_kv_index_to_req(req_to_token_indexs: torch.Tensor, b_req_idx: torch.Tensor, b_seq_len: torch.Tensor,
+                         memindex: torch.Tensor) -> None:
+    """req_to_token_indexs[b_req_idx[i], b_seq_len[i] - 1] = memindex[i]: registers the slot of each request's new token
+    in the decoding stage (loongserve/common/basemodel/triton_kernel/copy_kv_index_to_req.py:22-40, called
+    loongserve/models/llama/longserve_model.py:491, :497).  memindex is int32 or, as the allocator returns it, int64."""
+    _dev(req_to_token_indexs, "req_to_token_indexs"); _dev(memindex, "memindex")
+    B = b_seq_len.shape[0]
+    assert b_seq_len.shape[0] == memindex.shape[0] and b_req_idx.shape[0] == b_seq_len.shape[0]  # as the reference
+    _i32vec(b_req_idx, "b_req_idx", B); _i32vec(b_seq_len, "b_seq_len", B)
+    if req_to_token_indexs.dtype != torch.int32 or req_to_token_indexs.dim() != 2 or not req_to_token_indexs.is_contiguous():
+        raise ValueError("req_to_token_indexs must be a contiguous [max_req, max_seq] int32 tensor")
+    if memindex.dtype not in (torch.int32, torch.int64) or memindex.dim() != 1 or not memindex.is_contiguous():
+        raise ValueError("memindex must be a contiguous 1-D int32 or int64 tensor")
+    rc = _lib.load().lsattn_register_decode_tokens(req_to_token_indexs.data_ptr(), req_to_token_indexs.shape[1],
+                                                   b_req_idx.data_ptr(), b_seq_len.data_ptr(), memindex.data_ptr(),
+                                                   1 if memindex.dtype == torch.int64 else 0, B, _stream())
+    _lib.check(rc, "lsattn_register_decode_tokens")
+
+
 @torch.inference_mode()
 def init_req_to_token_indexes(req_to_token_indexs, b_req_idx, b_seq_len, alloc_mem_index,
                               b_start_loc: Optional[torch.Tensor] = None, max_len_in_batch: Optional[int] = None) -> None:

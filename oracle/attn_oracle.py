@@ -291,6 +291,13 @@ def register_tokens(req_to_tokens, b_req_idx, b_start_loc, b_seq_len, mem_index)
         req_to_tokens[int(b_req_idx[b]), 0:n] = mem_index[s:s + n].to(req_to_tokens.dtype)
 
 
+def copy_kv_index_to_req(req_to_token_indexs, b_req_idx, b_seq_len, memindex) -> None:
+    """req_to_token_indexs[b_req_idx[i], b_seq_len[i] - 1] = memindex[i], one entry per request
+    (loongserve/common/basemodel/triton_kernel/copy_kv_index_to_req.py:12-18)."""
+    for i in range(len(b_req_idx)):
+        req_to_token_indexs[int(b_req_idx[i]), int(b_seq_len[i]) - 1] = int(memindex[i])
+
+
 def kv_ranges(kv_cache_index_begin, kv_cache_index_end, kv_first_token_global_idx, peers: int):
     """(kv_range_begin, kv_range_end, new_kv_cache_len) of pre_copy_and_register_kv
     (loongserve/models/llama/triton_kernel/copy_and_register_kv.py:24-31, docstring :42-48):

@@ -70,7 +70,7 @@ def test_prefill_then_decode_through_the_pool(lsa, Hq, Hkv):
     qd, kvd = q.to(DEV), kv.to(DEV)
     lsa.longserve_cuda_kernels.rotary_emb(qd, kvd[:, :Hkv], cos.to(DEV), sin.to(DEV))
     assert torch.equal(qd.cpu(), q_ref) and torch.equal(kvd[:, :Hkv].cpu(), k_ref)
-    lsa.kv_scatter(kvd, slots, mm.kv_buffer[0])
+    lsa.destindex_copy_kv(kvd, slots, mm.kv_buffer[0])                     # longserve_transformer_layer_infer.py:377
     od = torch.empty(T, Hq, D, dtype=torch.float16, device=DEV)
     md = torch.full((T, Hq), float("-inf"), device=DEV)
     ld = torch.zeros(T, Hq, device=DEV)
@@ -101,9 +101,9 @@ def test_prefill_then_decode_through_the_pool(lsa, Hq, Hkv):
         held.append(new)
         qnd, kvnd = qn.to(DEV), kvn.to(DEV)
         lsa.longserve_cuda_kernels.rotary_emb(qnd, kvnd[:, :Hkv], cos.to(DEV), sin.to(DEV))
-        lsa.kv_scatter(kvnd, new, mm.kv_buffer[0])
-        rm.req_to_token_indexs[b_req_idx.long(), cur.to(DEV).long()] = new.to(torch.int32)
+        lsa.destindex_copy_kv(kvnd, new, mm.kv_buffer[0])
         cur = cur + 1
+        lsa.copy_kv_index_to_req(rm.req_to_token_indexs, b_req_idx, cur.to(DEV), new)   # longserve_model.py:491
         max_len = int(cur.max())
         nblk = (max_len + BLOCK_SEQ - 1) // BLOCK_SEQ
         mid_o = torch.empty(nblk, B, Hq, D, dtype=torch.float32, device=DEV)

@@ -181,6 +181,27 @@ def test_kv_scatter_and_register_bit_exact(lsa):
     lsa.init_req_to_token_indexes(table_d, b_req.to(DEV), ln.to(DEV), dest.to(DEV), st.to(DEV), max(lens))
     orc.register_tokens(table, b_req, st, ln, dest)
     assert torch.equal(table_d.cpu(), table)
+    # the operator names the reference's layer and model call: row scatter, one new slot per request in decode
+    pool2 = torch.zeros(pool_n, 2 * Hkv, D, dtype=torch.bfloat16, device=DEV)
+    lsa.destindex_copy_kv(src.to(DEV), dest.to(DEV).long(), pool2)
+    assert torch.equal(pool2, pool_d)
+    for dt in (torch.int32, torch.int64):
+        B = 1000
+        req = torch.randperm(1200, generator=g)[:B].to(torch.int32)
+        ln1 = torch.randint(1, 601, (B,), generator=g, dtype=torch.int32)
+        mem = torch.randint(0, 2_000_000, (B,), generator=g).to(dt)
+        t_ref = torch.full((1200, 600), orc.INT32_PAD, dtype=torch.int32)
+        t_dev = t_ref.to(DEV)
+        lsa.copy_kv_index_to_req(t_dev, req.to(DEV), ln1.to(DEV), mem.to(DEV))
+        orc.copy_kv_index_to_req(t_ref, req, ln1, mem)
+        assert torch.equal(t_dev.cpu(), t_ref)
+    # a length of 0 or beyond the row is skipped, nothing else is touched
+    t_dev = torch.full((3, 8), 5, dtype=torch.int32, device=DEV)
+    lsa.copy_kv_index_to_req(t_dev, torch.tensor([0, 1, 2], dtype=torch.int32, device=DEV),
+                             torch.tensor([0, 9, 8], dtype=torch.int32, device=DEV), torch.tensor([7, 7, 7], device=DEV))
+    want = torch.full((3, 8), 5, dtype=torch.int32)
+    want[2, 7] = 7
+    assert torch.equal(t_dev.cpu(), want)
 
 
 def test_bf16_v_converted_inside_the_kernel_or_before_it(lsa):

@@ -293,6 +293,17 @@ def test_kv_scatter_and_register():
     assert table[2].tolist() == [7, 2, 9, 0, orc.INT32_PAD]
     assert table[0].tolist() == [4, 5] + [orc.INT32_PAD] * 3
     assert torch.all(table[[1, 3]] == orc.INT32_PAD)
+    # the decode-stage registration: known answer, and the same as a numpy fancy-index assignment
+    orc.copy_kv_index_to_req(table, torch.tensor([0, 3]), torch.tensor([3, 1]), torch.tensor([11, 12]))
+    assert table[0].tolist() == [4, 5, 11] + [orc.INT32_PAD] * 2 and table[3].tolist() == [12] + [orc.INT32_PAD] * 4
+    import numpy as np
+    rng = np.random.default_rng(3)
+    t1 = torch.full((9, 20), orc.INT32_PAD, dtype=torch.int32)
+    t2 = t1.numpy().copy()
+    req, ln, mem = rng.permutation(9)[:6], rng.integers(1, 21, 6), rng.integers(0, 1000, 6)
+    orc.copy_kv_index_to_req(t1, torch.from_numpy(req), torch.from_numpy(ln), torch.from_numpy(mem))
+    t2[req, ln - 1] = mem
+    assert (t1.numpy() == t2).all()
 
 
 def test_kv_ranges_count_the_locally_held_tokens_of_the_window():
