@@ -38,3 +38,27 @@ def test_random_steps_match_the_oracle(lsa, seed):
         what = "seed %d case %d" % (seed, case)
         assert_o_close(o, o_ref, "O, " + what)
         assert_lse_close(lse, lse_ref, "LSE, " + what)
+        # a second random chunk folded into the first step's result, by the accumulating epilogue and by the in-place
+        # (o, m, l) one; the oracle merges the two steps' partials
+        klens2 = [rng.choice([0, 1, 64, 130, 512, 700, 1300]) for _ in range(B)]
+        kf2 = [rng.choice([0, 2, 50, 900]) for _ in range(B)]
+        Tk2 = max(sum(klens2), 1)
+        k2 = rand_t((Tk2, Hkv, 128), 1000 * seed + 300 + case, dtype)
+        v2 = rand_t((Tk2, Hkv, 128), 1000 * seed + 400 + case, dtype)
+        km2 = meta(klens2, kf2)
+        o2_ref, lse2_ref = orc.lse_merge([(o_ref, lse_ref), orc.attn_step(q, k2, v2, *qm, *km2, P)])
+        qd, qmd = q.to(DEV), [t.to(DEV) for t in qm]
+        lsa.prefill_attention_step(qd, k2.to(DEV), v2.to(DEV), *qmd, *[t.to(DEV) for t in km2], P, max(qlens), o, lse,
+                                   accumulate=True)
+        od = torch.full((Tq, Hq, 128), float("nan"), dtype=dtype, device=DEV)
+        md = torch.full((Tq, Hq), float("-inf"), device=DEV)
+        ld = torch.zeros(Tq, Hq, device=DEV)
+        for kk, vv, kmm in ((k, v, km), (k2, v2, km2)):
+            lsa.context_attention_fwd(qd, kk.to(DEV), vv.to(DEV), od, *qmd, *[t.to(DEV) for t in kmm], P, max(qlens), md, ld)
+        torch.cuda.synchronize()
+        assert_o_close(o, o2_ref, "accumulated O, " + what)
+        assert_lse_close(lse, lse2_ref, "accumulated LSE, " + what)
+        seen = ~torch.isinf(lse2_ref)
+        bars = dict(max_abs=2e-3, rel=1.5e-3) if dtype == torch.float16 else dict(max_abs=2e-2, rel=6e-3)  # o stored in q's dtype per step
+        assert_o_close(torch.where(seen[..., None], od.float().cpu(), torch.zeros(())), o2_ref, "in-place o, " + what, **bars)
+        assert_lse_close(orc.state_lse(md.cpu(), ld.cpu()).float(), lse2_ref, "in-place state, " + what)
