@@ -144,3 +144,24 @@ def test_stage2_alone_over_few_and_many_partials(lsa, nblk):
         else:
             assert_o_close(o, torch.where(dead[..., None], torch.zeros(()), o_ref), "o fp16", max_abs=4e-3, rel=1e-3)
         assert_lse_close(l, l_ref, "lse", rel=1e-5)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_peaked_softmax_keeps_the_bars(lsa, dtype):
+    """Scores of magnitude up to ~64: a few tokens carry each request."""
+    B, Hq, Hkv, D, BS = 3, 4, 2, 128, 256
+    lens = [3000, 700, 64]
+    q, kv, table, b_req, b_len = decode_case(5, B, Hq, Hkv, D, lens, 5000, dtype)
+    g = torch.Generator().manual_seed(9)
+    q = (torch.randn(q.shape, generator=g) * 4).to(dtype)
+    kv[:, :Hkv] = (torch.randn((5000, Hkv, D), generator=g) * 4).to(dtype)
+    o_ref, l_ref = orc.decode_full(q, kv[:, :Hkv], kv[:, Hkv:], table, b_req, b_len)
+    kvd = kv.to(DEV)
+    nblk = (max(lens) + BS - 1) // BS
+    mo = torch.empty(nblk, B, Hq, D, device=DEV)
+    ml = torch.empty(nblk, B, Hq, device=DEV)
+    o, l = lsa.longserve_token_decode_attention_flash_decoding(q.to(DEV), table.to(DEV), b_req.to(DEV), b_len.to(DEV), mo, ml, B,
+                                                               max(lens), Hq, D, kvd[:, :Hkv], kvd[:, Hkv:], BS)
+    torch.cuda.synchronize()
+    assert_o_close(o, o_ref, "o")
+    assert_lse_close(l, l_ref, "lse")

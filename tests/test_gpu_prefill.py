@@ -349,3 +349,22 @@ def test_ring_accumulated_in_the_epilogue_matches_monolithic(lsa, dtype):
         torch.cuda.synchronize()
         assert_o_close(o, o1_ref[r::P], "striped accumulated O rank %d" % r)
         assert_lse_close(l, lse1_ref[r::P], "striped accumulated LSE rank %d" % r)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("scale", [2.0, 4.0])
+def test_peaked_softmax_keeps_the_bars(lsa, dtype, scale):
+    """Scores of magnitude up to ~16 and ~64 (a few keys carry each row): the running max moves often and far, so the
+    main loop's late-maximum path and the rescaling of the accumulators run many times."""
+    print("case", dtype, scale, flush=True)
+    lens, Hq, Hkv = [2300, 700], 4, 2
+    T = sum(lens)
+    g = torch.Generator().manual_seed(int(scale))
+    q = (torch.randn((T, Hq, 128), generator=g) * scale).to(dtype)
+    k = (torch.randn((T, Hkv, 128), generator=g) * scale).to(dtype)
+    v = rand_t((T, Hkv, 128), 3, dtype)
+    m = meta(lens)
+    o, lse = _run_step(lsa, q, k, v, m, m, 1, max(lens))
+    o_ref, lse_ref = orc.attn_step(q, k, v, *m, *m, 1)
+    assert_o_close(o, o_ref, "O")
+    assert_lse_close(lse, lse_ref, "LSE")
