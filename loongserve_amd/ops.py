@@ -274,6 +274,22 @@ def rmsnorm_forward(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.
     return rms_norm(x.view(-1, x.shape[-1]), weight, eps).view(x.shape)
 
 
+def rotary_emb_fwd(q: torch.Tensor, k: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> None:
+    """Name and signature of the Triton rotary operator (loongserve/models/llama/triton_kernel/rotary_emb.py:119); nothing in
+    the reference calls it (the layer uses longserve_cuda_kernels.rotary_emb, which this runs)."""
+    from .longserve_cuda_kernels import rotary_emb
+    rotary_emb(q, k, cos, sin)
+
+
+def silu_and_mul_fwd(input: torch.Tensor) -> torch.Tensor:
+    """Name and signature of the Triton operator (loongserve/models/llama/triton_kernel/silu_and_mul.py:50-74): in place
+    on the first half of the columns, which is returned as a view; nothing in the reference calls it (ffn_block does the
+    same through longserve_cuda_kernels.silu_and_mul_inplace, which this runs)."""
+    from .longserve_cuda_kernels import silu_and_mul_inplace
+    silu_and_mul_inplace(input)
+    return input[:, 0:(input.shape[-1] // 2)]
+
+
 def destindex_copy_kv(K: torch.Tensor, DestLoc: torch.Tensor, Out: torch.Tensor) -> None:
     """Out[DestLoc[i]] = K[i]: name and argument order of the operator the layer calls to persist a step's K/V rows
     (loongserve/common/basemodel/triton_kernel/destindex_copy_kv.py:32, called

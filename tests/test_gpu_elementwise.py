@@ -89,6 +89,26 @@ def test_ffn_block_composition(lsa):
     assert err <= 2e-2 * max(1.0, np.abs(want).max()), err   # library GEMM accumulation order + fp16 outputs
 
 
+def test_triton_operator_names_run_the_same_kernels(lsa):
+    """rotary_emb_fwd / silu_and_mul_fwd (the Triton duplicates in the reference's tree) give what the extension-module
+    functions give, with the Triton wrappers' return convention."""
+    g = torch.Generator().manual_seed(3)
+    T, Hq, Hkv, D, I = 33, 4, 2, 128, 256
+    q = (torch.randn(T, Hq, D, generator=g)).half().to(DEV)
+    k = (torch.randn(T, Hkv, D, generator=g)).half().to(DEV)
+    ang = torch.rand(T, D // 2, generator=g) * 6
+    cos, sin = torch.cos(ang).half().to(DEV), torch.sin(ang).half().to(DEV)
+    q2, k2 = q.clone(), k.clone()
+    lsa.longserve_cuda_kernels.rotary_emb(q, k, cos, sin)
+    assert lsa.rotary_emb_fwd(q2, k2, cos, sin) is None
+    assert torch.equal(q, q2) and torch.equal(k, k2)
+    io = (torch.randn(T, 2 * I, generator=g) * 2).half().to(DEV)
+    io2 = io.clone()
+    lsa.longserve_cuda_kernels.silu_and_mul_inplace(io)
+    out = lsa.silu_and_mul_fwd(io2)
+    assert out.shape == (T, I) and out.data_ptr() == io2.data_ptr() and torch.equal(io, io2)
+
+
 def test_argument_checks(lsa):
     k = lsa.longserve_cuda_kernels
     with pytest.raises(ValueError):
