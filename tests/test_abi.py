@@ -145,7 +145,9 @@ def test_fused_decode_split_rule():
     assert _fused_block_seq(256, 64, 32768, 8) == 1024           # config 3: 64 x 32 blocks x 2 task groups
     assert _fused_block_seq(256, 4, 131072, 32) == 1024          # one instance of config 4
     assert _fused_block_seq(256, 1, 4096, 8) == 256              # a single short request: nothing to spare
-    assert _fused_block_seq(256, 16, 8192, 8) == 256
+    assert _fused_block_seq(256, 16, 8192, 8) == 1024            # 16 x 8 blocks x 2 task groups = one workgroup per CU
+    assert _fused_block_seq(256, 1, 131072, 8) == 1024
+    assert _fused_block_seq(256, 1, 32768, 8) == 256
     assert _fused_block_seq(2048, 64, 32768, 8) == 2048          # never below what the caller asked for
     assert _fused_block_seq(16, 4096, 16, 8) == 16
     for bs in (1, 16, 64, 256):
