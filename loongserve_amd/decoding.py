@@ -31,12 +31,23 @@ FUSED_SPLIT_TOKENS = 1024
 FUSED_MIN_WORKGROUPS = 256
 
 
+# Very long contexts go further, up to 4096 tokens, while the longest request still has this many blocks: there the last,
+# partly filled block of a request and the spread of lengths in the batch (which the host does not see) weigh little, and
+# the partials and their merge are what is left to save (one request of 1048576 tokens: 721 -> 675 us; four of 131072
+# with 32 KV heads: 1336 -> 1313 us).  With fewer blocks per request the coarser split loses to the ragged tail
+# (config 3, lengths 4096..32768: 903 us at 1024, 947 at 2048).
+FUSED_LONG_SPLIT_TOKENS = 4096
+FUSED_LONG_MIN_BLOCKS = 64
+
+
 def _fused_block_seq(block_seq: int, batch_size: int, max_len_in_batch: int, num_kv_heads: int) -> int:
     bs = int(block_seq)
     task_groups = (int(num_kv_heads) + 3) // 4
-    while bs * 2 <= FUSED_SPLIT_TOKENS and bs < int(max_len_in_batch):
+    while bs * 2 <= FUSED_LONG_SPLIT_TOKENS and bs < int(max_len_in_batch):
         blocks = (int(max_len_in_batch) + 2 * bs - 1) // (2 * bs)
         if int(batch_size) * blocks * task_groups < FUSED_MIN_WORKGROUPS:
+            break
+        if bs * 2 > FUSED_SPLIT_TOKENS and blocks < FUSED_LONG_MIN_BLOCKS:
             break
         bs *= 2
     return bs

@@ -141,15 +141,17 @@ def test_python_wrappers_reject_cpu_tensors():
 def test_fused_decode_split_rule():
     """The fused decode call may split the context more coarsely than BLOCK_SEQ, but only while the launch keeps enough
     workgroups; the stage functions called on their own never change the block size they are given."""
-    from loongserve_amd.decoding import FUSED_SPLIT_TOKENS, _fused_block_seq
+    from loongserve_amd.decoding import FUSED_LONG_SPLIT_TOKENS, _fused_block_seq
     assert _fused_block_seq(256, 64, 32768, 8) == 1024           # config 3: 64 x 32 blocks x 2 task groups
-    assert _fused_block_seq(256, 4, 131072, 32) == 1024          # one instance of config 4
     assert _fused_block_seq(256, 1, 4096, 8) == 256              # a single short request: nothing to spare
     assert _fused_block_seq(256, 16, 8192, 8) == 1024            # 16 x 8 blocks x 2 task groups = one workgroup per CU
     assert _fused_block_seq(256, 1, 131072, 8) == 1024
     assert _fused_block_seq(256, 1, 32768, 8) == 256
+    assert _fused_block_seq(256, 1, 1048576, 8) == 4096          # very long contexts: up to 4096 while >= 64 blocks remain
+    assert _fused_block_seq(256, 4, 131072, 32) == 2048
+    assert _fused_block_seq(256, 16, 32768, 8) == 1024
     assert _fused_block_seq(2048, 64, 32768, 8) == 2048          # never below what the caller asked for
     assert _fused_block_seq(16, 4096, 16, 8) == 16
     for bs in (1, 16, 64, 256):
         got = _fused_block_seq(bs, 1 << 14, 1 << 20, 32)
-        assert got % bs == 0 and got <= max(FUSED_SPLIT_TOKENS, bs)
+        assert got % bs == 0 and got <= max(FUSED_LONG_SPLIT_TOKENS, bs)
