@@ -89,7 +89,12 @@ __global__ __launch_bounds__(NW * 64) void decode_stage1_kernel(Stage1Params p) 
   int64_t nblk = len <= 0 ? 0 : ((int64_t)len + p.block_seq - 1) / p.block_seq;
   if (nblk > p.grid_blocks) nblk = p.grid_blocks;
   if (nblk > p.num_blocks) nblk = p.num_blocks;
-  const int64_t blk_begin = (int64_t)(p.tasks_on_x ? blockIdx.y : blockIdx.x) * p.blocks_per_wg;
+  // Workgroups go to the 8 XCDs round-robin in linear id order, so a fixed chunk index always lands on the same XCDs and
+  // the first chunks (all that short requests have) would load some XCDs more than others; the chunk index is rotated by
+  // the request index to spread them (batch 64 with lengths 4096..32768: 5.62 -> 5.9 TB/s).
+  const unsigned n_chunks = p.tasks_on_x ? gridDim.y : gridDim.x;
+  const unsigned chunk = ((p.tasks_on_x ? blockIdx.y : blockIdx.x) + (unsigned)b) % n_chunks;
+  const int64_t blk_begin = (int64_t)chunk * p.blocks_per_wg;
   int64_t blk_end = blk_begin + p.blocks_per_wg;
   if (blk_end > nblk) blk_end = nblk;
   if (blk_begin >= blk_end) return;
