@@ -24,7 +24,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
-PREFILL_TRAFFIC_BYTES = 1364.6e6  # per launch, averaged over a ring step: profiles/bench_default_hbm_traffic.txt
+PREFILL_TRAFFIC_BYTES = 1364.3e6  # per launch, averaged over a ring step: profiles/bench_default_hbm_traffic.txt
 PEAK_MFMA_TFLOPS = 2500.0  # dense fp16/bf16 MFMA, MI355X
 PEAK_HBM_GBS = 8000.0
 DEV = "cuda:0"
