@@ -27,6 +27,9 @@
 //     bounds-checked step; causal work is skipped per wave;
 //   * workgroup ids are mapped so that the workgroups sharing one KV head run on one XCD
 //     (ids are dealt round-robin to the 8 XCDs) and heavy (late) query tiles start first.
+//   * one kernel, three epilogues (MODE): 0 writes the step's fp32 partial (O, LSE) from the empty state, 1 folds the
+//     step into the reference's in-place (o, m, l) state (ring_context_flashattention_nopad.py:171-188), 2 LSE-merges it
+//     into a running fp32 (O, LSE); the folding ones read the old state of both row blocks of a wave at once.
 #include <type_traits>
 
 #include "common.hip.h"
