@@ -105,7 +105,7 @@ class RingPrefill:
                           torch.empty((self.shard, self.H), dtype=torch.float32, device=DEV)) for _ in self.order]
         ring_prefill_partials(self.q, self.chunks, self.qs, self.ql, self.qf, 1, self.shard, self.Hkv, self.bufs, self.out, self.lse)
 
-    def cpu_baseline(self, heads=8, rows=4096):
+    def cpu_baseline(self, heads=16, rows=6144):
         """Oracle (PyTorch CPU fp32) on a slice: `heads` heads, the last `rows` query rows of the
         shard, against all four KV shards; scaled by algorithmic FLOPs."""
         from oracle import attn_oracle as orc
