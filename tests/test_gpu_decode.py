@@ -165,3 +165,41 @@ def test_peaked_softmax_keeps_the_bars(lsa, dtype):
     torch.cuda.synchronize()
     assert_o_close(o, o_ref, "o")
     assert_lse_close(l, l_ref, "lse")
+
+
+def test_one_request_of_a_million_tokens(lsa):
+    """The longest context the serving configs name (1M tokens) in one request: the fused call's coarsest split, the wide
+    merge, 32-bit positions near 2^20 and slot numbers above 2^20.  Checked through closed forms rather than a CPU pass
+    over 1 GB of rows: q = 0 gives O = mean of the request's V rows and LSE = ln(n); a query equal to 40 x one key's
+    direction puts almost all weight on that token."""
+    n, Hq, Hkv, D, BS = 1_048_576, 4, 2, 128, 256
+    pool = n + 4096
+    g = torch.Generator(device=DEV).manual_seed(11)
+    kv = (torch.randn((pool, 2 * Hkv, D), generator=g, device=DEV) * 0.5).half()
+    perm = torch.randperm(pool, generator=g, device=DEV)[:n].to(torch.int32)
+    table = torch.full((2, n + 8), 2147483647, dtype=torch.int32, device=DEV)
+    table[1, :n] = perm
+    b_req = torch.tensor([1], dtype=torch.int32, device=DEV)
+    b_len = torch.tensor([n], dtype=torch.int32, device=DEV)
+    nblk = (n + BS - 1) // BS
+    mo = torch.empty(nblk, 1, Hq, D, device=DEV)
+    ml = torch.empty(nblk, 1, Hq, device=DEV)
+    q = torch.zeros(1, Hq, D, dtype=torch.float16, device=DEV)
+    o, lse = lsa.longserve_token_decode_attention_flash_decoding(q, table, b_req, b_len, mo, ml, 1, n, Hq, D, kv[:, :Hkv], kv[:, Hkv:], BS)
+    torch.cuda.synchronize()
+    v_mean = kv[perm.long(), Hkv:].double().mean(0)                        # [Hkv, D]
+    want = v_mean.repeat_interleave(Hq // Hkv, 0)[None].float()
+    assert (o - want).abs().max().item() <= 2e-5
+    assert (lse - math.log(n)).abs().max().item() <= 1e-4 * math.log(n)
+    # a peaked query: token t of the request (any position, here near the end) dominates
+    t = n - 12345
+    slot = int(perm[t])
+    kdir = kv[slot, :Hkv].float()                                          # [Hkv, D]
+    q2 = (kdir * (40.0 / kdir.norm(dim=-1, keepdim=True))).repeat_interleave(Hq // Hkv, 0)[None].half()
+    o2, lse2 = lsa.longserve_token_decode_attention_flash_decoding(q2, table, b_req, b_len, mo, ml, 1, n, Hq, D, kv[:, :Hkv], kv[:, Hkv:], BS)
+    torch.cuda.synchronize()
+    s = torch.einsum("hd,nhd->hn", q2[0].float().view(Hkv, Hq // Hkv, D).reshape(Hq, D)[::Hq // Hkv], kv[perm.long(), :Hkv].float()) / math.sqrt(D)
+    lse_ref = torch.logsumexp(s.double(), dim=-1).float().repeat_interleave(Hq // Hkv)
+    o_ref = torch.einsum("hn,nhd->hd", torch.softmax(s.double(), dim=-1), kv[perm.long(), Hkv:].double()).float().repeat_interleave(Hq // Hkv, 0)
+    assert_lse_close(lse2[0], lse_ref.cpu(), "peaked lse")
+    assert_o_close(o2[0], o_ref.cpu(), "peaked o")
