@@ -1,0 +1,65 @@
+"""The library keeps no state: calls on different streams, from different host threads, do not disturb each other.
+Prefill steps and decode steps are issued concurrently on two streams (default priority) from two threads and compared
+with the same calls made one after the other."""
+import threading
+
+import pytest
+import torch
+
+from tests.helpers import decode_case, meta, rand_t
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def test_two_threads_two_streams(lsa):
+    Hq, Hkv, D, BS = 8, 2, 128, 64
+    lens = [900, 300]
+    T = sum(lens)
+    q, k, v = [rand_t(s, i).to(DEV) for i, s in enumerate(((T, Hq, D), (T, Hkv, D), (T, Hkv, D)))]
+    m = [t.to(DEV) for t in meta(lens)]
+    dl = [700, 33, 1025]
+    dq, dkv, table, b_req, b_len = [t.to(DEV) for t in decode_case(77, 3, Hq, Hkv, D, dl, 3000)]
+    nblk = (max(dl) + BS - 1) // BS
+
+    def prefill(out, lse):
+        lsa.prefill_attention_step(q, k, v, *m, *m, 1, max(lens), out, lse)
+
+    def decode(mo, ml, o, l):
+        lsa.longserve_token_decode_attention_flash_decoding(dq, table, b_req, b_len, mo, ml, 3, max(dl), Hq, D, dkv[:, :Hkv],
+                                                            dkv[:, Hkv:], BS, o, l)
+
+    def bufs():
+        return (torch.empty(T, Hq, D, device=DEV), torch.empty(T, Hq, device=DEV), torch.empty(nblk, 3, Hq, D, device=DEV),
+                torch.empty(nblk, 3, Hq, device=DEV), torch.empty(3, Hq, D, device=DEV), torch.empty(3, Hq, device=DEV))
+
+    ref = bufs()
+    prefill(ref[0], ref[1]); decode(*ref[2:])
+    torch.cuda.synchronize()
+
+    got = [bufs() for _ in range(8)]
+    errors = []
+
+    def worker(kind):
+        try:
+            s = torch.cuda.Stream()
+            with torch.cuda.stream(s):
+                for b in got:
+                    if kind == 0:
+                        prefill(b[0], b[1])
+                    else:
+                        decode(*b[2:])
+            s.synchronize()
+        except Exception as e:  # surfaced below: an exception in a thread would otherwise be lost
+            errors.append(e)
+
+    threads = [threading.Thread(target=worker, args=(kind,)) for kind in (0, 1)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    torch.cuda.synchronize()
+    assert not errors, errors
+    for b in got:
+        assert torch.equal(b[0], ref[0]) and torch.equal(b[1], ref[1])
+        assert torch.equal(b[4], ref[4]) and torch.equal(b[5], ref[5])
