@@ -3,8 +3,9 @@
 //
 // Stage 1 replaces flash_decoding_stage1_kernel
 // (longserve_cuda_kernels/src/flash_decoding_stage1.cu:25-143).  Differences by design:
-//   * one wave64 serves one KV head and all (up to 8) query heads of its GQA group, so a
-//     K/V row is fetched once per KV head instead of once per query head;
+//   * one wave64 serves one KV head and up to four query heads of its GQA group (larger groups take
+//     several waves, sizes that are not a multiple of four a last wave with spare accumulators), so a
+//     K/V row is fetched once per four query heads instead of once per query head;
 //   * a K/V row of 128 16-bit elements is read by 16 lanes x 16 bytes; a wave has four
 //     such lane groups and every group keeps 8 K rows and 8 V rows in flight;
 //   * each lane group runs its own online softmax; groups are merged once per block with
@@ -80,10 +81,14 @@ __global__ __launch_bounds__(NW * 64) void decode_stage1_kernel(Stage1Params p) 
   // time (measured 2 % faster on GQA 32/8, two task groups per chunk).
   const int task = SPLIT ? (int)(p.tasks_on_x ? blockIdx.x : blockIdx.y) : (int)(p.tasks_on_x ? blockIdx.x : blockIdx.y) * NW + wave;
   if (task >= p.tasks) return;  // (SPLIT: the same for every wave of the workgroup, like the block range below)
+  // a task = one KV head and up to GT query heads of its group; the last task of a group whose size is not a multiple of
+  // GT has fewer (nh): its spare accumulators repeat the last query head and are not written
   const int group = (int)(p.hq / p.hkv);
-  const int sub_groups = group / GT;
+  const int sub_groups = (group + GT - 1) / GT;
   const int kvh = task / sub_groups;
-  const int qh0 = kvh * group + (task % sub_groups) * GT;
+  const int sg = task % sub_groups;
+  const int qh0 = kvh * group + sg * GT;
+  const int nh = group - sg * GT < GT ? group - sg * GT : GT;
 
   const int len = p.b_seqlen[b];  // positions inside a request are 32-bit (max_seq_len is checked on the host)
   int64_t nblk = len <= 0 ? 0 : ((int64_t)len + p.block_seq - 1) / p.block_seq;
@@ -107,7 +112,7 @@ __global__ __launch_bounds__(NW * 64) void decode_stage1_kernel(Stage1Params p) 
   // q stays packed (8 elements = 4 words per head and lane); the scale is applied to the reduced dot
   u32x4 qw[GT];
 #pragma unroll
-  for (int h = 0; h < GT; h++) qw[h] = *(const u32x4*)((const char*)p.q + ((b * p.hq + qh0 + h) * 128 + sub * 8) * 2);
+  for (int h = 0; h < GT; h++) qw[h] = *(const u32x4*)((const char*)p.q + ((b * p.hq + qh0 + (h < nh ? h : nh - 1)) * 128 + sub * 8) * 2);
 
   for (int64_t blk = blk_begin; blk < blk_end; blk++) {
     const int t0 = (int)(blk * p.block_seq);
@@ -286,6 +291,7 @@ __global__ __launch_bounds__(NW * 64) void decode_stage1_kernel(Stage1Params p) 
     // merge the four lane groups (and, SPLIT, the waves) and write the block's partial
     __shared__ float xw[SPLIT ? NW : 1][GT][16][10];  // per wave, head and column slot: 8 sums, running max, row sum
     auto write_partial = [&](int h, float M, float L, const float (&ov)[8]) {
+      if (h >= nh) return;
       const float inv = 1.f / L;
       const int64_t row = (blk * p.batch + b) * p.hq + qh0 + h;
       f32x4* dst = (f32x4*)(p.mid_o + row * 128 + sub * 8);
@@ -465,7 +471,7 @@ static int launch_stage1(const lsattn_decode_stage1_args* a, hipStream_t st) {
   p.block_seq = a->seq_block_size;
   p.grid_blocks = (a->max_len_in_batch + a->seq_block_size - 1) / a->seq_block_size;  // stage1.cu:211
   const int group = (int)(a->num_q_heads / a->num_kv_heads);
-  p.tasks = (int)a->num_kv_heads * (group / GT);
+  p.tasks = (int)a->num_kv_heads * ((group + GT - 1) / GT);
   const int wgs_y = (p.tasks + NW - 1) / NW;
   // tokens per workgroup: at least ~1024, and few enough workgroups-per-launch to stay cheap
 #ifndef LSATTN_DECODE_TOK_PER_WG
@@ -498,11 +504,10 @@ static int launch_stage1(const lsattn_decode_stage1_args* a, hipStream_t st) {
 
 template <typename T> static int dispatch_stage1(const lsattn_decode_stage1_args* a, hipStream_t st) {
   const int group = (int)(a->num_q_heads / a->num_kv_heads);
-#ifndef LSATTN_DECODE_MAX_GT
-#define LSATTN_DECODE_MAX_GT 4
-#endif
-  if (group % 4 == 0 && LSATTN_DECODE_MAX_GT >= 4) return launch_stage1<T, 4>(a, st);
-  if (group % 2 == 0) return launch_stage1<T, 2>(a, st);
+  // groups of 3 and more take four query heads per task (a group of 5, 6 or 7 as 4 + the rest, of 3 as one task with a
+  // spare): fetching a K/V row once per four query heads matters more than the spare accumulators cost
+  if (group >= 3) return launch_stage1<T, 4>(a, st);
+  if (group == 2) return launch_stage1<T, 2>(a, st);
   return launch_stage1<T, 1>(a, st);
 }
 
