@@ -83,6 +83,37 @@ def ring_prefill_accumulate(q, chunks: Sequence[KVChunk], q_b_start_loc, q_b_seq
     return out, lse
 
 
+def ring_prefill_with_migration(q, chunks: Sequence[KVChunk], q_b_start_loc, q_b_seq_len, q_first_token_global_idx,
+                                logical_sp_peers_num: int, max_q_len: int, num_kv_heads: int,
+                                kv_cache_index_begin, kv_cache_index_end, mem_index, mem_cache, req_to_token_indexs,
+                                b_req_idx, should_register_kv: bool = True):
+    """The in-place ring with the context migration of longserve_transformer_layer_infer.py:180-220: after each step the
+    rows of the chunk at hand whose global token index falls in this instance's window
+    [kv_cache_index_begin, kv_cache_index_end) are copied into the pool slots `mem_index` hands out, in the order the
+    chunks pass by, and (first layer) registered in the request table after the rows kept so far.  This is how a
+    prefill spread over several instances leaves its KV on fewer of them.  Returns (o, m, l, kept rows per request)."""
+    from .ops import destindex_copy_and_register_kv, pre_copy_and_register_kv
+    o = torch.zeros_like(q)
+    m = torch.full(q.shape[:2], float("-inf"), dtype=torch.float32, device=q.device)
+    l = torch.zeros(q.shape[:2], dtype=torch.float32, device=q.device)
+    batch = q_b_seq_len.shape[0]
+    cur_kv_cache_index = torch.zeros(batch, dtype=torch.int32, device=q.device)
+    num_used_mem_index = 0
+    for c in chunks:
+        context_attention_fwd(q, c.k(num_kv_heads), c.v(num_kv_heads), o, q_b_start_loc, q_b_seq_len,
+                              q_first_token_global_idx, c.b_start_loc, c.b_seq_len, c.first_token_global_idx,
+                              logical_sp_peers_num, max_q_len, m, l)
+        kv_range_begin, kv_range_end, new_kv_cache_len = pre_copy_and_register_kv(
+            kv_cache_index_begin, kv_cache_index_end, c.first_token_global_idx, logical_sp_peers_num)
+        new_kv_cache_len_sum = torch.cumsum(new_kv_cache_len, dim=0, dtype=torch.int64)
+        destindex_copy_and_register_kv(batch, new_kv_cache_len, kv_range_begin, kv_range_end, new_kv_cache_len_sum, c.kv,
+                                       c.b_start_loc, cur_kv_cache_index, mem_index, mem_cache, req_to_token_indexs,
+                                       b_req_idx, num_used_mem_index, max_q_len + 1, should_register_kv)
+        num_used_mem_index += int(new_kv_cache_len_sum[-1].item())  # as the reference: one read-back per step
+        cur_kv_cache_index += new_kv_cache_len
+    return o, m, l, cur_kv_cache_index
+
+
 def next_power_of_2(n: int) -> int:
     return 1 if n <= 1 else 1 << (n - 1).bit_length()
 

@@ -3,6 +3,7 @@ import pytest
 import torch
 
 from oracle import attn_oracle as orc
+from tests.helpers import meta
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -132,3 +133,54 @@ def test_decoding_stage_migration_matches_oracle(lsa, dtype):
     torch.cuda.synchronize()
     assert torch.equal(pool_d.cpu().view(torch.int16), pool_o.view(torch.int16))
     assert torch.equal(table_d.cpu(), table_o)
+
+
+def test_striped_ring_with_scale_down_then_decode(lsa):
+    """The elastic flow end to end: a striped prefill over P = 3 logical instances; rank r keeps, while the chunks pass
+    by, the rows of its window of global token positions (here rank 0 keeps [0, cut) and rank 1 the rest, rank 2 nothing);
+    afterwards a decode token attends to both kept parts through the multi-instance merge.  Prefill rows and the decode
+    result are compared with dense attention over the whole sequence."""
+    from loongserve_amd.simulate import DecodeInstance, KVChunk, multi_instance_decode, ring_prefill_with_migration
+    g = torch.Generator().manual_seed(31)
+    P, N, Hq, Hkv, D = 3, 1000, 8, 2, 128
+    cut = 617
+    q = (torch.randn(N, Hq, D, generator=g) * 0.5).half()
+    kv = (torch.randn(N, 2 * Hkv, D, generator=g) * 0.5).half()
+    m1 = meta([N])
+    o_ref, _ = orc.attn_step(q, kv[:, :Hkv], kv[:, Hkv:], *m1, *m1, 1)
+    chunks = []
+    for j in range(P):
+        kj = kv[j::P].contiguous()
+        st, ln, fr = meta([kj.shape[0]], [j])
+        chunks.append(KVChunk(kj.to(DEV), st.to(DEV), ln.to(DEV), fr.to(DEV)))
+    windows = [(0, cut), (cut, N), (N, N)]
+    kept = []
+    for r in range(P):
+        qi = q[r::P].contiguous().to(DEV)
+        qs, ql, qf = [t.to(DEV) for t in meta([qi.shape[0]], [r])]
+        order = [(r - i) % P for i in range(P)]
+        pool = torch.zeros(2000, 2 * Hkv, D, dtype=torch.float16, device=DEV)
+        table = torch.full((2, N + 8), orc.INT32_PAD, dtype=torch.int32, device=DEV)
+        mem_index = torch.randperm(2000, generator=g)[:N].to(torch.int32).to(DEV)
+        b, e = windows[r]
+        o, _, _, n_kept = ring_prefill_with_migration(qi, [chunks[i] for i in order], qs, ql, qf, P, qi.shape[0], Hkv,
+                                                      _i32([b]).to(DEV), _i32([e]).to(DEV), mem_index, pool, table,
+                                                      _i32([1]).to(DEV))
+        torch.cuda.synchronize()
+        assert (o.float().cpu() - o_ref[r::P]).abs().max().item() <= 2e-3
+        assert int(n_kept[0]) == e - b
+        # the kept rows are the window's tokens, stripe by stripe in the order the chunks passed by
+        want = torch.cat([torch.arange(j, N, P)[(torch.arange(j, N, P) >= b) & (torch.arange(j, N, P) < e)] for j in order])
+        slots = table[1, :e - b].long()
+        assert torch.equal(pool[slots].cpu(), kv[want])
+        assert bool((table[1, e - b:] == orc.INT32_PAD).all())
+        kept.append((pool, table, e - b))
+    # one decode token: instance 0 is the master, instance 1 a peer, instance 2 holds nothing
+    qd = (torch.randn(1, Hq, D, generator=g) * 0.5).half()
+    insts = [DecodeInstance(p, t, _i32([1]).to(DEV), _i32([n]).to(DEV), max(n, 1)) for p, t, n in kept]
+    o, lse = multi_instance_decode(qd.to(DEV), insts, Hkv)
+    torch.cuda.synchronize()
+    t_cpu = torch.arange(N, dtype=torch.int32)[None]
+    o_d, l_d = orc.decode_full(qd, kv[:, :Hkv], kv[:, Hkv:], t_cpu, _i32([0]), _i32([N]))
+    assert (o.float().cpu() - o_d).abs().max().item() <= 2e-3
+    assert torch.allclose(lse.cpu(), l_d, rtol=1e-4, atol=1e-4)
