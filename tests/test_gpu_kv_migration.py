@@ -184,3 +184,42 @@ def test_striped_ring_with_scale_down_then_decode(lsa):
     o_d, l_d = orc.decode_full(qd, kv[:, :Hkv], kv[:, Hkv:], t_cpu, _i32([0]), _i32([N]))
     assert (o.float().cpu() - o_d).abs().max().item() <= 2e-3
     assert torch.allclose(lse.cpu(), l_d, rtol=1e-4, atol=1e-4)
+
+
+def test_decoding_stage_migration_keeps_the_attention_result(lsa):
+    """Scale-out during decoding (longserve_model.py:588-619): instance A hands the last tokens of some requests to
+    instance B; attention over A's remaining tokens merged with B's received ones equals attention over what A held
+    before, and the slots A gave up are free again."""
+    from loongserve_amd.simulate import DecodeInstance, multi_instance_decode
+    g = torch.Generator().manual_seed(43)
+    Hq, Hkv, D, B = 8, 2, 128, 3
+    lens, moved = [900, 300, 64], [400, 0, 64]
+    mm_a = lsa.LongServeMemoryManager(3000, torch.float16, Hkv, D, 1)
+    mm_b = lsa.LongServeMemoryManager(2000, torch.float16, Hkv, D, 1)
+    rm_a, rm_b = lsa.LongServeReqManager(4, 1024, mm_a), lsa.LongServeReqManager(4, 1024, mm_b)
+    mm_a.kv_buffer.copy_((torch.randn(mm_a.kv_buffer.shape, generator=g) * 0.5).half())
+    rows = _i32([2, 0, 3]).to(DEV)
+    b_len = _i32(lens).to(DEV)
+    slots_a = mm_a.alloc(sum(lens))
+    lsa.init_req_to_token_indexes(rm_a.req_to_token_indexs, rows, b_len, slots_a)
+    q = (torch.randn(B, Hq, D, generator=g) * 0.5).half().to(DEV)
+    before, lse_before = multi_instance_decode(q, [DecodeInstance(mm_a.kv_buffer[0], rm_a.req_to_token_indexs, rows, b_len, max(lens))], Hkv)
+    before, lse_before = before.clone(), lse_before.clone()
+    # A sends, B receives into freshly allocated slots of its own pool
+    num = _i32(moved).to(DEV)
+    total = sum(moved)
+    buf = torch.empty(1, total, 2 * Hkv, D, dtype=torch.float16, device=DEV)
+    free_before = mm_a.can_use_mem_size
+    lsa.decoding_stage_migration_sender_kernel(buf, rm_a.req_to_token_indexs, mm_a.mem_state, mm_a.kv_buffer, rows, num, b_len)
+    mm_a.can_use_mem_size += total                         # the sender kernel cleared the reference counts of what it sent
+    assert int((mm_a.mem_state == 0).sum()) == mm_a.can_use_mem_size == free_before + total
+    slots_b = mm_b.alloc(total)
+    held_b = torch.zeros(B, dtype=torch.int32, device=DEV)
+    lsa.decoding_stage_migration_receiver_kernel(buf, rm_b.req_to_token_indexs, mm_b.kv_buffer, slots_b, rows, num, held_b)  # int64 slots, as alloc returns them
+    len_a, len_b = b_len - num, num
+    after, lse_after = multi_instance_decode(q, [
+        DecodeInstance(mm_a.kv_buffer[0], rm_a.req_to_token_indexs, rows, len_a, max(lens)),
+        DecodeInstance(mm_b.kv_buffer[0], rm_b.req_to_token_indexs, rows, len_b, max(max(moved), 1))], Hkv)
+    torch.cuda.synchronize()
+    assert (after.float() - before.float()).abs().max().item() <= 2e-3
+    assert torch.allclose(lse_after, lse_before, rtol=1e-4, atol=1e-4)
