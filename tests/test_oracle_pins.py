@@ -542,3 +542,22 @@ def test_pool_oracle_reference_counts_and_duplicates():
                 held.append(got[0].copy() if got is not None else m.alloc(need).copy())
         assert m.can_use_mem_size == int((m.mem_state == 0).sum())
         assert sum(len(h) for h in held) == int(m.mem_state.sum())
+
+
+def test_oracle_against_the_committed_known_answers():
+    """tests/golden/attention_known_answers.npz: answers computed once by float64 loops over the definition
+    (tests/golden/make_fixtures.py, no oracle code); the oracle must reproduce them."""
+    import os
+    import numpy as np
+    z = np.load(os.path.join(os.path.dirname(__file__), "golden", "attention_known_answers.npz"))
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a))
+    cum = lambda ln: torch.cumsum(t(ln), 0).to(torch.int32) - t(ln)
+    o, lse = orc.attn_step(t(z["pf_q"]), t(z["pf_k"]), t(z["pf_v"]), cum(z["pf_q_len"]), t(z["pf_q_len"]), t(z["pf_q_first"]),
+                           cum(z["pf_kv_len"]), t(z["pf_kv_len"]), t(z["pf_kv_first"]), int(z["pf_peers"]), dtype=torch.float64)
+    assert torch.allclose(o, t(z["pf_o"]), atol=1e-12) and torch.allclose(lse, t(z["pf_lse"]), atol=1e-12)
+    assert torch.equal(torch.isinf(lse), torch.isinf(t(z["pf_lse"])))
+    Hkv = z["dc_pool"].shape[1] // 2
+    pool = t(z["dc_pool"])
+    o, lse = orc.decode_full(t(z["dc_q"]), pool[:, :Hkv], pool[:, Hkv:], t(z["dc_table"]), t(z["dc_b_req"]), t(z["dc_b_len"]),
+                             dtype=torch.float64)
+    assert torch.allclose(o, t(z["dc_o"]), atol=1e-12) and torch.allclose(lse, t(z["dc_lse"]), atol=1e-12)
