@@ -445,10 +445,7 @@ __global__ __launch_bounds__(NT) void decode_stage2_kernel(Stage2Params p) {
 
 template <typename T, int GT>
 static int launch_stage1(const lsattn_decode_stage1_args* a, hipStream_t st) {
-#ifndef LSATTN_DECODE_NW
-#define LSATTN_DECODE_NW 4
-#endif
-  constexpr int NW = LSATTN_DECODE_NW;
+  constexpr int NW = 4;  // waves (tasks) per workgroup; 8 measured no faster
   Stage1Params p;
   p.mid_o = a->mid_o;
   p.mid_lse = a->mid_o_logexpsum;
@@ -473,11 +470,10 @@ static int launch_stage1(const lsattn_decode_stage1_args* a, hipStream_t st) {
   const int group = (int)(a->num_q_heads / a->num_kv_heads);
   p.tasks = (int)a->num_kv_heads * ((group + GT - 1) / GT);
   const int wgs_y = (p.tasks + NW - 1) / NW;
-  // tokens per workgroup: at least ~1024, and few enough workgroups-per-launch to stay cheap
-#ifndef LSATTN_DECODE_TOK_PER_WG
-#define LSATTN_DECODE_TOK_PER_WG 256
-#endif
-  int64_t per_wg = (LSATTN_DECODE_TOK_PER_WG + a->seq_block_size - 1) / a->seq_block_size;
+  // a workgroup walks consecutive blocks until it has covered at least 256 tokens (smaller units measured slower for
+  // short blocks, larger ones lose to tail imbalance)
+  constexpr int64_t kTokensPerWorkgroup = 256;
+  int64_t per_wg = (kTokensPerWorkgroup + a->seq_block_size - 1) / a->seq_block_size;
   if (per_wg < 1) per_wg = 1;
   int64_t nblk = p.grid_blocks < a->num_blocks ? p.grid_blocks : a->num_blocks;
   if (nblk < 1) return LSATTN_OK;
