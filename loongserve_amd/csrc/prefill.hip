@@ -25,8 +25,9 @@
 //     other does the exponentials of its own step, a workgroup barrier ends each phase;
 //   * tiles that straddle the diagonal or the end of the KV chunk take a general, masked,
 //     bounds-checked step; causal work is skipped per wave;
-//   * workgroup ids are mapped so that the workgroups sharing one KV head run on one XCD
-//     (ids are dealt round-robin to the 8 XCDs) and heavy (late) query tiles start first.
+//   * workgroup ids are mapped so that the workgroups sharing one KV head run on one XCD (ids are dealt
+//     round-robin to the 8 XCDs; with fewer KV heads than XCDs a head's work is dealt to several of them)
+//     and heavy (late) query tiles start first.
 //   * one kernel, three epilogues (MODE): 0 writes the step's fp32 partial (O, LSE) from the empty state, 1 folds the
 //     step into the reference's in-place (o, m, l) state (ring_context_flashattention_nopad.py:171-188), 2 LSE-merges it
 //     into a running fp32 (O, LSE); the folding ones read the old state of both row blocks of a wave at once.
@@ -47,7 +48,7 @@ struct PrefillParams {
   const int32_t* kv_start;
   const int32_t* kv_len;
   const int32_t* kv_first;
-  int32_t batch, hq, hkv, peers, nz, kv_slots;
+  int32_t batch, hq, hkv, peers, nz, kv_slots, slices, units_per_slice;
   float scale_log2;
   void* o;
   int64_t o_st, o_sh;
@@ -248,17 +249,21 @@ template <typename T, int MODE, bool DV>
 __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p) {
   __shared__ __attribute__((aligned(1024))) char lds[kLdsBytes];
 
+  // Workgroup ids go to the 8 XCDs round-robin.  The (query head, query tile) units of one KV head are dealt to p.slices
+  // XCDs (1 when the KV heads are a multiple of 8, else as many as it takes for hkv * slices to be one), so that the
+  // workgroups sharing a KV head's K/V meet in few L2s and every XCD has work whatever the head count.
   const int group = p.hq / p.hkv;
   int j = blockIdx.x >> 3;
   const int xcd = blockIdx.x & 7;
-  const int gq = j % group;
-  j /= group;
-  const int zr = j % p.nz;
-  j /= p.nz;
+  const int up = j % p.units_per_slice;
+  j /= p.units_per_slice;
   const int slot = j % p.kv_slots;
   const int b = j / p.kv_slots;
-  const int kvh = xcd + 8 * slot;
-  if (kvh >= p.hkv) return;
+  const int vh = xcd + 8 * slot;  // (KV head, slice) pair: always < hkv * slices
+  const int kvh = vh / p.slices;
+  const int u = up * p.slices + vh % p.slices;
+  if (u >= group * p.nz) return;
+  const int gq = u % group, zr = u / group;
   const int h = kvh * group + gq;
   const int z = p.nz - 1 - zr;
 
@@ -812,7 +817,12 @@ template <typename T, int MODE, bool DV> static int launch_prefill(const lsattn_
   p.hkv = a->num_kv_heads;
   p.peers = a->sp_peers;
   p.nz = (a->max_q_len + BM - 1) / BM;
-  p.kv_slots = (a->num_kv_heads + 7) / 8;
+  {
+    int g8 = 8;  // gcd(num_kv_heads, 8)
+    while (a->num_kv_heads % g8) g8 >>= 1;
+    p.slices = 8 / g8;
+    p.kv_slots = a->num_kv_heads / g8;  // hkv * slices / 8
+  }
   p.scale_log2 = a->sm_scale * kLog2e;
   p.o = a->o;
   p.o_st = a->o_stride_t;
@@ -823,7 +833,8 @@ template <typename T, int MODE, bool DV> static int launch_prefill(const lsattn_
   p.ml_st = a->ml_stride_t;
   p.ml_sh = a->ml_stride_h;
   const int group = a->num_q_heads / a->num_kv_heads;
-  const int64_t wgs = (int64_t)8 * group * p.nz * p.kv_slots * a->batch;
+  p.units_per_slice = (int32_t)(((int64_t)group * p.nz + p.slices - 1) / p.slices);
+  const int64_t wgs = (int64_t)8 * p.units_per_slice * p.kv_slots * a->batch;
   if (wgs > 0x7fffffff) return LSATTN_ERR_INVALID_ARG;
   hipLaunchKernelGGL((prefill_kernel<T, MODE, DV>), dim3((unsigned)wgs), dim3(NWAVE * 64), 0, st, p);
   return check_launch();
