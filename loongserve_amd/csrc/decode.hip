@@ -68,7 +68,10 @@ template <> struct Dot<BF16> {
 // SPLIT: the NW waves of a workgroup share one task and take every NW-th batch of 32 tokens of a block; their partials
 // meet in LDS.  For launches too small to fill the chip otherwise (short contexts at small batch): NW times as many rows
 // in flight.
-template <typename T, int GT, int NW, bool SPLIT>
+// ONCE: every K/V row is read by one wave only (at most GT query heads per KV head), so the rows are loaded
+// non-temporally; otherwise the waves that take the other query heads of the group read them again and ordinary loads let
+// those find the rows in L2.
+template <typename T, int GT, int NW, bool SPLIT, bool ONCE>
 __global__ __launch_bounds__(NW * 64) void decode_stage1_kernel(Stage1Params p) {
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -147,12 +150,14 @@ __global__ __launch_bounds__(NW * 64) void decode_stage1_kernel(Stage1Params p) 
 #pragma unroll
       for (int j = 0; j < kTok; j++) {
         asm volatile("" : "+v"(slot[j]));
-        kr[j] = __builtin_nontemporal_load((const u32x4*)(kbase + (int64_t)slot[j] * k_row_bytes));
+        kr[j] = ONCE ? __builtin_nontemporal_load((const u32x4*)(kbase + (int64_t)slot[j] * k_row_bytes))
+                     : *(const u32x4*)(kbase + (int64_t)slot[j] * k_row_bytes);
       }
 #pragma unroll
       for (int j = 0; j < kTok; j++) {
         asm volatile("" : "+v"(slot[j]));
-        vr[j] = __builtin_nontemporal_load((const u32x4*)(vbase + (int64_t)slot[j] * v_row_bytes));
+        vr[j] = ONCE ? __builtin_nontemporal_load((const u32x4*)(vbase + (int64_t)slot[j] * v_row_bytes))
+                     : *(const u32x4*)(vbase + (int64_t)slot[j] * v_row_bytes);
       }
       // The rows are read once: non-temporal loads.  As ordinary loads they push the block partials (which stage 2
       // reads back) out of the caches early, and the trickle of write-backs between the reads costs the gather 5 %.
@@ -483,18 +488,21 @@ static int launch_stage1(const lsattn_decode_stage1_args* a, hipStream_t st) {
   // A launch of less than one workgroup per CU leaves most of the chip's load slots empty: the waves of a workgroup then
   // share one task and split each block's tokens (measured: 64 workgroups, one request of 8192 tokens with 8 KV heads,
   // 19.9 -> 10.0 us; from 256 workgroups on it gains nothing; blocks shorter than 32 tokens per wave cannot use it).
+  const bool once = group <= GT;
   const bool split = chunks * wgs_y * a->batch < 256 && a->seq_block_size >= 32 * NW && p.tasks <= 65535;
   if (split) {
     p.tasks_on_x = chunks <= 65535;
     dim3 grid = p.tasks_on_x ? dim3((unsigned)p.tasks, (unsigned)chunks, (unsigned)a->batch)
                              : dim3((unsigned)chunks, (unsigned)p.tasks, (unsigned)a->batch);
-    hipLaunchKernelGGL((decode_stage1_kernel<T, GT, NW, true>), grid, dim3(NW * 64), 0, st, p);
+    if (once) hipLaunchKernelGGL((decode_stage1_kernel<T, GT, NW, true, true>), grid, dim3(NW * 64), 0, st, p);
+    else hipLaunchKernelGGL((decode_stage1_kernel<T, GT, NW, true, false>), grid, dim3(NW * 64), 0, st, p);
     return check_launch();
   }
   p.tasks_on_x = wgs_y <= 2 && chunks <= 65535;  // with more task groups per chunk (MHA, 32 KV heads) it measured 2 % slower
   dim3 grid = p.tasks_on_x ? dim3((unsigned)wgs_y, (unsigned)chunks, (unsigned)a->batch)
                            : dim3((unsigned)chunks, (unsigned)wgs_y, (unsigned)a->batch);
-  hipLaunchKernelGGL((decode_stage1_kernel<T, GT, NW, false>), grid, dim3(NW * 64), 0, st, p);
+  if (once) hipLaunchKernelGGL((decode_stage1_kernel<T, GT, NW, false, true>), grid, dim3(NW * 64), 0, st, p);
+  else hipLaunchKernelGGL((decode_stage1_kernel<T, GT, NW, false, false>), grid, dim3(NW * 64), 0, st, p);
   return check_launch();
 }
 
