@@ -527,7 +527,7 @@ def main():
                                    "2.5M-slot scattered pool; fused stage1 + stage2 call with BLOCK_SEQ %d (mid_o is scratch there: "
                                    "split-K at %d tokens between the stages)" % (d.BS, d.split),
                        "tokens": d.tokens, "algorithmic_gb_per_step": d.bytes / 1e9, "step_stats": st},
-            "roofline": {"kernel": "decode_stage1_kernel<F16,4,4,false>", "bound": "hbm", "achieved": ach, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+            "roofline": {"kernel": "decode_stage1_kernel<F16,4,4,false,true>", "bound": "hbm", "achieved": ach, "peak": PEAK_HBM_GBS, "unit": "GB/s",
                          "frac": ach / PEAK_HBM_GBS,
                          # HBM bytes per launch (read 5174.6 MB + written 20.8 MB), same source as above
                          "traffic": 5195.4e6, "per_launch_ms": s1},
