@@ -173,6 +173,14 @@ class TokenDecode:
                                                             self.max_len, self.Hq, self.D, self.kv[:, :self.Hkv], self.kv[:, self.Hkv:],
                                                             self.BS, self.o, self.lse)
 
+    def step_separate_stages(self):
+        """Stage 1 and stage 2 as two calls at BLOCK_SEQ, the way the master of a decode step makes them
+        (longserve_transformer_layer_infer.py:272-281, :360-367)."""
+        import loongserve_amd as lsa
+        lsa.longserve_flash_decode_stage1(self.q, self.kv[:, :self.Hkv], self.kv[:, self.Hkv:], self.table, self.b_req, self.b_len,
+                                          self.max_len, self.mid_o, self.mid_l, self.BS)
+        lsa.longserve_flash_decode_stage2(self.mid_o, self.mid_l, self.b_len, self.o, self.lse, self.BS)
+
     def stage1_only(self):
         import loongserve_amd as lsa
         lsa.longserve_flash_decode_stage1(self.q, self.kv[:, :self.Hkv], self.kv[:, self.Hkv:], self.table, self.b_req, self.b_len,
@@ -517,6 +525,7 @@ def main():
         dsteps = max(args.steps, 10)
         d_ms = _time_events(d.step, dsteps, max(args.warmup, 2))
         s1_ms = _time_events(d.stage1_only, dsteps, 1)
+        sep = _stats(_time_events(d.step_separate_stages, dsteps, 2))
         st = _stats(d_ms)
         gbs = d.bytes / (st["mean_ms"] * 1e-3) / 1e9
         s1 = sum(s1_ms) / len(s1_ms)
@@ -526,7 +535,10 @@ def main():
             "config": {"workload": "config 3: token-indexed decode, batch 64, ctx U[4096,32768], GQA 32/8, head_dim 128, fp16, "
                                    "2.5M-slot scattered pool; fused stage1 + stage2 call with BLOCK_SEQ %d (mid_o is scratch there: "
                                    "split-K at %d tokens between the stages)" % (d.BS, d.split),
-                       "tokens": d.tokens, "algorithmic_gb_per_step": d.bytes / 1e9, "step_stats": st},
+                       "tokens": d.tokens, "algorithmic_gb_per_step": d.bytes / 1e9, "step_stats": st,
+                       "separate_stages": {"what": "stage 1 and stage 2 as two calls at BLOCK_SEQ %d (the master path of a decode "
+                                                   "step); stage 1 merges groups of blocks into one partial" % d.BS,
+                                           "ms_per_step": sep["mean_ms"], "value": d.bytes / (sep["mean_ms"] * 1e-3) / 1e9}},
             "roofline": {"kernel": "decode_stage1_kernel<F16,4,4,false,true>", "bound": "hbm", "achieved": ach, "peak": PEAK_HBM_GBS, "unit": "GB/s",
                          "frac": ach / PEAK_HBM_GBS,
                          # HBM bytes per launch (read 5174.6 MB + written 20.8 MB), same source as above

@@ -150,6 +150,12 @@ typedef struct lsattn_decode_stage1_args {
   int64_t max_seq_len;     /* req_to_tokens.size(1) */
   int64_t seq_block_size;  /* tokens per partial, >= 1 */
   int64_t max_len_in_batch;
+  int64_t merge_blocks;    /* 0 or 1: one partial per block, as the reference.  m in 2..16: one partial per m consecutive
+                              blocks, written to the row of the first of them; the rows of the others (as far as the
+                              request reaches) get LSE = -inf, i.e. "empty", and their mid_o is left alone.  Any LSE
+                              merge over the rows (stage 2 with the same seq_block_size, or with block_seq = 1 and the
+                              block count as length, longserve_model.py:514-516) gives the same result with a quarter
+                              (m = 4) of the partial bytes written while the gather runs */
 } lsattn_decode_stage1_args;
 int lsattn_decode_stage1(const lsattn_decode_stage1_args* a, void* stream);
 

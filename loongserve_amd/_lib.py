@@ -52,6 +52,7 @@ class DecodeStage1Args(C.Structure):
         ("req_to_tokens", _vp), ("b_req_idx", _vp), ("b_seqlen", _vp),
         ("batch", _i64), ("num_q_heads", _i64), ("num_kv_heads", _i64), ("num_blocks", _i64),
         ("head_dim", _i64), ("max_seq_len", _i64), ("seq_block_size", _i64), ("max_len_in_batch", _i64),
+        ("merge_blocks", _i64),
     ]
 
 

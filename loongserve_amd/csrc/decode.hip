@@ -30,7 +30,8 @@ struct Stage1Params {
   const int32_t* req_to_tokens;
   const int32_t* b_req_idx;
   const int32_t* b_seqlen;
-  int64_t batch, hq, hkv, num_blocks, max_seq_len, block_seq, grid_blocks;
+  int64_t batch, hq, hkv, num_blocks, max_seq_len, block_seq, grid_blocks;  // block_seq: tokens per partial computed
+  int64_t row_mul, fine_block_seq;  // partial of coarse block i goes to row i * row_mul; rows in between are marked empty
   int32_t blocks_per_wg;  // consecutive blocks walked by one workgroup
   int32_t tasks;          // hkv * (group / GT) wave tasks
   int32_t tasks_on_x;     // grid = (task groups, chunks, batch) instead of (chunks, task groups, batch)
@@ -96,7 +97,9 @@ __global__ __launch_bounds__(NW * 64) void decode_stage1_kernel(Stage1Params p) 
   const int len = p.b_seqlen[b];  // positions inside a request are 32-bit (max_seq_len is checked on the host)
   int64_t nblk = len <= 0 ? 0 : ((int64_t)len + p.block_seq - 1) / p.block_seq;
   if (nblk > p.grid_blocks) nblk = p.grid_blocks;
-  if (nblk > p.num_blocks) nblk = p.num_blocks;
+  if (nblk > (p.num_blocks + p.row_mul - 1) / p.row_mul) nblk = (p.num_blocks + p.row_mul - 1) / p.row_mul;
+  int64_t fine_nblk = len <= 0 ? 0 : ((int64_t)len + p.fine_block_seq - 1) / p.fine_block_seq;  // rows the request reaches
+  if (fine_nblk > p.num_blocks) fine_nblk = p.num_blocks;
   // Workgroups go to the 8 XCDs round-robin in linear id order, so a fixed chunk index always lands on the same XCDs and
   // the first chunks (all that short requests have) would load some XCDs more than others; the chunk index is rotated by
   // the request index to spread them (batch 64 with lengths 4096..32768: 5.62 -> 5.9 TB/s).
@@ -298,11 +301,14 @@ __global__ __launch_bounds__(NW * 64) void decode_stage1_kernel(Stage1Params p) 
     auto write_partial = [&](int h, float M, float L, const float (&ov)[8]) {
       if (h >= nh) return;
       const float inv = 1.f / L;
-      const int64_t row = (blk * p.batch + b) * p.hq + qh0 + h;
+      const int64_t row = (blk * p.row_mul * p.batch + b) * p.hq + qh0 + h;
       f32x4* dst = (f32x4*)(p.mid_o + row * 128 + sub * 8);
       dst[0] = f32x4{ov[0] * inv, ov[1] * inv, ov[2] * inv, ov[3] * inv};
       dst[1] = f32x4{ov[4] * inv, ov[5] * inv, ov[6] * inv, ov[7] * inv};
       if (sub == 0) p.mid_lse[row] = (M + __builtin_amdgcn_logf(L)) * kLn2;
+      // the rows of the blocks merged into this partial (row_mul <= 16: lane `sub` takes the sub-th of them)
+      if (sub >= 1 && sub < p.row_mul && blk * p.row_mul + sub < fine_nblk)
+        p.mid_lse[((blk * p.row_mul + sub) * p.batch + b) * p.hq + qh0 + h] = -INFINITY;
     };
 #pragma unroll
     for (int h = 0; h < GT; h++) {
@@ -410,17 +416,21 @@ __global__ __launch_bounds__(NT) void decode_stage2_kernel(Stage2Params p) {
     float lse[U];
     f32x4 tv[U];
 #pragma unroll
+    for (int u = 0; u < U; u++) lse[u] = p.mid_lse[(i + u * SL) * row_stride + row0];
+    // an empty partial's row of mid_o is not read (stage 1 leaves the rows it merged into another one untouched)
+#pragma unroll
     for (int u = 0; u < U; u++) {
       const int64_t row = (i + u * SL) * row_stride + row0;
-      lse[u] = p.mid_lse[row];
-      tv[u] = *(const f32x4*)(p.mid_o + row * D + c * 4);
+      tv[u] = f32x4{0.f, 0.f, 0.f, 0.f};
+      if (lse[u] != -INFINITY) tv[u] = *(const f32x4*)(p.mid_o + row * D + c * 4);
     }
 #pragma unroll
     for (int u = 0; u < U; u++) fold(lse[u], tv[u]);
   }
   for (; i < n; i += SL) {
     const int64_t row = i * row_stride + row0;
-    fold(p.mid_lse[row], *(const f32x4*)(p.mid_o + row * D + c * 4));
+    const float lse = p.mid_lse[row];
+    if (lse != -INFINITY) fold(lse, *(const f32x4*)(p.mid_o + row * D + c * 4));
   }
   __shared__ float sM[SL], sL[SL];
   __shared__ f32x4 sAcc[SL][LPR];
@@ -470,17 +480,20 @@ static int launch_stage1(const lsattn_decode_stage1_args* a, hipStream_t st) {
   p.hkv = a->num_kv_heads;
   p.num_blocks = a->num_blocks;
   p.max_seq_len = a->max_seq_len;
-  p.block_seq = a->seq_block_size;
-  p.grid_blocks = (a->max_len_in_batch + a->seq_block_size - 1) / a->seq_block_size;  // stage1.cu:211
+  p.row_mul = a->merge_blocks > 1 ? a->merge_blocks : 1;
+  p.fine_block_seq = a->seq_block_size;
+  p.block_seq = a->seq_block_size * p.row_mul;
+  p.grid_blocks = (a->max_len_in_batch + p.block_seq - 1) / p.block_seq;  // stage1.cu:211, in partials computed
   const int group = (int)(a->num_q_heads / a->num_kv_heads);
   p.tasks = (int)a->num_kv_heads * ((group + GT - 1) / GT);
   const int wgs_y = (p.tasks + NW - 1) / NW;
   // a workgroup walks consecutive blocks until it has covered at least 256 tokens (smaller units measured slower for
   // short blocks, larger ones lose to tail imbalance)
   constexpr int64_t kTokensPerWorkgroup = 256;
-  int64_t per_wg = (kTokensPerWorkgroup + a->seq_block_size - 1) / a->seq_block_size;
+  int64_t per_wg = (kTokensPerWorkgroup + p.block_seq - 1) / p.block_seq;
   if (per_wg < 1) per_wg = 1;
-  int64_t nblk = p.grid_blocks < a->num_blocks ? p.grid_blocks : a->num_blocks;
+  const int64_t rows_avail = (a->num_blocks + p.row_mul - 1) / p.row_mul;
+  int64_t nblk = p.grid_blocks < rows_avail ? p.grid_blocks : rows_avail;
   if (nblk < 1) return LSATTN_OK;
   p.blocks_per_wg = (int32_t)per_wg;
   const int64_t chunks = (nblk + per_wg - 1) / per_wg;
@@ -489,7 +502,7 @@ static int launch_stage1(const lsattn_decode_stage1_args* a, hipStream_t st) {
   // share one task and split each block's tokens (measured: 64 workgroups, one request of 8192 tokens with 8 KV heads,
   // 19.9 -> 10.0 us; from 256 workgroups on it gains nothing; blocks shorter than 32 tokens per wave cannot use it).
   const bool once = group <= GT;
-  const bool split = chunks * wgs_y * a->batch < 256 && a->seq_block_size >= 32 * NW && p.tasks <= 65535;
+  const bool split = chunks * wgs_y * a->batch < 256 && p.block_seq >= 32 * NW && p.tasks <= 65535;
   if (split) {
     p.tasks_on_x = chunks <= 65535;
     dim3 grid = p.tasks_on_x ? dim3((unsigned)p.tasks, (unsigned)chunks, (unsigned)a->batch)
@@ -522,6 +535,8 @@ using namespace lsattn;
 extern "C" int lsattn_decode_stage1(const lsattn_decode_stage1_args* a, void* stream) {
   if (!a || !a->mid_o || !a->mid_o_logexpsum || !a->q || !a->k || !a->v || !a->req_to_tokens || !a->b_req_idx ||
       !a->b_seqlen)
+    return LSATTN_ERR_INVALID_ARG;
+  if (a->merge_blocks < 0 || a->merge_blocks > 16 || a->seq_block_size * (a->merge_blocks > 1 ? a->merge_blocks : 1) > 0x40000000)
     return LSATTN_ERR_INVALID_ARG;
   if (a->batch < 0 || a->num_q_heads <= 0 || a->num_kv_heads <= 0 || a->num_blocks < 0 || a->seq_block_size < 1 ||
       a->max_len_in_batch < 0 || a->max_seq_len < 0 || a->max_seq_len > 0x7fffff00)  // 32-bit token positions in the kernel

@@ -8,10 +8,22 @@ import torch
 from . import longserve_cuda_kernels
 
 
+# The stage functions called on their own (the master path, longserve_transformer_layer_infer.py:272-281 then :360-367)
+# must leave rows that an LSE merge over ceil(len / block_seq) rows per request turns into the right result; nothing in
+# the reference looks at a single block's partial.  With this switch on, stage 1 computes one partial per group of
+# consecutive blocks (the same rule as the fused call below, at most 16 blocks), writes it to the row of the group's first
+# block and marks the rows of the others empty (LSE = -inf): a quarter of the partial bytes at BLOCK_SEQ 256, and the
+# separate calls run as fast as the fused one.  Off: one partial per block, exactly the reference's buffers.
+STAGE1_MERGES_BLOCKS = True
+
+
 def longserve_flash_decode_stage1(q, k, v, Req_to_tokens, B_req_idx, B_Seqlen, max_len_in_batch, mid_out,
                                   mid_out_logsumexp, block_seq):
+    merge = 1
+    if STAGE1_MERGES_BLOCKS:
+        merge = min(16, _fused_block_seq(block_seq, q.shape[0], max_len_in_batch, k.shape[1]) // int(block_seq))
     longserve_cuda_kernels.flash_decoding_stage1(mid_out, mid_out_logsumexp, q, k, v, Req_to_tokens, B_req_idx,
-                                                 B_Seqlen, max_len_in_batch, block_seq)
+                                                 B_Seqlen, max_len_in_batch, block_seq, merge)
     return
 
 

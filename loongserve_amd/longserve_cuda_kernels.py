@@ -25,7 +25,7 @@ def _req(cond: bool, what: str) -> None:
 
 
 def _stage1_args(mid_o, mid_o_logexpsum, q, k, v, req_to_tokens, b_req_idx, b_seqlen,
-                 max_len_in_batch: int, seq_block_size: int) -> _lib.DecodeStage1Args:
+                 max_len_in_batch: int, seq_block_size: int, merge_blocks: int = 1) -> _lib.DecodeStage1Args:
     """The checks of ENTRY:115-160 and the argument block of lsattn_decode_stage1."""
     # ENTRY:115-122
     _req(mid_o.is_contiguous(), "mid_o.is_contiguous()")
@@ -68,14 +68,18 @@ def _stage1_args(mid_o, mid_o_logexpsum, q, k, v, req_to_tokens, b_req_idx, b_se
     a.batch, a.num_q_heads, a.num_kv_heads = B, Hq, k.size(1)
     a.num_blocks, a.head_dim, a.max_seq_len = mid_o.size(0), D, req_to_tokens.size(1)
     a.seq_block_size, a.max_len_in_batch = int(seq_block_size), int(max_len_in_batch)
+    _req(1 <= int(merge_blocks) <= 16, "1 <= merge_blocks <= 16")
+    a.merge_blocks = int(merge_blocks)
     return a
 
 
 @torch.inference_mode()
 def flash_decoding_stage1(mid_o, mid_o_logexpsum, q, k, v, req_to_tokens, b_req_idx, b_seqlen,
-                          max_len_in_batch: int, seq_block_size: int) -> None:
-    """ENTRY:103-164, same argument order."""
-    a = _stage1_args(mid_o, mid_o_logexpsum, q, k, v, req_to_tokens, b_req_idx, b_seqlen, max_len_in_batch, seq_block_size)
+                          max_len_in_batch: int, seq_block_size: int, merge_blocks: int = 1) -> None:
+    """ENTRY:103-164, same argument order.  merge_blocks > 1 (not in the reference): one partial per that many consecutive
+    blocks, in the row of the first; the rows of the others are marked empty (LSE = -inf)."""
+    a = _stage1_args(mid_o, mid_o_logexpsum, q, k, v, req_to_tokens, b_req_idx, b_seqlen, max_len_in_batch, seq_block_size,
+                     merge_blocks)
     _lib.check(_lib.load().lsattn_decode_stage1(C.byref(a), _stream()), "lsattn_decode_stage1")
 
 

@@ -124,6 +124,17 @@ def test_validation_rejects_bad_arguments_without_gpu():
     s2.mid_o = 0x1000
     s1.seq_block_size, s2.block_seq = 256, 128
     assert lib.lsattn_decode_attention(C.byref(s1), C.byref(s2), None) == -1
+    # stage 1 merges at most 16 blocks into one partial
+    s3 = _lib.DecodeStage1Args()
+    for f in ("mid_o", "mid_o_logexpsum", "q", "k", "v", "req_to_tokens", "b_req_idx", "b_seqlen"):
+        setattr(s3, f, 0x1000)
+    s3.batch, s3.num_q_heads, s3.num_kv_heads, s3.num_blocks, s3.head_dim = 1, 4, 2, 4, 128
+    s3.max_seq_len, s3.seq_block_size, s3.max_len_in_batch, s3.dtype = 1024, 256, 1024, _lib.LSATTN_F16
+    s3.k_stride_0 = s3.v_stride_0 = 512
+    s3.k_stride_1 = s3.v_stride_1 = 128
+    for bad in (-1, 17):
+        s3.merge_blocks = bad
+        assert lib.lsattn_decode_stage1(C.byref(s3), None) == -1, bad
 
 
 def test_python_wrappers_reject_cpu_tensors():

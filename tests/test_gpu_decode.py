@@ -25,11 +25,35 @@ def test_stage1_stage2_vs_oracle(lsa, dtype, Hq, Hkv, BS):
     mid_l = torch.full((nblk, B, Hq), float("nan"))
     orc.decode_stage1(q, k, v, table, b_req, b_len, max(lens), mid_o, mid_l, BS)
     kvd = kv.to(DEV)
+    from loongserve_amd import decoding
+    # first with groups of blocks merged into one partial (the default of the stage function called on its own): the rows
+    # of a group's other blocks are marked empty, rows past the request stay untouched, and the merge gives the same result
+    assert decoding.STAGE1_MERGES_BLOCKS
     mo_d = torch.full((nblk, B, Hq, D), float("nan"), device=DEV)
     ml_d = torch.full((nblk, B, Hq), float("nan"), device=DEV)
     lsa.longserve_flash_decode_stage1(q.to(DEV), kvd[:, :Hkv], kvd[:, Hkv:], table.to(DEV), b_req.to(DEV),
                                       b_len.to(DEV), max(lens), mo_d, ml_d, BS)
+    o_d = torch.empty(B, Hq, D, device=DEV)
+    l_d = torch.empty(B, Hq, device=DEV)
+    lsa.longserve_flash_decode_stage2(mo_d, ml_d, b_len.to(DEV), o_d, l_d, BS)
     torch.cuda.synchronize()
+    assert torch.equal(torch.isnan(ml_d.cpu()), torch.isnan(mid_l))                 # the same rows are written
+    merge = min(16, decoding._fused_block_seq(BS, B, max(lens), Hkv) // BS)
+    first = (torch.arange(nblk) % merge == 0)[:, None, None]
+    assert bool((torch.isinf(ml_d.cpu()) == (~first & ~torch.isnan(mid_l))).all())   # -inf exactly on a group's other rows
+    o_ref, l_ref = orc.decode_full(q, k, v, table, b_req, b_len)
+    assert_o_close(o_d, o_ref, "o from merged groups")
+    assert_lse_close(l_d, l_ref, "lse from merged groups")
+    # then one partial per block, the reference's buffers
+    decoding.STAGE1_MERGES_BLOCKS = False
+    try:
+        mo_d = torch.full((nblk, B, Hq, D), float("nan"), device=DEV)
+        ml_d = torch.full((nblk, B, Hq), float("nan"), device=DEV)
+        lsa.longserve_flash_decode_stage1(q.to(DEV), kvd[:, :Hkv], kvd[:, Hkv:], table.to(DEV), b_req.to(DEV),
+                                          b_len.to(DEV), max(lens), mo_d, ml_d, BS)
+        torch.cuda.synchronize()
+    finally:
+        decoding.STAGE1_MERGES_BLOCKS = True
     # blocks past a request's length are left untouched, like the reference
     written = ~torch.isnan(mid_l)
     assert torch.equal(torch.isnan(ml_d.cpu()), ~written)
