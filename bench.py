@@ -539,7 +539,7 @@ def main():
                        "separate_stages": {"what": "stage 1 and stage 2 as two calls at BLOCK_SEQ %d (the master path of a decode "
                                                    "step); stage 1 merges groups of blocks into one partial" % d.BS,
                                            "ms_per_step": sep["mean_ms"], "value": d.bytes / (sep["mean_ms"] * 1e-3) / 1e9}},
-            "roofline": {"kernel": "decode_stage1_kernel<F16,4,4,false,true>", "bound": "hbm", "achieved": ach, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+            "roofline": {"kernel": "decode_stage1_kernel<F16,4,4,false,true,1>", "bound": "hbm", "achieved": ach, "peak": PEAK_HBM_GBS, "unit": "GB/s",
                          "frac": ach / PEAK_HBM_GBS,
                          # HBM bytes per launch (read 5174.6 MB + written 20.8 MB), same source as above
                          "traffic": 5195.4e6, "per_launch_ms": s1},

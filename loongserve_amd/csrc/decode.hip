@@ -3,9 +3,9 @@
 //
 // Stage 1 replaces flash_decoding_stage1_kernel
 // (longserve_cuda_kernels/src/flash_decoding_stage1.cu:25-143).  Differences by design:
-//   * one wave64 serves one KV head and up to four query heads of its GQA group (larger groups take
-//     several waves, sizes that are not a multiple of four a last wave with spare accumulators), so a
-//     K/V row is fetched once per four query heads instead of once per query head;
+//   * one wave64 serves one KV head and up to eight query heads of its GQA group (four at a time, in
+//     up to two rounds over the rows it has loaded; larger groups take several waves), so a K/V row is
+//     fetched once per group instead of once per query head;
 //   * a K/V row of 128 16-bit elements is read by 16 lanes x 16 bytes; a wave has four
 //     such lane groups and every group keeps 8 K rows and 8 V rows in flight;
 //   * each lane group runs its own online softmax; groups are merged once per block with
@@ -72,8 +72,9 @@ template <> struct Dot<BF16> {
 // ONCE: every K/V row is read by one wave only (at most GT query heads per KV head), so the rows are loaded
 // non-temporally; otherwise the waves that take the other query heads of the group read them again and ordinary loads let
 // those find the rows in L2.
-template <typename T, int GT, int NW, bool SPLIT, bool ONCE>
+template <typename T, int GT, int NW, bool SPLIT, bool ONCE, int HR>
 __global__ __launch_bounds__(NW * 64) void decode_stage1_kernel(Stage1Params p) {
+  constexpr int GH = GT * HR;  // query heads per task
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int grp = lane >> 4;   // which of the 4 row slots of the wave
@@ -88,11 +89,11 @@ __global__ __launch_bounds__(NW * 64) void decode_stage1_kernel(Stage1Params p) 
   // a task = one KV head and up to GT query heads of its group; the last task of a group whose size is not a multiple of
   // GT has fewer (nh): its spare accumulators repeat the last query head and are not written
   const int group = (int)(p.hq / p.hkv);
-  const int sub_groups = (group + GT - 1) / GT;
+  const int sub_groups = (group + GH - 1) / GH;
   const int kvh = task / sub_groups;
   const int sg = task % sub_groups;
-  const int qh0 = kvh * group + sg * GT;
-  const int nh = group - sg * GT < GT ? group - sg * GT : GT;
+  const int qh0 = kvh * group + sg * GH;
+  const int nh = group - sg * GH < GH ? group - sg * GH : GH;
 
   const int len = p.b_seqlen[b];  // positions inside a request are 32-bit (max_seq_len is checked on the host)
   int64_t nblk = len <= 0 ? 0 : ((int64_t)len + p.block_seq - 1) / p.block_seq;
@@ -116,9 +117,9 @@ __global__ __launch_bounds__(NW * 64) void decode_stage1_kernel(Stage1Params p) 
   const int64_t k_row_bytes = p.k_s0 * 2, v_row_bytes = p.v_s0 * 2;
 
   // q stays packed (8 elements = 4 words per head and lane); the scale is applied to the reduced dot
-  u32x4 qw[GT];
+  u32x4 qw[GH];
 #pragma unroll
-  for (int h = 0; h < GT; h++) qw[h] = *(const u32x4*)((const char*)p.q + ((b * p.hq + qh0 + (h < nh ? h : nh - 1)) * 128 + sub * 8) * 2);
+  for (int h = 0; h < GH; h++) qw[h] = *(const u32x4*)((const char*)p.q + ((b * p.hq + qh0 + (h < nh ? h : nh - 1)) * 128 + sub * 8) * 2);
 
   for (int64_t blk = blk_begin; blk < blk_end; blk++) {
     const int t0 = (int)(blk * p.block_seq);
@@ -126,9 +127,9 @@ __global__ __launch_bounds__(NW * 64) void decode_stage1_kernel(Stage1Params p) 
     const int t1 = t1_64 > len ? len : (int)t1_64;
     const int t_last = t1 - 1;
 
-    float m[GT], l[GT], o[GT][8];
+    float m[GH], l[GH], o[GH][8];
 #pragma unroll
-    for (int h = 0; h < GT; h++) {
+    for (int h = 0; h < GH; h++) {
       m[h] = -INFINITY;
       l[h] = 0.f;
 #pragma unroll
@@ -175,129 +176,134 @@ __global__ __launch_bounds__(NW * 64) void decode_stage1_kernel(Stage1Params p) 
       }
       __builtin_amdgcn_sched_barrier(0);
 
-      // Partial dots over this lane's 8 elements for the 8 rows x GT heads of the group (value index
-      // v = GT*j + h), then a transposing reduction over the 16 lanes of the row group: two halving steps
-      // with bank-masked DPP adds (lanes with sub bits (3,2) = (B3,B2) keep values [NV/2*B3 + NV/4*B2, +NV/4))
-      // and a sum over the quad.  Every lane ends with the finished raw scores of two rows,
-      // jbase = 4*B3 + 2*B2 and jbase + 1, for all GT heads: w[GT*r + h].  The softmax scale is folded
-      // into the exp2 argument.
-      constexpr int NV = kTok * GT;
-      float u[NV / 2], w[NV / 4];
-      // Everything up to the quad sums is volatile inline assembly in a fixed order: a DPP read needs two
-      // wait states after the write of its source, the compiler's hazard recogniser does not look into inline
-      // assembly, and it would otherwise move the dots between the DPP adds.  The first halving step of a
-      // value pair (v, v + NV/2) follows the dots of the next pair, so only two partial dots are live at a time.
-      float lo_prev = 0.f, hi_prev = 0.f;
-#pragma unroll
-      for (int i = 0; i < NV / 2; i++) {
-        const int j = i / GT, h = i % GT;
-        float lo, hi;
-        Dot<T>::first(lo, qw[h][0], kr[j][0]);
-        Dot<T>::first(hi, qw[h][0], kr[j + kTok / 2][0]);
-#pragma unroll
-        for (int c = 1; c < 4; c++) {
-          Dot<T>::next(lo, qw[h][c], kr[j][c]);
-          Dot<T>::next(hi, qw[h][c], kr[j + kTok / 2][c]);
+      // HR rounds of GT query heads each over the rows just loaded (HR = 2: groups of 5 to 8 query heads per KV head
+      // fetch every row once, not once per four heads)
+      static_for<HR>([&](auto hr_tag) {
+        constexpr int HB = decltype(hr_tag)::value * GT;
+        // Partial dots over this lane's 8 elements for the 8 rows x GT heads of the group (value index
+        // v = GT*j + h), then a transposing reduction over the 16 lanes of the row group: two halving steps
+        // with bank-masked DPP adds (lanes with sub bits (3,2) = (B3,B2) keep values [NV/2*B3 + NV/4*B2, +NV/4))
+        // and a sum over the quad.  Every lane ends with the finished raw scores of two rows,
+        // jbase = 4*B3 + 2*B2 and jbase + 1, for all GT heads: w[GT*r + h].  The softmax scale is folded
+        // into the exp2 argument.
+        constexpr int NV = kTok * GT;
+        float u[NV / 2], w[NV / 4];
+        // Everything up to the quad sums is volatile inline assembly in a fixed order: a DPP read needs two
+        // wait states after the write of its source, the compiler's hazard recogniser does not look into inline
+        // assembly, and it would otherwise move the dots between the DPP adds.  The first halving step of a
+        // value pair (v, v + NV/2) follows the dots of the next pair, so only two partial dots are live at a time.
+        float lo_prev = 0.f, hi_prev = 0.f;
+  #pragma unroll
+        for (int i = 0; i < NV / 2; i++) {
+          const int j = i / GT, h = i % GT;
+          float lo, hi;
+          Dot<T>::first(lo, qw[HB + h][0], kr[j][0]);
+          Dot<T>::first(hi, qw[HB + h][0], kr[j + kTok / 2][0]);
+  #pragma unroll
+          for (int c = 1; c < 4; c++) {
+            Dot<T>::next(lo, qw[HB + h][c], kr[j][c]);
+            Dot<T>::next(hi, qw[HB + h][c], kr[j + kTok / 2][c]);
+          }
+          if (i > 0) {
+            asm volatile("v_add_f32_dpp %0, %1, %1 row_ror:8 row_mask:0xf bank_mask:0x3" : "=v"(u[i - 1]) : "v"(lo_prev));
+            asm volatile("v_add_f32_dpp %0, %1, %1 row_ror:8 row_mask:0xf bank_mask:0xc" : "+v"(u[i - 1]) : "v"(hi_prev));
+          }
+          lo_prev = lo;
+          hi_prev = hi;
         }
-        if (i > 0) {
-          asm volatile("v_add_f32_dpp %0, %1, %1 row_ror:8 row_mask:0xf bank_mask:0x3" : "=v"(u[i - 1]) : "v"(lo_prev));
-          asm volatile("v_add_f32_dpp %0, %1, %1 row_ror:8 row_mask:0xf bank_mask:0xc" : "+v"(u[i - 1]) : "v"(hi_prev));
+        asm volatile("s_nop 1");
+        asm volatile("v_add_f32_dpp %0, %1, %1 row_ror:8 row_mask:0xf bank_mask:0x3" : "=v"(u[NV / 2 - 1]) : "v"(lo_prev));
+        asm volatile("v_add_f32_dpp %0, %1, %1 row_ror:8 row_mask:0xf bank_mask:0xc" : "+v"(u[NV / 2 - 1]) : "v"(hi_prev));
+        asm volatile("s_nop 1");
+  #pragma unroll
+        for (int i = 0; i < NV / 4; i++) asm volatile("v_add_f32_dpp %0, %1, %1 row_ror:12 row_mask:0xf bank_mask:0x5" : "=v"(w[i]) : "v"(u[i]));
+        asm volatile("s_nop 1");
+  #pragma unroll
+        for (int i = 0; i < NV / 4; i++) asm volatile("v_add_f32_dpp %0, %1, %1 row_ror:4 row_mask:0xf bank_mask:0xa" : "+v"(w[i]) : "v"(u[i + NV / 4]));
+        asm volatile("s_nop 1");
+  #pragma unroll
+        for (int i = 0; i < NV / 4; i++) {
+          w[i] += dpp_mov<0xB1>(w[i]);  // quad_perm [1,0,3,2]
+          w[i] += dpp_mov<0x4E>(w[i]);  // quad_perm [2,3,0,1]
         }
-        lo_prev = lo;
-        hi_prev = hi;
-      }
-      asm volatile("s_nop 1");
-      asm volatile("v_add_f32_dpp %0, %1, %1 row_ror:8 row_mask:0xf bank_mask:0x3" : "=v"(u[NV / 2 - 1]) : "v"(lo_prev));
-      asm volatile("v_add_f32_dpp %0, %1, %1 row_ror:8 row_mask:0xf bank_mask:0xc" : "+v"(u[NV / 2 - 1]) : "v"(hi_prev));
-      asm volatile("s_nop 1");
-#pragma unroll
-      for (int i = 0; i < NV / 4; i++) asm volatile("v_add_f32_dpp %0, %1, %1 row_ror:12 row_mask:0xf bank_mask:0x5" : "=v"(w[i]) : "v"(u[i]));
-      asm volatile("s_nop 1");
-#pragma unroll
-      for (int i = 0; i < NV / 4; i++) asm volatile("v_add_f32_dpp %0, %1, %1 row_ror:4 row_mask:0xf bank_mask:0xa" : "+v"(w[i]) : "v"(u[i + NV / 4]));
-      asm volatile("s_nop 1");
-#pragma unroll
-      for (int i = 0; i < NV / 4; i++) {
-        w[i] += dpp_mov<0xB1>(w[i]);  // quad_perm [1,0,3,2]
-        w[i] += dpp_mov<0x4E>(w[i]);  // quad_perm [2,3,0,1]
-      }
-      // rows past the block only exist in its last batch and are masked there
-      const bool tail = it + 4 * kTok > t1;
-      if (tail) {
-#pragma unroll
-        for (int r = 0; r < 2; r++) {
-          const bool valid = it + (jbase + r) * 4 + grp < t1;
-#pragma unroll
-          for (int h = 0; h < GT; h++) w[GT * r + h] = valid ? w[GT * r + h] : -INFINITY;
+        // rows past the block only exist in its last batch and are masked there
+        const bool tail = it + 4 * kTok > t1;
+        if (tail) {
+  #pragma unroll
+          for (int r = 0; r < 2; r++) {
+            const bool valid = it + (jbase + r) * 4 + grp < t1;
+  #pragma unroll
+            for (int h = 0; h < GT; h++) w[GT * r + h] = valid ? w[GT * r + h] : -INFINITY;
+          }
         }
-      }
-      float pw[2 * GT];
-      float alpha[GT];
-      bool grow = false;
-#pragma unroll
-      for (int h = 0; h < GT; h++) {
-        float mx = fmaxf(w[h], w[GT + h]);
-        mx = fmaxf(mx, dpp_mov<0x124>(mx));  // row_ror:4
-        mx = fmaxf(mx, dpp_mov<0x128>(mx));  // row_ror:8: now the maximum over the 8 rows, in every lane
-        const float m_new = fmaxf(m[h], mx * p.scale_log2);  // scale > 0
-        const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
-        alpha[h] = __builtin_amdgcn_exp2f(m[h] - m_safe);
-        grow |= m_new != m[h];
-        pw[h] = __builtin_amdgcn_exp2f(__builtin_fmaf(w[h], p.scale_log2, -m_safe));
-        pw[GT + h] = __builtin_amdgcn_exp2f(__builtin_fmaf(w[GT + h], p.scale_log2, -m_safe));
-        float ps = pw[h] + pw[GT + h];
-        ps += dpp_mov<0x124>(ps);
-        ps += dpp_mov<0x128>(ps);
-        l[h] = l[h] * alpha[h] + ps;
-        m[h] = m_new;
-      }
-      // the accumulators only need rescaling when some running max moved (rare once warmed up)
-      if (__builtin_amdgcn_ballot_w64(grow) != 0) {
-#pragma unroll
-        for (int h = 0; h < GT; h++)
-#pragma unroll
-          for (int i = 0; i < 8; i++) o[h][i] *= alpha[h];
-      }
-      if (std::is_same<T, F16>::value) {
-        // O += P V on pairs of rows: the owners pack (p[2q], p[2q+1]) to fp16 (p <= 1), row pair q is
-        // broadcast from lane 4q of the group, the two V rows are interleaved element by element
-        uint32_t pp[GT];
-#pragma unroll
-        for (int h = 0; h < GT; h++) pp[h] = pack2<F16>(pw[h], pw[GT + h]);
-        static_for<kTok / 2>([&](auto q_tag) {
-          constexpr int q = decltype(q_tag)::value;
-          uint32_t bq[GT];
-#pragma unroll
-          for (int h = 0; h < GT; h++) bq[h] = __builtin_bit_cast(uint32_t, dpp_mov<0x150 + 4 * q>(__builtin_bit_cast(float, pp[h])));  // row_newbcast
-#pragma unroll
-          for (int w4 = 0; w4 < 4; w4++) {
-            const uint32_t lo = __builtin_amdgcn_perm(vr[2 * q + 1][w4], vr[2 * q][w4], 0x05040100u);
-            const uint32_t hi = __builtin_amdgcn_perm(vr[2 * q + 1][w4], vr[2 * q][w4], 0x07060302u);
-#pragma unroll
-            for (int h = 0; h < GT; h++) {
-              o[h][2 * w4] = dot2acc<F16>(bq[h], lo, o[h][2 * w4]);
-              o[h][2 * w4 + 1] = dot2acc<F16>(bq[h], hi, o[h][2 * w4 + 1]);
+        float pw[2 * GT];
+        float alpha[GT];
+        bool grow = false;
+  #pragma unroll
+        for (int h = 0; h < GT; h++) {
+          float mx = fmaxf(w[h], w[GT + h]);
+          mx = fmaxf(mx, dpp_mov<0x124>(mx));  // row_ror:4
+          mx = fmaxf(mx, dpp_mov<0x128>(mx));  // row_ror:8: now the maximum over the 8 rows, in every lane
+          const float m_new = fmaxf(m[HB + h], mx * p.scale_log2);  // scale > 0
+          const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+          alpha[h] = __builtin_amdgcn_exp2f(m[HB + h] - m_safe);
+          grow |= m_new != m[HB + h];
+          pw[h] = __builtin_amdgcn_exp2f(__builtin_fmaf(w[h], p.scale_log2, -m_safe));
+          pw[GT + h] = __builtin_amdgcn_exp2f(__builtin_fmaf(w[GT + h], p.scale_log2, -m_safe));
+          float ps = pw[h] + pw[GT + h];
+          ps += dpp_mov<0x124>(ps);
+          ps += dpp_mov<0x128>(ps);
+          l[HB + h] = l[HB + h] * alpha[h] + ps;
+          m[HB + h] = m_new;
+        }
+        // the accumulators only need rescaling when some running max moved (rare once warmed up)
+        if (__builtin_amdgcn_ballot_w64(grow) != 0) {
+  #pragma unroll
+          for (int h = 0; h < GT; h++)
+  #pragma unroll
+            for (int i = 0; i < 8; i++) o[HB + h][i] *= alpha[h];
+        }
+        if (std::is_same<T, F16>::value) {
+          // O += P V on pairs of rows: the owners pack (p[2q], p[2q+1]) to fp16 (p <= 1), row pair q is
+          // broadcast from lane 4q of the group, the two V rows are interleaved element by element
+          uint32_t pp[GT];
+  #pragma unroll
+          for (int h = 0; h < GT; h++) pp[h] = pack2<F16>(pw[h], pw[GT + h]);
+          static_for<kTok / 2>([&](auto q_tag) {
+            constexpr int q = decltype(q_tag)::value;
+            uint32_t bq[GT];
+  #pragma unroll
+            for (int h = 0; h < GT; h++) bq[h] = __builtin_bit_cast(uint32_t, dpp_mov<0x150 + 4 * q>(__builtin_bit_cast(float, pp[h])));  // row_newbcast
+  #pragma unroll
+            for (int w4 = 0; w4 < 4; w4++) {
+              const uint32_t lo = __builtin_amdgcn_perm(vr[2 * q + 1][w4], vr[2 * q][w4], 0x05040100u);
+              const uint32_t hi = __builtin_amdgcn_perm(vr[2 * q + 1][w4], vr[2 * q][w4], 0x07060302u);
+  #pragma unroll
+              for (int h = 0; h < GT; h++) {
+                o[HB + h][2 * w4] = dot2acc<F16>(bq[h], lo, o[HB + h][2 * w4]);
+                o[HB + h][2 * w4 + 1] = dot2acc<F16>(bq[h], hi, o[HB + h][2 * w4 + 1]);
+              }
             }
-          }
-        });
-      } else {
-        // bf16: a bf16 P would cost ~1e-3 relative error, so P stays fp32 and is broadcast row by row
-        static_for<kTok>([&](auto j_tag) {
-          constexpr int j = decltype(j_tag)::value;
-          float vf[8];
-          unpack8<T>(vr[j], vf);
-#pragma unroll
-          for (int h = 0; h < GT; h++) {
-            const float pb = dpp_mov<0x150 + 4 * (j >> 1)>(pw[GT * (j & 1) + h]);  // row_newbcast
-#pragma unroll
-            for (int i = 0; i < 8; i++) o[h][i] = __builtin_fmaf(pb, vf[i], o[h][i]);
-          }
-        });
-      }
+          });
+        } else {
+          // bf16: a bf16 P would cost ~1e-3 relative error, so P stays fp32 and is broadcast row by row
+          static_for<kTok>([&](auto j_tag) {
+            constexpr int j = decltype(j_tag)::value;
+            float vf[8];
+            unpack8<T>(vr[j], vf);
+  #pragma unroll
+            for (int h = 0; h < GT; h++) {
+              const float pb = dpp_mov<0x150 + 4 * (j >> 1)>(pw[GT * (j & 1) + h]);  // row_newbcast
+  #pragma unroll
+              for (int i = 0; i < 8; i++) o[HB + h][i] = __builtin_fmaf(pb, vf[i], o[HB + h][i]);
+            }
+          });
+        }
+      });
     }
 
     // merge the four lane groups (and, SPLIT, the waves) and write the block's partial
-    __shared__ float xw[SPLIT ? NW : 1][GT][16][10];  // per wave, head and column slot: 8 sums, running max, row sum
+    __shared__ float xw[SPLIT ? NW : 1][GH][16][10];  // per wave, head and column slot: 8 sums, running max, row sum
     auto write_partial = [&](int h, float M, float L, const float (&ov)[8]) {
       if (h >= nh) return;
       const float inv = 1.f / L;
@@ -311,7 +317,7 @@ __global__ __launch_bounds__(NW * 64) void decode_stage1_kernel(Stage1Params p) 
         p.mid_lse[((blk * p.row_mul + sub) * p.batch + b) * p.hq + qh0 + h] = -INFINITY;
     };
 #pragma unroll
-    for (int h = 0; h < GT; h++) {
+    for (int h = 0; h < GH; h++) {
       float M = fmaxf(m[h], __shfl_xor(m[h], 16));
       M = fmaxf(M, __shfl_xor(M, 32));
       const float w = exp2_diff(m[h], M);  // 0 for a group (or, SPLIT, a whole wave) that saw no row
@@ -342,7 +348,7 @@ __global__ __launch_bounds__(NW * 64) void decode_stage1_kernel(Stage1Params p) 
       __syncthreads();
       if (wave == 0 && grp == 0) {
 #pragma unroll
-        for (int h = 0; h < GT; h++) {
+        for (int h = 0; h < GH; h++) {
           float M = xw[0][h][sub][8];
 #pragma unroll
           for (int w = 1; w < NW; w++) M = fmaxf(M, xw[w][h][sub][8]);
@@ -458,7 +464,7 @@ __global__ __launch_bounds__(NT) void decode_stage2_kernel(Stage2Params p) {
   }
 }
 
-template <typename T, int GT>
+template <typename T, int GT, int HR>
 static int launch_stage1(const lsattn_decode_stage1_args* a, hipStream_t st) {
   constexpr int NW = 4;  // waves (tasks) per workgroup; 8 measured no faster
   Stage1Params p;
@@ -485,7 +491,7 @@ static int launch_stage1(const lsattn_decode_stage1_args* a, hipStream_t st) {
   p.block_seq = a->seq_block_size * p.row_mul;
   p.grid_blocks = (a->max_len_in_batch + p.block_seq - 1) / p.block_seq;  // stage1.cu:211, in partials computed
   const int group = (int)(a->num_q_heads / a->num_kv_heads);
-  p.tasks = (int)a->num_kv_heads * ((group + GT - 1) / GT);
+  p.tasks = (int)a->num_kv_heads * ((group + GT * HR - 1) / (GT * HR));
   const int wgs_y = (p.tasks + NW - 1) / NW;
   // a workgroup walks consecutive blocks until it has covered at least 256 tokens (smaller units measured slower for
   // short blocks, larger ones lose to tail imbalance)
@@ -501,31 +507,34 @@ static int launch_stage1(const lsattn_decode_stage1_args* a, hipStream_t st) {
   // A launch of less than one workgroup per CU leaves most of the chip's load slots empty: the waves of a workgroup then
   // share one task and split each block's tokens (measured: 64 workgroups, one request of 8192 tokens with 8 KV heads,
   // 19.9 -> 10.0 us; from 256 workgroups on it gains nothing; blocks shorter than 32 tokens per wave cannot use it).
-  const bool once = group <= GT;
-  const bool split = chunks * wgs_y * a->batch < 256 && p.block_seq >= 32 * NW && p.tasks <= 65535;
+  const bool once = group <= GT * HR;
+  // ... and so does a launch with fewer tasks than a workgroup has waves (one or two KV heads: the other waves would idle)
+  const bool split = (chunks * wgs_y * a->batch < 256 || p.tasks < NW) && p.block_seq >= 32 * NW && p.tasks <= 65535;
   if (split) {
     p.tasks_on_x = chunks <= 65535;
     dim3 grid = p.tasks_on_x ? dim3((unsigned)p.tasks, (unsigned)chunks, (unsigned)a->batch)
                              : dim3((unsigned)chunks, (unsigned)p.tasks, (unsigned)a->batch);
-    if (once) hipLaunchKernelGGL((decode_stage1_kernel<T, GT, NW, true, true>), grid, dim3(NW * 64), 0, st, p);
-    else hipLaunchKernelGGL((decode_stage1_kernel<T, GT, NW, true, false>), grid, dim3(NW * 64), 0, st, p);
+    if (once) hipLaunchKernelGGL((decode_stage1_kernel<T, GT, NW, true, true, HR>), grid, dim3(NW * 64), 0, st, p);
+    else hipLaunchKernelGGL((decode_stage1_kernel<T, GT, NW, true, false, HR>), grid, dim3(NW * 64), 0, st, p);
     return check_launch();
   }
   p.tasks_on_x = wgs_y <= 2 && chunks <= 65535;  // with more task groups per chunk (MHA, 32 KV heads) it measured 2 % slower
   dim3 grid = p.tasks_on_x ? dim3((unsigned)wgs_y, (unsigned)chunks, (unsigned)a->batch)
                            : dim3((unsigned)chunks, (unsigned)wgs_y, (unsigned)a->batch);
-  if (once) hipLaunchKernelGGL((decode_stage1_kernel<T, GT, NW, false, true>), grid, dim3(NW * 64), 0, st, p);
-  else hipLaunchKernelGGL((decode_stage1_kernel<T, GT, NW, false, false>), grid, dim3(NW * 64), 0, st, p);
+  if (once) hipLaunchKernelGGL((decode_stage1_kernel<T, GT, NW, false, true, HR>), grid, dim3(NW * 64), 0, st, p);
+  else hipLaunchKernelGGL((decode_stage1_kernel<T, GT, NW, false, false, HR>), grid, dim3(NW * 64), 0, st, p);
   return check_launch();
 }
 
 template <typename T> static int dispatch_stage1(const lsattn_decode_stage1_args* a, hipStream_t st) {
   const int group = (int)(a->num_q_heads / a->num_kv_heads);
-  // groups of 3 and more take four query heads per task (a group of 5, 6 or 7 as 4 + the rest, of 3 as one task with a
-  // spare): fetching a K/V row once per four query heads matters more than the spare accumulators cost
-  if (group >= 3) return launch_stage1<T, 4>(a, st);
-  if (group == 2) return launch_stage1<T, 2>(a, st);
-  return launch_stage1<T, 1>(a, st);
+  // groups of 3 and 4 take four query heads per task (3: one spare): fetching a K/V row once per group matters more than
+  // the spare accumulators cost
+  // groups of more than four: eight query heads per task in two rounds of four over the same rows
+  if (group >= 5) return launch_stage1<T, 4, 2>(a, st);
+  if (group >= 3) return launch_stage1<T, 4, 1>(a, st);
+  if (group == 2) return launch_stage1<T, 2, 1>(a, st);
+  return launch_stage1<T, 1, 1>(a, st);
 }
 
 }  // namespace lsattn
