@@ -13,7 +13,7 @@ DEV = "cuda:0"
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("Hq,Hkv,BS", [(32, 8, 256), (4, 4, 64), (16, 8, 16), (10, 5, 128), (12, 4, 256), (8, 1, 32), (14, 2, 256),
-                                       (5, 1, 64), (12, 2, 128), (3, 1, 16), (8, 1, 256), (16, 2, 64), (9, 1, 128), (32, 2, 256)])
+                                       (5, 1, 64), (12, 2, 128), (3, 1, 16), (8, 1, 256), (16, 2, 64), (9, 1, 128), (32, 2, 256), (8, 2, 100), (4, 4, 7)])
 def test_stage1_stage2_vs_oracle(lsa, dtype, Hq, Hkv, BS):
     print("case", dtype, Hq, Hkv, BS, flush=True)
     B, D = 5, 128
