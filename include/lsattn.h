@@ -190,6 +190,23 @@ int lsattn_decode_stage2(const lsattn_decode_stage2_args* a, void* stream);
 int lsattn_decode_attention(const lsattn_decode_stage1_args* s1, const lsattn_decode_stage2_args* s2, void* stream);
 
 /*
+ * lsattn_decode_attention for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc): the split-K partials live in a device array inside the library instead of
+ * caller memory.  It has no counterpart in the reference, whose callers allocate mid_o / mid_o_logexpsum themselves
+ * (longserve_model.py:514-517).  Both argument blocks are filled as for lsattn_decode_attention, except that mid_o and
+ * mid_o_logexpsum must be NULL in both; num_blocks (= num_seq_blocks) is the number of partial rows the caller would
+ * have allocated, and min(num_blocks, ceil(max_len_in_batch / seq_block_size)) * batch * Hq * (D + 1) * 4 bytes must not
+ * exceed LSATTN_STATIC_SCRATCH_BYTES (else LSATTN_ERR_WORKSPACE); merge_blocks must be 0 or 1.  Results are those of
+ * lsattn_decode_attention bit for bit.  The call allocates and frees nothing.  Each GPU has one such array (held until
+ * the process ends) and every call on that GPU uses it: calls that overlap on one GPU (two streams, two threads) race;
+ * calls in stream order on one stream do not.  Nothing needs clearing between calls: stage 2 reads only rows that
+ * stage 1 of the same call has written.  The first call on a device looks the array's address up
+ * (hipGetSymbolAddress); make that call outside any stream capture.
+ */
+#define LSATTN_STATIC_SCRATCH_BYTES (64 * 1024 * 1024)
+int lsattn_decode_attention_static(const lsattn_decode_stage1_args* s1, const lsattn_decode_stage2_args* s2, void* stream);
+
+/*
  * Row scatter into the KV pool: dst[dest_index[i]] = src[i] for i < n_rows, bit-exact.
  * Replaces _fwd_kernel_destindex_copy_kv
  * (loongserve/common/basemodel/triton_kernel/destindex_copy_kv.py:7-51).

@@ -15,6 +15,7 @@ LIB_PATH = os.environ.get("LSATTN_LIB_PATH") or os.path.join(os.path.dirname(os.
 
 LSATTN_F16, LSATTN_BF16, LSATTN_F32 = 0, 1, 2
 LSATTN_MAX_PARTS = 16
+LSATTN_STATIC_SCRATCH_BYTES = 64 * 1024 * 1024
 
 _vp, _i32, _i64, _f32 = C.c_void_p, C.c_int32, C.c_int64, C.c_float
 
@@ -91,6 +92,7 @@ EXPORTS = {
     "lsattn_decode_stage1": (C.c_int, [C.POINTER(DecodeStage1Args), _vp]),
     "lsattn_decode_stage2": (C.c_int, [C.POINTER(DecodeStage2Args), _vp]),
     "lsattn_decode_attention": (C.c_int, [C.POINTER(DecodeStage1Args), C.POINTER(DecodeStage2Args), _vp]),
+    "lsattn_decode_attention_static": (C.c_int, [C.POINTER(DecodeStage1Args), C.POINTER(DecodeStage2Args), _vp]),
     "lsattn_kv_scatter": (C.c_int, [_vp, _i64, _vp, _i64, _vp, _i64, _i64, _vp]),
     "lsattn_register_tokens": (C.c_int, [_vp, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _vp]),
     "lsattn_register_decode_tokens": (C.c_int, [_vp, _i64, _vp, _vp, _vp, C.c_int32, _i64, _vp]),

@@ -13,6 +13,7 @@
 //     result is deterministic;
 //   * a workgroup walks several consecutive blocks, so the launch is sized for the chip
 //     and not for block_seq.
+#include <atomic>
 #include <type_traits>
 
 #include "common.hip.h"
@@ -607,4 +608,65 @@ extern "C" int lsattn_decode_attention(const lsattn_decode_stage1_args* s1, cons
   const int rc = lsattn_decode_stage1(s1, stream);
   if (rc != LSATTN_OK) return rc;
   return lsattn_decode_stage2(s2, stream);
+}
+
+// ------------------------------------------------------------------------------------
+// lsattn_decode_attention with the split-K partials in a file-scope device array instead of caller memory, for callers
+// that cannot allocate.  Every device the library runs on holds its own copy of the array at its own address; the name
+// below is only the host-side handle of it, so host code uses the address hipGetSymbolAddress returns for the current
+// device (looked up once per device) and nothing else.
+// ------------------------------------------------------------------------------------
+static __device__ __align__(256) unsigned char scratch[LSATTN_STATIC_SCRATCH_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::atomic<void*> g_scratch_ptr[kMaxDevices];  // zero-initialised: not looked up yet
+
+// device address of `scratch` on the current device, or nullptr
+void* scratch_on_current_device() {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+  void* ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (ptr) return ptr;
+  // two threads that race here look the same address up twice; either store is right
+  if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) {
+    (void)hipGetLastError();
+    return nullptr;
+  }
+  g_scratch_ptr[dev].store(ptr, std::memory_order_release);
+  return ptr;
+}
+}  // namespace
+
+extern "C" int lsattn_decode_attention_static(const lsattn_decode_stage1_args* s1, const lsattn_decode_stage2_args* s2,
+                                              void* stream) {
+  if (!s1 || !s2) return LSATTN_ERR_INVALID_ARG;
+  // the partials are the library's here: the caller names none
+  if (s1->mid_o || s1->mid_o_logexpsum || s2->mid_o || s2->mid_o_logexpsum) return LSATTN_ERR_INVALID_ARG;
+  if (s1->b_seqlen != s2->b_seqlen || s1->batch != s2->batch || s1->num_q_heads != s2->num_heads ||
+      s1->num_blocks != s2->num_seq_blocks || s1->head_dim != s2->head_dim || s1->seq_block_size != s2->block_seq)
+    return LSATTN_ERR_INVALID_ARG;
+  if (s1->batch < 0 || s1->num_q_heads <= 0 || s1->num_blocks < 0 || s1->seq_block_size < 1 || s1->max_len_in_batch < 0 ||
+      s1->merge_blocks > 1)
+    return LSATTN_ERR_INVALID_ARG;
+  if (s1->head_dim != 128) return LSATTN_ERR_UNSUPPORTED;
+  // Rows of partials this call can touch: stage 1 writes block i of a request only for i below both bounds, and stage 2
+  // is told the same count, so it reads no row that this call has not written (the array keeps the last call's bytes).
+  int64_t rows = (s1->max_len_in_batch + s1->seq_block_size - 1) / s1->seq_block_size;
+  if (rows > s1->num_blocks) rows = s1->num_blocks;
+  const int64_t per_row = s1->batch * s1->num_q_heads;  // (request, head) pairs per block row
+  if (per_row > 0 && rows > (int64_t)LSATTN_STATIC_SCRATCH_BYTES / 4 / 129 / per_row) return LSATTN_ERR_WORKSPACE;
+  const int64_t o_floats = rows * per_row * 128;         // a multiple of 128 floats: the LSE part stays 16-byte aligned
+  if ((uint64_t)(o_floats + rows * per_row) * 4 > (uint64_t)LSATTN_STATIC_SCRATCH_BYTES) return LSATTN_ERR_WORKSPACE;
+  float* base = (float*)scratch_on_current_device();
+  if (!base) return LSATTN_ERR_LAUNCH;
+  lsattn_decode_stage1_args a1 = *s1;
+  lsattn_decode_stage2_args a2 = *s2;
+  a1.mid_o = base;
+  a1.mid_o_logexpsum = base + o_floats;
+  a1.num_blocks = rows;
+  a2.mid_o = a1.mid_o;
+  a2.mid_o_logexpsum = a1.mid_o_logexpsum;
+  a2.num_seq_blocks = rows;
+  return lsattn_decode_attention(&a1, &a2, stream);
 }

@@ -25,8 +25,10 @@ def _req(cond: bool, what: str) -> None:
 
 
 def _stage1_args(mid_o, mid_o_logexpsum, q, k, v, req_to_tokens, b_req_idx, b_seqlen,
-                 max_len_in_batch: int, seq_block_size: int, merge_blocks: int = 1) -> _lib.DecodeStage1Args:
-    """The checks of ENTRY:115-160 and the argument block of lsattn_decode_stage1."""
+                 max_len_in_batch: int, seq_block_size: int, merge_blocks: int = 1,
+                 partials_in_library: bool = False) -> _lib.DecodeStage1Args:
+    """The checks of ENTRY:115-160 and the argument block of lsattn_decode_stage1.  partials_in_library: mid_o and
+    mid_o_logexpsum only carry the shape (meta tensors) and the block names no partial buffers."""
     # ENTRY:115-122
     _req(mid_o.is_contiguous(), "mid_o.is_contiguous()")
     _req(mid_o_logexpsum.is_contiguous(), "mid_o_logexpsum.is_contiguous()")
@@ -39,9 +41,10 @@ def _stage1_args(mid_o, mid_o_logexpsum, q, k, v, req_to_tokens, b_req_idx, b_se
     # ENTRY:124-131
     for t, d, n in ((mid_o, 4, "mid_o"), (mid_o_logexpsum, 3, "mid_o_logexpsum"), (q, 3, "q"), (k, 3, "k"), (v, 3, "v"),
                     (req_to_tokens, 2, "req_to_tokens"), (b_req_idx, 1, "b_req_idx"), (b_seqlen, 1, "b_seqlen")):
-        if t.dim() != d or not t.is_cuda:  # (the message is only built on failure: this runs once per decode step)
+        on_gpu = t.is_cuda or (partials_in_library and t.is_meta)
+        if t.dim() != d or not on_gpu:  # (the message is only built on failure: this runs once per decode step)
             _req(t.dim() == d, "%s.dim() == %d" % (n, d))
-            _req(t.is_cuda, "%s on the GPU" % n)
+            _req(on_gpu, "%s on the GPU" % n)
     # ENTRY:133-140 (bfloat16 accepted in addition to half)
     _req(mid_o.dtype == torch.float32, "mid_o float32")
     _req(mid_o_logexpsum.dtype == torch.float32, "mid_o_logexpsum float32")
@@ -58,7 +61,8 @@ def _stage1_args(mid_o, mid_o_logexpsum, q, k, v, req_to_tokens, b_req_idx, b_se
     _req(b_req_idx.size(0) == B and b_seqlen.size(0) == B, "b_req_idx/b_seqlen length == batch")
     _req(seq_block_size >= 1, "seq_block_size >= 1")
     a = _lib.DecodeStage1Args()
-    a.mid_o, a.mid_o_logexpsum = mid_o.data_ptr(), mid_o_logexpsum.data_ptr()
+    if not partials_in_library:
+        a.mid_o, a.mid_o_logexpsum = mid_o.data_ptr(), mid_o_logexpsum.data_ptr()
     a.q, a.k, a.v = q.data_ptr(), k.data_ptr(), v.data_ptr()
     a.k_stride_0, a.k_stride_1 = k.stride(0), k.stride(1)
     a.v_stride_0, a.v_stride_1 = v.stride(0), v.stride(1)
@@ -83,15 +87,17 @@ def flash_decoding_stage1(mid_o, mid_o_logexpsum, q, k, v, req_to_tokens, b_req_
     _lib.check(_lib.load().lsattn_decode_stage1(C.byref(a), _stream()), "lsattn_decode_stage1")
 
 
-def _stage2_args(o, out_logexpsum, b_seqlen, mid_o, mid_o_logexpsum, block_seq: int) -> _lib.DecodeStage2Args:
+def _stage2_args(o, out_logexpsum, b_seqlen, mid_o, mid_o_logexpsum, block_seq: int,
+                 partials_in_library: bool = False) -> _lib.DecodeStage2Args:
     """The checks of ENTRY:174-190 and the argument block of lsattn_decode_stage2."""
     # ENTRY:174-190
     for t, d, n in ((o, 3, "o"), (out_logexpsum, 2, "out_logexpsum"), (b_seqlen, 1, "b_seqlen"), (mid_o, 4, "mid_o"),
                     (mid_o_logexpsum, 3, "mid_o_logexpsum")):
-        if not t.is_contiguous() or t.dim() != d or not t.is_cuda:
+        on_gpu = t.is_cuda or (partials_in_library and t.is_meta)
+        if not t.is_contiguous() or t.dim() != d or not on_gpu:
             _req(t.is_contiguous(), "%s.is_contiguous()" % n)
             _req(t.dim() == d, "%s.dim() == %d" % (n, d))
-            _req(t.is_cuda, "%s on the GPU" % n)
+            _req(on_gpu, "%s on the GPU" % n)
     _req(o.dtype in (torch.float16, torch.float32, torch.bfloat16), "o half, bfloat16 or float")
     _req(out_logexpsum.dtype == torch.float32, "out_logexpsum float32")
     _req(b_seqlen.dtype == torch.int32, "b_seqlen int32")
@@ -105,7 +111,8 @@ def _stage2_args(o, out_logexpsum, b_seqlen, mid_o, mid_o_logexpsum, block_seq: 
     _req(block_seq >= 1, "block_seq >= 1")
     a = _lib.DecodeStage2Args()
     a.o, a.o_dtype, a.out_logexpsum, a.b_seqlen = o.data_ptr(), _DT[o.dtype], out_logexpsum.data_ptr(), b_seqlen.data_ptr()
-    a.mid_o, a.mid_o_logexpsum = mid_o.data_ptr(), mid_o_logexpsum.data_ptr()
+    if not partials_in_library:
+        a.mid_o, a.mid_o_logexpsum = mid_o.data_ptr(), mid_o_logexpsum.data_ptr()
     a.batch, a.num_heads, a.num_seq_blocks, a.head_dim, a.block_seq = B, H, mid_o.size(0), D, int(block_seq)
     return a
 
@@ -125,6 +132,26 @@ def flash_decoding(mid_o, mid_o_logexpsum, q, k, v, req_to_tokens, b_req_idx, b_
     a1 = _stage1_args(mid_o, mid_o_logexpsum, q, k, v, req_to_tokens, b_req_idx, b_seqlen, max_len_in_batch, block_seq)
     a2 = _stage2_args(o, out_logexpsum, b_seqlen, mid_o, mid_o_logexpsum, block_seq)
     _lib.check(_lib.load().lsattn_decode_attention(C.byref(a1), C.byref(a2), _stream()), "lsattn_decode_attention")
+
+
+@torch.inference_mode()
+def flash_decoding_static(q, k, v, req_to_tokens, b_req_idx, b_seqlen, max_len_in_batch: int, o, out_logexpsum,
+                          block_seq: int) -> None:
+    """flash_decoding without mid_o / mid_o_logexpsum: the partials live in the library's per-GPU static array
+    (lsattn_decode_attention_static), so the call needs no scratch tensors.  Raises if
+    ceil(max_len_in_batch / block_seq) * batch * heads * (head_dim + 1) * 4 bytes exceed
+    _lib.LSATTN_STATIC_SCRATCH_BYTES.  Calls that overlap on one GPU share the array and race."""
+    _req(q.dim() == 3 and q.is_contiguous() and q.is_cuda, "q contiguous [batch, heads, head_dim] on the GPU")
+    B, Hq, D = q.shape
+    rows = max((int(max_len_in_batch) + int(block_seq) - 1) // int(block_seq), 1)
+    # the argument blocks are checked as usual against tensors of the partials' shape that own no memory
+    mid_o = torch.empty((rows, B, Hq, D), dtype=torch.float32, device="meta")
+    mid_lse = torch.empty((rows, B, Hq), dtype=torch.float32, device="meta")
+    a1 = _stage1_args(mid_o, mid_lse, q, k, v, req_to_tokens, b_req_idx, b_seqlen, max_len_in_batch, block_seq,
+                      partials_in_library=True)
+    a2 = _stage2_args(o, out_logexpsum, b_seqlen, mid_o, mid_lse, block_seq, partials_in_library=True)
+    _lib.check(_lib.load().lsattn_decode_attention_static(C.byref(a1), C.byref(a2), _stream()),
+               "lsattn_decode_attention_static")
 
 
 def _half2d(t: torch.Tensor, name: str, dim: int) -> None:
