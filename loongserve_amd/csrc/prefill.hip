@@ -31,6 +31,7 @@
 //   * one kernel, three epilogues (MODE): 0 writes the step's fp32 partial (O, LSE) from the empty state, 1 folds the
 //     step into the reference's in-place (o, m, l) state (ring_context_flashattention_nopad.py:171-188), 2 LSE-merges it
 //     into a running fp32 (O, LSE); the folding ones read the old state of both row blocks of a wave at once.
+#include <cstdlib>
 #include <type_traits>
 
 #include "common.hip.h"
@@ -62,6 +63,7 @@ constexpr int BM = 256;   // query rows per workgroup (32 per wave)
 constexpr int BN = 64;    // keys per LDS tile
 constexpr int SUB = 32;   // keys per pipeline step (the contraction length of one P V MFMA)
 constexpr int NWAVE = 8;  // two per SIMD
+constexpr int64_t kSplitBelowWorkgroups = 1024;  // 256-row workgroups in a launch below which the 128-row variant runs
 constexpr float kLazyRescale = 8.f;  // log2 units the running max may lag before O is rescaled
 
 template <typename T> struct Mfma;
@@ -192,62 +194,16 @@ __device__ __forceinline__ const char* uniform_ptr(const char* ptr) {
   return (const char*)(((uint64_t)hi << 32) | lo);
 }
 
-// Online-softmax update for one 32-key sub-tile in the general path.  s[kb][qb][r] is the score of key
-// n0 + 16 kb + 4 g + r for the lane's query row of block qb; on return pk[qb] holds that row's eight P values as
-// the B operand of the P V MFMA, in the key order the V^T operands use.  The running maximum only moves when some
-// row of the wave exceeds it by more than kLazyRescale (then every row takes its true maximum).
-template <bool MASK>
-__device__ __forceinline__ bool softmax32(f32x4 (&s)[2][2], u32x4 (&pk)[2], float (&m_run)[2], float (&l_run)[2], float (&alpha)[2],
-                                          float scale_log2, int g, int n0, int kv_len, int kf, int P, const int (&qpos)[2]) {
-  float mx[2];
-  bool over = false;
-#pragma unroll
-  for (int qb = 0; qb < 2; qb++) {
-    if (MASK) {
-#pragma unroll
-      for (int kb = 0; kb < 2; kb++)
-#pragma unroll
-        for (int r = 0; r < 4; r++) {
-          const int n = n0 + 16 * kb + 4 * g + r;
-          const bool vis = (n < kv_len) && (kf + n * P <= qpos[qb]);
-          s[kb][qb][r] = vis ? s[kb][qb][r] : -INFINITY;
-        }
-    }
-    float m8 = fmaxf(fmaxf(s[0][qb][0], s[0][qb][1]), fmaxf(s[0][qb][2], s[0][qb][3]));
-    m8 = fmaxf(m8, fmaxf(fmaxf(s[1][qb][0], s[1][qb][1]), fmaxf(s[1][qb][2], s[1][qb][3])));
-    mx[qb] = column_max(m8) * scale_log2;
-    over = over || (mx[qb] > m_run[qb] + kLazyRescale);
-  }
-  const bool any = __builtin_amdgcn_ballot_w64(over) != 0;
-#pragma unroll
-  for (int qb = 0; qb < 2; qb++) {
-    const float m_new = any ? fmaxf(m_run[qb], mx[qb]) : m_run[qb];
-    const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-    alpha[qb] = (m_run[qb] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m_run[qb] - m_use);
-    m_run[qb] = m_new;
-    float ps0 = 0.f, ps1 = 0.f;
-    u32x4 w;
-#pragma unroll
-    for (int kb = 0; kb < 2; kb++)
-#pragma unroll
-      for (int e = 0; e < 2; e++) {
-        const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kb][qb][2 * e], scale_log2, -m_use));
-        const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kb][qb][2 * e + 1], scale_log2, -m_use));
-        w[2 * kb + e] = pack2<F16>(p0, p1);
-        ps0 += p0;
-        ps1 += p1;
-      }
-    pk[qb] = w;
-    l_run[qb] = l_run[qb] * alpha[qb] + (ps0 + ps1);
-  }
-  return any;
-}
-
 // DV: the V tiles are fp16 in memory and go straight into LDS; otherwise (bf16 V) they pass through registers and are
 // converted on the way.
-template <typename T, int MODE, bool DV>
+// SPLIT: a workgroup owns 128 query rows instead of 256: waves w and w + 4 (one SIMD) hold the same 32 rows and take the
+// even and the odd 32-key sub-tiles of every tile; their partial results meet in LDS after the loop.  Half the rows per
+// workgroup at the same per-wave shape: for launches with too few 256-row workgroups to fill and balance the chip.
+template <typename T, int MODE, bool DV, bool SPLIT>
 __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p) {
+  static_assert(DV || !SPLIT, "the split variant takes fp16 V tiles only");
   __shared__ __attribute__((aligned(1024))) char lds[kLdsBytes];
+  constexpr int BMW = SPLIT ? BM / 2 : BM;  // query rows of this workgroup
 
   // Workgroup ids go to the 8 XCDs round-robin.  The (query head, query tile) units of one KV head are dealt to p.slices
   // XCDs (1 when the KV heads are a multiple of 8, else as many as it takes for hkv * slices to be one), so that the
@@ -268,7 +224,7 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
   const int z = p.nz - 1 - zr;
 
   const int q_len = p.q_len[b];
-  const int m_lo = z * BM;
+  const int m_lo = z * BMW;
   if (m_lo >= q_len) return;
   const int kv_len = p.kv_len[b];
   const int64_t q_start = p.q_start[b], kv_start = p.kv_start[b];
@@ -278,23 +234,23 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int qc = lane & 15, g = lane >> 4;  // query column within a 16-row block, lane group
+  const int wrow = SPLIT ? (wave & 3) : wave;  // which 32 rows of the workgroup
+  const int kp = SPLIT ? (wave >> 2) : 0;      // SPLIT: parity of the sub-tiles this wave takes
 
+  // keys of this KV chunk visible to global query position qpos (RING:156-159)
   auto visible_keys = [&](int qpos) -> int {
     const int dq = qpos - kf;
     const int n = dq >= 0 ? dq / P + 1 : 0;
     return n > kv_len ? kv_len : n;
   };
-  const int m_hi = (m_lo + BM < q_len ? m_lo + BM : q_len) - 1;
-  const int nt = (visible_keys(qf + m_hi * P) + BN - 1) / BN;
+  const int m_hi = (m_lo + BMW < q_len ? m_lo + BMW : q_len) - 1;
+  const int nt = (visible_keys(qf + m_hi * P) + BN - 1) / BN;  // tiles the workgroup walks
 
-  const int m_w0 = m_lo + wave * 32;
-  const bool wave_has_rows = m_w0 < q_len;
-  const int m_wlast = m_w0 + 31 > q_len - 1 ? q_len - 1 : m_w0 + 31;
-  const int ns_w = wave_has_rows ? (visible_keys(qf + m_wlast * P) + SUB - 1) / SUB : 0;
-  const int i_mask = wave_has_rows ? visible_keys(qf + m_w0 * P) / SUB : 0;
+  const int m_w0 = m_lo + wrow * 32;
 
-  // Q as B operands: qreg[qb][ks] = Q[row 16 qb + qc][32 ks + 8g .. +7]
+  // Q as B operands: qreg[qb][ks] = Q[row 16 qb + qc][32 ks + 8g .. +7]; cnt[qb] = keys that row sees (0 past the end)
   u32x4 qreg[2][4];
+  int cnt[2];
 #pragma unroll
   for (int qb = 0; qb < 2; qb++) {
     const int m = m_w0 + 16 * qb + qc;
@@ -302,6 +258,7 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
     const char* src = (const char*)p.q + ((q_start + (ok ? m : 0)) * p.q_st + (int64_t)h * p.q_sh + 8 * g) * 2;
 #pragma unroll
     for (int ks = 0; ks < 4; ks++) qreg[qb][ks] = ok ? *(const u32x4*)(src + ks * 64) : u32x4{0, 0, 0, 0};
+    cnt[qb] = ok ? visible_keys(qf + m * P) : 0;
   }
 
   int koff0 = qc * 256 + ((g ^ swz_k(qc)) << 4);
@@ -315,84 +272,90 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
   }
   const int lds_base = (int)(uintptr_t)(__attribute__((address_space(3))) char*)lds;
 
-  // staging: wave w owns rows [8w, 8w+8) of every tile, 4 rows per instruction
-  const char* kg = (const char*)p.k + (kv_start * p.k_st + (int64_t)kvh * p.k_sh) * 2;
-  const char* vg = (const char*)p.v + (kv_start * p.v_st + (int64_t)kvh * p.v_sh) * 2;
-  const int64_t k_row_bytes = p.k_st * 2, v_row_bytes = p.v_st * 2;
-  const int st_row = lane >> 4;
+  // staging: wave w owns rows [8w, 8w+8) of every tile, 4 rows per instruction.  The chunk bases and row strides are
+  // wave-uniform and held in scalar registers.
+  const char* kg = uniform_ptr((const char*)p.k + (kv_start * p.k_st + (int64_t)kvh * p.k_sh) * 2);
+  const char* vg = uniform_ptr((const char*)p.v + (kv_start * p.v_st + (int64_t)kvh * p.v_sh) * 2);
+  const int k_row_bytes = __builtin_amdgcn_readfirstlane((int)p.k_st * 2), v_row_bytes = __builtin_amdgcn_readfirstlane((int)p.v_st * 2);
+  const int st_row = 8 * wave + (lane >> 4);  // the lane's row of the tile in the first of its two instructions
   const int last_row = kv_len - 1;
+  // byte offset of the lane's 16 bytes from the tile's first row, row and swizzled chunk
   uint32_t k_lane_off[2], v_lane_off[2];
-  int st_chunk_k[2], st_chunk_v[2];
 #pragma unroll
   for (int i = 0; i < 2; i++) {
-    const int r = 8 * wave + 4 * i + st_row;
-    st_chunk_k[i] = ((lane & 15) ^ swz_k(r)) << 4;
-    st_chunk_v[i] = ((lane & 15) ^ swz_v(r)) << 4;
-    k_lane_off[i] = (uint32_t)(r * k_row_bytes) + st_chunk_k[i];
-    v_lane_off[i] = (uint32_t)(r * v_row_bytes) + st_chunk_v[i];
+    const int r = st_row + 4 * i;
+    k_lane_off[i] = (uint32_t)(r * k_row_bytes) + (((lane & 15) ^ swz_k(r)) << 4);
+    v_lane_off[i] = (uint32_t)(r * v_row_bytes) + (((lane & 15) ^ swz_v(r)) << 4);
   }
+  const int st_lds = lds_base + 8 * wave * 256;
   u32x4 vst[2];
-  auto load_tiles = [&](auto full_tag, int tk, int tv) __attribute__((always_inline)) {
-    constexpr bool FULL = decltype(full_tag)::value;
+  // All tile loads are issued from inline assembly: behind a load to LDS that the compiler sees, it waits for vmcnt(0)
+  // before every later LDS read (it cannot tell which LDS bytes the load writes); the waits for these loads are the
+  // explicit wait_vmem calls.  The s_nop is the wait state a write of m0 needs before an LDS-DMA load reads it.
+  //
+  // Tile `t` of K (of V) into ring slot S, rows past the end of the chunk replaced by its last row (they are masked
+  // where they are used, and a tile that lies wholly past the end is never read): any tile index is safe.  The tile
+  // pointer is scalar (a tile past the end becomes the last one), the lane's offset moves back to the last row.
+  const int last_tile = last_row / BN;
+  auto clamped_tile = [&](const char* base, int row_bytes, uint32_t lane_off, int i, int t, const char*& tile, uint32_t& off)
+                          __attribute__((always_inline)) {
+    const int tc = __builtin_amdgcn_readfirstlane(t < last_tile ? t : last_tile);
+    tile = base + (int64_t)tc * BN * row_bytes;
+    // rows of the tile between the lane's row, st_row + 4 i, and the last one of the chunk (the scalar part on its own,
+    // so that no further per-lane values are kept across the loop)
+    const int lim = __builtin_amdgcn_readfirstlane(last_row - tc * BN - 4 * i);
+    int back = st_row - lim;
+    back = back < 0 ? 0 : back;
+    off = lane_off - (uint32_t)(back * row_bytes);
+  };
+  auto load_k_clamped = [&](auto slot_tag, int t) __attribute__((always_inline)) {
+    constexpr int S = decltype(slot_tag)::value;
 #pragma unroll
     for (int i = 0; i < 2; i++) {
-      const int r = 8 * wave + 4 * i + st_row;
-      const char* ksrc;
-      const char* vsrc;
-      if (FULL) {
-        const char* kt = kg + (int64_t)__builtin_amdgcn_readfirstlane(tk) * BN * k_row_bytes;
-        const char* vt = vg + (int64_t)__builtin_amdgcn_readfirstlane(tv) * BN * v_row_bytes;
-        kt = uniform_ptr(kt);
-        vt = uniform_ptr(vt);
-        ksrc = kt + k_lane_off[i];
-        vsrc = vt + v_lane_off[i];
-      } else {
-        int nk = tk * BN + r, nv = tv * BN + r;
-        nk = nk > last_row ? last_row : nk;
-        nv = nv > last_row ? last_row : nv;
-        nv = nv < 0 ? 0 : nv;
-        ksrc = kg + nk * k_row_bytes + st_chunk_k[i];
-        vsrc = vg + nv * v_row_bytes + st_chunk_v[i];
-      }
-      const int kdst = (tk & (kRing - 1)) * kTileBytes + (8 * wave + 4 * i) * 256;
-      const int vdst = kLdsV + (tv & (kRing - 1)) * kTileBytes + (8 * wave + 4 * i) * 256;
-      if (FULL) {
-        // issued from inline assembly: behind a load to LDS that the compiler sees, it waits for
-        // vmcnt(0) before every later LDS read (it cannot tell which LDS bytes the load writes);
-        // the waits for these loads are the explicit wait_vmem calls
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_base + kdst), "v"(ksrc) : "m0");
-        if (DV)
-          asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_base + vdst), "v"(vsrc) : "m0");
-        else
-          vst[i] = *(const u32x4*)vsrc;
-        continue;
-      }
-      __builtin_amdgcn_global_load_lds((global_void_ptr)ksrc, (lds_void_ptr)(lds + kdst), 16, 0, 0);
+      const char* tile;
+      uint32_t off;
+      clamped_tile(kg, k_row_bytes, k_lane_off[i], i, t, tile, off);
+      const int dst = st_lds + S * kTileBytes + i * 1024;
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(off), "s"(tile) : "m0", "memory");
+    }
+  };
+  auto load_v_clamped = [&](auto slot_tag, int t) __attribute__((always_inline)) {
+    constexpr int S = decltype(slot_tag)::value;
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+      const char* tile;
+      uint32_t off;
+      clamped_tile(vg, v_row_bytes, v_lane_off[i], i, t, tile, off);
       if (DV) {
-        __builtin_amdgcn_global_load_lds((global_void_ptr)vsrc, (lds_void_ptr)(lds + vdst), 16, 0, 0);
+        const int dst = st_lds + kLdsV + S * kTileBytes + i * 1024;
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(off), "s"(tile) : "m0", "memory");
       } else {
-        vst[i] = *(const u32x4*)vsrc;
+        u32x4 w;  // into registers: see store_v_tile
+        asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(w) : "v"(off), "s"(tile) : "memory");
+        vst[i] = w;
       }
     }
   };
-  auto store_v_tile = [&](int tv) __attribute__((always_inline)) {
+  // (bf16 V only) the tile held in registers, converted, into ring slot S
+  auto store_v_tile = [&](auto slot_tag) __attribute__((always_inline)) {
+    constexpr int S = decltype(slot_tag)::value;
     if (!DV) {
 #pragma unroll
       for (int i = 0; i < 2; i++)
-        *(u32x4*)(lds + kLdsV + (tv & (kRing - 1)) * kTileBytes + (8 * wave + 4 * i) * 256 + lane * 16) = to_pv_operand<T>(vst[i]);
+        *(u32x4*)(lds + kLdsV + S * kTileBytes + (8 * wave + 4 * i) * 256 + lane * 16) = to_pv_operand<T>(vst[i]);
     }
   };
 
-  // Full tiles in the fast loop: running scalar tile pointers, the lane's 32-bit offset and the LDS
-  // destination of a compile-time ring slot, issued from inline assembly (as in load_tiles).
+  // Tiles that lie wholly inside the chunk: running scalar tile pointers and the lane's 32-bit offset, K tile it + KA
+  // and V tile it + VA of iteration `it` into their ring slots.
+  constexpr int KA = SPLIT ? 4 : 3, VA = SPLIT ? 3 : 2;  // how far ahead of the tile in work the loads run
   const char* kt_run = kg;
   const char* vt_run = vg;
-  const int st_lds = lds_base + 8 * wave * 256;
   auto load_tiles_fast = [&](auto r_tag) __attribute__((always_inline)) {
     constexpr int R = decltype(r_tag)::value;
-    constexpr int kslot = ((R + 3) & 3) * kTileBytes, vslot = kLdsV + ((R + 2) & 3) * kTileBytes;
+    constexpr int kslot = ((R + KA) & 3) * kTileBytes, vslot = kLdsV + ((R + VA) & 3) * kTileBytes;
     // one block, so that nothing is put between the loads (a wave issues an instruction every five cycles or so,
-    // whatever it is); the s_nop is the wait state a write of m0 needs before an LDS-DMA load reads it
+    // whatever it is)
     if (DV) {
       asm volatile(
           "s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %4, %8\n\t"
@@ -409,17 +372,16 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
           "s"(st_lds + kslot + 1024), "v"(k_lane_off[0]), "v"(k_lane_off[1]), "s"(kt_run)
           : "m0", "memory");
     }
-    kt_run += BN * k_row_bytes;
-    if (DV) vt_run += BN * v_row_bytes;
+    kt_run += (int64_t)BN * k_row_bytes;
+    if (DV) vt_run += (int64_t)BN * v_row_bytes;
   };
   // A V tile that has to be converted on its way into LDS goes through registers: loaded one iteration before it is
   // stored (three tiles ahead of its use), so the wait in front of the store is for loads a whole iteration old.
-  // The compiler does not see these loads: fast_iteration waits for them before it stores the tile.
   auto load_v_regs_fast = [&]() __attribute__((always_inline)) {
 #pragma unroll
     for (int i = 0; i < 2; i++)
       asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(vst[i]) : "v"(v_lane_off[i]), "s"(vt_run) : "memory");
-    vt_run += BN * v_row_bytes;
+    vt_run += (int64_t)BN * v_row_bytes;
   };
 
   // O^T accumulators: oacc[db][qb][r] = O[row 16 qb + qc][16 db + 4g + r]
@@ -428,63 +390,19 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
   for (int db = 0; db < 8; db++)
 #pragma unroll
     for (int qb = 0; qb < 2; qb++) oacc[db][qb] = f32x4{0.f, 0.f, 0.f, 0.f};
-  float m_run[2] = {-INFINITY, -INFINITY}, l_run[2] = {0.f, 0.f}, alpha[2] = {1.f, 1.f};
+  float m_run[2] = {-INFINITY, -INFINITY}, l_run[2] = {0.f, 0.f};
   f32x4 s[2][2];  // s[kb][qb][r] = S[row 16 qb + qc][key 16 kb + 4g + r of the sub-tile]
   u32x4 pk[2];
   u32x4 ka[2][4], va[8];
-  const int qpos[2] = {qf + (m_w0 + qc) * P, qf + (m_w0 + 16 + qc) * P};
 
-  // General step for sub-tile i: bounds-checked, masked, nothing carried over between steps.
-  auto step = [&](int i) __attribute__((always_inline)) {
-    if (i >= ns_w) return;  // no row of this wave sees a key of this sub-tile (wave-uniform)
-    const int ksub = lds_base + ((i >> 1) & (kRing - 1)) * kTileBytes + (i & 1) * (SUB * 256);
-    asm volatile("" : "+v"(koff0), "+v"(voff0));
-    load_k_operands(ksub, koff0, ka);
-    load_v_operands(ksub + kLdsV, voff0, va);
-#pragma unroll
-    for (int kb = 0; kb < 2; kb++)
-#pragma unroll
-      for (int qb = 0; qb < 2; qb++) s[kb][qb] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int ks = 0; ks < 4; ks++)
-#pragma unroll
-      for (int kb = 0; kb < 2; kb++)
-#pragma unroll
-        for (int qb = 0; qb < 2; qb++) s[kb][qb] = Mfma<T>::run(ka[kb][ks], qreg[qb][ks], s[kb][qb]);
-    // sub-tiles below i_mask are visible to the first row of the wave, hence to all of them: no mask to compute
-    const bool any = i < i_mask ? softmax32<false>(s, pk, m_run, l_run, alpha, p.scale_log2, g, i * SUB, kv_len, kf, P, qpos)
-                                : softmax32<true>(s, pk, m_run, l_run, alpha, p.scale_log2, g, i * SUB, kv_len, kf, P, qpos);
-    if (any) {
-#pragma unroll
-      for (int db = 0; db < 8; db++)
-#pragma unroll
-        for (int qb = 0; qb < 2; qb++) oacc[db][qb] *= alpha[qb];
-    }
-#pragma unroll
-    for (int db = 0; db < 8; db++)
-#pragma unroll
-      for (int qb = 0; qb < 2; qb++) oacc[db][qb] = Mfma<F16>::run(va[db], pk[qb], oacc[db][qb]);
-  };
-  // Iteration `it` works on tile `it` (sub-tiles 2it, 2it+1) and issues the loads of K tile it+3 and
-  // V tile it+2.  The wait in the middle leaves only this iteration's loads in flight, so the previous
-  // iteration's are complete for every wave after the next barrier.
-  auto iteration = [&](int it) __attribute__((always_inline)) {
-    __syncthreads();
-    load_tiles(std::false_type{}, it + 3, it + 2);
-    step(2 * it);
-    if (DV) wait_vmem<4>();
-    step(2 * it + 1);
-    store_v_tile(it + 2);
-  };
-
-  // Fast iterations: every key of the tile exists and is visible to every row of the workgroup, and the
-  // ring slot (it & 3 == R) is a compile-time constant, so every LDS read is a fixed register plus an
-  // immediate.  A step has an MFMA phase (S(i) = K(i) Q^T, then O += V(i-1) P(i-1), each operand register
-  // refilled for the next step right behind the MFMA that consumed it) and a softmax phase (P(i)).
-  // Running state in this form, per 16-row block qb: neg_m = -m, thr_raw = (m + 2^kLazyRescale) / scale,
-  // l = lacc[qb] (any element).
+  // Every tile goes through the same pipelined loop, and the ring slot of a tile (it & 3 == R) is a compile-time
+  // constant there, so every LDS read is a fixed register plus an immediate.  A 32-key step has an MFMA phase
+  // (S(i) = K(i) Q^T, then O += V(i') P(i') for the wave's previous sub-tile i', each operand register refilled for the
+  // next step right behind the MFMA that consumed it) and a softmax phase (P(i)).
+  // Running state, per 16-row block qb: neg_m = -m (+inf while the row has seen no key), thr_raw = (m + 2^kLazyRescale)
+  // / scale, l = lacc[qb] (any element).
   int kaddr[4], vaddr[8];
-  float neg_m[2] = {0.f, 0.f}, thr_raw[2] = {0.f, 0.f};
+  float neg_m[2] = {INFINITY, INFINITY}, thr_raw[2] = {-INFINITY, -INFINITY};
   // row sums of P on the matrix pipe: lacc[qb] += ones(16 x 32) P^T, every element of a lane's lacc[qb] is the sum of
   // its query column over all keys so far (of the fp16 P values, the ones that multiply V)
   f32x4 lacc[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};
@@ -493,11 +411,13 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
   u32x4 ones = u32x4{0x3C003C00u, 0x3C003C00u, 0x3C003C00u, 0x3C003C00u};
   asm volatile("" : "+v"(ones));
   const float scale = p.scale_log2, inv_scale = 1.f / p.scale_log2;
-  auto fphase_mfma = [&](auto par_tag, auto r_tag) __attribute__((always_inline)) {
-    constexpr int PAR = decltype(par_tag)::value;  // sub-tile i = 2it + PAR
+  auto fphase_mfma = [&](auto par_tag, auto r_tag, auto lsum_tag) __attribute__((always_inline)) {
+    constexpr int PAR = decltype(par_tag)::value;  // sub-tile i = 2it + PAR (SPLIT: the parity is in the address registers)
     constexpr int R = decltype(r_tag)::value;
-    constexpr int koff = (PAR ? ((R + 1) & 3) : R) * kTileBytes + (PAR ^ 1) * (SUB * 256);  // K sub-tile i+1
-    constexpr int voff = R * kTileBytes + PAR * (SUB * 256);                               // V sub-tile i
+    constexpr bool LSUM = decltype(lsum_tag)::value;  // the row sums of the P consumed here go through the matrix pipe
+    // K operands of the wave's next sub-tile, V operands of this one
+    constexpr int koff = SPLIT ? ((R + 1) & 3) * kTileBytes : (PAR ? ((R + 1) & 3) : R) * kTileBytes + (PAR ^ 1) * (SUB * 256);
+    constexpr int voff = SPLIT ? R * kTileBytes : R * kTileBytes + PAR * (SUB * 256);
 #pragma unroll
     for (int ks = 0; ks < 4; ks++)
 #pragma unroll
@@ -522,16 +442,35 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
       va[db] = u32x4{wa[0], wa[1], wb[0], wb[1]};
       __builtin_amdgcn_sched_barrier(0);
     }
-    MfmaAsm<F16>::acc(lacc[0], ones, pk[0]);
-    MfmaAsm<F16>::acc(lacc[1], ones, pk[1]);
-    __builtin_amdgcn_sched_barrier(0);
+    if (LSUM) {
+      MfmaAsm<F16>::acc(lacc[0], ones, pk[0]);
+      MfmaAsm<F16>::acc(lacc[1], ones, pk[1]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
   };
   // P(i) = exp2(S(i) * scale - m) with the current m, and the lane's largest score of each block in mx[qb].  Sixteen
   // independent operations at a time, the levels of the maxima's trees spread between them: this wave's vector work
   // runs beside the other wave's MFMAs only without short dependent chains and without dot-product instructions
   // (those queue behind the MFMAs).
-  auto compute_p = [&](float (&mx)[2]) __attribute__((always_inline)) {
-    float ma[2], mb[2], t[2][8];
+  // MASKED (tiles on the diagonal or at the end of the chunk): key n of the chunk counts for a row only if n < cnt,
+  // the others' scores become -inf first; a row that has seen no key yet (neg_m = +inf) computes with m = 0.
+  // MASKED iterations also return the sums of the lane's P values in fp32 (ps): a row that sees only a few keys needs its
+  // row sum more exact than the fp16 P values give it.
+  auto compute_p = [&](auto masked_tag, int i, float (&mx)[2], float (&ps)[2]) __attribute__((always_inline)) {
+    constexpr bool MASKED = decltype(masked_tag)::value;
+    float ma[2], mb[2], t[2][8], nm[2];
+#pragma unroll
+    for (int qb = 0; qb < 2; qb++) {
+      nm[qb] = neg_m[qb];
+      if (MASKED) {
+        nm[qb] = neg_m[qb] == INFINITY ? 0.f : neg_m[qb];
+        const int rel = cnt[qb] - i * SUB - 4 * g;  // keys from the lane's first one of key block 0 to the row's limit
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+          for (int r = 0; r < 4; r++) s[kb][qb][r] = (16 * kb + r < rel) ? s[kb][qb][r] : -INFINITY;
+      }
+    }
 #pragma unroll
     for (int qb = 0; qb < 2; qb++) {
       ma[qb] = fmaxf(fmaxf(s[0][qb][0], s[0][qb][1]), s[0][qb][2]);
@@ -542,131 +481,230 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
 #pragma unroll
       for (int kb = 0; kb < 2; kb++)
 #pragma unroll
-        for (int r = 0; r < 4; r++) t[qb][4 * kb + r] = __builtin_fmaf(s[kb][qb][r], scale, neg_m[qb]);
+        for (int r = 0; r < 4; r++) t[qb][4 * kb + r] = __builtin_fmaf(s[kb][qb][r], scale, nm[qb]);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int qb = 0; qb < 2; qb++) ma[qb] = fmaxf(fmaxf(ma[qb], s[1][qb][2]), s[1][qb][3]);
 #pragma unroll
     for (int qb = 0; qb < 2; qb++)
 #pragma unroll
-      for (int i = 0; i < 8; i++) t[qb][i] = __builtin_amdgcn_exp2f(t[qb][i]);
+      for (int e = 0; e < 8; e++) t[qb][e] = __builtin_amdgcn_exp2f(t[qb][e]);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int qb = 0; qb < 2; qb++) mx[qb] = fmaxf(ma[qb], mb[qb]);
+    if (MASKED) {
+#pragma unroll
+      for (int qb = 0; qb < 2; qb++)
+        ps[qb] = ((t[qb][0] + t[qb][1]) + (t[qb][2] + t[qb][3])) + ((t[qb][4] + t[qb][5]) + (t[qb][6] + t[qb][7]));
+    }
 #pragma unroll
     for (int qb = 0; qb < 2; qb++)
 #pragma unroll
       for (int e = 0; e < 4; e++) pk[qb][e] = pack2<F16>(t[qb][2 * e], t[qb][2 * e + 1]);
     __builtin_amdgcn_sched_barrier(0);
   };
-  auto fphase_softmax = [&]() __attribute__((always_inline)) {
-    float mx[2];
-    compute_p(mx);
+  auto fphase_softmax = [&](auto masked_tag, int i) __attribute__((always_inline)) {
+    constexpr bool MASKED = decltype(masked_tag)::value;
+    float mx[2], ps[2];
+    compute_p(masked_tag, i, mx, ps);
     if (__builtin_amdgcn_ballot_w64((mx[0] > thr_raw[0]) | (mx[1] > thr_raw[1])) != 0) {
-      // rare: some score is above the lazy threshold; raise the running maxima and redo the sub-tile
-      // (the accumulators' last MFMAs were issued before this phase's barrier and the whole of compute_p lies
-      // between them and these multiplies)
+      // rare: some score is above the lazy threshold (always so for the first key a row sees); raise the running maxima
+      // and redo the sub-tile (the accumulators' last MFMAs were issued before this phase's barrier and the whole of
+      // compute_p lies between them and these multiplies)
 #pragma unroll
       for (int qb = 0; qb < 2; qb++) {
         const float m_new = fminf(neg_m[qb], -column_max(mx[qb]) * scale);  // -max(m, mx*scale)
-        const float al = __builtin_amdgcn_exp2f(m_new - neg_m[qb]);
+        // (a block of rows that still has seen no key keeps neg_m = +inf: no inf - inf)
+        const float al = (MASKED && m_new == neg_m[qb]) ? 1.f : __builtin_amdgcn_exp2f(m_new - neg_m[qb]);
         neg_m[qb] = m_new;
         thr_raw[qb] = (kLazyRescale - m_new) * inv_scale;
-        lacc[qb] *= al;
+        if (MASKED) l_run[qb] *= al;
+        else lacc[qb] *= al;
 #pragma unroll
         for (int db = 0; db < 8; db++) oacc[db][qb] *= al;
       }
-      compute_p(mx);
+      compute_p(masked_tag, i, mx, ps);
+    }
+    if (MASKED) {
+      l_run[0] += ps[0];
+      l_run[1] += ps[1];
     }
     __builtin_amdgcn_sched_barrier(0);
   };
-  // The two waves that share a SIMD (w and w + 4) run the fast loop half a step apart, one in its MFMA
-  // phase while the other is in its softmax phase (wave priorities make no measurable difference with this MFMA shape);
-  // a workgroup barrier ends every phase.  The loads of K tile it+3 and V tile it+2 go out in the first
-  // softmax phase of iteration it; the wait before the iteration's second MFMA phase leaves only those
-  // in flight, so a tile is complete for both groups one barrier before its first read, and no read of
-  // the slot a load overwrites is still pending when the load is issued.
-  auto fast_iteration = [&](auto r_tag, int it) __attribute__((always_inline)) {
-    fphase_mfma(std::integral_constant<int, 0>{}, r_tag);
-    __builtin_amdgcn_s_barrier();
-    load_tiles_fast(r_tag);
-    fphase_softmax();
-    __builtin_amdgcn_s_barrier();
-    if (DV) wait_vmem<4>();
-    fphase_mfma(std::integral_constant<int, 1>{}, r_tag);
-    __builtin_amdgcn_s_barrier();
-    fphase_softmax();
-    if (!DV) {
-      // everything but this iteration's two K loads has arrived: the registers hold V tile it+2, and K tile it+2
-      // (loaded one iteration ago) is complete as well
-      asm volatile("s_waitcnt vmcnt(2)" : "+v"(vst[0]), "+v"(vst[1]));
-      store_v_tile(it + 2);
-      load_v_regs_fast();  // V tile it+3
+  // The two waves that share a SIMD (w and w + 4) run the loop half a step apart, one in its MFMA phase while the other
+  // is in its softmax phase (wave priorities make no measurable difference with this MFMA shape); a workgroup barrier
+  // ends every phase.
+  // Not SPLIT: iteration `it` is tile `it`, sub-tiles 2it and 2it+1.  The loads of K tile it+3 and V tile it+2 go out in
+  // its first softmax phase; the wait before its second MFMA phase leaves only those in flight, so a tile is complete for
+  // both groups one barrier before its first read, and no read of the slot a load overwrites is still pending when the
+  // load is issued.
+  // SPLIT: iteration `it` is sub-tile 2it + kp of tile `it`: one MFMA phase and one softmax phase, in which K tile it+4
+  // and V tile it+3 are requested.  The group of waves 4-7 runs one phase behind: the last reads of the slots these loads
+  // overwrite (K tile it, V tile it-1) were issued in its MFMA phase of iteration it-1, two barriers before its loads and
+  // one before those of waves 0-3.  The wait at the end of an iteration leaves that iteration's loads in flight, so
+  // tile it+4 is complete for everyone after iteration it+1 of waves 4-7, one phase before waves 0-3 first read it.
+  // MASKED iterations clamp the rows they load to the end of the chunk and mask the scores; the others assume that the
+  // tiles they load lie inside the chunk and that every row of the workgroup sees every key of the tile.
+  auto request_tiles = [&](auto r_tag, auto masked_tag, int it) __attribute__((always_inline)) {
+    constexpr int R = decltype(r_tag)::value;
+    if constexpr (decltype(masked_tag)::value) {
+      load_k_clamped(std::integral_constant<int, (R + KA) & 3>{}, it + KA);
+      if constexpr (DV) load_v_clamped(std::integral_constant<int, (R + VA) & 3>{}, it + VA);
+    } else {
+      load_tiles_fast(r_tag);
     }
-    __builtin_amdgcn_s_barrier();
+  };
+  auto iteration = [&](auto r_tag, auto masked_tag, int it) __attribute__((always_inline)) {
+    constexpr int R = decltype(r_tag)::value;
+    constexpr bool MASKED = decltype(masked_tag)::value;
+    if (SPLIT) {
+      fphase_mfma(std::integral_constant<int, 0>{}, r_tag, std::integral_constant<bool, !MASKED>{});
+      __builtin_amdgcn_s_barrier();
+      request_tiles(r_tag, masked_tag, it);
+      fphase_softmax(masked_tag, 2 * it + kp);
+      wait_vmem<4>();
+      __builtin_amdgcn_s_barrier();
+    } else {
+      fphase_mfma(std::integral_constant<int, 0>{}, r_tag, std::integral_constant<bool, !MASKED>{});
+      __builtin_amdgcn_s_barrier();
+      request_tiles(r_tag, masked_tag, it);
+      fphase_softmax(masked_tag, 2 * it);
+      __builtin_amdgcn_s_barrier();
+      if (DV) wait_vmem<4>();
+      fphase_mfma(std::integral_constant<int, 1>{}, r_tag, std::integral_constant<bool, !MASKED>{});
+      __builtin_amdgcn_s_barrier();
+      fphase_softmax(masked_tag, 2 * it + 1);
+      if (!DV) {
+        // everything but this iteration's two K loads has arrived: the registers hold V tile it+2, and K tile it+2
+        // (loaded one iteration ago) is complete as well
+        asm volatile("s_waitcnt vmcnt(2)" : "+v"(vst[0]), "+v"(vst[1]));
+        store_v_tile(std::integral_constant<int, (R + 2) & 3>{});
+        if (MASKED) {
+          load_v_clamped(std::integral_constant<int, 0>{}, it + 3);  // (into registers: the slot is not used)
+        } else {
+          load_v_regs_fast();  // V tile it+3
+        }
+      }
+      __builtin_amdgcn_s_barrier();
+    }
   };
 
   if (nt > 0) {
-    load_tiles(std::false_type{}, 0, 0);
-    store_v_tile(0);
-    load_tiles(std::false_type{}, 1, 1);
-    store_v_tile(1);
-    load_tiles(std::false_type{}, 2, 1);
-    store_v_tile(1);
-    wait_vmem<0>();
-    // the fast loop's trip count is the same for every wave of the workgroup (it holds barriers):
-    // sub-tiles below i_mask_wg are visible to the first row of the workgroup, hence to all of them
-    const int i_mask_wg = visible_keys(qf + m_lo * P) / SUB;
-    int fast_end = i_mask_wg / 2;
-    if (fast_end > kv_len / BN - 3) fast_end = kv_len / BN - 3;
-    if (fast_end > nt) fast_end = nt;
+    // K tiles 0 .. KA-1 and V tiles 0 .. VA-1
+    load_k_clamped(std::integral_constant<int, 0>{}, 0);
+    load_k_clamped(std::integral_constant<int, 1>{}, 1);
+    load_k_clamped(std::integral_constant<int, 2>{}, 2);
+    if (SPLIT) load_k_clamped(std::integral_constant<int, 3>{}, 3);
+    if (DV) {
+      load_v_clamped(std::integral_constant<int, 0>{}, 0);
+      load_v_clamped(std::integral_constant<int, 1>{}, 1);
+      if (SPLIT) load_v_clamped(std::integral_constant<int, 2>{}, 2);
+    } else {
+      load_v_clamped(std::integral_constant<int, 0>{}, 0);
+      asm volatile("s_waitcnt vmcnt(0)" : "+v"(vst[0]), "+v"(vst[1]));
+      store_v_tile(std::integral_constant<int, 0>{});
+      load_v_clamped(std::integral_constant<int, 0>{}, 1);
+      asm volatile("s_waitcnt vmcnt(0)" : "+v"(vst[0]), "+v"(vst[1]));
+      store_v_tile(std::integral_constant<int, 1>{});
+      load_v_clamped(std::integral_constant<int, 0>{}, 2);  // stays in registers until the end of iteration 0
+    }
+    // The loop's trip count is the same for every wave of the workgroup (it holds barriers).  Tiles below n_plain are
+    // visible to the first row of the workgroup, hence to all of them, hold 64 keys, and the tiles requested while they
+    // are worked on lie inside the chunk; the loop over them is unrolled over the four ring slots.
+    int n_plain = visible_keys(qf + m_lo * P) / BN;
+    if (n_plain > kv_len / BN - KA) n_plain = kv_len / BN - KA;
+    if (n_plain > nt) n_plain = nt;
+    n_plain = n_plain < 0 ? 0 : (n_plain & ~3);
+    const int par_off = kp * (SUB * 256);
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++) {
+      kaddr[ks] = ((lds_base + koff0) ^ (ks << 6)) + par_off;
+      asm volatile("" : "+v"(kaddr[ks]));
+    }
+#pragma unroll
+    for (int db = 0; db < 8; db++) {
+      vaddr[db] = ((lds_base + kLdsV + voff0) ^ (db << 5)) + par_off;
+      asm volatile("" : "+v"(vaddr[db]));
+    }
+    if (DV) wait_vmem<0>();
+    else wait_vmem<2>();
+    __syncthreads();
+    // operands of the wave's first step; its "previous" product is a V tile times a zero P
+    load_k_operands(lds_base + par_off, koff0, ka);
+    load_v_operands(lds_base + kLdsV + par_off, voff0, va);
+    pk[0] = u32x4{0, 0, 0, 0};
+    pk[1] = u32x4{0, 0, 0, 0};
+    kt_run = uniform_ptr(kg + (int64_t)KA * BN * k_row_bytes);
+    vt_run = uniform_ptr(vg + (int64_t)(DV ? VA : 3) * BN * v_row_bytes);
     int it = 0;
-    if (fast_end >= 4) {
+    if (wave >= 4) __builtin_amdgcn_s_barrier();
+    for (; it < n_plain; it += 4) {
+      iteration(std::integral_constant<int, 0>{}, std::false_type{}, it);
+      iteration(std::integral_constant<int, 1>{}, std::false_type{}, it + 1);
+      iteration(std::integral_constant<int, 2>{}, std::false_type{}, it + 2);
+      iteration(std::integral_constant<int, 3>{}, std::false_type{}, it + 3);
+    }
+    // (the row sums of the last plain step's P, which the masked MFMA phases leave out; from here on the sums are kept
+    // lane by lane in l_run)
 #pragma unroll
-      for (int ks = 0; ks < 4; ks++) {
-        kaddr[ks] = (lds_base + koff0) ^ (ks << 6);
-        asm volatile("" : "+v"(kaddr[ks]));
-      }
+    for (int qb = 0; qb < 2; qb++) {
+      lacc[qb] = Mfma<F16>::run(ones, pk[qb], lacc[qb]);
+      l_run[qb] = g == 0 ? lacc[qb][0] : 0.f;
+    }
+    // The rest, with masks.  (Guarded iterations, not early exits from the unrolled body: those cost the register
+    // allocation of the whole kernel.)
+    for (; it < nt; it += 4) {
+      iteration(std::integral_constant<int, 0>{}, std::true_type{}, it);
+      if (it + 1 < nt) iteration(std::integral_constant<int, 1>{}, std::true_type{}, it + 1);
+      if (it + 2 < nt) iteration(std::integral_constant<int, 2>{}, std::true_type{}, it + 2);
+      if (it + 3 < nt) iteration(std::integral_constant<int, 3>{}, std::true_type{}, it + 3);
+    }
+    if (wave < 4) __builtin_amdgcn_s_barrier();
+    // (a V tile loaded ahead is dropped; its loads must have landed before the registers are used for anything else)
+    if (!DV) asm volatile("s_waitcnt vmcnt(0)" : "+v"(vst[0]), "+v"(vst[1]));
+    // the product of the wave's last step is still owed
 #pragma unroll
-      for (int db = 0; db < 8; db++) {
-        vaddr[db] = (lds_base + kLdsV + voff0) ^ (db << 5);
-        asm volatile("" : "+v"(vaddr[db]));
-      }
-      neg_m[0] = neg_m[1] = INFINITY;
-      thr_raw[0] = thr_raw[1] = -INFINITY;
-      __syncthreads();
-      // operands of step 0; its "previous" product is V(tile 0) times a zero P
-      load_k_operands(lds_base, koff0, ka);
-      load_v_operands(lds_base + kLdsV, voff0, va);
-      pk[0] = u32x4{0, 0, 0, 0};
-      pk[1] = u32x4{0, 0, 0, 0};
-      kt_run = uniform_ptr(kg + (int64_t)3 * BN * k_row_bytes);
-      vt_run = uniform_ptr(vg + (int64_t)2 * BN * v_row_bytes);
-      if (!DV) load_v_regs_fast();  // V tile 2
-      if (wave >= 4) __builtin_amdgcn_s_barrier();
-      for (; it + 3 < fast_end; it += 4) {
-        fast_iteration(std::integral_constant<int, 0>{}, it);
-        fast_iteration(std::integral_constant<int, 1>{}, it + 1);
-        fast_iteration(std::integral_constant<int, 2>{}, it + 2);
-        fast_iteration(std::integral_constant<int, 3>{}, it + 3);
-      }
-      if (wave < 4) __builtin_amdgcn_s_barrier();
-      // (a V tile loaded ahead is dropped: the general steps load what they need themselves; its loads must have
-      // landed before the registers are used for anything else)
-      if (!DV) asm volatile("s_waitcnt vmcnt(0)" : "+v"(vst[0]), "+v"(vst[1]));
-      // the product of the last fast step is still owed
+    for (int db = 0; db < 8; db++)
+#pragma unroll
+      for (int qb = 0; qb < 2; qb++) oacc[db][qb] = Mfma<F16>::run(va[db], pk[qb], oacc[db][qb]);
+    // (the masked iterations, of which the last one always is, keep the row sums in l_run lane by lane; the epilogues
+    // add the lanes of a column up)
+#pragma unroll
+    for (int qb = 0; qb < 2; qb++) m_run[qb] = -neg_m[qb];
+  }
+
+  if (SPLIT) {
+    // the partial of the odd sub-tiles (waves 4-7) joins that of the even ones through LDS; waves 0-3 go on alone
+    wait_vmem<0>();  // (loads requested ahead for tiles that were never used may still be writing the rings)
+    __syncthreads();
+    float* xch = (float*)lds + wrow * (68 * 64) + lane;  // [value][lane]: 64 accumulators, 2 maxima, 2 sums
+    if (kp == 1) {
 #pragma unroll
       for (int db = 0; db < 8; db++)
 #pragma unroll
-        for (int qb = 0; qb < 2; qb++) oacc[db][qb] = Mfma<F16>::run(va[db], pk[qb], oacc[db][qb]);
+        for (int qb = 0; qb < 2; qb++)
+#pragma unroll
+          for (int r = 0; r < 4; r++) xch[((db * 2 + qb) * 4 + r) * 64] = oacc[db][qb][r];
 #pragma unroll
       for (int qb = 0; qb < 2; qb++) {
-        lacc[qb] = Mfma<F16>::run(ones, pk[qb], lacc[qb]);
-        m_run[qb] = -neg_m[qb];
-        l_run[qb] = g == 0 ? lacc[qb][0] : 0.f;  // the general steps keep per-lane partial sums, added up over the column at the end
+        xch[(64 + qb) * 64] = m_run[qb];
+        xch[(66 + qb) * 64] = l_run[qb];
       }
     }
-    for (; it < nt; it++) iteration(it);
+    __syncthreads();
+    if (kp == 1) return;
+#pragma unroll
+    for (int qb = 0; qb < 2; qb++) {
+      const float m1 = xch[(64 + qb) * 64], l1 = xch[(66 + qb) * 64];
+      const float M = fmaxf(m_run[qb], m1);
+      const float w0 = exp2_diff(m_run[qb], M), w1 = exp2_diff(m1, M);  // 0 for a side that saw no key
+      l_run[qb] = l_run[qb] * w0 + l1 * w1;
+      m_run[qb] = M;
+#pragma unroll
+      for (int db = 0; db < 8; db++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) oacc[db][qb][r] = oacc[db][qb][r] * w0 + xch[((db * 2 + qb) * 4 + r) * 64] * w1;
+    }
   }
 
   // ---- epilogue ----
@@ -795,7 +833,8 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
   }
 }
 
-template <typename T, int MODE, bool DV> static int launch_prefill(const lsattn_prefill_args* a, hipStream_t st) {
+template <typename T, int MODE, bool DV, bool SPLIT> static int launch_prefill_rows(const lsattn_prefill_args* a, hipStream_t st) {
+  constexpr int BMW = SPLIT ? BM / 2 : BM;
   PrefillParams p;
   p.q = a->q;
   p.k = a->k;
@@ -816,7 +855,7 @@ template <typename T, int MODE, bool DV> static int launch_prefill(const lsattn_
   p.hq = a->num_q_heads;
   p.hkv = a->num_kv_heads;
   p.peers = a->sp_peers;
-  p.nz = (a->max_q_len + BM - 1) / BM;
+  p.nz = (a->max_q_len + BMW - 1) / BMW;
   {
     int g8 = 8;  // gcd(num_kv_heads, 8)
     while (a->num_kv_heads % g8) g8 >>= 1;
@@ -836,8 +875,26 @@ template <typename T, int MODE, bool DV> static int launch_prefill(const lsattn_
   p.units_per_slice = (int32_t)(((int64_t)group * p.nz + p.slices - 1) / p.slices);
   const int64_t wgs = (int64_t)8 * p.units_per_slice * p.kv_slots * a->batch;
   if (wgs > 0x7fffffff) return LSATTN_ERR_INVALID_ARG;
-  hipLaunchKernelGGL((prefill_kernel<T, MODE, DV>), dim3((unsigned)wgs), dim3(NWAVE * 64), 0, st, p);
+  hipLaunchKernelGGL((prefill_kernel<T, MODE, DV, SPLIT>), dim3((unsigned)wgs), dim3(NWAVE * 64), 0, st, p);
   return check_launch();
+}
+
+// Rows per workgroup.  256 is the efficient shape (each staged K/V tile serves twice the rows); 128 (the split variant)
+// when 256-row workgroups would be too few for the chip: under causal masking their work runs from 1 to nz tiles of
+// rows, and with less than a few of them per CU the heaviest one is the launch's duration.  LSATTN_PREFILL_ROWS = 128
+// or 256 in the environment overrides the choice (tuning and tests).
+template <typename T, int MODE, bool DV> static int launch_prefill(const lsattn_prefill_args* a, hipStream_t st) {
+  if constexpr (!DV) {
+    return launch_prefill_rows<T, MODE, false, false>(a, st);
+  } else {
+    const int64_t wgs256 = (int64_t)a->batch * a->num_q_heads * ((a->max_q_len + BM - 1) / BM);
+    bool split = wgs256 < kSplitBelowWorkgroups;
+    if (const char* e = getenv("LSATTN_PREFILL_ROWS")) {
+      if (e[0] == '1' && e[1] == '2' && e[2] == '8' && !e[3]) split = true;
+      if (e[0] == '2' && e[1] == '5' && e[2] == '6' && !e[3]) split = false;
+    }
+    return split ? launch_prefill_rows<T, MODE, true, true>(a, st) : launch_prefill_rows<T, MODE, true, false>(a, st);
+  }
 }
 
 static int validate(const lsattn_prefill_args* a, int mode) {
