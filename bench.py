@@ -3,11 +3,14 @@
 
 A step is one pass of the ring-prefill workload (BASELINE config 2): the 16384 queries of
 shard 3 of a 131072-token sequence attend to KV shards 3 (causal), 0, 1, 2 (full), one
-kernel launch per shard, then the fp32 partials are LSE-merged.  The same run also times
-the token-indexed decode workload (config 3) and reports it next to the prefill number.
+kernel launch per shard, each later launch LSE-merging its partial into the running result.
+The same run times the token-indexed decode workload (config 3, under "decode"), the other
+three baseline configs (1, 4, 5, under "workloads", each with its own roofline block) and
+small-batch decode latency against the host's call overhead ("decode_latency").
 Inputs are synthetic (seeded N(0,1)*0.5) and resident in HBM before the timed region.
 
-One JSON line goes to stdout; `--all` adds the other baseline configs under `other_configs`.
+One JSON line goes to stdout; `--all` adds the steps around attention (element-wise kernels,
+migration, allocator) under `other`.
 """
 from __future__ import annotations
 
@@ -24,7 +27,17 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
-PREFILL_TRAFFIC_BYTES = 1364.3e6  # per launch, averaged over a ring step: profiles/bench_default_hbm_traffic.txt
+# HBM bytes per launch of each workload's dominant kernel: rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled by what the same
+# counter reads for a plain copy of 1 GiB.  Not measured by this run: taken from profiles/bench_default_hbm_traffic.txt,
+# which is regenerated with the kernels (the JSON line says so in "traffic_source").
+TRAFFIC_SOURCE = "profiles/bench_default_hbm_traffic.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this command, scaled by a 1 GiB copy); a constant of bench.py, not measured in this run"
+TRAFFIC_BYTES = {
+    "config2": 1364.3e6,   # per launch, averaged over the four launches of a ring step
+    "config3": 5195.4e6,   # stage 1 of the fused call
+    "config1": None,
+    "config4": None,
+    "config5": None,
+}
 PEAK_MFMA_TFLOPS = 2500.0  # dense fp16/bf16 MFMA, MI355X
 PEAK_HBM_GBS = 8000.0
 DEV = "cuda:0"
@@ -57,6 +70,38 @@ def _time_events(fn, steps, warmup):
         b.record()
     torch.cuda.synchronize()
     return [a.elapsed_time(b) for a, b in evs]
+
+
+def _time_graph(fn, launches=20, reps=10):
+    """Device time (ms) of one call of `fn`, for calls too short to time from the host: `launches` calls are recorded
+    into one HIP graph, whose replays are timed with HIP events; the median over `reps` replays, per call."""
+    for _ in range(3):
+        fn()
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        for _ in range(launches):
+            fn()
+    g.replay()
+    torch.cuda.synchronize()
+    ts = []
+    for _ in range(reps):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        g.replay()
+        b.record()
+        torch.cuda.synchronize()
+        ts.append(a.elapsed_time(b) / launches)
+    return sorted(ts)[len(ts) // 2]
+
+
+def _roof(kernel, bound, achieved, per_launch_ms, traffic_key, **extra):
+    peak = PEAK_MFMA_TFLOPS if bound == "mfma" else PEAK_HBM_GBS
+    r = {"kernel": kernel, "bound": bound, "achieved": achieved, "peak": peak, "unit": "TFLOP/s" if bound == "mfma" else "GB/s",
+         "frac": achieved / peak, "traffic": TRAFFIC_BYTES.get(traffic_key), "traffic_source": TRAFFIC_SOURCE,
+         "per_launch_ms": per_launch_ms}
+    r.update(extra)
+    return r
 
 
 # --------------------------------------------------------------------------------------
@@ -181,6 +226,15 @@ class TokenDecode:
                                           self.max_len, self.mid_o, self.mid_l, self.BS)
         lsa.longserve_flash_decode_stage2(self.mid_o, self.mid_l, self.b_len, self.o, self.lse, self.BS)
 
+    def step_separate_stages_merged(self):
+        """The same two calls with groups of blocks merged into one partial by stage 1 (the opt-in layout)."""
+        from loongserve_amd import decoding
+        decoding.STAGE1_MERGES_BLOCKS = True
+        try:
+            self.step_separate_stages()
+        finally:
+            decoding.STAGE1_MERGES_BLOCKS = False
+
     def stage1_only(self):
         import loongserve_amd as lsa
         lsa.longserve_flash_decode_stage1(self.q, self.kv[:, :self.Hkv], self.kv[:, self.Hkv:], self.table, self.b_req, self.b_len,
@@ -244,6 +298,23 @@ class ElasticDecode:
         from loongserve_amd.simulate import multi_instance_decode
         return multi_instance_decode(self.q, self.instances, self.H, out=self.out, workspace=self.ws)
 
+    def stage1_of_one_instance(self):
+        """Stage 1 alone over the 4 x 131072 tokens of one instance, at the split the fused call uses there."""
+        import loongserve_amd as lsa
+        from loongserve_amd.decoding import _fused_block_seq
+        from loongserve_amd.simulate import decode_block_seq
+        inst = self.instances[1]
+        part = self.ctx // self.n_inst
+        if not hasattr(self, "s1"):
+            split = _fused_block_seq(decode_block_seq(part), self.B, part, self.H)
+            nblk = (part + split - 1) // split
+            self.s1 = (split, torch.empty((nblk, self.B, self.H, self.D), dtype=torch.float32, device=DEV),
+                       torch.empty((nblk, self.B, self.H), dtype=torch.float32, device=DEV), _i32([part] * self.B))
+        split, mo, ml, blen = self.s1
+        lsa.longserve_cuda_kernels.flash_decoding_stage1(mo, ml, self.q, self.kv[:, :self.H], self.kv[:, self.H:], inst.req_to_token,
+                                                         self.b_req, blen, part, split)
+        return part * self.B * (2 * self.H * self.D * 2 + 4)
+
 
 # --------------------------------------------------------------------------------------
 # config 5: mixed varlen prefill, 24 sequences log-uniform in [1024, 200000], GQA 32/8, bf16,
@@ -276,13 +347,21 @@ class VarlenPrefill:
         self.pairs = sum(n * (n + 1) // 2 for n in lens)
         self.flops = 4 * D * Hq * self.pairs
         self.scatter_bytes = T * 2 * Hkv * D * 2 * 2  # read + write of every K/V row
+        self.v_f16 = torch.empty((T, Hkv, D), dtype=torch.float16, device=DEV)  # the caller's buffer for the fp16 copy of V
 
     def attention(self):
         import loongserve_amd as lsa
         self.m.fill_(float("-inf"))
         self.l.zero_()
         lsa.context_attention_fwd(self.q, self.kv[:, :self.Hkv], self.kv[:, self.Hkv:], self.o, self.start, self.len, self.first,
-                                  self.start, self.len, self.first, 1, self.max_len, self.m, self.l)
+                                  self.start, self.len, self.first, 1, self.max_len, self.m, self.l, v_f16=self.v_f16)
+
+    def attention_kernel_only(self):
+        """The attention launch alone: (m, l) not reset (the result is not used), V's fp16 copy taken as it stands."""
+        import loongserve_amd as lsa
+        lsa.context_attention_fwd(self.q, self.kv[:, :self.Hkv], self.kv[:, self.Hkv:], self.o, self.start, self.len, self.first,
+                                  self.start, self.len, self.first, 1, self.max_len, self.m, self.l, v_f16=self.v_f16,
+                                  v_f16_valid=True)
 
     def persist(self):
         import loongserve_amd as lsa
@@ -310,44 +389,105 @@ def _stats(ms):
     return {"median_ms": s[n // 2], "p10_ms": s[int(0.1 * (n - 1))], "p90_ms": s[int(math.ceil(0.9 * (n - 1)))], "mean_ms": sum(s) / n}
 
 
-def other_configs(steps):
-    """Configs 1, 4 and 5 of the baseline, timed the same way (not part of the one-line contract)."""
+def workloads(steps):
+    """Configs 1, 4 and 5 of the baseline: each timed as a whole and with the launch duration of its dominant kernel."""
     import loongserve_amd as lsa
     out = {}
-    # config 1: single causal prefill, 2048 tokens, 32/32 heads
+    # ---- config 1: single causal prefill, 2048 tokens, 32/32 heads, fp16, one ring step
     T, H, D = 2048, 32, 128
     q, kv = _randn_half((T, H, D), 1001), _randn_half((T, 2 * H, D), 1002)
     s0, ln, f0 = _i32([0]), _i32([T]), _i32([0])
     ob = torch.empty((T, H, D), dtype=torch.float32, device=DEV)
     lb = torch.empty((T, H), dtype=torch.float32, device=DEV)
-    ms = _time_events(lambda: lsa.prefill_attention_step(q, kv[:, :H], kv[:, H:], s0, ln, f0, s0, ln, f0, 1, T, ob, lb), 50, 10)
+    call = lambda: lsa.prefill_attention_step(q, kv[:, :H], kv[:, H:], s0, ln, f0, s0, ln, f0, 1, T, ob, lb)  # noqa: E731
+    st = _stats(_time_events(call, 50, 10))
+    dev_ms = _time_graph(call, launches=20, reps=10)
     fl = 4 * D * H * (T * (T + 1) // 2)
-    st = _stats(ms)
-    out["config1"] = {"workload": "1 x 2048 causal, 32/32 heads, fp16", "median_ms": st["median_ms"], "tflops": fl / (st["median_ms"] * 1e-3) / 1e12,
-                      "pct_of_mfma_peak": 100 * fl / (st["median_ms"] * 1e-3) / 1e12 / PEAK_MFMA_TFLOPS}
+    out["config1"] = {
+        "workload": "config 1: 1 x 2048 tokens causal, 32/32 heads, head_dim 128, fp16, fp32 (O, LSE) out, one launch",
+        "value": fl / (dev_ms * 1e-3) / 1e12, "unit": "TFLOP/s", "ms_per_step": dev_ms, "pct_of_mfma_peak": 100 * fl / (dev_ms * 1e-3) / 1e12 / PEAK_MFMA_TFLOPS,
+        "algorithmic_tflop_per_step": fl / 1e12,
+        "timing": "device time per launch: 20 launches recorded in one HIP graph, replays timed with HIP events (the launch "
+                  "is shorter than the host's call overhead); eager_call_ms is one call bracketed by HIP events, host overhead included",
+        "eager_call_ms": st["median_ms"],
+        "roofline": _roof("prefill_kernel<F16,0,true,false> (256-row workgroups: 256 of them)", "mfma", fl / (dev_ms * 1e-3) / 1e12, dev_ms, "config1",
+                          algorithmic_tflop_per_launch=fl / 1e12)}
     del q, kv, ob, lb
-    # config 4
+    # ---- config 4: long-context elastic decode, 4 x 524288, MHA 32, four instances, merge at the master
     e = ElasticDecode()
-    ms = _time_events(e.step, steps, 2)
-    st = _stats(ms)
-    out["config4"] = {"workload": "decode 4 x 524288, MHA 32, 4 instances x (stage1+stage2) + merge", "median_ms": st["median_ms"],
-                      "gbs": e.bytes / (st["median_ms"] * 1e-3) / 1e9, "pct_of_hbm_peak": 100 * e.bytes / (st["median_ms"] * 1e-3) / 1e9 / PEAK_HBM_GBS}
+    st = _stats(_time_events(e.step, steps, 2))
+    nbytes1 = e.stage1_of_one_instance()
+    s1 = _stats(_time_events(e.stage1_of_one_instance, max(steps, 5), 2))
+    out["config4"] = {
+        "workload": "config 4: decode 4 x 524288 tokens, MHA 32 heads, head_dim 128, fp16, scattered pool; four simulated instances "
+                    "(three peers through the fused call, the master through stage 1 + the block_seq = 1 merge of all partials)",
+        "value": e.bytes / (st["median_ms"] * 1e-3) / 1e9, "unit": "GB/s", "ms_per_step": st["median_ms"],
+        "pct_of_hbm_peak": 100 * e.bytes / (st["median_ms"] * 1e-3) / 1e9 / PEAK_HBM_GBS, "algorithmic_gb_per_step": e.bytes / 1e9,
+        "step_stats": st,
+        "roofline": _roof("decode_stage1_kernel<F16,1,4,false,true,1> (one instance: 4 x 131072 tokens x 32 KV heads)", "hbm",
+                          nbytes1 / (s1["median_ms"] * 1e-3) / 1e9, s1["median_ms"], "config4", algorithmic_gb_per_launch=nbytes1 / 1e9)}
     del e
     torch.cuda.empty_cache()
-    # config 5
+    # ---- config 5: mixed varlen prefill, bf16, GQA 32/8, K/V rows written to pool slots and registered
     v = VarlenPrefill()
-    ms_a = _time_events(v.attention, 3, 1)
-    ms_p = _time_events(v.persist, 5, 1)
-    ms_m = _time_events(v.migrate, 5, 1)
-    sa, sp, sm = _stats(ms_a), _stats(ms_p), _stats(ms_m)
-    out["config5"] = {"workload": "24 packed sequences, %d tokens, GQA 32/8, bf16, causal + KV scatter/registration" % v.T,
-                      "attention_median_ms": sa["median_ms"], "tflops": v.flops / (sa["median_ms"] * 1e-3) / 1e12,
-                      "pct_of_mfma_peak": 100 * v.flops / (sa["median_ms"] * 1e-3) / 1e12 / PEAK_MFMA_TFLOPS,
-                      "scatter_median_ms": sp["median_ms"], "scatter_gbs": v.scatter_bytes / (sp["median_ms"] * 1e-3) / 1e9,
-                      "migration_copy_register_median_ms": sm["median_ms"],
-                      "migration_copy_register_gbs": v.scatter_bytes / (sm["median_ms"] * 1e-3) / 1e9}
+    sa = _stats(_time_events(v.attention, 3, 1))
+    sk = _stats(_time_events(v.attention_kernel_only, 3, 0))
+    sp = _stats(_time_events(v.persist, 5, 1))
+    sm = _stats(_time_events(v.migrate, 5, 1))
+    whole_ms = sa["median_ms"] + sp["median_ms"]
+    out["config5"] = {
+        "workload": "config 5: 24 packed sequences, lengths log-uniform in [1024, 200000], %d tokens, GQA 32/8, head_dim 128, bf16, "
+                    "causal, through context_attention_fwd ((m, l) reset, fp16 copy of V into the caller's buffer, one attention "
+                    "launch), then the K/V rows scattered to pool slots and registered" % v.T,
+        "value": v.flops / (whole_ms * 1e-3) / 1e12, "unit": "TFLOP/s", "ms_per_step": whole_ms,
+        "pct_of_mfma_peak": 100 * v.flops / (whole_ms * 1e-3) / 1e12 / PEAK_MFMA_TFLOPS, "algorithmic_tflop_per_step": v.flops / 1e12,
+        "attention_ms": sa["median_ms"], "attention_tflops": v.flops / (sa["median_ms"] * 1e-3) / 1e12,
+        "kv_write": {"what": "lsattn_kv_scatter + lsattn_register_tokens: every K/V row (4096 B) read and written once",
+                     "ms": sp["median_ms"], "gbs": v.scatter_bytes / (sp["median_ms"] * 1e-3) / 1e9,
+                     "pct_of_hbm_peak": 100 * v.scatter_bytes / (sp["median_ms"] * 1e-3) / 1e9 / PEAK_HBM_GBS},
+        "migration_copy_register": {"what": "the same rows through lsattn_kv_copy_register (copy + registration in one launch)",
+                                    "ms": sm["median_ms"], "gbs": v.scatter_bytes / (sm["median_ms"] * 1e-3) / 1e9},
+        "roofline": _roof("prefill_kernel<BF16,1,true,false>", "mfma", v.flops / (sk["median_ms"] * 1e-3) / 1e12, sk["median_ms"], "config5",
+                          algorithmic_tflop_per_launch=v.flops / 1e12)}
     del v
     torch.cuda.empty_cache()
+    return out
+
+
+def decode_latency():
+    """Small-batch decode: the host's cost of a call against the device's.  GQA 32/8, head_dim 128, fp16, scattered slots,
+    fused stage 1 + stage 2 call (the operator a decode step of the layer makes, longserve_transformer_layer_infer.py:293-308).
+    eager_us: wall clock per call over 200 back-to-back calls and one synchronize (host-bound when the host is slower
+    than the kernels); graph_us: the same call replayed from a HIP graph of 20 of them, per call (device time)."""
+    import loongserve_amd as lsa
+    rows = []
+    for B in (1, 4, 16):
+        for ctx in (2048, 8192, 32768):
+            d = TokenDecode(B=B, lens=[ctx] * B, pool=B * ctx + 1024, seed=3100 + B)
+            for _ in range(5):
+                d.step()
+            torch.cuda.synchronize()
+            n = 200
+            t0 = time.perf_counter()
+            for _ in range(n):
+                d.step()
+            torch.cuda.synchronize()
+            eager = (time.perf_counter() - t0) / n * 1e6
+            graph = _time_graph(d.step, launches=20, reps=10) * 1e3
+            rows.append({"batch": B, "ctx": ctx, "eager_us": round(eager, 2), "graph_us": round(graph, 2),
+                         "kv_gbs_at_graph_rate": round(d.bytes / (graph * 1e-6) / 1e9, 1)})
+            del d
+    torch.cuda.empty_cache()
+    return {"what": decode_latency.__doc__.split("\n")[0].strip() + " eager_us = wall clock per call over 200 back-to-back calls + one "
+                    "synchronize; graph_us = per call when 20 calls are replayed from one HIP graph (device time)",
+            "reference_launch_overhead_us": "100-400 (Triton launch overhead the reference reports, longserve_cuda_kernels/README.md:7-9)",
+            "cases": rows}
+
+
+def other_steps(steps):
+    """The steps around attention (not part of the five baseline configs)."""
+    import loongserve_amd as lsa
+    out = {}
     # the element-wise steps around attention at config 2's per-GPU shape (16384 tokens, hidden 4096, 32 heads, inter 11008)
     from loongserve_amd import longserve_cuda_kernels as lk
     T, H, I, NH, D = 16384, 4096, 11008, 32, 128
@@ -450,7 +590,7 @@ def main():
     ap.add_argument("--only", choices=["prefill", "decode"], default=None, help="time one workload only (profiling aid)")
     ap.add_argument("--calib-copy", action="store_true",
                     help="only run three plain 1 GiB device-to-device copies (known traffic, for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE)")
-    ap.add_argument("--all", action="store_true", help="also time configs 1, 4 and 5 (reported under 'other_configs')")
+    ap.add_argument("--all", action="store_true", help="also time the steps around attention: element-wise kernels, migration, allocator (under 'other')")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU (no collectives, no second GPU); --gpus %d is not supported" % args.gpus,
@@ -506,13 +646,8 @@ def main():
                                           "launches_per_step": w.launches + 1},
                        "in_place": {"what": "the same steps through context_attention_fwd: (o fp16, m, l) reset and updated in place",
                                     "ms_per_step": inp["mean_ms"], "value": w.flops / (inp["mean_ms"] * 1e-3) / 1e12}},
-            "roofline": {"kernel": "prefill_kernel<F16,0,true> (diagonal launch) + prefill_kernel<F16,2,true> (three full launches)",
-                         "bound": "mfma", "achieved": ach, "peak": PEAK_MFMA_TFLOPS, "unit": "TFLOP/s",
-                         "frac": ach / PEAK_MFMA_TFLOPS,
-                         # HBM bytes per launch, averaged over the step's four launches: rocprofv3 FETCH_SIZE / WRITE_SIZE scaled
-                         # by a plain copy, profiles/bench_default_hbm_traffic.txt
-                         "traffic": PREFILL_TRAFFIC_BYTES,
-                         "per_launch_ms": per_launch_ms, "algorithmic_tflop_per_launch": w.flops / w.launches / 1e12},
+            "roofline": _roof("prefill_kernel<F16,0,true,false> (diagonal launch) + prefill_kernel<F16,2,true,false> (three full launches)",
+                              "mfma", ach, per_launch_ms, "config2", algorithmic_tflop_per_launch=w.flops / w.launches / 1e12),
         })
         if not args.no_cpu:
             line["cpu_baseline"] = w.cpu_baseline()
@@ -526,6 +661,7 @@ def main():
         d_ms = _time_events(d.step, dsteps, max(args.warmup, 2))
         s1_ms = _time_events(d.stage1_only, dsteps, 1)
         sep = _stats(_time_events(d.step_separate_stages, dsteps, 2))
+        sepm = _stats(_time_events(d.step_separate_stages_merged, dsteps, 2))
         st = _stats(d_ms)
         gbs = d.bytes / (st["mean_ms"] * 1e-3) / 1e9
         s1 = sum(s1_ms) / len(s1_ms)
@@ -537,12 +673,12 @@ def main():
                                    "split-K at %d tokens between the stages)" % (d.BS, d.split),
                        "tokens": d.tokens, "algorithmic_gb_per_step": d.bytes / 1e9, "step_stats": st,
                        "separate_stages": {"what": "stage 1 and stage 2 as two calls at BLOCK_SEQ %d (the master path of a decode "
-                                                   "step); stage 1 merges groups of blocks into one partial" % d.BS,
-                                           "ms_per_step": sep["mean_ms"], "value": d.bytes / (sep["mean_ms"] * 1e-3) / 1e9}},
-            "roofline": {"kernel": "decode_stage1_kernel<F16,4,4,false,true,1>", "bound": "hbm", "achieved": ach, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                         "frac": ach / PEAK_HBM_GBS,
-                         # HBM bytes per launch (read 5174.6 MB + written 20.8 MB), same source as above
-                         "traffic": 5195.4e6, "per_launch_ms": s1},
+                                                   "step), one partial per block: the reference's buffers" % d.BS,
+                                           "ms_per_step": sep["mean_ms"], "value": d.bytes / (sep["mean_ms"] * 1e-3) / 1e9,
+                                           "merged_blocks": {"what": "the same two calls with decoding.STAGE1_MERGES_BLOCKS = True (opt-in, "
+                                                                     "not the reference's layout): one partial per group of blocks",
+                                                             "ms_per_step": sepm["mean_ms"], "value": d.bytes / (sepm["mean_ms"] * 1e-3) / 1e9}}},
+            "roofline": _roof("decode_stage1_kernel<F16,4,4,false,true,1>", "hbm", ach, s1, "config3"),
         }
         if not args.no_cpu:
             dec["cpu_baseline"] = d.cpu_baseline()
@@ -552,8 +688,13 @@ def main():
                 line["cpu_baseline"] = dec["cpu_baseline"]
         else:
             line["decode"] = dec
+        del d
+        torch.cuda.empty_cache()
+    if args.only is None:
+        line["workloads"] = workloads(max(3, min(args.steps, 10)))
+        line["decode_latency"] = decode_latency()
     if args.all:
-        line["other_configs"] = other_configs(max(3, min(args.steps, 10)))
+        line["other"] = other_steps(max(3, min(args.steps, 10)))
     print(json.dumps(line))
 
 

@@ -17,7 +17,12 @@ LIB_PATH = os.path.join(PKG_DIR, "liblsattn.so")
 SOURCES = ["prefill.hip", "decode.hip", "merge_scatter.hip", "elementwise.hip", "pool.hip"]
 # elementwise.hip reproduces the reference's half arithmetic operation by operation: no fused multiply-adds
 # other than the ones it writes
-FILE_FLAGS = {"elementwise.hip": ["-ffp-contract=off"]}
+FILE_FLAGS = {
+    "elementwise.hip": ["-ffp-contract=off"],
+    # prefill.hip only: no NaN is ever produced on a valid path of its loop (infinities are, and stay honoured); this drops
+    # the v_max x,x,x canonicalisation in front of every fmaxf of the softmax phase, the scarce one there
+    "prefill.hip": ["-fno-honor-nans"],
+}
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
@@ -25,9 +30,6 @@ FLAGS = [
     # packed-fp32 VALU forms are switched off for every kernel in this library
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-I" + os.path.join(ROOT, "include"), "-I" + CSRC,
-    # no NaN is ever produced on a valid path (infinities are, and stay honoured); this drops the
-    # v_max x,x,x canonicalisation in front of every fmaxf
-    "-fno-honor-nans",
     "-Wno-unused-result",
 ]
 

@@ -9,12 +9,14 @@ from . import longserve_cuda_kernels
 
 
 # The stage functions called on their own (the master path, longserve_transformer_layer_infer.py:272-281 then :360-367)
-# must leave rows that an LSE merge over ceil(len / block_seq) rows per request turns into the right result; nothing in
-# the reference looks at a single block's partial.  With this switch on, stage 1 computes one partial per group of
-# consecutive blocks (the same rule as the fused call below, at most 16 blocks), writes it to the row of the group's first
-# block and marks the rows of the others empty (LSE = -inf): a quarter of the partial bytes at BLOCK_SEQ 256, and the
-# separate calls run as fast as the fused one.  Off: one partial per block, exactly the reference's buffers.
-STAGE1_MERGES_BLOCKS = True
+# leave the reference's buffers: one partial per block of block_seq tokens, row i of mid_out = block i.
+# Opt-in (STAGE1_MERGES_BLOCKS = True; not the reference's layout): stage 1 computes one partial per group of consecutive
+# blocks (the same rule as the fused call below, at most 16 blocks), writes it to the row of the group's first block and
+# marks the rows of the others empty (LSE = -inf, mid_out row left as it was).  Any LSE merge over ceil(len / block_seq)
+# rows per request that skips empty rows (this package's stage 2 does) gives the same result, with a quarter of the
+# partial bytes at BLOCK_SEQ 256; a consumer that multiplies an empty row's mid_out by a zero weight instead must not use
+# it (the stale row may hold anything).
+STAGE1_MERGES_BLOCKS = False
 
 
 def longserve_flash_decode_stage1(q, k, v, Req_to_tokens, B_req_idx, B_Seqlen, max_len_in_batch, mid_out,

@@ -64,11 +64,15 @@ def _slots(t: torch.Tensor, name: str, n: Optional[int] = None) -> torch.Tensor:
 PRECONVERT_BF16_V = True
 
 
-def _v_as_f16(v: torch.Tensor) -> torch.Tensor:
+def _v_as_f16(v: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """fp16 copy of a [tokens, heads, head_dim] bfloat16 tensor (any token / head strides), made on the device by
-    lsattn_bf16_to_f16_rows; values beyond fp16's range become +-65504."""
+    lsattn_bf16_to_f16_rows into `out` (the caller's contiguous fp16 [tokens, heads, head_dim] buffer; a new tensor if
+    None); values beyond fp16's range become +-65504."""
     T, H, D = v.shape
-    out = torch.empty((T, H, D), dtype=torch.float16, device=v.device)
+    if out is None:
+        out = torch.empty((T, H, D), dtype=torch.float16, device=v.device)
+    elif out.dtype != torch.float16 or tuple(out.shape) != (T, H, D) or not out.is_contiguous() or out.device != v.device:
+        raise ValueError("v_f16 must be a contiguous float16 tensor of v's shape on v's device")
     if T == 0:
         return out
     lib = _lib.load()
@@ -94,7 +98,8 @@ def _pad_head_dim(t: torch.Tensor) -> torch.Tensor:
 
 
 def _prefill_args(q, k, v, o, q_b_start_loc, q_b_seq_len, q_first, kv_b_start_loc, kv_b_seq_len, kv_first,
-                  peers: int, max_q_len: int, sm_scale: Optional[float]) -> _lib.PrefillArgs:
+                  peers: int, max_q_len: int, sm_scale: Optional[float], v_f16: Optional[torch.Tensor] = None,
+                  v_f16_valid: bool = False) -> _lib.PrefillArgs:
     for t, n in ((q, "q"), (k, "k"), (v, "v"), (o, "o")):
         _dev(t, n)
         if t.dim() != 3:
@@ -116,8 +121,13 @@ def _prefill_args(q, k, v, o, q_b_start_loc, q_b_seq_len, q_first, kv_b_start_lo
                  (kv_b_start_loc, "kv_b_start_loc"), (kv_b_seq_len, "kv_b_seq_len"), (kv_first, "kv_first_token_global_idx")):
         _i32vec(t, n, B)
     a = _lib.PrefillArgs()
-    if q.dtype == torch.bfloat16 and PRECONVERT_BF16_V:
-        v = _v_as_f16(v)
+    if q.dtype == torch.bfloat16 and (PRECONVERT_BF16_V or v_f16 is not None):
+        if v_f16_valid:
+            if v_f16 is None or v_f16.dtype != torch.float16 or v_f16.shape != v.shape or v_f16.stride(2) != 1:
+                raise ValueError("v_f16_valid needs v_f16, the float16 copy of v")
+            v = v_f16
+        else:
+            v = _v_as_f16(v, v_f16)
         a.v_is_f16 = 1
         a._v_f16 = v  # keeps the copy alive as long as the argument block
     a.q, a.k, a.v = q.data_ptr(), k.data_ptr(), v.data_ptr()
@@ -140,8 +150,14 @@ def _prefill_args(q, k, v, o, q_b_start_loc, q_b_seq_len, q_first, kv_b_start_lo
 @torch.inference_mode()
 def context_attention_fwd(q, k, v, o, q_b_start_loc, q_b_seq_len, q_first_token_global_idx,
                           kv_b_start_loc, kv_b_seq_len, kv_first_token_global_idx,
-                          logical_sp_peers_num: int, max_q_b_seq_len: int, m, l) -> None:
+                          logical_sp_peers_num: int, max_q_b_seq_len: int, m, l, *, v_f16: Optional[torch.Tensor] = None,
+                          v_f16_valid: bool = False) -> None:
     """One ring-attention step folded in place into (o, m, l); signature of RING:191-206.
+
+    Keyword-only additions for bfloat16 inputs (the reference is fp16 only): the kernel multiplies P and V in fp16, so V is
+    rewritten as fp16 first.  v_f16 is the caller's buffer for that copy (contiguous float16, v's shape): with it the call
+    allocates nothing; v_f16_valid=True says it already holds the copy of this v (e.g. from an earlier step over the same
+    chunk) and skips the conversion.
 
     Call it repeatedly with the same local q/o/m/l and a different kv chunk each time.
     Start from m = -inf, l = 0 (o need not be zeroed).  After k calls o is the
@@ -158,7 +174,7 @@ def context_attention_fwd(q, k, v, o, q_b_start_loc, q_b_seq_len, q_first_token_
         q, k, v = _pad_head_dim(q), _pad_head_dim(k), _pad_head_dim(v)
     a = _prefill_args(q, k, v, o, q_b_start_loc, q_b_seq_len, q_first_token_global_idx, kv_b_start_loc,
                       kv_b_seq_len, kv_first_token_global_idx, logical_sp_peers_num, max_q_b_seq_len,
-                      1.0 / (D ** 0.5))
+                      1.0 / (D ** 0.5), v_f16 if o_user is None else None, v_f16_valid and o_user is None)
     for t, n in ((m, "m"), (l, "l")):
         _dev(t, n)
         if t.dtype != torch.float32 or t.dim() != 2 or tuple(t.shape) != (q.shape[0], q.shape[1]):
@@ -177,8 +193,10 @@ def prefill_attention_step(q, k, v, q_b_start_loc, q_b_seq_len, q_first_token_gl
                            kv_b_start_loc, kv_b_seq_len, kv_first_token_global_idx,
                            logical_sp_peers_num: int, max_q_b_seq_len: int,
                            out: Optional[torch.Tensor] = None, lse: Optional[torch.Tensor] = None,
-                           sm_scale: Optional[float] = None, accumulate: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
+                           sm_scale: Optional[float] = None, accumulate: bool = False, v_f16: Optional[torch.Tensor] = None,
+                           v_f16_valid: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
     """One step as a mergeable partial: (O fp32 [Tq,Hq,D] normalised, LSE fp32 [Tq,Hq]).
+    v_f16 / v_f16_valid: as in context_attention_fwd (the caller's buffer for the fp16 copy of a bfloat16 v).
 
     Same inputs as context_attention_fwd; rows that see no key get O = 0, LSE = -inf.
     With accumulate=True the step is LSE-merged into the (out, lse) passed in (a running partial of earlier steps over
@@ -202,7 +220,8 @@ def prefill_attention_step(q, k, v, q_b_start_loc, q_b_seq_len, q_first_token_gl
         if sm_scale is None:
             sm_scale = 1.0 / (D ** 0.5)
     a = _prefill_args(q, k, v, out, q_b_start_loc, q_b_seq_len, q_first_token_global_idx, kv_b_start_loc,
-                      kv_b_seq_len, kv_first_token_global_idx, logical_sp_peers_num, max_q_b_seq_len, sm_scale)
+                      kv_b_seq_len, kv_first_token_global_idx, logical_sp_peers_num, max_q_b_seq_len, sm_scale,
+                      v_f16 if out_user is None else None, v_f16_valid and out_user is None)
     a.lse = lse.data_ptr()
     if accumulate:
         _lib.check(_lib.load().lsattn_prefill_step_accumulate(C.byref(a), _stream()), "lsattn_prefill_step_accumulate")
@@ -254,7 +273,9 @@ def kv_scatter(src: torch.Tensor, dest_index: torch.Tensor, pool: torch.Tensor) 
     dest_index = _slots(dest_index, "dest_index", src.shape[0])
     if src.dtype != pool.dtype or src.shape[1:] != pool.shape[1:]:
         raise ValueError("src and pool rows must match")
-    if not src[0].is_contiguous() or not pool[0].is_contiguous():
+    if src.shape[0] == 0:
+        return  # an empty chunk writes nothing
+    if pool.shape[0] == 0 or not src[0].is_contiguous() or not pool[0].is_contiguous():
         raise ValueError("rows must be contiguous")
     row_bytes = src[0].numel() * src.element_size()
     rc = _lib.load().lsattn_kv_scatter(src.data_ptr(), src.stride(0) * src.element_size(), pool.data_ptr(),
@@ -386,7 +407,9 @@ def destindex_copy_and_register_kv(batch_size: int, new_kv_cache_len: torch.Tens
     _dev(kv, "kv"); _dev(total_kv_cache, "total_kv_cache"); _dev(req_to_token_indexs, "req_to_token_indexs")
     if kv.dtype != total_kv_cache.dtype or kv.shape[1:] != total_kv_cache.shape[1:]:
         raise ValueError("kv and total_kv_cache rows must match")
-    if not kv[0].is_contiguous() or not total_kv_cache[0].is_contiguous():
+    if kv.shape[0] == 0:
+        return  # no rows held: nothing can migrate
+    if total_kv_cache.shape[0] == 0 or not kv[0].is_contiguous() or not total_kv_cache[0].is_contiguous():
         raise ValueError("rows must be contiguous")
     if req_to_token_indexs.dtype != torch.int32 or not req_to_token_indexs.is_contiguous():
         raise ValueError("req_to_token_indexs must be contiguous int32")

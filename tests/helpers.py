@@ -34,6 +34,20 @@ def assert_o_close(o_gpu, o_ref, what="", max_abs=O_MAX_ABS, rel=O_REL):
     assert fro <= rel, "%s: relative %.3e > %.1e" % (what, fro, rel)
 
 
+def assert_inplace_o_close(o_gpu, o_state_ref, o_exact, what=""):
+    """The running `o` of context_attention_fwd, stored in q's dtype and re-rounded to it at every step.
+    o_state_ref is the oracle's state after the same steps with the same storage dtype (oracle.context_attention_fwd
+    rounds at every step too): held to the stated bars for float16; for bfloat16 to the same relative bar doubled and to
+    one unit in the last place of that format below |o| = 2 (two roundings of nearly equal fp32 values differ by at
+    most that).  o_exact, the fp32 answer, is a second, looser check that the state has not drifted."""
+    if o_gpu.dtype == torch.float16:
+        assert_o_close(o_gpu, o_state_ref, what + " (vs the oracle's fp16 state)", max_abs=O_MAX_ABS, rel=O_REL)
+        assert_o_close(o_gpu, o_exact, what + " (vs the fp32 answer)", max_abs=2e-3, rel=1.5e-3)
+    else:
+        assert_o_close(o_gpu, o_state_ref, what + " (vs the oracle's bf16 state)", max_abs=2.0 ** -7, rel=2 * O_REL)
+        assert_o_close(o_gpu, o_exact, what + " (vs the fp32 answer)", max_abs=2e-2, rel=6e-3)
+
+
 def assert_lse_close(l_gpu, l_ref, what="", rel=LSE_REL):
     a = l_gpu.detach().float().cpu()
     b = l_ref.float()

@@ -26,13 +26,17 @@ def test_stage1_stage2_vs_oracle(lsa, dtype, Hq, Hkv, BS):
     orc.decode_stage1(q, k, v, table, b_req, b_len, max(lens), mid_o, mid_l, BS)
     kvd = kv.to(DEV)
     from loongserve_amd import decoding
-    # first with groups of blocks merged into one partial (the default of the stage function called on its own): the rows
-    # of a group's other blocks are marked empty, rows past the request stay untouched, and the merge gives the same result
-    assert decoding.STAGE1_MERGES_BLOCKS
-    mo_d = torch.full((nblk, B, Hq, D), float("nan"), device=DEV)
-    ml_d = torch.full((nblk, B, Hq), float("nan"), device=DEV)
-    lsa.longserve_flash_decode_stage1(q.to(DEV), kvd[:, :Hkv], kvd[:, Hkv:], table.to(DEV), b_req.to(DEV),
-                                      b_len.to(DEV), max(lens), mo_d, ml_d, BS)
+    # opt-in layout first: groups of blocks merged into one partial; the rows of a group's other blocks are marked empty,
+    # rows past the request stay untouched, and the merge gives the same result
+    assert not decoding.STAGE1_MERGES_BLOCKS  # the default is the reference's one partial per block
+    decoding.STAGE1_MERGES_BLOCKS = True
+    try:
+        mo_d = torch.full((nblk, B, Hq, D), float("nan"), device=DEV)
+        ml_d = torch.full((nblk, B, Hq), float("nan"), device=DEV)
+        lsa.longserve_flash_decode_stage1(q.to(DEV), kvd[:, :Hkv], kvd[:, Hkv:], table.to(DEV), b_req.to(DEV),
+                                          b_len.to(DEV), max(lens), mo_d, ml_d, BS)
+    finally:
+        decoding.STAGE1_MERGES_BLOCKS = False
     o_d = torch.empty(B, Hq, D, device=DEV)
     l_d = torch.empty(B, Hq, device=DEV)
     lsa.longserve_flash_decode_stage2(mo_d, ml_d, b_len.to(DEV), o_d, l_d, BS)
@@ -44,16 +48,12 @@ def test_stage1_stage2_vs_oracle(lsa, dtype, Hq, Hkv, BS):
     o_ref, l_ref = orc.decode_full(q, k, v, table, b_req, b_len)
     assert_o_close(o_d, o_ref, "o from merged groups")
     assert_lse_close(l_d, l_ref, "lse from merged groups")
-    # then one partial per block, the reference's buffers
-    decoding.STAGE1_MERGES_BLOCKS = False
-    try:
-        mo_d = torch.full((nblk, B, Hq, D), float("nan"), device=DEV)
-        ml_d = torch.full((nblk, B, Hq), float("nan"), device=DEV)
-        lsa.longserve_flash_decode_stage1(q.to(DEV), kvd[:, :Hkv], kvd[:, Hkv:], table.to(DEV), b_req.to(DEV),
-                                          b_len.to(DEV), max(lens), mo_d, ml_d, BS)
-        torch.cuda.synchronize()
-    finally:
-        decoding.STAGE1_MERGES_BLOCKS = True
+    # then the default: one partial per block, the reference's buffers
+    mo_d = torch.full((nblk, B, Hq, D), float("nan"), device=DEV)
+    ml_d = torch.full((nblk, B, Hq), float("nan"), device=DEV)
+    lsa.longserve_flash_decode_stage1(q.to(DEV), kvd[:, :Hkv], kvd[:, Hkv:], table.to(DEV), b_req.to(DEV),
+                                      b_len.to(DEV), max(lens), mo_d, ml_d, BS)
+    torch.cuda.synchronize()
     # blocks past a request's length are left untouched, like the reference
     written = ~torch.isnan(mid_l)
     assert torch.equal(torch.isnan(ml_d.cpu()), ~written)
@@ -72,6 +72,54 @@ def test_stage1_stage2_vs_oracle(lsa, dtype, Hq, Hkv, BS):
         else:
             assert_o_close(o_d, o_ref, "o")
         assert_lse_close(l_d, l_ref, "lse")
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("merge", [2, 8, 16])
+@pytest.mark.parametrize("Hq,Hkv,BS,lens", [
+    (32, 8, 16, [700, 1, 256, 33, 1025]),      # group 4, many short blocks
+    (8, 1, 128, [5000]),                       # group 8 (two rounds of four heads), one request: the waves split a block
+    (16, 1, 256, [3000, 9000]),                # group 16 (two tasks per KV head), few workgroups: split path
+    (16, 4, 32, [100, 2049, 17, 640, 1, 999]),  # group 4, ragged
+    (4, 4, 128, [4097, 130]),                  # one query head per KV head
+])
+def test_stage1_forced_merge_blocks(lsa, dtype, merge, Hq, Hkv, BS, lens):
+    """merge_blocks = m of flash_decoding_stage1: the partial of blocks [m j, m j + m) of a request in row m j, the other
+    rows the request reaches marked empty, rows past it untouched; checked row by row against the oracle's stage 1 at
+    block size m * BS, and through stage 2 at the caller's block size."""
+    print("case", dtype, merge, Hq, Hkv, BS, lens, flush=True)
+    B, D = len(lens), 128
+    q, kv, table, b_req, b_len = decode_case(500 + merge, B, Hq, Hkv, D, lens, sum(lens) + 300, dtype)
+    k, v = kv[:, :Hkv], kv[:, Hkv:]
+    nblk = (max(lens) + BS - 1) // BS
+    ngrp = (nblk + merge - 1) // merge
+    ref_o = torch.full((ngrp, B, Hq, D), float("nan"))
+    ref_l = torch.full((ngrp, B, Hq), float("nan"))
+    orc.decode_stage1(q, k, v, table, b_req, b_len, max(lens), ref_o, ref_l, BS * merge)
+    kvd = kv.to(DEV)
+    mo_d = torch.full((nblk, B, Hq, D), float("nan"), device=DEV)
+    ml_d = torch.full((nblk, B, Hq), float("nan"), device=DEV)
+    lsa.longserve_cuda_kernels.flash_decoding_stage1(mo_d, ml_d, q.to(DEV), kvd[:, :Hkv], kvd[:, Hkv:], table.to(DEV), b_req.to(DEV),
+                                                     b_len.to(DEV), max(lens), BS, merge)
+    torch.cuda.synchronize()
+    mo_c, ml_c = mo_d.cpu(), ml_d.cpu()
+    for b in range(B):
+        reach = (lens[b] + BS - 1) // BS
+        for i in range(nblk):
+            if i >= reach:
+                assert torch.isnan(ml_c[i, b]).all() and torch.isnan(mo_c[i, b]).all(), (b, i)   # untouched
+            elif i % merge:
+                assert (ml_c[i, b] == float("-inf")).all() and torch.isnan(mo_c[i, b]).all(), (b, i)  # empty, mid_o left alone
+            else:
+                assert_o_close(mo_c[i, b], ref_o[i // merge, b], "mid_o row %d request %d" % (i, b))
+                assert_lse_close(ml_c[i, b], ref_l[i // merge, b], "mid_lse row %d request %d" % (i, b))
+    o_d = torch.empty(B, Hq, D, device=DEV)
+    l_d = torch.empty(B, Hq, device=DEV)
+    lsa.longserve_flash_decode_stage2(mo_d, ml_d, b_len.to(DEV), o_d, l_d, BS)
+    torch.cuda.synchronize()
+    o_ref, l_ref = orc.decode_full(q, k, v, table, b_req, b_len)
+    assert_o_close(o_d, o_ref, "o")
+    assert_lse_close(l_d, l_ref, "lse")
 
 
 def test_gather_indices_bit_exact(lsa):

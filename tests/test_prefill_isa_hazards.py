@@ -4,7 +4,19 @@ assembly block, that
   * no vector-ALU instruction writes one of its source registers in the two instructions before it (the compiler
     rebuilding a constant or copying a register right in front of the MFMA), and
   * no other instruction touches its result in the six instructions after it.
-Loads from LDS / scratch into the sources are ordered by s_waitcnt, which the compiler does insert for inline assembly."""
+Loads from LDS / scratch into the sources are ordered by s_waitcnt, which the compiler does insert for inline assembly.
+
+The K/V tile loads (global -> LDS, and global -> registers for a bfloat16 V) are issued from inline assembly too, with
+hand-placed `s_waitcnt vmcnt(N)`: the compiler neither counts them nor waits for them.  For every loop of every kernel
+that holds such loads the test checks the budget the pipeline is built on: after a group of tile loads, and before the
+next group is issued, there is a wait that leaves at most that one group in flight (so the group before it has landed),
+and a workgroup barrier follows that wait before the next group goes out (the other waves' parts have landed too before
+anyone reads the tile, and nobody still reads the slot the next loads overwrite).  In the kernels that take fp16 V tiles
+no other vector-memory instruction (a register spill) sits in those loops: its compiler-placed vmcnt(0) would wait for
+the tile loads just issued.
+
+decode.hip orders DPP additions by hand: a DPP operand needs two wait states after a vector write of it, so no vector
+instruction may write the DPP source of an inline-assembly DPP instruction in the two instructions before it."""
 import os
 import re
 import shutil
@@ -101,5 +113,178 @@ def test_no_vector_write_next_to_an_inline_assembly_mfma():
         text = open(out).read()
     ins, bad = find_hazards(text)
     n_asm_mfma = sum(1 for _, op, _, in_asm in ins if in_asm and op.startswith("v_mfma"))
-    assert n_asm_mfma >= 9 * 8 * 34, n_asm_mfma   # nine kernels (dtype / V route x three epilogues), eight unrolled phases of 34 MFMAs
+    # fifteen kernels (dtype / V route / rows per workgroup x three epilogues); the 256-row ones hold eight unrolled
+    # plain phases of 34 MFMAs and eight masked ones of 32
+    assert n_asm_mfma >= 15 * 4 * (34 + 32), n_asm_mfma
+    assert not bad, "\n".join(bad[:20])
+    bad = tile_load_budget_violations(text)
+    assert not bad, "\n".join(bad[:20])
+
+
+def _kernels(text):
+    """{kernel symbol: its lines} for every prefill_kernel instantiation in the assembly text."""
+    out, name = {}, None
+    for raw in text.split("\n"):
+        m = re.match(r"^(_ZN6lsattn14prefill_kernel\w+):", raw)
+        if m:
+            name = m.group(1)
+            out[name] = []
+        elif raw.startswith("\t.end_amdhsa_kernel") or raw.startswith(".Lfunc_end"):
+            name = None
+        if name:
+            out[name].append(raw)
+    return out
+
+
+def _loops(lines):
+    """(first line index, last line index) of every loop: a label and a later branch back to it."""
+    labels = {}
+    loops = []
+    for i, raw in enumerate(lines):
+        m = re.match(r"^(\.LBB\d+_\d+):", raw)
+        if m:
+            labels[m.group(1)] = i
+        m = re.match(r"^\s+s_cbranch_\w+\s+(\.LBB\d+_\d+)", raw) or re.match(r"^\s+s_branch\s+(\.LBB\d+_\d+)", raw)
+        if m and m.group(1) in labels:
+            loops.append((labels[m.group(1)], i))
+    return loops
+
+
+def tile_load_budget_violations(text, min_loops=2 * 15):
+    """Plays the vector-memory counter over every loop that issues tile loads (three trips; loads complete in order, a
+    wait for vmcnt(n) retires all but the n youngest) and reports, in the steady state:
+      * a group of global -> LDS loads issued while a group older than the previous one is still in flight,
+      * a group of global -> LDS loads issued after a hand-placed wait (vmcnt(n), n > 0) retired LDS loads with no
+        barrier in between,
+      * (fp16-V kernels) any other vector-memory instruction in the loop."""
+    bad = []
+    n_loops = 0
+    for name, lines in _kernels(text).items():
+        fp16_v = bool(re.search(r"ELi\dELb1ELb[01]E", name))  # DV = true
+        for lo, hi in _loops(lines):
+            ev, in_asm = [], False  # ("L",) load to LDS, ("R",) load to registers, ("W", n), ("B",), ("X", text) other vmem
+            for raw in lines[lo:hi + 1]:
+                if "#ASMSTART" in raw:
+                    in_asm = True
+                    continue
+                if "#ASMEND" in raw:
+                    in_asm = False
+                    continue
+                ins = raw.split(";")[0].strip()
+                if not ins:
+                    continue
+                op = ins.split()[0]
+                if op.startswith(("global_", "scratch_", "buffer_", "flat_")):
+                    if in_asm and op.startswith("global_load_lds"):
+                        ev.append(("L",))
+                    elif in_asm and op.startswith("global_load"):
+                        ev.append(("R",))
+                    else:
+                        ev.append(("X", ins))
+                elif op == "s_waitcnt":
+                    m = re.search(r"vmcnt\((\d+)\)", ins)
+                    if m:
+                        ev.append(("W", int(m.group(1))))
+                elif op == "s_barrier":
+                    ev.append(("B",))
+            if not any(e[0] == "L" for e in ev):
+                continue
+            n_loops += 1
+            if fp16_v:
+                bad += ["%s: %s inside a loop with tile loads" % (name, e[1]) for e in ev if e[0] == "X"]
+            ev = [e for e in ev if e[0] != "X"]
+            queue, group, prev, need_barrier = [], 0, None, False  # queue of (LDS group id or None), oldest first
+            found = set()
+            for trip in range(3):
+                for e in ev:
+                    if e[0] == "L":
+                        if prev != "L":
+                            group += 1
+                            older = {g for g in queue if g is not None and g < group - 1}
+                            if trip and older:
+                                found.add("%s: tile loads issued with more than the previous group still in flight" % name)
+                            if trip and need_barrier:
+                                found.add("%s: tile loads issued after a wait for earlier ones with no barrier in between" % name)
+                        queue.append(group)
+                    elif e[0] == "R":
+                        queue.append(None)
+                    elif e[0] == "W":
+                        done, queue = queue[:max(len(queue) - e[1], 0)], queue[max(len(queue) - e[1], 0):]
+                        # (a vmcnt(0) in a loop is the compiler's, behind a spill reload: it only makes this wave wait
+                        # longer and is not the wait the pipeline relies on)
+                        if e[1] > 0 and any(g is not None for g in done):
+                            need_barrier = True
+                    elif e[0] == "B":
+                        need_barrier = False
+                    prev = e[0]
+            bad += sorted(found)
+    assert n_loops >= min_loops, n_loops  # a plain and a masked loop in each of the fifteen kernels
+    return bad
+
+
+def test_budget_scanner_flags_a_lax_wait():
+    ok = """_ZN6lsattn14prefill_kernelINS_3F16ELi0ELb1ELb0EEEvNS_13PrefillParamsE:
+.LBB0_1:
+	;;#ASMSTART
+	global_load_lds_dwordx4 v1, s[2:3]
+	global_load_lds_dwordx4 v2, s[2:3]
+	;;#ASMEND
+	s_barrier
+	s_waitcnt vmcnt(%d)
+	s_barrier
+	s_cbranch_scc1 .LBB0_1
+"""
+    scan = lambda t: tile_load_budget_violations(t, min_loops=1)
+    assert not scan(ok % 2)
+    assert any("still in flight" in b for b in scan(ok % 3))
+    assert any("no barrier" in b for b in scan((ok % 2).replace("\ts_barrier\n\ts_cbranch", "\ts_cbranch")))
+    assert any("inside a loop" in b for b in scan((ok % 2).replace("\ts_barrier\n\ts_waitcnt", "\tscratch_load_dword v3, off, off\n\ts_barrier\n\ts_waitcnt")))
+
+
+def find_dpp_hazards(text):
+    ins, bad = _instructions(text), []
+    for idx, (ln, op, ops, in_asm) in enumerate(ins):
+        if not (in_asm and op.endswith("_dpp")):
+            continue
+        srcs = set().union(*[_regs(t) for t in ops[1:3]])
+        for back in (1, 2):
+            if idx - back < 0:
+                break
+            l2, op2, ops2, _ = ins[idx - back]
+            if op2.startswith("v_") and not op2.startswith("v_cmp") and ops2 and (_regs(ops2[0]) & srcs):
+                bad.append("line %d: DPP source written by %s at line %d" % (ln, op2, l2))
+    return ins, bad
+
+
+def test_dpp_scanner_flags_a_close_write():
+    text = """
+	;;#ASMSTART
+	v_dot2c_f32_f16 v5, v1, v2
+	;;#ASMEND
+	v_mov_b32_e32 v7, v5
+	;;#ASMSTART
+	v_add_f32_dpp v9, v7, v7 row_ror:8 row_mask:0xf bank_mask:0x3
+	;;#ASMEND
+	;;#ASMSTART
+	v_add_f32_dpp v10, v5, v5 row_ror:8 row_mask:0xf bank_mask:0x3
+	;;#ASMEND
+"""
+    _, bad = find_dpp_hazards(text)
+    assert len(bad) == 1 and "written by v_mov_b32_e32" in bad[0], bad
+
+
+@pytest.mark.skipif(shutil.which(HIPCC) is None, reason="hipcc not available")
+def test_no_vector_write_next_to_an_inline_assembly_dpp_in_decode():
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("_lsattn_build_flags", os.path.join(REPO, "loongserve_amd", "build.py"))
+    recipe = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(recipe)
+    src = os.path.join(REPO, "loongserve_amd", "csrc", "decode.hip")
+    with tempfile.TemporaryDirectory() as tmp:
+        out = os.path.join(tmp, "decode.s")
+        cmd = [recipe.HIPCC, *recipe.FLAGS, *recipe.FILE_FLAGS.get("decode.hip", []), "-S", "--cuda-device-only", src, "-o", out]
+        subprocess.run(cmd, check=True, stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)
+        text = open(out).read()
+    ins, bad = find_dpp_hazards(text)
+    assert sum(1 for _, op, _, in_asm in ins if in_asm and op.endswith("_dpp")) >= 1000
     assert not bad, "\n".join(bad[:20])
