@@ -261,6 +261,9 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
     cnt[qb] = ok ? visible_keys(qf + m * P) : 0;
   }
 
+  // keys every row of the wave sees: sub-tiles below this need no mask (rows past the end of the sequence count as rows
+  // that see nothing, so a wave that holds some masks everywhere)
+  const int cnt_wave = __builtin_amdgcn_readfirstlane(m_w0 + 31 < q_len ? visible_keys(qf + m_w0 * P) : 0);
   int koff0 = qc * 256 + ((g ^ swz_k(qc)) << 4);
   int voff0;
   {
@@ -410,7 +413,13 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
   // written by vector moves the compiler cannot order against them)
   u32x4 ones = u32x4{0x3C003C00u, 0x3C003C00u, 0x3C003C00u, 0x3C003C00u};
   asm volatile("" : "+v"(ones));
-  const float scale = p.scale_log2, inv_scale = 1.f / p.scale_log2;
+  const float scale = p.scale_log2;
+  // (wave-uniform: kept in a scalar register, the vector registers are all taken)
+  float inv_scale;
+  {
+    const float inv = 1.f / p.scale_log2;
+    asm volatile("v_readfirstlane_b32 %0, %1" : "=s"(inv_scale) : "v"(inv));
+  }
   auto fphase_mfma = [&](auto par_tag, auto r_tag, auto lsum_tag) __attribute__((always_inline)) {
     constexpr int PAR = decltype(par_tag)::value;  // sub-tile i = 2it + PAR (SPLIT: the parity is in the address registers)
     constexpr int R = decltype(r_tag)::value;
@@ -462,8 +471,11 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
 #pragma unroll
     for (int qb = 0; qb < 2; qb++) {
       nm[qb] = neg_m[qb];
-      if (MASKED) {
-        nm[qb] = neg_m[qb] == INFINITY ? 0.f : neg_m[qb];
+      if (MASKED) nm[qb] = neg_m[qb] == INFINITY ? 0.f : neg_m[qb];
+    }
+    if (MASKED && (i + 1) * SUB > cnt_wave) {  // (wave-uniform: the wave's first row sees the fewest keys)
+#pragma unroll
+      for (int qb = 0; qb < 2; qb++) {
         const int rel = cnt[qb] - i * SUB - 4 * g;  // keys from the lane's first one of key block 0 to the row's limit
 #pragma unroll
         for (int kb = 0; kb < 2; kb++)
@@ -471,10 +483,12 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
           for (int r = 0; r < 4; r++) s[kb][qb][r] = (16 * kb + r < rel) ? s[kb][qb][r] : -INFINITY;
       }
     }
+    if (MASKED) {
 #pragma unroll
-    for (int qb = 0; qb < 2; qb++) {
-      ma[qb] = fmaxf(fmaxf(s[0][qb][0], s[0][qb][1]), s[0][qb][2]);
-      mb[qb] = fmaxf(fmaxf(s[0][qb][3], s[1][qb][0]), s[1][qb][1]);
+      for (int qb = 0; qb < 2; qb++) {
+        ma[qb] = fmaxf(fmaxf(s[0][qb][0], s[0][qb][1]), s[0][qb][2]);
+        mb[qb] = fmaxf(fmaxf(s[0][qb][3], s[1][qb][0]), s[1][qb][1]);
+      }
     }
 #pragma unroll
     for (int qb = 0; qb < 2; qb++)
@@ -483,15 +497,19 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
 #pragma unroll
         for (int r = 0; r < 4; r++) t[qb][4 * kb + r] = __builtin_fmaf(s[kb][qb][r], scale, nm[qb]);
     __builtin_amdgcn_sched_barrier(0);
+    if (MASKED) {
 #pragma unroll
-    for (int qb = 0; qb < 2; qb++) ma[qb] = fmaxf(fmaxf(ma[qb], s[1][qb][2]), s[1][qb][3]);
+      for (int qb = 0; qb < 2; qb++) ma[qb] = fmaxf(fmaxf(ma[qb], s[1][qb][2]), s[1][qb][3]);
+    }
 #pragma unroll
     for (int qb = 0; qb < 2; qb++)
 #pragma unroll
       for (int e = 0; e < 8; e++) t[qb][e] = __builtin_amdgcn_exp2f(t[qb][e]);
     __builtin_amdgcn_sched_barrier(0);
+    if (MASKED) {
 #pragma unroll
-    for (int qb = 0; qb < 2; qb++) mx[qb] = fmaxf(ma[qb], mb[qb]);
+      for (int qb = 0; qb < 2; qb++) mx[qb] = fmaxf(ma[qb], mb[qb]);
+    }
     if (MASKED) {
 #pragma unroll
       for (int qb = 0; qb < 2; qb++)
@@ -507,10 +525,26 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
     constexpr bool MASKED = decltype(masked_tag)::value;
     float mx[2], ps[2];
     compute_p(masked_tag, i, mx, ps);
-    if (__builtin_amdgcn_ballot_w64((mx[0] > thr_raw[0]) | (mx[1] > thr_raw[1])) != 0) {
+    bool over;
+    if (MASKED) {
+      over = (mx[0] > thr_raw[0]) | (mx[1] > thr_raw[1]);
+    } else {
+      // Every key counts here, so no maxima are needed to tell whether the running ones still hold: some P is 2 or more
+      // (also infinite, as for the first keys a row sees, when m is still -inf) exactly if bit 14 of one of the packed
+      // fp16 values, the top bit of its exponent, is set.  Six instructions instead of the eleven of the maxima.
+      const uint32_t any = (pk[0][0] | pk[0][1] | pk[0][2]) | (pk[0][3] | pk[1][0] | pk[1][1]) | (pk[1][2] | pk[1][3]);
+      over = (any & 0x40004000u) != 0;
+    }
+    if (__builtin_amdgcn_ballot_w64(over) != 0) {
       // rare: some score is above the lazy threshold (always so for the first key a row sees); raise the running maxima
       // and redo the sub-tile (the accumulators' last MFMAs were issued before this phase's barrier and the whole of
       // compute_p lies between them and these multiplies)
+      if (!MASKED) {
+#pragma unroll
+        for (int qb = 0; qb < 2; qb++)
+          mx[qb] = fmaxf(fmaxf(fmaxf(s[0][qb][0], s[0][qb][1]), fmaxf(s[0][qb][2], s[0][qb][3])),
+                         fmaxf(fmaxf(s[1][qb][0], s[1][qb][1]), fmaxf(s[1][qb][2], s[1][qb][3])));
+      }
 #pragma unroll
       for (int qb = 0; qb < 2; qb++) {
         const float m_new = fminf(neg_m[qb], -column_max(mx[qb]) * scale);  // -max(m, mx*scale)
@@ -548,8 +582,15 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
   auto request_tiles = [&](auto r_tag, auto masked_tag, int it) __attribute__((always_inline)) {
     constexpr int R = decltype(r_tag)::value;
     if constexpr (decltype(masked_tag)::value) {
-      load_k_clamped(std::integral_constant<int, (R + KA) & 3>{}, it + KA);
-      if constexpr (DV) load_v_clamped(std::integral_constant<int, (R + VA) & 3>{}, it + VA);
+      // (tiles that lie inside the chunk take the cheaper loads here too; the running pointers advance either way)
+      if (it + KA < kv_len / BN) {
+        load_tiles_fast(r_tag);
+      } else {
+        load_k_clamped(std::integral_constant<int, (R + KA) & 3>{}, it + KA);
+        if constexpr (DV) load_v_clamped(std::integral_constant<int, (R + VA) & 3>{}, it + VA);
+        kt_run += (int64_t)BN * k_row_bytes;
+        if (DV) vt_run += (int64_t)BN * v_row_bytes;
+      }
     } else {
       load_tiles_fast(r_tag);
     }
