@@ -3,6 +3,8 @@ loongserve/models/llama/triton_kernel/longserve_flash_decoding_stage1.py:78,
 longserve_flash_decoding_stage2.py:53 and longserve_flash_decoding.py:3."""
 from __future__ import annotations
 
+import functools
+
 import torch
 
 from . import longserve_cuda_kernels
@@ -54,6 +56,7 @@ FUSED_LONG_SPLIT_TOKENS = 4096
 FUSED_LONG_MIN_BLOCKS = 64
 
 
+@functools.lru_cache(maxsize=4096)
 def _fused_block_seq(block_seq: int, batch_size: int, max_len_in_batch: int, num_kv_heads: int) -> int:
     bs = int(block_seq)
     task_groups = (int(num_kv_heads) + 3) // 4

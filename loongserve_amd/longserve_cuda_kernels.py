@@ -124,14 +124,34 @@ def flash_decoding_stage2(o, out_logexpsum, b_seqlen, mid_o, mid_o_logexpsum, bl
     _lib.check(_lib.load().lsattn_decode_stage2(C.byref(a), _stream()), "lsattn_decode_stage2")
 
 
-@torch.inference_mode()
+# Argument blocks of the fused call, by the full metadata of its tensors.  A decode step of a serving loop calls with the
+# same buffers every time (the request table, the length vector and the KV pool are updated in place), and the checks and
+# the filling of the two blocks then cost more host time than a small batch's kernels run: a call whose tensors all have
+# the address, shape, strides and dtype of an earlier, validated call reuses that call's blocks.
+_FUSED_CACHE: dict = {}
+_FUSED_CACHE_MAX = 64
+
+
+def _meta(t):
+    return (t.data_ptr(), t.shape, t.stride(), t.dtype)
+
+
 def flash_decoding(mid_o, mid_o_logexpsum, q, k, v, req_to_tokens, b_req_idx, b_seqlen, max_len_in_batch: int,
                    o, out_logexpsum, block_seq: int) -> None:
     """Stage 1 and stage 2 with the same block size from one library call (what FDPY:12-27 does with two): the checks of
     both, one argument pass, the two launches back to back."""
-    a1 = _stage1_args(mid_o, mid_o_logexpsum, q, k, v, req_to_tokens, b_req_idx, b_seqlen, max_len_in_batch, block_seq)
-    a2 = _stage2_args(o, out_logexpsum, b_seqlen, mid_o, mid_o_logexpsum, block_seq)
-    _lib.check(_lib.load().lsattn_decode_attention(C.byref(a1), C.byref(a2), _stream()), "lsattn_decode_attention")
+    key = (_meta(mid_o), _meta(mid_o_logexpsum), _meta(q), _meta(k), _meta(v), _meta(req_to_tokens), _meta(b_req_idx),
+           _meta(b_seqlen), _meta(o), _meta(out_logexpsum), max_len_in_batch, block_seq, q.device.index)
+    blocks = _FUSED_CACHE.get(key)
+    if blocks is None:
+        a1 = _stage1_args(mid_o, mid_o_logexpsum, q, k, v, req_to_tokens, b_req_idx, b_seqlen, max_len_in_batch, block_seq)
+        a2 = _stage2_args(o, out_logexpsum, b_seqlen, mid_o, mid_o_logexpsum, block_seq)
+        if len(_FUSED_CACHE) >= _FUSED_CACHE_MAX:
+            _FUSED_CACHE.clear()
+        blocks = _FUSED_CACHE[key] = (a1, a2, C.byref(a1), C.byref(a2), _lib.load().lsattn_decode_attention)
+    rc = blocks[4](blocks[2], blocks[3], _stream())
+    if rc:
+        _lib.check(rc, "lsattn_decode_attention")
 
 
 @torch.inference_mode()
