@@ -378,6 +378,29 @@ class VarlenPrefill:
         lsa.destindex_copy_and_register_kv(len(self.lens), self.len, self.zero, self.len, self.len_sum, self.kv, self.start, self.zero,
                                            self.mem_index, self.pool, self.req_to_token, self.b_req, 0, self.max_len, True)
 
+    def write_back_setup(self):
+        """The write-back of the step's tokens (rotary of q and k, K/V rows to their pool slots, registration) runs in
+        fp16, as the reference's rotary kernel does: the same buffers are read as fp16 bit patterns (timing only, the
+        rotation overwrites q and k)."""
+        self.q16, self.kv16, self.pool16 = self.q.view(torch.float16), self.kv.view(torch.float16), self.pool.view(torch.float16)
+        self.cos = _randn_half((self.T, self.D // 2), 5101, torch.float16)
+        self.sin = _randn_half((self.T, self.D // 2), 5102, torch.float16)
+        # bytes the fused launch has to move: q read + written, K/V rows read, K written back in place, pool rows written,
+        # cos/sin read, slot numbers read, table written
+        self.write_back_bytes = self.T * (2 * self.Hq * self.D * 2 + 2 * self.Hkv * self.D * 2 + self.Hkv * self.D * 2
+                                          + 2 * self.Hkv * self.D * 2 + 2 * (self.D // 2) * 2 + 8)
+
+    def write_back_separate(self):
+        import loongserve_amd as lsa
+        lsa.longserve_cuda_kernels.rotary_emb(self.q16, self.kv16[:, :self.Hkv], self.cos, self.sin)
+        lsa.kv_scatter(self.kv16, self.mem_index, self.pool16)
+        lsa.init_req_to_token_indexes(self.req_to_token, self.b_req, self.len, self.mem_index, self.start, self.max_len)
+
+    def write_back_fused(self):
+        import loongserve_amd as lsa
+        lsa.rotary_emb_write_kv(self.q16, self.kv16, self.cos, self.sin, self.mem_index, self.pool16, self.req_to_token, self.b_req,
+                                self.len, self.start, self.max_len)
+
     def step(self):
         self.attention()
         self.persist()
@@ -434,6 +457,9 @@ def workloads(steps):
     sk = _stats(_time_events(v.attention_kernel_only, 3, 0))
     sp = _stats(_time_events(v.persist, 5, 1))
     sm = _stats(_time_events(v.migrate, 5, 1))
+    v.write_back_setup()
+    wsep = _stats(_time_events(v.write_back_separate, 5, 1))
+    wfus = _stats(_time_events(v.write_back_fused, 5, 1))
     whole_ms = sa["median_ms"] + sp["median_ms"]
     out["config5"] = {
         "workload": "config 5: 24 packed sequences, lengths log-uniform in [1024, 200000], %d tokens, GQA 32/8, head_dim 128, bf16, "
@@ -445,6 +471,13 @@ def workloads(steps):
         "kv_write": {"what": "lsattn_kv_scatter + lsattn_register_tokens: every K/V row (4096 B) read and written once",
                      "ms": sp["median_ms"], "gbs": v.scatter_bytes / (sp["median_ms"] * 1e-3) / 1e9,
                      "pct_of_hbm_peak": 100 * v.scatter_bytes / (sp["median_ms"] * 1e-3) / 1e9 / PEAK_HBM_GBS},
+        "write_back_with_rotary": {
+            "what": "rotary embedding of q and k + K/V rows to their pool slots + registration, on the same buffers read as fp16 "
+                    "(the reference's rotary kernel is fp16 only): the four launches the layer makes (rotary of q, rotary of k, "
+                    "scatter, registration) against the one launch of lsattn_rotary_kv_write; GB/s on the bytes the fused launch moves",
+            "separate_ms": wsep["median_ms"], "fused_ms": wfus["median_ms"], "bytes": v.write_back_bytes,
+            "separate_gbs": v.write_back_bytes / (wsep["median_ms"] * 1e-3) / 1e9, "fused_gbs": v.write_back_bytes / (wfus["median_ms"] * 1e-3) / 1e9,
+            "fused_pct_of_hbm_peak": 100 * v.write_back_bytes / (wfus["median_ms"] * 1e-3) / 1e9 / PEAK_HBM_GBS},
         "migration_copy_register": {"what": "the same rows through lsattn_kv_copy_register (copy + registration in one launch)",
                                     "ms": sm["median_ms"], "gbs": v.scatter_bytes / (sm["median_ms"] * 1e-3) / 1e9},
         "roofline": _roof("prefill_kernel<BF16,1,true,false>", "mfma", v.flops / (sk["median_ms"] * 1e-3) / 1e12, sk["median_ms"], "config5",

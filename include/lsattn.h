@@ -349,6 +349,46 @@ int lsattn_rotary_emb(void* x, const void* cos, const void* sin, int64_t x_strid
                       int64_t num_tokens, int64_t num_heads, int64_t head_dim, void* stream);
 
 /*
+ * The write-back of a step's new tokens in one launch instead of the reference's three passes over K and V:
+ *   rotary embedding of q and of the K heads of kv, in place, as lsattn_rotary_emb
+ *     (longserve_cuda_kernels.rotary_emb, called longserve_transformer_layer_infer.py:88-93);
+ *   pool[dest_index[t]] = the token's row of kv after the rotation, K heads then V heads, bit-exact
+ *     (destindex_copy_kv, longserve_transformer_layer_infer.py:377; skipped when pool is NULL);
+ *   register_mode 1: req_to_tokens[b_req_idx[b], 0:b_seq_len[b]] = dest_index[b_start_loc[b] : +b_seq_len[b]]
+ *     (init_req_to_token_indexes, loongserve/common/infer_utils.py:1-13);
+ *   register_mode 2: req_to_tokens[b_req_idx[i], b_seq_len[i] - 1] = dest_index[i], one new token per request
+ *     (copy_kv_index_to_req, longserve_model.py:491); register_mode 0: the table is left alone.
+ * q [T, Hq, D] and kv [T, 2*Hkv, D] are fp16 with the last dimension contiguous (strides in elements, multiples of 8),
+ * cos / sin [T, D/2] contiguous, a pool slot holds 2*Hkv*D contiguous elements, pool_slot_stride elements apart.
+ * head_dim % 16 == 0.  kv stays valid for the attention step that follows (K rotated in place).
+ */
+typedef struct lsattn_rotary_kv_write_args {
+  void* q;
+  int64_t q_stride_t, q_stride_h;
+  int64_t num_q_heads;
+  void* kv;
+  int64_t kv_stride_t, kv_stride_h;
+  int64_t num_kv_heads;
+  const void* cos;
+  const void* sin;
+  int64_t num_tokens;
+  int64_t head_dim;
+  void* pool;                   /* [slots, 2*Hkv*D] or NULL */
+  int64_t pool_slot_stride;
+  const int32_t* dest_index;    /* [num_tokens] */
+  int32_t* req_to_tokens;       /* [max_req, max_seq_len] */
+  int64_t max_seq_len;
+  const int32_t* b_req_idx;     /* [batch] */
+  const int32_t* b_start_loc;   /* [batch], register_mode 1 */
+  const int32_t* b_seq_len;     /* [batch] */
+  int64_t batch;
+  int64_t max_len_in_batch;     /* register_mode 1: upper bound of b_seq_len[] (sizes the launch) */
+  int32_t register_mode;
+  int32_t reserved;
+} lsattn_rotary_kv_write_args;
+int lsattn_rotary_kv_write(const lsattn_rotary_kv_write_args* a, void* stream);
+
+/*
  * Slot allocator of the KV pool.  mem_state is int32 [pool_size] on the device (16-byte aligned), 0 = free slot,
  * otherwise the slot's reference count.  The searches need a device workspace of
  * lsattn_pool_search_workspace_bytes(pool_size) bytes (16-byte aligned); nothing is allocated or kept by the library

@@ -24,12 +24,12 @@ from .decoding import (longserve_flash_decode_stage1, longserve_flash_decode_sta
 from .ops import (context_attention_fwd, copy_kv_index_to_req, decoding_stage_migration_receiver_kernel,  # noqa: E402
                   decoding_stage_migration_sender_kernel, destindex_copy_and_register_kv, destindex_copy_kv,
                   init_req_to_token_indexes, kv_scatter, lse_merge, pre_copy_and_register_kv, prefill_attention_step,
-                  rmsnorm_forward, rotary_emb_fwd, silu_and_mul_fwd)
+                  rmsnorm_forward, rotary_emb_fwd, rotary_emb_write_kv, silu_and_mul_fwd)
 
 __all__ = [
     "context_attention_fwd", "prefill_attention_step", "lse_merge", "kv_scatter", "init_req_to_token_indexes",
     "pre_copy_and_register_kv", "destindex_copy_and_register_kv", "destindex_copy_kv", "copy_kv_index_to_req",
-    "rmsnorm_forward", "rotary_emb_fwd", "silu_and_mul_fwd",
+    "rmsnorm_forward", "rotary_emb_fwd", "rotary_emb_write_kv", "silu_and_mul_fwd",
     "decoding_stage_migration_sender_kernel", "decoding_stage_migration_receiver_kernel",
     "longserve_flash_decode_stage1", "longserve_flash_decode_stage2",
     "longserve_token_decode_attention_flash_decoding", "longserve_cuda_kernels",

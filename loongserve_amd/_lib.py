@@ -84,6 +84,15 @@ class DecodeMigrationArgs(C.Structure):  # mirrors lsattn_decode_migration_args
                 ("num_tokens_cumsum", C.c_void_p), ("b_seq_len", C.c_void_p), ("batch", C.c_int64), ("max_num_tokens", C.c_int64)]
 
 
+class RotaryKvWriteArgs(C.Structure):  # mirrors lsattn_rotary_kv_write_args
+    _fields_ = [("q", _vp), ("q_stride_t", _i64), ("q_stride_h", _i64), ("num_q_heads", _i64),
+                ("kv", _vp), ("kv_stride_t", _i64), ("kv_stride_h", _i64), ("num_kv_heads", _i64),
+                ("cos", _vp), ("sin", _vp), ("num_tokens", _i64), ("head_dim", _i64),
+                ("pool", _vp), ("pool_slot_stride", _i64), ("dest_index", _vp),
+                ("req_to_tokens", _vp), ("max_seq_len", _i64), ("b_req_idx", _vp), ("b_start_loc", _vp), ("b_seq_len", _vp),
+                ("batch", _i64), ("max_len_in_batch", _i64), ("register_mode", _i32), ("reserved", _i32)]
+
+
 EXPORTS = {
     "lsattn_prefill_step": (C.c_int, [C.POINTER(PrefillArgs), _vp]),
     "lsattn_prefill_step_merge": (C.c_int, [C.POINTER(PrefillArgs), _vp]),
@@ -102,6 +111,7 @@ EXPORTS = {
     "lsattn_decode_migration_recv": (C.c_int, [C.POINTER(DecodeMigrationArgs), _vp]),
     "lsattn_rms_norm": (C.c_int, [_vp, _vp, _vp, _i64, _i64, C.c_float, _vp]),
     "lsattn_silu_and_mul_inplace": (C.c_int, [_vp, _i64, _i64, _vp]),
+    "lsattn_rotary_kv_write": (C.c_int, [C.POINTER(RotaryKvWriteArgs), _vp]),
     "lsattn_rotary_emb": (C.c_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp]),
     "lsattn_pool_search_workspace_bytes": (C.c_size_t, [_i64]),
     "lsattn_pool_alloc": (C.c_int, [_vp, _i64, _i64, _vp, _vp, C.c_size_t, _vp]),

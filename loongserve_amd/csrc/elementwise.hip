@@ -133,6 +133,91 @@ __global__ __launch_bounds__(256) void rotary_emb_kernel(uint16_t* __restrict__ 
 }
 
 // ---------------------------------------------------------------------------------------------------
+// The write-back of a step's new tokens in one launch: rotary embedding of q and of the K heads in place (the arithmetic
+// of rotary_emb_kernel), every token's rotated K heads and its V heads copied to the token's slot of the KV pool, and the
+// slots entered in the request table.  A unit is 32 bytes of one (token, head): the two 16-byte halves a rotary lane
+// owns, or two consecutive 16-byte pieces of a V head.  Blocks past the data units do the registration, one table entry
+// per lane.
+// ---------------------------------------------------------------------------------------------------
+struct RotaryWriteParams {
+  uint16_t* q;
+  int64_t q_st, q_sh, hq;
+  uint16_t* kv;
+  int64_t kv_st, kv_sh, hkv;
+  const uint16_t* cos_t;
+  const uint16_t* sin_t;
+  int64_t num_tokens, head_dim;
+  uint16_t* pool;
+  int64_t pool_stride;  // elements per slot
+  const int32_t* dest;
+  int32_t* req_to_tokens;
+  int64_t max_seq_len;
+  const int32_t* b_req_idx;
+  const int32_t* b_start_loc;
+  const int32_t* b_seq_len;
+  int64_t batch, data_blocks, reg_blocks_per_req;
+  int32_t reg_mode;  // 0 none, 1 every token of every request (prefill), 2 the last token of every request (decode)
+};
+
+__global__ __launch_bounds__(256) void rotary_kv_write_kernel(RotaryWriteParams p) {
+  if ((int64_t)blockIdx.x >= p.data_blocks) {
+    const int64_t rb = (int64_t)blockIdx.x - p.data_blocks;
+    if (p.reg_mode == 1) {
+      const int64_t b = rb / p.reg_blocks_per_req;
+      const int64_t j = (rb % p.reg_blocks_per_req) * 256 + threadIdx.x;
+      if (j >= p.b_seq_len[b] || j >= p.max_seq_len) return;
+      p.req_to_tokens[(int64_t)p.b_req_idx[b] * p.max_seq_len + j] = p.dest[(int64_t)p.b_start_loc[b] + j];
+    } else {
+      const int64_t i = rb * 256 + threadIdx.x;
+      if (i >= p.batch) return;
+      const int64_t pos = (int64_t)p.b_seq_len[i] - 1;
+      if (pos < 0 || pos >= p.max_seq_len) return;
+      p.req_to_tokens[(int64_t)p.b_req_idx[i] * p.max_seq_len + pos] = p.dest[i];
+    }
+    return;
+  }
+  const int64_t pieces = p.head_dim / 16;  // units per head
+  const int64_t heads = p.hq + 2 * p.hkv;
+  const int64_t gid = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (gid >= p.num_tokens * heads * pieces) return;
+  const int64_t c = gid % pieces;
+  const int64_t h = (gid / pieces) % heads;
+  const int64_t t = gid / (pieces * heads);
+  if (h >= p.hq + p.hkv) {
+    // V head: 32 bytes to the pool
+    if (!p.pool) return;
+    const int64_t hv = h - p.hq;  // head index inside the token's K/V row
+    const f16x8* src = (const f16x8*)(p.kv + t * p.kv_st + hv * p.kv_sh) + 2 * c;
+    f16x8* dst = (f16x8*)(p.pool + (int64_t)p.dest[t] * p.pool_stride + hv * p.head_dim) + 2 * c;
+    const f16x8 a = src[0], b = src[1];
+    dst[0] = a;
+    dst[1] = b;
+    return;
+  }
+  const bool is_k = h >= p.hq;
+  uint16_t* base = is_k ? p.kv + t * p.kv_st + (h - p.hq) * p.kv_sh : p.q + t * p.q_st + h * p.q_sh;
+  f16x8* p1 = (f16x8*)base + c;
+  f16x8* p2 = (f16x8*)(base + p.head_dim / 2) + c;
+  const f16x8 x1 = *p1, x2 = *p2;
+  const f16x8 co = *((const f16x8*)(p.cos_t + t * (p.head_dim / 2)) + c);
+  const f16x8 si = *((const f16x8*)(p.sin_t + t * (p.head_dim / 2)) + c);
+  const f16x8 t1 = x2 * si, t2 = x2 * co;  // rounded to half (this file is compiled without contraction)
+  f16x8 n1, n2;
+#pragma unroll
+  for (int e = 0; e < 8; e++) {
+    n1[e] = __builtin_fmaf16(x1[e], co[e], -t1[e]);
+    n2[e] = __builtin_fmaf16(x1[e], si[e], t2[e]);
+  }
+  *p1 = n1;
+  *p2 = n2;
+  if (is_k && p.pool) {
+    uint16_t* prow = p.pool + (int64_t)p.dest[t] * p.pool_stride + (h - p.hq) * p.head_dim;
+    *((f16x8*)prow + c) = n1;
+    *((f16x8*)(prow + p.head_dim / 2) + c) = n2;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------
 // bf16 -> fp16 row copy, rounded toward zero (exact inside fp16's normal range, +-65504 beyond it): prepares a bf16 V
 // for the prefill kernel, whose P V product runs in fp16.  One 16-byte piece per lane.
 // ---------------------------------------------------------------------------------------------------
@@ -204,5 +289,59 @@ extern "C" int lsattn_rotary_emb(void* x, const void* cos, const void* sin, int6
   if (blocks > 0x7fffffff) return LSATTN_ERR_INVALID_ARG;
   hipLaunchKernelGGL(rotary_emb_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (uint16_t*)x,
                      (const uint16_t*)cos, (const uint16_t*)sin, x_stride_t, x_stride_h, num_tokens, num_heads, head_dim);
+  return check_launch();
+}
+
+extern "C" int lsattn_rotary_kv_write(const lsattn_rotary_kv_write_args* a, void* stream) {
+  if (!a || !a->q || !a->kv || !a->cos || !a->sin || a->num_tokens < 0 || a->num_q_heads <= 0 || a->num_kv_heads <= 0 ||
+      a->head_dim <= 0 || a->batch < 0)
+    return LSATTN_ERR_INVALID_ARG;
+  if (a->head_dim % 16 || a->q_stride_t % 8 || a->q_stride_h % 8 || a->kv_stride_t % 8 || a->kv_stride_h % 8 ||
+      (((uintptr_t)a->q | (uintptr_t)a->kv | (uintptr_t)a->cos | (uintptr_t)a->sin | (uintptr_t)a->pool) & 15))
+    return LSATTN_ERR_INVALID_ARG;
+  if (a->pool && (!a->dest_index || a->pool_slot_stride % 8 || a->pool_slot_stride < 2 * a->num_kv_heads * a->head_dim))
+    return LSATTN_ERR_INVALID_ARG;
+  if (a->register_mode < 0 || a->register_mode > 2) return LSATTN_ERR_INVALID_ARG;
+  if (a->register_mode != 0 &&
+      (!a->req_to_tokens || !a->dest_index || !a->b_req_idx || !a->b_seq_len || a->max_seq_len <= 0 ||
+       (a->register_mode == 1 && (!a->b_start_loc || a->max_len_in_batch < 0 || a->max_len_in_batch > a->max_seq_len))))
+    return LSATTN_ERR_INVALID_ARG;
+  RotaryWriteParams p;
+  p.q = (uint16_t*)a->q;
+  p.q_st = a->q_stride_t;
+  p.q_sh = a->q_stride_h;
+  p.hq = a->num_q_heads;
+  p.kv = (uint16_t*)a->kv;
+  p.kv_st = a->kv_stride_t;
+  p.kv_sh = a->kv_stride_h;
+  p.hkv = a->num_kv_heads;
+  p.cos_t = (const uint16_t*)a->cos;
+  p.sin_t = (const uint16_t*)a->sin;
+  p.num_tokens = a->num_tokens;
+  p.head_dim = a->head_dim;
+  p.pool = (uint16_t*)a->pool;
+  p.pool_stride = a->pool_slot_stride;
+  p.dest = a->dest_index;
+  p.req_to_tokens = a->req_to_tokens;
+  p.max_seq_len = a->max_seq_len;
+  p.b_req_idx = a->b_req_idx;
+  p.b_start_loc = a->b_start_loc;
+  p.b_seq_len = a->b_seq_len;
+  p.batch = a->batch;
+  p.reg_mode = a->register_mode;
+  const int64_t units = a->num_tokens * (a->num_q_heads + 2 * a->num_kv_heads) * (a->head_dim / 16);
+  p.data_blocks = (units + 255) / 256;
+  p.reg_blocks_per_req = 0;
+  int64_t reg_blocks = 0;
+  if (a->register_mode == 1) {
+    p.reg_blocks_per_req = (a->max_len_in_batch + 255) / 256;
+    reg_blocks = p.reg_blocks_per_req * a->batch;
+  } else if (a->register_mode == 2) {
+    reg_blocks = (a->batch + 255) / 256;
+  }
+  const int64_t blocks = p.data_blocks + reg_blocks;
+  if (blocks == 0) return LSATTN_OK;
+  if (blocks > 0x7fffffff) return LSATTN_ERR_INVALID_ARG;
+  hipLaunchKernelGGL(rotary_kv_write_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, p);
   return check_launch();
 }

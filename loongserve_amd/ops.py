@@ -319,6 +319,72 @@ def destindex_copy_kv(K: torch.Tensor, DestLoc: torch.Tensor, Out: torch.Tensor)
 
 
 @torch.inference_mode()
+def rotary_emb_write_kv(q: torch.Tensor, cache_kv: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor,
+                        mem_index: Optional[torch.Tensor] = None, pool: Optional[torch.Tensor] = None,
+                        req_to_token_indexs: Optional[torch.Tensor] = None, b_req_idx: Optional[torch.Tensor] = None,
+                        b_seq_len: Optional[torch.Tensor] = None, b_start_loc: Optional[torch.Tensor] = None,
+                        max_len_in_batch: Optional[int] = None, decode: bool = False) -> None:
+    """A step's write-back of its new tokens in one launch (lsattn_rotary_kv_write) instead of the three operators the
+    layer calls one after the other:
+      longserve_cuda_kernels.rotary_emb(q, cache_kv[:, :Hkv], cos, sin)           (..._layer_infer.py:88-93), in place;
+      destindex_copy_kv(cache_kv, mem_index, pool)                                (..._layer_infer.py:377), if pool is given;
+      init_req_to_token_indexes(req_to_token_indexs, b_req_idx, b_seq_len, mem_index)  (prefill, decode=False) or
+      copy_kv_index_to_req(req_to_token_indexs, b_req_idx, b_seq_len, mem_index)       (decode=True), if the table is given.
+    q [T, Hq, D], cache_kv [T, 2*Hkv, D] (K heads then V heads), float16; the results are those of the separate
+    operators bit for bit."""
+    for t, n in ((q, "q"), (cache_kv, "cache_kv")):
+        _dev(t, n)
+        if t.dim() != 3 or t.dtype != torch.float16 or t.stride(2) != 1:
+            raise ValueError("%s must be a 3-d float16 tensor with a contiguous last dimension" % n)
+    T, Hq, D = q.shape
+    if cache_kv.shape[0] != T or cache_kv.shape[2] != D or cache_kv.shape[1] % 2:
+        raise ValueError("cache_kv must be [tokens, 2 * kv_heads, head_dim] for q's tokens and head_dim")
+    for t, n in ((cos, "cos"), (sin, "sin")):
+        _dev(t, n)
+        if t.dtype != torch.float16 or tuple(t.shape) != (T, D // 2) or not t.is_contiguous():
+            raise ValueError("%s must be a contiguous float16 [tokens, head_dim / 2] tensor" % n)
+    a = _lib.RotaryKvWriteArgs()
+    a.q, a.q_stride_t, a.q_stride_h, a.num_q_heads = q.data_ptr(), q.stride(0), q.stride(1), Hq
+    a.kv, a.kv_stride_t, a.kv_stride_h, a.num_kv_heads = cache_kv.data_ptr(), cache_kv.stride(0), cache_kv.stride(1), cache_kv.shape[1] // 2
+    a.cos, a.sin, a.num_tokens, a.head_dim = cos.data_ptr(), sin.data_ptr(), T, D
+    keep = []
+    if mem_index is not None:
+        mem_index = _slots(mem_index, "mem_index")
+        keep.append(mem_index)
+        a.dest_index = mem_index.data_ptr()
+    if pool is not None:
+        _dev(pool, "pool")
+        if mem_index is None or mem_index.shape[0] != T:
+            raise ValueError("mem_index must name one slot per token")
+        if pool.dtype != torch.float16 or pool.shape[1:] != cache_kv.shape[1:] or (pool.shape[0] and not pool[0].is_contiguous()):
+            raise ValueError("pool must be float16 [slots, 2 * kv_heads, head_dim] with contiguous slots")
+        a.pool, a.pool_slot_stride = pool.data_ptr(), pool.stride(0)
+    if req_to_token_indexs is not None:
+        _dev(req_to_token_indexs, "req_to_token_indexs")
+        if req_to_token_indexs.dtype != torch.int32 or req_to_token_indexs.dim() != 2 or not req_to_token_indexs.is_contiguous():
+            raise ValueError("req_to_token_indexs must be a contiguous [max_req, max_seq] int32 tensor")
+        if mem_index is None or b_req_idx is None or b_seq_len is None:
+            raise ValueError("registration needs mem_index, b_req_idx and b_seq_len")
+        B = b_req_idx.shape[0]
+        _i32vec(b_req_idx, "b_req_idx", B); _i32vec(b_seq_len, "b_seq_len", B)
+        a.req_to_tokens, a.max_seq_len = req_to_token_indexs.data_ptr(), req_to_token_indexs.shape[1]
+        a.b_req_idx, a.b_seq_len, a.batch = b_req_idx.data_ptr(), b_seq_len.data_ptr(), B
+        if decode:
+            if mem_index.shape[0] != B:
+                raise ValueError("decode registration: one slot per request")
+            a.register_mode = 2
+        else:
+            if b_start_loc is None:
+                b_start_loc = (torch.cumsum(b_seq_len, 0, dtype=torch.int32) - b_seq_len).to(torch.int32)
+            if max_len_in_batch is None:
+                max_len_in_batch = int(b_seq_len.max().item()) if B else 0
+            _i32vec(b_start_loc, "b_start_loc", B)
+            keep.append(b_start_loc)
+            a.b_start_loc, a.max_len_in_batch, a.register_mode = b_start_loc.data_ptr(), int(max_len_in_batch), 1
+    _lib.check(_lib.load().lsattn_rotary_kv_write(C.byref(a), _stream()), "lsattn_rotary_kv_write")
+
+
+@torch.inference_mode()
 def copy_kv_index_to_req(req_to_token_indexs: torch.Tensor, b_req_idx: torch.Tensor, b_seq_len: torch.Tensor,
                          memindex: torch.Tensor) -> None:
     """req_to_token_indexs[b_req_idx[i], b_seq_len[i] - 1] = memindex[i]: registers the slot of each request's new token

@@ -42,6 +42,7 @@ int main(void) {
   printf("%zu %zu %zu %zu %zu\n", sizeof(lsattn_prefill_args), sizeof(lsattn_merge_args),
          sizeof(lsattn_decode_stage1_args), sizeof(lsattn_decode_stage2_args), sizeof(lsattn_kv_copy_register_args));
   printf("%zu %zu\n", sizeof(lsattn_decode_migration_args), offsetof(lsattn_decode_migration_args, b_seq_len));
+  printf("%zu %zu\n", sizeof(lsattn_rotary_kv_write_args), offsetof(lsattn_rotary_kv_write_args, register_mode));
   printf("%zu %zu %zu %zu %zu %zu\n", offsetof(lsattn_prefill_args, sm_scale), offsetof(lsattn_prefill_args, ml_stride_h),
          offsetof(lsattn_decode_stage1_args, req_to_tokens), offsetof(lsattn_decode_stage2_args, block_seq),
          offsetof(lsattn_kv_copy_register_args, req_to_tokens), offsetof(lsattn_kv_copy_register_args, should_register));
@@ -55,7 +56,9 @@ int main(void) {
         out = subprocess.check_output([exe]).decode().split()
     sizes = [int(x) for x in out[:5]]
     mig = [int(x) for x in out[5:7]]
-    offs = [int(x) for x in out[7:]]
+    rot = [int(x) for x in out[7:9]]
+    offs = [int(x) for x in out[9:]]
+    assert rot == [C.sizeof(_lib.RotaryKvWriteArgs), _lib.RotaryKvWriteArgs.register_mode.offset]
     assert mig == [C.sizeof(_lib.DecodeMigrationArgs), _lib.DecodeMigrationArgs.b_seq_len.offset]
     assert sizes == [C.sizeof(_lib.PrefillArgs), C.sizeof(_lib.MergeArgs), C.sizeof(_lib.DecodeStage1Args),
                      C.sizeof(_lib.DecodeStage2Args), C.sizeof(_lib.KvCopyRegisterArgs)]
@@ -75,6 +78,9 @@ def test_validation_rejects_bad_arguments_without_gpu():
     mg = _lib.DecodeMigrationArgs()
     assert lib.lsattn_decode_migration_send(C.byref(mg), None) == -1
     assert lib.lsattn_decode_migration_recv(None, None) == -1
+    rw = _lib.RotaryKvWriteArgs()
+    assert lib.lsattn_rotary_kv_write(C.byref(rw), None) == -1
+    assert lib.lsattn_rotary_kv_write(None, None) == -1
     cr = _lib.KvCopyRegisterArgs()
     assert lib.lsattn_kv_copy_register(C.byref(cr), None) == -1
     assert lib.lsattn_kv_ranges(None, None, None, 1, 0, None, None, None, None) == -1

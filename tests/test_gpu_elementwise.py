@@ -70,6 +70,54 @@ def test_rotary_emb_bit_exact_on_strided_views(lsa, T, Hq, Hkv, D):
     assert np.array_equal(d.cpu().numpy().view(np.int16), want.view(np.int16))   # v heads untouched, q/k bit-exact
 
 
+@pytest.mark.parametrize("decode", [False, True])
+@pytest.mark.parametrize("Hq,Hkv,D", [(32, 8, 128), (4, 4, 64), (6, 1, 32)])
+def test_fused_rotary_kv_write_register_matches_the_separate_operators(lsa, decode, Hq, Hkv, D):
+    """lsattn_rotary_kv_write against the oracles of the three steps it replaces: rotary of q and k (bit-exact), the
+    rotated K rows and the V rows in their pool slots (bit-exact row scatter), and the request table (prefill: every
+    token of every request; decode: the last token of every request)."""
+    from oracle import attn_oracle as orc
+    rng = np.random.default_rng(Hq * 13 + D + decode)
+    lens = [5, 1, 40, 17] if not decode else [9, 300, 1, 64, 2]
+    B = len(lens)
+    T = B if decode else sum(lens)
+    qkv = rng.standard_normal((T, Hq + 2 * Hkv, D)).astype(np.float16)   # q and kv are views of one buffer, as in the model
+    ang = rng.uniform(0, 6.28, (T, D // 2))
+    cos, sin = np.cos(ang).astype(np.float16), np.sin(ang).astype(np.float16)
+    slots = 3 * T + 7
+    g = torch.Generator().manual_seed(5)
+    mem_index = torch.randperm(slots, generator=g)[:T].to(torch.int32)
+    pool0 = torch.from_numpy(rng.standard_normal((slots, 2 * Hkv, D)).astype(np.float16))
+    max_seq = max(lens) + 3
+    table0 = torch.full((B + 2, max_seq), orc.INT32_PAD, dtype=torch.int32)
+    b_req = torch.randperm(B + 2, generator=g)[:B].to(torch.int32)
+    b_len = torch.tensor(lens, dtype=torch.int32)
+    b_start = (torch.cumsum(b_len, 0) - b_len).to(torch.int32)
+    d = torch.from_numpy(qkv).to(DEV)
+    pool, table = pool0.clone().to(DEV), table0.clone().to(DEV)
+    lsa.rotary_emb_write_kv(d[:, :Hq], d[:, Hq:], torch.from_numpy(cos).to(DEV), torch.from_numpy(sin).to(DEV), mem_index.to(DEV), pool,
+                            table, b_req.to(DEV), b_len.to(DEV), None if decode else b_start.to(DEV), None if decode else max(lens),
+                            decode=decode)
+    torch.cuda.synchronize()
+    want = qkv.copy()
+    ew.rotary_emb(want[:, :Hq], cos, sin)
+    ew.rotary_emb(want[:, Hq:Hq + Hkv], cos, sin)
+    assert np.array_equal(d.cpu().numpy().view(np.int16), want.view(np.int16))          # q, k rotated in place, v untouched
+    pool_ref, table_ref = pool0.clone(), table0.clone()
+    orc.kv_scatter(torch.from_numpy(want[:, Hq:].copy()), mem_index, pool_ref)
+    if decode:
+        orc.copy_kv_index_to_req(table_ref, b_req, b_len, mem_index)
+    else:
+        orc.register_tokens(table_ref, b_req, b_start, b_len, mem_index)
+    assert torch.equal(pool.cpu().view(torch.int16), pool_ref.view(torch.int16))         # every slot: written rows and the rest
+    assert torch.equal(table.cpu(), table_ref)
+    # without a pool and without a table it is the rotary step alone
+    d2 = torch.from_numpy(qkv).to(DEV)
+    lsa.rotary_emb_write_kv(d2[:, :Hq], d2[:, Hq:], torch.from_numpy(cos).to(DEV), torch.from_numpy(sin).to(DEV))
+    torch.cuda.synchronize()
+    assert np.array_equal(d2.cpu().numpy().view(np.int16), want.view(np.int16))
+
+
 def test_ffn_block_composition(lsa):
     rng = np.random.default_rng(9)
     T, H, I = 17, 512, 1024
