@@ -211,10 +211,22 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
   const int group = p.hq / p.hkv;
   int j = blockIdx.x >> 3;
   const int xcd = blockIdx.x & 7;
-  const int up = j % p.units_per_slice;
-  j /= p.units_per_slice;
-  const int slot = j % p.kv_slots;
-  const int b = j / p.kv_slots;
+  int up, slot;
+  if (SPLIT) {
+    // Small launches: the heaviest query tiles of all KV heads first, so that a CU that has finished a light tile of the
+    // first round takes a heavy one of the rest and the other way round.
+    slot = j % p.kv_slots;
+    j /= p.kv_slots;
+    up = j % p.units_per_slice;
+    j /= p.units_per_slice;
+  } else {
+    // Large launches: one KV head at a time per XCD, whose K/V then serves all the workgroups the XCD runs.
+    up = j % p.units_per_slice;
+    j /= p.units_per_slice;
+    slot = j % p.kv_slots;
+    j /= p.kv_slots;
+  }
+  const int b = j;
   const int vh = xcd + 8 * slot;  // (KV head, slice) pair: always < hkv * slices
   const int kvh = vh / p.slices;
   const int u = up * p.slices + vh % p.slices;
