@@ -32,11 +32,11 @@ if ROOT not in sys.path:
 # which is regenerated with the kernels (the JSON line says so in "traffic_source").
 TRAFFIC_SOURCE = "profiles/bench_default_hbm_traffic.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this command, scaled by a 1 GiB copy); a constant of bench.py, not measured in this run"
 TRAFFIC_BYTES = {
-    "config2": 1364.3e6,   # per launch, averaged over the four launches of a ring step
-    "config3": 5195.4e6,   # stage 1 of the fused call
-    "config1": None,
-    "config4": None,
-    "config5": None,
+    "config2": 1307.6e6,    # per launch, averaged over the four launches of a ring step (one diagonal + three full)
+    "config3": 5195.2e6,    # stage 1 of the fused call
+    "config1": 108.6e6,
+    "config4": 8596.5e6,    # stage 1 over one instance's 4 x 131072 tokens
+    "config5": 105164e6,    # the attention launch
 }
 PEAK_MFMA_TFLOPS = 2500.0  # dense fp16/bf16 MFMA, MI355X
 PEAK_HBM_GBS = 8000.0
@@ -433,7 +433,7 @@ def workloads(steps):
         "timing": "device time per launch: 20 launches recorded in one HIP graph, replays timed with HIP events (the launch "
                   "is shorter than the host's call overhead); eager_call_ms is one call bracketed by HIP events, host overhead included",
         "eager_call_ms": st["median_ms"],
-        "roofline": _roof("prefill_kernel<F16,0,true,false> (256-row workgroups: 256 of them)", "mfma", fl / (dev_ms * 1e-3) / 1e12, dev_ms, "config1",
+        "roofline": _roof("prefill_kernel<F16,0,true,true> (128-row workgroups: 512 of them)", "mfma", fl / (dev_ms * 1e-3) / 1e12, dev_ms, "config1",
                           algorithmic_tflop_per_launch=fl / 1e12)}
     del q, kv, ob, lb
     # ---- config 4: long-context elastic decode, 4 x 524288, MHA 32, four instances, merge at the master
