@@ -172,3 +172,13 @@ def test_fused_decode_split_rule():
     for bs in (1, 16, 64, 256):
         got = _fused_block_seq(bs, 1 << 14, 1 << 20, 32)
         assert got % bs == 0 and got <= max(FUSED_LONG_SPLIT_TOKENS, bs)
+
+
+def test_extension_module_resolves_by_its_reference_name():
+    """`import longserve_cuda_kernels`, as loongserve/models/llama/triton_kernel/longserve_flash_decoding_stage1.py:4 does."""
+    import importlib
+    m = importlib.import_module("longserve_cuda_kernels")
+    from loongserve_amd import longserve_cuda_kernels as real
+    for name in ("flash_decoding_stage1", "flash_decoding_stage2", "rms_norm", "silu_and_mul_inplace", "rotary_emb", "ffn_block",
+                 "hello_world"):
+        assert getattr(m, name) is getattr(real, name)
