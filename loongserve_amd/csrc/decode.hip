@@ -14,6 +14,7 @@
 //   * a workgroup walks several consecutive blocks, so the launch is sized for the chip
 //     and not for block_seq.
 #include <atomic>
+#include <cstdlib>
 #include <type_traits>
 
 #include "common.hip.h"
@@ -371,6 +372,282 @@ __global__ __launch_bounds__(NW * 64) void decode_stage1_kernel(Stage1Params p) 
 }
 
 // ------------------------------------------------------------------------------------
+// Stage 1 for large GQA groups (five or more query heads per KV head, large launches): both products on the matrix pipe.
+// One wave64 = one KV head, up to 16 query heads of its group (the 16 columns of a 16x16x32 MFMA) and a run of
+// consecutive blocks; the waves of a workgroup are independent (no barrier).  A batch is 32 tokens:
+//   the K and V rows are loaded the way the other stage-1 kernels load them, a whole 256-byte row per 16 lanes (loading the
+//     MFMA operand layout straight from memory, 16 rows x 64 bytes per instruction, ran 20 % slower), double-buffered in
+//     registers so that the rows of batch j + 1 are in flight while batch j is computed;
+//   at compute time the wave turns its rows into operand layout through its own 17.5 KB of LDS (rows padded to 272 and
+//     288 bytes, so that the sixteen rows of a K read and the eight rows of a transposing V read fall into different banks
+//     and every address is one register plus an immediate): K rows are read back as the A operand of S = K Q^T (Q^T, the B operand, stays in registers), V rows are
+//     read back transposed (ds_read_b64_tr_b16) as the A operand of O^T += V^T P^T;
+//   the softmax runs on the accumulators (a lane holds one query head's scores of eight tokens), and P, converted in
+//     place, is the B operand of the second product.  A bfloat16 P would cost about 1e-3 relative error, so bfloat16
+//     inputs multiply V by the high and by the low part of P.
+// All global loads are issued from inline assembly, so that the hand-placed waits leave exactly the next batch's rows
+// outstanding; tests/test_prefill_isa_hazards.py checks that no register of a load in flight is touched before its wait.
+// ------------------------------------------------------------------------------------
+__device__ __forceinline__ float xlane16(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x401F));  // lane ^ 16
+}
+__device__ __forceinline__ float xlane32(float v) {
+  const unsigned u = __builtin_bit_cast(unsigned, v);
+  auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return __builtin_bit_cast(float, (threadIdx.x & 32) ? r[0] : r[1]);
+}
+template <typename T> struct Mfma16;
+template <> struct Mfma16<F16> {
+  static __device__ __forceinline__ f32x4 run(const u32x4& a, const u32x4& b, const f32x4& c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  }
+};
+template <> struct Mfma16<BF16> {
+  static __device__ __forceinline__ f32x4 run(const u32x4& a, const u32x4& b, const f32x4& c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  }
+};
+
+constexpr int kMfmaWaves = 4;        // waves per workgroup (independent)
+constexpr int kMfmaBatch = 32;       // tokens per batch
+constexpr int kMfmaKRow = 272, kMfmaVRow = 288;  // padded row lengths in LDS (bytes)
+constexpr int kMfmaStage = kMfmaBatch * (kMfmaKRow + kMfmaVRow);  // LDS bytes per wave: the K rows and the V rows of one batch
+
+template <typename T>
+__global__ __launch_bounds__(kMfmaWaves * 64, 2) void decode_stage1_mfma_kernel(Stage1Params p) {
+  __shared__ __attribute__((aligned(1024))) char lds[kMfmaWaves * kMfmaStage];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int n = lane & 15, g = lane >> 4;  // query head (column) or 16-byte chunk of a row / token group or row of four
+  const int64_t b = blockIdx.z;
+  const int task = blockIdx.y;
+  const int group = (int)(p.hq / p.hkv);
+  const int sub_groups = (group + 15) / 16;
+  const int kvh = task / sub_groups;
+  const int sg = task % sub_groups;
+  const int qh0 = kvh * group + sg * 16;
+  const int nh = group - sg * 16 < 16 ? group - sg * 16 : 16;
+
+  const int len = p.b_seqlen[b];
+  int64_t nblk = len <= 0 ? 0 : ((int64_t)len + p.block_seq - 1) / p.block_seq;
+  if (nblk > p.grid_blocks) nblk = p.grid_blocks;
+  if (nblk > (p.num_blocks + p.row_mul - 1) / p.row_mul) nblk = (p.num_blocks + p.row_mul - 1) / p.row_mul;
+  int64_t fine_nblk = len <= 0 ? 0 : ((int64_t)len + p.fine_block_seq - 1) / p.fine_block_seq;
+  if (fine_nblk > p.num_blocks) fine_nblk = p.num_blocks;
+  const unsigned n_chunks = gridDim.x * kMfmaWaves;
+  const unsigned chunk = (blockIdx.x * kMfmaWaves + wave + (unsigned)b) % n_chunks;  // (rotated by the request, as above)
+  const int64_t blk_begin = (int64_t)chunk * p.blocks_per_wg;
+  int64_t blk_end = blk_begin + p.blocks_per_wg;
+  if (blk_end > nblk) blk_end = nblk;
+  if (blk_begin >= blk_end) return;
+  const int bs = (int)p.block_seq;                    // a multiple of 32 (checked on the host)
+  const int t_begin = (int)(blk_begin * bs);
+  const int t_end = blk_end * bs > len ? len : (int)(blk_end * bs);
+  const int t_last = t_end - 1;
+  const int n_batches = (t_end - t_begin + kMfmaBatch - 1) / kMfmaBatch;
+
+  const int32_t* table = p.req_to_tokens + (int64_t)p.b_req_idx[b] * p.max_seq_len;
+  const char* kbase = (const char*)p.k + ((int64_t)kvh * p.k_s1) * 2 + n * 16;
+  const char* vbase = (const char*)p.v + ((int64_t)kvh * p.v_s1) * 2 + n * 16;
+  const int64_t k_row_bytes = p.k_s0 * 2, v_row_bytes = p.v_s0 * 2;
+
+  // Q^T as B operands: qb[ks] = Q[head n][32 ks + 8 g .. + 7] (zero for the spare columns)
+  u32x4 qb[4];
+  {
+    const char* qrow = (const char*)p.q + ((b * p.hq + qh0 + (n < nh ? n : 0)) * 128 + 8 * g) * 2;
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++) qb[ks] = n < nh ? *(const u32x4*)(qrow + ks * 64) : u32x4{0, 0, 0, 0};
+  }
+  char* lds_k = lds + wave * kMfmaStage;
+  char* lds_v = lds_k + kMfmaBatch * kMfmaKRow;
+  // the lane writes chunk n of row 4 i + g (one register + 4 i rows as immediate), reads K row n (and 16 + n), chunk
+  // 4 ks + g, and V through the transposing read: lane n of a group points at row 4 g + n / 4, elements 4 (n % 4) .. + 3 of a d-block
+  char* kwrite0 = lds_k + g * kMfmaKRow + n * 16;
+  char* vwrite0 = lds_v + g * kMfmaVRow + n * 16;
+  const char* kread0 = lds_k + n * kMfmaKRow + g * 16;
+  const int vread0 = (int)(uintptr_t)(__attribute__((address_space(3))) char*)lds_v + (4 * g + (n >> 2)) * kMfmaVRow + 8 * (n & 3);
+  // Slot numbers of a batch: the lane loads chunk n of the rows of tokens 4 i + g; positions past the end repeat the last
+  // row.  Issued from inline assembly like the data loads (one hand-kept count of outstanding loads).
+  struct Slots {
+    int v[8];
+  };
+  auto load_slots = [&](int t0, Slots& sl) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      const int tok = t0 + 4 * i + g;
+      const uint32_t off = (uint32_t)(tok < t_last ? tok : t_last) * 4u;  // (a row of the table is shorter than 2^31 entries)
+      asm volatile("global_load_dword %0, %1, %2" : "=v"(sl.v[i]) : "v"(off), "s"(table) : "memory");
+    }
+  };
+  // waits until at most N loads are outstanding and makes the slot numbers of `sl` usable
+  auto wait_slots = [&](auto n_tag, Slots& sl) __attribute__((always_inline)) {
+    constexpr int N = decltype(n_tag)::value;
+    asm volatile("s_waitcnt vmcnt(%8)"
+                 : "+v"(sl.v[0]), "+v"(sl.v[1]), "+v"(sl.v[2]), "+v"(sl.v[3]), "+v"(sl.v[4]), "+v"(sl.v[5]), "+v"(sl.v[6]), "+v"(sl.v[7])
+                 : "n"(N)
+                 : "memory");
+  };
+  // the 16 row loads of a batch: K rows into kr, V rows into vr (rows are read once: non-temporal)
+  auto issue = [&](const Slots& sl, u32x4 (&kr)[8], u32x4 (&vr)[8]) __attribute__((always_inline)) {
+    // (the 64-bit row address is formed next to its load, in a scratch register pair that dies with it: sixteen addresses
+    // formed ahead of their loads would not fit the register file beside two batches of rows)
+    const uint32_t krb = (uint32_t)k_row_bytes, vrb = (uint32_t)v_row_bytes;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      uint64_t addr;
+      asm volatile("v_mad_u64_u32 %1, vcc, %2, %3, %4\n\tglobal_load_dwordx4 %0, %1, off nt"
+                   : "=v"(kr[i]), "=&v"(addr) : "v"(sl.v[i]), "s"(krb), "v"(kbase) : "vcc", "memory");
+    }
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      uint64_t addr;
+      asm volatile("v_mad_u64_u32 %1, vcc, %2, %3, %4\n\tglobal_load_dwordx4 %0, %1, off nt"
+                   : "=v"(vr[i]), "=&v"(addr) : "v"(sl.v[i]), "s"(vrb), "v"(vbase) : "vcc", "memory");
+    }
+  };
+  // waits until at most 16 loads (the next batch's rows) are outstanding and makes kr / vr usable
+  auto wait_rows = [&](u32x4 (&kr)[8], u32x4 (&vr)[8]) __attribute__((always_inline)) {
+    asm volatile("s_waitcnt vmcnt(16)"
+                 : "+v"(kr[0]), "+v"(kr[1]), "+v"(kr[2]), "+v"(kr[3]), "+v"(kr[4]), "+v"(kr[5]), "+v"(kr[6]), "+v"(kr[7]), "+v"(vr[0]),
+                   "+v"(vr[1]), "+v"(vr[2]), "+v"(vr[3]), "+v"(vr[4]), "+v"(vr[5]), "+v"(vr[6]), "+v"(vr[7])
+                 :
+                 : "memory");
+  };
+
+  f32x4 oacc[8];
+  float m = -INFINITY, l = 0.f;  // running maximum (log2 domain, the same in the four lanes of a head) / the lane's part of the sum
+  auto reset = [&]() __attribute__((always_inline)) {
+#pragma unroll
+    for (int db = 0; db < 8; db++) oacc[db] = f32x4{0.f, 0.f, 0.f, 0.f};
+    m = -INFINITY;
+    l = 0.f;
+  };
+  reset();
+  auto flush = [&](int64_t blk) __attribute__((always_inline)) {
+    float lt = l + xlane16(l);
+    lt += xlane32(lt);
+    if (n < nh) {
+      const float inv = 1.f / lt;  // a block holds at least one token
+      const int64_t row = (blk * p.row_mul * p.batch + b) * p.hq + qh0 + n;
+      float* dst = p.mid_o + row * 128 + 4 * g;
+#pragma unroll
+      for (int db = 0; db < 8; db++) *(f32x4*)(dst + 16 * db) = oacc[db] * inv;
+      if (g == 0) p.mid_lse[row] = (m + __builtin_amdgcn_logf(lt)) * kLn2;
+      // the rows of the blocks merged into this partial (row_mul <= 16: lane group g takes every fourth of them)
+      for (int r = 1 + g; r < p.row_mul; r += 4)
+        if (blk * p.row_mul + r < fine_nblk) p.mid_lse[((blk * p.row_mul + r) * p.batch + b) * p.hq + qh0 + n] = -INFINITY;
+    }
+  };
+  // one batch whose rows have arrived in kr / vr
+  auto compute = [&](int t0, const u32x4 (&kr)[8], const u32x4 (&vr)[8]) __attribute__((always_inline)) {
+    // rows into operand layout through the wave's LDS (the reads of the previous batch were consumed by its MFMAs)
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      *(u32x4*)(kwrite0 + 4 * i * kMfmaKRow) = kr[i];
+      *(u32x4*)(vwrite0 + 4 * i * kMfmaVRow) = vr[i];
+    }
+    f32x4 s[2];
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+      s[h] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < 4; ks++) {
+        const u32x4 ka = *(const u32x4*)(kread0 + h * 16 * kMfmaKRow + ks * 64);
+        s[h] = Mfma16<T>::run(ka, qb[ks], s[h]);
+      }
+    }
+    // s[h][r] = score of token t0 + 16 h + 4 g + r for head n
+    float mx = -INFINITY;
+#pragma unroll
+    for (int h = 0; h < 2; h++)
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        const bool valid = t0 + 16 * h + 4 * g + r < t_end;
+        s[h][r] = valid ? s[h][r] * p.scale_log2 : -INFINITY;
+        mx = fmaxf(mx, s[h][r]);
+      }
+    mx = fmaxf(mx, xlane16(mx));
+    mx = fmaxf(mx, xlane32(mx));            // over the batch's 32 tokens (at least one is valid)
+    const float m_new = fmaxf(m, mx);
+    const float alpha = exp2_diff(m, m_new);
+    if (__builtin_amdgcn_ballot_w64(m_new != m) != 0) {
+#pragma unroll
+      for (int db = 0; db < 8; db++) oacc[db] *= alpha;
+      l *= alpha;
+    }
+    m = m_new;
+    float pv[8];
+    float ps = 0.f;
+#pragma unroll
+    for (int h = 0; h < 2; h++)
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        pv[4 * h + r] = __builtin_amdgcn_exp2f(s[h][r] - m_new);
+        ps += pv[4 * h + r];
+      }
+    l += ps;
+    // P^T as B operand: the lane's eight tokens are the contraction slots 8 g .. 8 g + 7, the order the V^T operand uses
+    u32x4 phi, plo;
+    if (std::is_same<T, F16>::value) {
+#pragma unroll
+      for (int e = 0; e < 4; e++) phi[e] = pack2<F16>(pv[2 * e], pv[2 * e + 1]);
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        // high part: P truncated to bfloat16; low part: the rest, rounded
+        const uint32_t h0 = __builtin_bit_cast(uint32_t, pv[2 * e]) & 0xffff0000u, h1 = __builtin_bit_cast(uint32_t, pv[2 * e + 1]) & 0xffff0000u;
+        phi[e] = (h0 >> 16) | h1;
+        plo[e] = pack2<BF16>(pv[2 * e] - __builtin_bit_cast(float, h0), pv[2 * e + 1] - __builtin_bit_cast(float, h1));
+      }
+    }
+#pragma unroll
+    for (int db = 0; db < 8; db++) {
+      const i16x4 xa = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) i16x4*)(vread0 + db * 32));
+      const i16x4 xb = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) i16x4*)(vread0 + db * 32 + 16 * kMfmaVRow));
+      const u32x2 wa = __builtin_bit_cast(u32x2, xa), wb = __builtin_bit_cast(u32x2, xb);
+      const u32x4 va = u32x4{wa[0], wa[1], wb[0], wb[1]};
+      oacc[db] = Mfma16<T>::run(va, phi, oacc[db]);
+      if (!std::is_same<T, F16>::value) oacc[db] = Mfma16<T>::run(va, plo, oacc[db]);
+    }
+  };
+  auto finish_batch = [&](int t0) __attribute__((always_inline)) {
+    if ((t0 + kMfmaBatch - t_begin) % bs == 0 || t0 + kMfmaBatch >= t_end) {
+      flush(blk_begin + (t0 - t_begin) / bs);
+      reset();
+    }
+  };
+
+  // Order of the loads, oldest first, when batch j is about to be computed:  rows(j) | slots(j+2) | rows(j+1).  The wait for
+  // vmcnt(16) then leaves exactly rows(j+1) in flight; slots(j+1), which rows(j+1) were addressed with, were complete one
+  // wait earlier (the vmcnt(24) in front of an issue is a no-op except in the first trip).
+  u32x4 kr0[8], vr0[8], kr1[8], vr1[8];
+  Slots s_even, s_odd;
+  load_slots(t_begin, s_even);
+  load_slots(t_begin + kMfmaBatch, s_odd);
+  wait_slots(std::integral_constant<int, 8>{}, s_even);
+  issue(s_even, kr0, vr0);
+  // two batches per trip, so that the register set of a batch is a compile-time choice
+  for (int j = 0; j < n_batches; j += 2) {
+    const int t0 = t_begin + j * kMfmaBatch;
+    load_slots(t0 + 2 * kMfmaBatch, s_even);                // slots(j+2): rows(j) have been addressed
+    wait_slots(std::integral_constant<int, 24>{}, s_odd);   // slots(j+1) usable
+    issue(s_odd, kr1, vr1);                                 // rows(j+1) (past the end: the last row again, never used)
+    wait_rows(kr0, vr0);
+    compute(t0, kr0, vr0);
+    finish_batch(t0);
+    load_slots(t0 + 3 * kMfmaBatch, s_odd);                 // slots(j+3)
+    wait_slots(std::integral_constant<int, 24>{}, s_even);  // slots(j+2) usable
+    issue(s_even, kr0, vr0);                                // rows(j+2)
+    wait_rows(kr1, vr1);
+    if (j + 1 < n_batches) {
+      compute(t0 + kMfmaBatch, kr1, vr1);
+      finish_batch(t0 + kMfmaBatch);
+    }
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // (rows requested past the end land before the registers are given back)
+}
+
+// ------------------------------------------------------------------------------------
 // Stage 2: grid (batch, heads); SL slices of D/4 lanes walk the block axis in parallel
 // (the reference walks it serially, flash_decoding_stage2.cu:38-48), then merge through LDS.
 // ------------------------------------------------------------------------------------
@@ -527,8 +804,65 @@ static int launch_stage1(const lsattn_decode_stage1_args* a, hipStream_t st) {
   return check_launch();
 }
 
+// Large groups: the matrix-pipe kernel, when its conditions hold (blocks a multiple of 32 tokens, enough waves to fill
+// the chip); LSATTN_DECODE_MFMA = 0 / 1 in the environment forces the choice where the conditions allow it (tuning, tests).
+template <typename T> static int launch_stage1_mfma(const lsattn_decode_stage1_args* a, hipStream_t st, bool* taken) {
+  *taken = false;
+  const int group = (int)(a->num_q_heads / a->num_kv_heads);
+  Stage1Params p;
+  p.mid_o = a->mid_o;
+  p.mid_lse = a->mid_o_logexpsum;
+  p.q = a->q;
+  p.k = a->k;
+  p.v = a->v;
+  p.k_s0 = a->k_stride_0;
+  p.k_s1 = a->k_stride_1;
+  p.v_s0 = a->v_stride_0;
+  p.v_s1 = a->v_stride_1;
+  p.scale_log2 = a->sm_scale * kLog2e;
+  p.req_to_tokens = a->req_to_tokens;
+  p.b_req_idx = a->b_req_idx;
+  p.b_seqlen = a->b_seqlen;
+  p.batch = a->batch;
+  p.hq = a->num_q_heads;
+  p.hkv = a->num_kv_heads;
+  p.num_blocks = a->num_blocks;
+  p.max_seq_len = a->max_seq_len;
+  p.row_mul = a->merge_blocks > 1 ? a->merge_blocks : 1;
+  p.fine_block_seq = a->seq_block_size;
+  p.block_seq = a->seq_block_size * p.row_mul;
+  p.grid_blocks = (a->max_len_in_batch + p.block_seq - 1) / p.block_seq;
+  if (p.block_seq % kMfmaBatch || a->k_stride_0 >= (1 << 30) || a->v_stride_0 >= (1 << 30)) return LSATTN_OK;
+  p.tasks = (int)a->num_kv_heads * ((group + 15) / 16);
+  int64_t per_wave = (256 + p.block_seq - 1) / p.block_seq;  // a wave walks at least 256 tokens
+  if (per_wave < 1) per_wave = 1;
+  const int64_t rows_avail = (a->num_blocks + p.row_mul - 1) / p.row_mul;
+  const int64_t nblk = p.grid_blocks < rows_avail ? p.grid_blocks : rows_avail;
+  if (nblk < 1) return LSATTN_OK;
+  p.blocks_per_wg = (int32_t)per_wave;
+  const int64_t chunks = (nblk + per_wave - 1) / per_wave;
+  const int64_t wgs_x = (chunks + kMfmaWaves - 1) / kMfmaWaves;
+  if (wgs_x > 0x7fffffff || a->batch > 65535 || p.tasks > 65535) return LSATTN_OK;
+  bool use = group >= 5 && chunks * p.tasks * a->batch >= 1024;
+  if (const char* e = getenv("LSATTN_DECODE_MFMA")) {
+    if (e[0] == '0' && !e[1]) use = false;
+    if (e[0] == '1' && !e[1]) use = true;
+  }
+  if (!use) return LSATTN_OK;
+  *taken = true;
+  p.tasks_on_x = 0;
+  hipLaunchKernelGGL((decode_stage1_mfma_kernel<T>), dim3((unsigned)wgs_x, (unsigned)p.tasks, (unsigned)a->batch), dim3(kMfmaWaves * 64), 0,
+                     st, p);
+  return check_launch();
+}
+
 template <typename T> static int dispatch_stage1(const lsattn_decode_stage1_args* a, hipStream_t st) {
   const int group = (int)(a->num_q_heads / a->num_kv_heads);
+  {
+    bool taken;
+    const int rc = launch_stage1_mfma<T>(a, st, &taken);
+    if (taken) return rc;
+  }
   // groups of 3 and 4 take four query heads per task (3: one spare): fetching a K/V row once per group matters more than
   // the spare accumulators cost
   // groups of more than four: eight query heads per task in two rounds of four over the same rows

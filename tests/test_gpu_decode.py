@@ -15,6 +15,10 @@ DEV = "cuda:0"
 @pytest.mark.parametrize("Hq,Hkv,BS", [(32, 8, 256), (4, 4, 64), (16, 8, 16), (10, 5, 128), (12, 4, 256), (8, 1, 32), (14, 2, 256),
                                        (5, 1, 64), (12, 2, 128), (3, 1, 16), (8, 1, 256), (16, 2, 64), (9, 1, 128), (32, 2, 256), (8, 2, 100), (4, 4, 7)])
 def test_stage1_stage2_vs_oracle(lsa, dtype, Hq, Hkv, BS):
+    _check_stage1_stage2(lsa, dtype, Hq, Hkv, BS)
+
+
+def _check_stage1_stage2(lsa, dtype, Hq, Hkv, BS):
     print("case", dtype, Hq, Hkv, BS, flush=True)
     B, D = 5, 128
     lens = [700, 1, 256, 33, 1025]
@@ -84,6 +88,10 @@ def test_stage1_stage2_vs_oracle(lsa, dtype, Hq, Hkv, BS):
     (4, 4, 128, [4097, 130]),                  # one query head per KV head
 ])
 def test_stage1_forced_merge_blocks(lsa, dtype, merge, Hq, Hkv, BS, lens):
+    _check_merge_blocks(lsa, dtype, merge, Hq, Hkv, BS, lens)
+
+
+def _check_merge_blocks(lsa, dtype, merge, Hq, Hkv, BS, lens):
     """merge_blocks = m of flash_decoding_stage1: the partial of blocks [m j, m j + m) of a request in row m j, the other
     rows the request reaches marked empty, rows past it untouched; checked row by row against the oracle's stage 1 at
     block size m * BS, and through stage 2 at the caller's block size."""
@@ -120,6 +128,68 @@ def test_stage1_forced_merge_blocks(lsa, dtype, merge, Hq, Hkv, BS, lens):
     o_ref, l_ref = orc.decode_full(q, k, v, table, b_req, b_len)
     assert_o_close(o_d, o_ref, "o")
     assert_lse_close(l_d, l_ref, "lse")
+
+
+@pytest.fixture
+def matrix_pipe(monkeypatch):
+    """Stage 1 through the matrix-pipe kernel wherever its conditions hold (blocks a multiple of 32 tokens), whatever the
+    launch's size: by itself the library takes it for groups of five or more query heads per KV head in launches of
+    1024 waves or more."""
+    monkeypatch.setenv("LSATTN_DECODE_MFMA", "1")
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("Hq,Hkv,BS", [(32, 8, 256), (4, 4, 64), (10, 5, 128), (8, 1, 32), (5, 1, 64), (9, 1, 128), (16, 2, 64), (32, 2, 256),
+                                       (17, 1, 96), (66, 2, 32), (7, 7, 160)])
+def test_matrix_pipe_stage1_stage2_vs_oracle(lsa, matrix_pipe, dtype, Hq, Hkv, BS):
+    """Groups of 1 to 33 query heads (padded to 16-row operands, 17 and 33: a second / third task with one live row),
+    blocks of one to eight 32-token batches, requests of 1 token, of a partial batch and of a partial block."""
+    _check_stage1_stage2(lsa, dtype, Hq, Hkv, BS)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("merge", [2, 16])
+@pytest.mark.parametrize("Hq,Hkv,BS,lens", [
+    (8, 1, 128, [5000]),
+    (16, 1, 256, [3000, 9000]),
+    (16, 4, 32, [100, 2049, 17, 640, 1, 999]),
+    (40, 8, 64, [4097, 130]),
+])
+def test_matrix_pipe_stage1_forced_merge_blocks(lsa, matrix_pipe, dtype, merge, Hq, Hkv, BS, lens):
+    _check_merge_blocks(lsa, dtype, merge, Hq, Hkv, BS, lens)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_large_group_launch_that_takes_the_matrix_pipe_by_itself(lsa, dtype):
+    """64 query heads over 8 KV heads, 2 requests of about 17000 tokens: 2 x 8 x 67 waves of the matrix-pipe kernel, the
+    library's own choice (no environment override), through the fused call and through the two stages."""
+    assert "LSATTN_DECODE_MFMA" not in __import__("os").environ
+    B, Hq, Hkv, D, BS = 2, 64, 8, 128, 256
+    lens = [17000, 16411]
+    q, kv, table, b_req, b_len = decode_case(77, B, Hq, Hkv, D, lens, sum(lens) + 1000, dtype)
+    k, v = kv[:, :Hkv], kv[:, Hkv:]
+    o_ref, l_ref = orc.decode_full(q, k, v, table, b_req, b_len)
+    kvd = kv.to(DEV)
+    nblk = (max(lens) + BS - 1) // BS
+    mo_d = torch.full((nblk, B, Hq, D), float("nan"), device=DEV)
+    ml_d = torch.full((nblk, B, Hq), float("nan"), device=DEV)
+    o_d = torch.empty(B, Hq, D, device=DEV)
+    l_d = torch.empty(B, Hq, device=DEV)
+    lsa.longserve_token_decode_attention_flash_decoding(q.to(DEV), table.to(DEV), b_req.to(DEV), b_len.to(DEV), mo_d, ml_d, B, max(lens),
+                                                        Hq, D, kvd[:, :Hkv], kvd[:, Hkv:], BS, o_d, l_d)
+    torch.cuda.synchronize()
+    assert_o_close(o_d, o_ref, "o, fused call")
+    assert_lse_close(l_d, l_ref, "lse, fused call")
+    mo_d.fill_(float("nan"))
+    ml_d.fill_(float("nan"))
+    lsa.longserve_flash_decode_stage1(q.to(DEV), kvd[:, :Hkv], kvd[:, Hkv:], table.to(DEV), b_req.to(DEV), b_len.to(DEV), max(lens),
+                                      mo_d, ml_d, BS)
+    lsa.longserve_flash_decode_stage2(mo_d, ml_d, b_len.to(DEV), o_d, l_d, BS)
+    torch.cuda.synchronize()
+    reach = torch.tensor([(n + BS - 1) // BS for n in lens])
+    assert torch.equal(torch.isnan(ml_d.cpu()), (torch.arange(nblk)[:, None] >= reach[None, :])[:, :, None].expand(nblk, B, Hq))
+    assert_o_close(o_d, o_ref, "o, two stages")
+    assert_lse_close(l_d, l_ref, "lse, two stages")
 
 
 def test_gather_indices_bit_exact(lsa):

@@ -273,18 +273,120 @@ def test_dpp_scanner_flags_a_close_write():
     assert len(bad) == 1 and "written by v_mov_b32_e32" in bad[0], bad
 
 
+_DECODE_ASM = []
+
+
+def _decode_asm():
+    """The device assembly of decode.hip under the library's own flags (compiled once per session)."""
+    if not _DECODE_ASM:
+        import importlib.util
+        spec = importlib.util.spec_from_file_location("_lsattn_build_flags", os.path.join(REPO, "loongserve_amd", "build.py"))
+        recipe = importlib.util.module_from_spec(spec)
+        spec.loader.exec_module(recipe)
+        src = os.path.join(REPO, "loongserve_amd", "csrc", "decode.hip")
+        with tempfile.TemporaryDirectory() as tmp:
+            out = os.path.join(tmp, "decode.s")
+            cmd = [recipe.HIPCC, *recipe.FLAGS, *recipe.FILE_FLAGS.get("decode.hip", []), "-S", "--cuda-device-only", src, "-o", out]
+            subprocess.run(cmd, check=True, stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)
+            _DECODE_ASM.append(open(out).read())
+    return _DECODE_ASM[0]
+
+
 @pytest.mark.skipif(shutil.which(HIPCC) is None, reason="hipcc not available")
 def test_no_vector_write_next_to_an_inline_assembly_dpp_in_decode():
-    import importlib.util
-    spec = importlib.util.spec_from_file_location("_lsattn_build_flags", os.path.join(REPO, "loongserve_amd", "build.py"))
-    recipe = importlib.util.module_from_spec(spec)
-    spec.loader.exec_module(recipe)
-    src = os.path.join(REPO, "loongserve_amd", "csrc", "decode.hip")
-    with tempfile.TemporaryDirectory() as tmp:
-        out = os.path.join(tmp, "decode.s")
-        cmd = [recipe.HIPCC, *recipe.FLAGS, *recipe.FILE_FLAGS.get("decode.hip", []), "-S", "--cuda-device-only", src, "-o", out]
-        subprocess.run(cmd, check=True, stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)
-        text = open(out).read()
-    ins, bad = find_dpp_hazards(text)
+    ins, bad = find_dpp_hazards(_decode_asm())
     assert sum(1 for _, op, _, in_asm in ins if in_asm and op.endswith("_dpp")) >= 1000
     assert not bad, "\n".join(bad[:20])
+
+
+def loads_in_flight_violations(text, kernel_pattern):
+    """The matrix-pipe decode kernel issues its global loads from inline assembly and waits for them with hand-placed
+    `s_waitcnt vmcnt(N)`; the compiler knows of neither, so nothing but data flow through the asm operands keeps it from
+    using a destination register early.  Walk each matching kernel in program order: a register that such a load is still
+    to write (vmcnt retires loads oldest first: `vmcnt(N)` leaves the N youngest in flight) may appear in no instruction,
+    not even as the address of the next load.  Returns {kernel: (asm loads seen, violations)}.  The walk is linear over the
+    text; a loop's back edge is covered by the prologue putting the counters into the state the loop's end leaves."""
+    res, kernels, name = {}, {}, None
+    for ln, raw in enumerate(text.split("\n"), 1):
+        m = re.match(r"^(_ZN6lsattn\w+):", raw)
+        if m:
+            name = m.group(1)
+            kernels[name] = []
+        elif raw.startswith("\t.end_amdhsa_kernel") or raw.startswith(".Lfunc_end"):
+            name = None
+        if name:
+            kernels[name].append((ln, raw))
+    for name, lines in kernels.items():
+        if kernel_pattern not in name:
+            continue
+        pending, bad, in_asm, nload = {}, [], False, 0
+        for ln, raw in lines:
+            if "#ASMSTART" in raw:
+                in_asm = True
+                continue
+            if "#ASMEND" in raw:
+                in_asm = False
+                continue
+            ins = raw.split(";")[0].strip()
+            if not ins or ins.endswith(":") or ins.startswith("."):
+                continue
+            parts = ins.split(None, 1)
+            op = parts[0]
+            ops = [t.strip().split(" ")[0] for t in parts[1].split(",")] if len(parts) > 1 else []
+            if op == "s_waitcnt":
+                m = re.search(r"vmcnt\((\d+)\)", ins)
+                if m:
+                    n = int(m.group(1))
+                    keep = set(sorted(set(pending.values()))[-n:]) if n > 0 else set()
+                    pending = {r: v for r, v in pending.items() if v in keep}
+                continue
+            touched = set().union(*[_regs(t) for t in ops]) if ops else set()
+            if in_asm and op.startswith("global_load_dword"):
+                nload += 1
+                hit = set().union(*[_regs(t) for t in ops[1:]]) & set(pending) if len(ops) > 1 else set()
+                if hit:
+                    bad.append("line %d: %s addresses with v%s, which a load in flight writes" % (ln, ins, sorted(hit)))
+                for r in _regs(ops[0]):
+                    pending[r] = nload
+                continue
+            hit = touched & set(pending)
+            if hit:
+                bad.append("line %d: %s touches v%s, which a load in flight writes" % (ln, ins, sorted(hit)))
+        res[name] = (nload, bad)
+    return res
+
+
+def test_in_flight_scanner_flags_an_early_use():
+    text = """
+_ZN6lsattn4demoEv:
+	;;#ASMSTART
+	global_load_dwordx4 v[4:7], v[20:21], off nt
+	;;#ASMEND
+	;;#ASMSTART
+	global_load_dwordx4 v[8:11], v[22:23], off nt
+	;;#ASMEND
+	;;#ASMSTART
+	s_waitcnt vmcnt(1)
+	;;#ASMEND
+	v_add_f32_e32 v30, v4, v5
+	%s
+	;;#ASMSTART
+	s_waitcnt vmcnt(0)
+	;;#ASMEND
+	v_add_f32_e32 v31, v8, v9
+	s_endpgm
+.Lfunc_end0:
+"""
+    (n, bad), = loads_in_flight_violations(text % "v_mov_b32_e32 v32, v6", "demo").values()
+    assert n == 2 and not bad, bad
+    (n, bad), = loads_in_flight_violations(text % "v_mov_b32_e32 v32, v10", "demo").values()
+    assert len(bad) == 1 and "touches v[10]" in bad[0], bad
+
+
+@pytest.mark.skipif(shutil.which(HIPCC) is None, reason="hipcc not available")
+def test_decode_matrix_pipe_kernel_touches_no_register_of_a_load_in_flight():
+    res = loads_in_flight_violations(_decode_asm(), "decode_stage1_mfma_kernel")
+    assert len(res) == 2, list(res)                       # fp16 and bf16
+    for name, (n, bad) in res.items():
+        assert n >= 3 * 8 + 3 * 16, (name, n)             # slot and row loads of the prologue and of both halves of the loop
+        assert not bad, name + "\n" + "\n".join(bad[:20])
