@@ -38,6 +38,20 @@
 
 namespace lsattn {
 
+// Division of 0 <= n < 2^31 by a launch constant d >= 1 without the divide sequence (some thirty instructions each, and
+// the prologue of a workgroup needs ten): n / d = umulhi(n, mul) >> shr with mul = ceil(2^(31 + L) / d), shr = L - 1,
+// L = ceil(log2 d); d = 1 is mul = 0.
+struct FastDiv {
+  uint32_t mul, shr;
+};
+static FastDiv fast_div(uint32_t d) {
+  if (d <= 1) return FastDiv{0, 0};
+  uint32_t L = 0;
+  while ((1u << L) < d) L++;
+  return FastDiv{(uint32_t)((((uint64_t)1 << (31 + L)) + d - 1) / d), L - 1};
+}
+__device__ __forceinline__ uint32_t div_by(uint32_t n, const FastDiv& f) { return f.mul ? __umulhi(n, f.mul) >> f.shr : n; }
+
 struct PrefillParams {
   const void* q;
   const void* k;
@@ -49,7 +63,8 @@ struct PrefillParams {
   const int32_t* kv_start;
   const int32_t* kv_len;
   const int32_t* kv_first;
-  int32_t batch, hq, hkv, peers, nz, kv_slots, slices, units_per_slice;
+  int32_t batch, hq, hkv, peers, nz, kv_slots, slices, units_per_slice, group;
+  FastDiv d_peers, d_kv_slots, d_slices, d_units, d_group;
   float scale_log2;
   void* o;
   int64_t o_st, o_sh;
@@ -208,39 +223,41 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
   // Workgroup ids go to the 8 XCDs round-robin.  The (query head, query tile) units of one KV head are dealt to p.slices
   // XCDs (1 when the KV heads are a multiple of 8, else as many as it takes for hkv * slices to be one), so that the
   // workgroups sharing a KV head's K/V meet in few L2s and every XCD has work whatever the head count.
-  const int group = p.hq / p.hkv;
-  int j = blockIdx.x >> 3;
+  const int group = p.group;
+  uint32_t j = blockIdx.x >> 3;
   const int xcd = blockIdx.x & 7;
   int up, slot;
   if (SPLIT) {
     // Small launches: the heaviest query tiles of all KV heads first, so that a CU that has finished a light tile of the
     // first round takes a heavy one of the rest and the other way round.
-    slot = j % p.kv_slots;
-    j /= p.kv_slots;
-    up = j % p.units_per_slice;
-    j /= p.units_per_slice;
+    const uint32_t j1 = div_by(j, p.d_kv_slots);
+    slot = (int)(j - j1 * p.kv_slots);
+    j = div_by(j1, p.d_units);
+    up = (int)(j1 - j * p.units_per_slice);
   } else {
     // Large launches: one KV head at a time per XCD, whose K/V then serves all the workgroups the XCD runs.
-    up = j % p.units_per_slice;
-    j /= p.units_per_slice;
-    slot = j % p.kv_slots;
-    j /= p.kv_slots;
+    const uint32_t j1 = div_by(j, p.d_units);
+    up = (int)(j - j1 * p.units_per_slice);
+    j = div_by(j1, p.d_kv_slots);
+    slot = (int)(j1 - j * p.kv_slots);
   }
-  const int b = j;
+  const int b = (int)j;  // < batch for every workgroup of the grid
+  // The request's six numbers, all requested before the first of them is used (one memory latency instead of three on
+  // the way to the first tile load; a workgroup's start-up is what a short launch is made of).
+  const int q_len = p.q_len[b], kv_len = p.kv_len[b], qf = p.q_first[b], kf = p.kv_first[b];
+  const int q_start32 = p.q_start[b], kv_start32 = p.kv_start[b];
+  asm volatile("" ::"s"(q_len), "s"(kv_len), "s"(qf), "s"(kf), "s"(q_start32), "s"(kv_start32));
+  const int64_t q_start = q_start32, kv_start = kv_start32;
   const int vh = xcd + 8 * slot;  // (KV head, slice) pair: always < hkv * slices
-  const int kvh = vh / p.slices;
-  const int u = up * p.slices + vh % p.slices;
+  const int kvh = (int)div_by((uint32_t)vh, p.d_slices);
+  const int u = up * p.slices + (vh - kvh * p.slices);
   if (u >= group * p.nz) return;
-  const int gq = u % group, zr = u / group;
+  const int zr = (int)div_by((uint32_t)u, p.d_group), gq = u - zr * group;
   const int h = kvh * group + gq;
   const int z = p.nz - 1 - zr;
 
-  const int q_len = p.q_len[b];
   const int m_lo = z * BMW;
   if (m_lo >= q_len) return;
-  const int kv_len = p.kv_len[b];
-  const int64_t q_start = p.q_start[b], kv_start = p.kv_start[b];
-  const int qf = p.q_first[b], kf = p.kv_first[b];
   const int P = p.peers;
 
   const int tid = threadIdx.x;
@@ -252,7 +269,7 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
   // keys of this KV chunk visible to global query position qpos (RING:156-159)
   auto visible_keys = [&](int qpos) -> int {
     const int dq = qpos - kf;
-    const int n = dq >= 0 ? dq / P + 1 : 0;
+    const int n = dq >= 0 ? (int)div_by((uint32_t)dq, p.d_peers) + 1 : 0;
     return n > kv_len ? kv_len : n;
   };
   const int m_hi = (m_lo + BMW < q_len ? m_lo + BMW : q_len) - 1;
@@ -269,7 +286,9 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
     const bool ok = m < q_len;
     const char* src = (const char*)p.q + ((q_start + (ok ? m : 0)) * p.q_st + (int64_t)h * p.q_sh + 8 * g) * 2;
 #pragma unroll
-    for (int ks = 0; ks < 4; ks++) qreg[qb][ks] = ok ? *(const u32x4*)(src + ks * 64) : u32x4{0, 0, 0, 0};
+    // (a row past the end holds the request's first row instead: it sees no key, cnt = 0, and is never stored; no select
+    // stands between the loads and the tile loads that follow)
+    for (int ks = 0; ks < 4; ks++) qreg[qb][ks] = *(const u32x4*)(src + ks * 64);
     cnt[qb] = ok ? visible_keys(qf + m * P) : 0;
   }
 
@@ -726,163 +745,200 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
     for (int qb = 0; qb < 2; qb++) m_run[qb] = -neg_m[qb];
   }
 
-  if (SPLIT) {
-    // the partial of the odd sub-tiles (waves 4-7) joins that of the even ones through LDS; waves 0-3 go on alone
-    wait_vmem<0>();  // (loads requested ahead for tiles that were never used may still be writing the rings)
-    __syncthreads();
-    float* xch = (float*)lds + wrow * (68 * 64) + lane;  // [value][lane]: 64 accumulators, 2 maxima, 2 sums
-    if (kp == 1) {
-#pragma unroll
-      for (int db = 0; db < 8; db++)
-#pragma unroll
-        for (int qb = 0; qb < 2; qb++)
-#pragma unroll
-          for (int r = 0; r < 4; r++) xch[((db * 2 + qb) * 4 + r) * 64] = oacc[db][qb][r];
-#pragma unroll
-      for (int qb = 0; qb < 2; qb++) {
-        xch[(64 + qb) * 64] = m_run[qb];
-        xch[(66 + qb) * 64] = l_run[qb];
-      }
-    }
-    __syncthreads();
-    if (kp == 1) return;
-#pragma unroll
-    for (int qb = 0; qb < 2; qb++) {
-      const float m1 = xch[(64 + qb) * 64], l1 = xch[(66 + qb) * 64];
-      const float M = fmaxf(m_run[qb], m1);
-      const float w0 = exp2_diff(m_run[qb], M), w1 = exp2_diff(m1, M);  // 0 for a side that saw no key
-      l_run[qb] = l_run[qb] * w0 + l1 * w1;
-      m_run[qb] = M;
-#pragma unroll
-      for (int db = 0; db < 8; db++)
-#pragma unroll
-        for (int r = 0; r < 4; r++) oacc[db][qb][r] = oacc[db][qb][r] * w0 + xch[((db * 2 + qb) * 4 + r) * 64] * w1;
-    }
-  }
-
-  // ---- epilogue ----
-  if (MODE == 0) {
-    // the step's partial from the empty state
+  // Old state of the rows for the epilogues that fold into one.  The two waves of a split pair both need it and one of
+  // them writes it: there it is read before the barrier that the writes come after.
+  float st_a[2] = {0.f, 0.f}, st_b[2] = {0.f, 0.f};
+  auto read_state = [&]() __attribute__((always_inline)) {
 #pragma unroll
     for (int qb = 0; qb < 2; qb++) {
       const int m = m_w0 + 16 * qb + qc;
-      const float l_tot = column_sum(l_run[qb]);
-      if (m < q_len) {
-        const int64_t tok = q_start + m;
-        const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
-        float* orow = (float*)p.o + tok * p.o_st + (int64_t)h * p.o_sh;
+      const int64_t tok = q_start + (m < q_len ? m : 0);
+      if (MODE == 1) {
+        st_a[qb] = p.m[tok * p.ml_st + (int64_t)h * p.ml_sh];
+        st_b[qb] = p.l[tok * p.ml_st + (int64_t)h * p.ml_sh];
+      }
+      if (MODE == 2) st_a[qb] = p.lse[tok * p.hq + h] * kLog2e;
+    }
+  };
+
+  if (SPLIT) {
+    // The partials of the even and of the odd sub-tiles meet through LDS.  Each wave of a pair keeps four of the eight
+    // d-blocks (the even side 0-3, the odd side 4-7), hands the other four to its partner with its maxima and sums, and
+    // finishes its half of every row: merge and stores are shared by all eight waves.
+    wait_vmem<0>();  // (loads requested ahead for tiles that were never used may still be writing the rings)
+    __syncthreads();
+    f32x4* xout = (f32x4*)lds + (wrow * 2 + kp) * (9 * 64) + lane;         // [8 blocks + (m, m, l, l)][lane]
+    const f32x4* xin = (const f32x4*)lds + (wrow * 2 + (kp ^ 1)) * (9 * 64) + lane;
+    auto give = [&](auto db0_tag) __attribute__((always_inline)) {
+      constexpr int DB0 = decltype(db0_tag)::value;
 #pragma unroll
-        for (int db = 0; db < 8; db++) *(f32x4*)(orow + db * 16 + 4 * g) = oacc[db][qb] * inv;
-        if (g == 0) p.lse[tok * p.hq + h] = l_tot > 0.f ? (m_run[qb] + __builtin_amdgcn_logf(l_tot)) * kLn2 : -INFINITY;
+      for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int qb = 0; qb < 2; qb++) xout[(i * 2 + qb) * 64] = oacc[DB0 + i][qb];
+    };
+    if (kp == 0) give(std::integral_constant<int, 4>{});
+    else give(std::integral_constant<int, 0>{});
+    xout[8 * 64] = f32x4{m_run[0], m_run[1], l_run[0], l_run[1]};
+    if (MODE != 0) read_state();
+    __syncthreads();
+    const f32x4 ml = xin[8 * 64];
+    float w_own[2], w_in[2];
+#pragma unroll
+    for (int qb = 0; qb < 2; qb++) {
+      const float m1 = ml[qb], l1 = ml[2 + qb];
+      const float M = fmaxf(m_run[qb], m1);
+      w_own[qb] = exp2_diff(m_run[qb], M);  // 0 for a side that saw no key
+      w_in[qb] = exp2_diff(m1, M);
+      // (the even side's term first on both sides: the two waves hold the same sum to the last bit)
+      l_run[qb] = kp == 0 ? __builtin_fmaf(l_run[qb], w_own[qb], l1 * w_in[qb]) : __builtin_fmaf(l1, w_in[qb], l_run[qb] * w_own[qb]);
+      m_run[qb] = M;
+    }
+    auto take = [&](auto db0_tag) __attribute__((always_inline)) {
+      constexpr int DB0 = decltype(db0_tag)::value;
+#pragma unroll
+      for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int qb = 0; qb < 2; qb++) oacc[DB0 + i][qb] = oacc[DB0 + i][qb] * w_own[qb] + xin[(i * 2 + qb) * 64] * w_in[qb];
+    };
+    if (kp == 0) take(std::integral_constant<int, 0>{});
+    else take(std::integral_constant<int, 4>{});
+  } else if (MODE != 0) {
+    read_state();
+  }
+
+  // ---- epilogue: d-blocks DB0 .. DB0 + NDB - 1 of the wave's rows; the per-row scalars are written by the side that holds block 0 ----
+  constexpr int NDB = SPLIT ? 4 : 8;
+  auto finish = [&](auto db0_tag) __attribute__((always_inline)) {
+    constexpr int DB0 = decltype(db0_tag)::value;
+    if (MODE == 0) {
+      // the step's partial from the empty state
+#pragma unroll
+      for (int qb = 0; qb < 2; qb++) {
+        const int m = m_w0 + 16 * qb + qc;
+        const float l_tot = column_sum(l_run[qb]);
+        if (m < q_len) {
+          const int64_t tok = q_start + m;
+          const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+          float* orow = (float*)p.o + tok * p.o_st + (int64_t)h * p.o_sh;
+#pragma unroll
+          for (int i = 0; i < NDB; i++) *(f32x4*)(orow + (DB0 + i) * 16 + 4 * g) = oacc[DB0 + i][qb] * inv;
+          if (g == 0 && DB0 == 0) p.lse[tok * p.hq + h] = l_tot > 0.f ? (m_run[qb] + __builtin_amdgcn_logf(l_tot)) * kLn2 : -INFINITY;
+        }
       }
     }
-  }
-  if (MODE == 1) {
-    // the reference's update of (o, m, l) (RING:171-188).  NB row blocks at a time: all reads of their old state are in
-    // flight together
-    auto fold_state = [&](auto nb_tag, int qb0) __attribute__((always_inline)) {
-      constexpr int NB = decltype(nb_tag)::value;
-      float l_tot[NB], m_old[NB], l_old[NB];
-      u32x2 old[NB][8];
-      bool in_range[NB];
+    if (MODE == 1) {
+      // the reference's update of (o, m, l) (RING:171-188).  NB row blocks at a time: all reads of their old o are in
+      // flight together
+      auto fold_state = [&](auto nb_tag, int qb0) __attribute__((always_inline)) {
+        constexpr int NB = decltype(nb_tag)::value;
+        float l_tot[NB];
+        u32x2 old[NB][NDB];
+        bool in_range[NB];
 #pragma unroll
-      for (int i = 0; i < NB; i++) {
-        const int qb = qb0 + i;
-        const int m = m_w0 + 16 * qb + qc;
-        l_tot[i] = column_sum(l_run[qb]);
-        in_range[i] = m < q_len;
-        const int64_t tok = q_start + (in_range[i] ? m : 0);
-        m_old[i] = p.m[tok * p.ml_st + (int64_t)h * p.ml_sh];
-        l_old[i] = p.l[tok * p.ml_st + (int64_t)h * p.ml_sh];
-        const uint16_t* orow = (const uint16_t*)p.o + tok * p.o_st + (int64_t)h * p.o_sh;
+        for (int i = 0; i < NB; i++) {
+          const int qb = qb0 + i;
+          const int m = m_w0 + 16 * qb + qc;
+          l_tot[i] = column_sum(l_run[qb]);
+          in_range[i] = m < q_len;
+          const int64_t tok = q_start + (in_range[i] ? m : 0);
+          const uint16_t* orow = (const uint16_t*)p.o + tok * p.o_st + (int64_t)h * p.o_sh;
 #pragma unroll
-        for (int db = 0; db < 8; db++) old[i][db] = *(const u32x2*)(orow + db * 16 + 4 * g);
-      }
+          for (int d = 0; d < NDB; d++) old[i][d] = *(const u32x2*)(orow + (DB0 + d) * 16 + 4 * g);
+        }
 #pragma unroll
-      for (int i = 0; i < NB; i++) {
-        const int qb = qb0 + i;
-        const float M = fmaxf(m_run[qb], m_old[i]);
-        if (!in_range[i] || M == -INFINITY || !(l_tot[i] > 0.f)) continue;
-        const int64_t tok = q_start + m_w0 + 16 * qb + qc;
-        const float w_old = l_old[i] * exp2_diff(m_old[i], M);
-        const float w_new = exp2_diff(m_run[qb], M);
-        const float L = w_old + l_tot[i] * w_new;
-        const float inv = 1.f / L;
-        uint16_t* orow = (uint16_t*)p.o + tok * p.o_st + (int64_t)h * p.o_sh;
+        for (int i = 0; i < NB; i++) {
+          const int qb = qb0 + i;
+          const float m_old = st_a[qb], l_old = st_b[qb];
+          const float M = fmaxf(m_run[qb], m_old);
+          if (!in_range[i] || M == -INFINITY || !(l_tot[i] > 0.f)) continue;
+          const int64_t tok = q_start + m_w0 + 16 * qb + qc;
+          const float w_old = l_old * exp2_diff(m_old, M);
+          const float w_new = exp2_diff(m_run[qb], M);
+          const float L = w_old + l_tot[i] * w_new;
+          const float inv = 1.f / L;
+          uint16_t* orow = (uint16_t*)p.o + tok * p.o_st + (int64_t)h * p.o_sh;
 #pragma unroll
-        for (int db = 0; db < 8; db++) {
-          float o0 = 0.f, o1 = 0.f, o2 = 0.f, o3 = 0.f;
-          if (w_old != 0.f) {  // a row in its start state (m = -inf, l = 0) may hold anything in o
-            unpack2<T>(old[i][db][0], o0, o1);
-            unpack2<T>(old[i][db][1], o2, o3);
+          for (int d = 0; d < NDB; d++) {
+            const int db = DB0 + d;
+            float o0 = 0.f, o1 = 0.f, o2 = 0.f, o3 = 0.f;
+            if (w_old != 0.f) {  // a row in its start state (m = -inf, l = 0) may hold anything in o
+              unpack2<T>(old[i][d][0], o0, o1);
+              unpack2<T>(old[i][d][1], o2, o3);
+            }
+            const float r0 = (o0 * w_old + oacc[db][qb][0] * w_new) * inv;
+            const float r1 = (o1 * w_old + oacc[db][qb][1] * w_new) * inv;
+            const float r2 = (o2 * w_old + oacc[db][qb][2] * w_new) * inv;
+            const float r3 = (o3 * w_old + oacc[db][qb][3] * w_new) * inv;
+            *(u32x2*)(orow + db * 16 + 4 * g) = u32x2{pack2<T>(r0, r1), pack2<T>(r2, r3)};
           }
-          const float r0 = (o0 * w_old + oacc[db][qb][0] * w_new) * inv;
-          const float r1 = (o1 * w_old + oacc[db][qb][1] * w_new) * inv;
-          const float r2 = (o2 * w_old + oacc[db][qb][2] * w_new) * inv;
-          const float r3 = (o3 * w_old + oacc[db][qb][3] * w_new) * inv;
-          *(u32x2*)(orow + db * 16 + 4 * g) = u32x2{pack2<T>(r0, r1), pack2<T>(r2, r3)};
+          if (g == 0 && DB0 == 0) {  // every reader of the old state has it (read_state)
+            p.m[tok * p.ml_st + (int64_t)h * p.ml_sh] = M;
+            p.l[tok * p.ml_st + (int64_t)h * p.ml_sh] = L;
+          }
         }
-        if (g == 0) {  // every lane of the column has read the old state above
-          p.m[tok * p.ml_st + (int64_t)h * p.ml_sh] = M;
-          p.l[tok * p.ml_st + (int64_t)h * p.ml_sh] = L;
-        }
+      };
+      if (DV) {
+        fold_state(std::integral_constant<int, 2>{}, 0);
+      } else {
+        fold_state(std::integral_constant<int, 1>{}, 0);
+        fold_state(std::integral_constant<int, 1>{}, 1);
       }
-    };
-    if (DV) {
-      fold_state(std::integral_constant<int, 2>{}, 0);
-    } else {
-      fold_state(std::integral_constant<int, 1>{}, 0);
-      fold_state(std::integral_constant<int, 1>{}, 1);
     }
-  }
-  if (MODE == 2) {
-    // fold this step's partial into the running fp32 (O, LSE) of each row; a row that saw no key stays as it is.
-    // NB row blocks at a time: all reads of their old state are in flight together
-    auto fold = [&](auto nb_tag, int qb0) __attribute__((always_inline)) {
-      constexpr int NB = decltype(nb_tag)::value;
-      float l_tot[NB], a_old[NB];
-      f32x4 old[NB][8];
-      bool live[NB];
+    if (MODE == 2) {
+      // fold this step's partial into the running fp32 (O, LSE) of each row; a row that saw no key stays as it is.
+      // NB row blocks at a time: all reads of their old O are in flight together
+      auto fold = [&](auto nb_tag, int qb0) __attribute__((always_inline)) {
+        constexpr int NB = decltype(nb_tag)::value;
+        float l_tot[NB];
+        f32x4 old[NB][NDB];
+        bool live[NB];
 #pragma unroll
-      for (int i = 0; i < NB; i++) {
-        const int qb = qb0 + i;
-        const int m = m_w0 + 16 * qb + qc;
-        l_tot[i] = column_sum(l_run[qb]);
-        live[i] = m < q_len && l_tot[i] > 0.f;
-        const int64_t tok = q_start + (m < q_len ? m : 0);
-        a_old[i] = p.lse[tok * p.hq + h] * kLog2e;
-        const float* orow = (const float*)p.o + tok * p.o_st + (int64_t)h * p.o_sh;
+        for (int i = 0; i < NB; i++) {
+          const int qb = qb0 + i;
+          const int m = m_w0 + 16 * qb + qc;
+          l_tot[i] = column_sum(l_run[qb]);
+          live[i] = m < q_len && l_tot[i] > 0.f;
+          const int64_t tok = q_start + (m < q_len ? m : 0);
+          const float* orow = (const float*)p.o + tok * p.o_st + (int64_t)h * p.o_sh;
 #pragma unroll
-        for (int db = 0; db < 8; db++) old[i][db] = *(const f32x4*)(orow + db * 16 + 4 * g);
-      }
-#pragma unroll
-      for (int i = 0; i < NB; i++) {
-        if (!live[i]) continue;
-        const int qb = qb0 + i;
-        const int64_t tok = q_start + m_w0 + 16 * qb + qc;
-        const float a_new = m_run[qb] + __builtin_amdgcn_logf(l_tot[i]);
-        const float top = fmaxf(a_old[i], a_new);
-        const float w_old = exp2_diff(a_old[i], top);
-        const float w_new = __builtin_amdgcn_exp2f(a_new - top);
-        const float W = w_old + w_new;
-        const float c_old = w_old / W, c_new = w_new / (W * l_tot[i]);
-        float* orow = (float*)p.o + tok * p.o_st + (int64_t)h * p.o_sh;
-#pragma unroll
-        for (int db = 0; db < 8; db++) {
-          // an empty row (lse = -inf) may hold anything: its old values are dropped, not multiplied by zero
-          const f32x4 keep = w_old != 0.f ? old[i][db] : f32x4{0.f, 0.f, 0.f, 0.f};
-          *(f32x4*)(orow + db * 16 + 4 * g) = keep * c_old + oacc[db][qb] * c_new;
+          for (int d = 0; d < NDB; d++) old[i][d] = *(const f32x4*)(orow + (DB0 + d) * 16 + 4 * g);
         }
-        if (g == 0) p.lse[tok * p.hq + h] = (top + __builtin_amdgcn_logf(W)) * kLn2;  // the column's lanes read the old value above
+#pragma unroll
+        for (int i = 0; i < NB; i++) {
+          if (!live[i]) continue;
+          const int qb = qb0 + i;
+          const int64_t tok = q_start + m_w0 + 16 * qb + qc;
+          const float a_old = st_a[qb];
+          const float a_new = m_run[qb] + __builtin_amdgcn_logf(l_tot[i]);
+          const float top = fmaxf(a_old, a_new);
+          const float w_old = exp2_diff(a_old, top);
+          const float w_new = __builtin_amdgcn_exp2f(a_new - top);
+          const float W = w_old + w_new;
+          const float c_old = w_old / W, c_new = w_new / (W * l_tot[i]);
+          float* orow = (float*)p.o + tok * p.o_st + (int64_t)h * p.o_sh;
+#pragma unroll
+          for (int d = 0; d < NDB; d++) {
+            // an empty row (lse = -inf) may hold anything: its old values are dropped, not multiplied by zero
+            const f32x4 keep = w_old != 0.f ? old[i][d] : f32x4{0.f, 0.f, 0.f, 0.f};
+            *(f32x4*)(orow + (DB0 + d) * 16 + 4 * g) = keep * c_old + oacc[DB0 + d][qb] * c_new;
+          }
+          if (g == 0 && DB0 == 0) p.lse[tok * p.hq + h] = (top + __builtin_amdgcn_logf(W)) * kLn2;  // (old value: read_state)
+        }
+      };
+      if (DV) {
+        fold(std::integral_constant<int, 2>{}, 0);
+      } else {
+        // the variant that converts V in registers has none to spare: one block at a time
+        fold(std::integral_constant<int, 1>{}, 0);
+        fold(std::integral_constant<int, 1>{}, 1);
       }
-    };
-    if (DV) {
-      fold(std::integral_constant<int, 2>{}, 0);
-    } else {
-      // the variant that converts V in registers has none to spare: one block at a time
-      fold(std::integral_constant<int, 1>{}, 0);
-      fold(std::integral_constant<int, 1>{}, 1);
     }
+  };
+  if constexpr (SPLIT) {
+    if (kp == 1) finish(std::integral_constant<int, 4>{});
+    else finish(std::integral_constant<int, 0>{});
+  } else {
+    finish(std::integral_constant<int, 0>{});
   }
 }
 
@@ -908,6 +964,7 @@ template <typename T, int MODE, bool DV, bool SPLIT> static int launch_prefill_r
   p.hq = a->num_q_heads;
   p.hkv = a->num_kv_heads;
   p.peers = a->sp_peers;
+  p.d_peers = fast_div((uint32_t)a->sp_peers);
   p.nz = (a->max_q_len + BMW - 1) / BMW;
   {
     int g8 = 8;  // gcd(num_kv_heads, 8)
@@ -925,7 +982,12 @@ template <typename T, int MODE, bool DV, bool SPLIT> static int launch_prefill_r
   p.ml_st = a->ml_stride_t;
   p.ml_sh = a->ml_stride_h;
   const int group = a->num_q_heads / a->num_kv_heads;
+  p.group = group;
   p.units_per_slice = (int32_t)(((int64_t)group * p.nz + p.slices - 1) / p.slices);
+  p.d_group = fast_div((uint32_t)group);
+  p.d_slices = fast_div((uint32_t)p.slices);
+  p.d_kv_slots = fast_div((uint32_t)p.kv_slots);
+  p.d_units = fast_div((uint32_t)p.units_per_slice);
   const int64_t wgs = (int64_t)8 * p.units_per_slice * p.kv_slots * a->batch;
   if (wgs > 0x7fffffff) return LSATTN_ERR_INVALID_ARG;
   hipLaunchKernelGGL((prefill_kernel<T, MODE, DV, SPLIT>), dim3((unsigned)wgs), dim3(NWAVE * 64), 0, st, p);
