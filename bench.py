@@ -32,11 +32,14 @@ if ROOT not in sys.path:
 # which is regenerated with the kernels (the JSON line says so in "traffic_source").
 TRAFFIC_SOURCE = "profiles/bench_default_hbm_traffic.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this command, scaled by a 1 GiB copy); a constant of bench.py, not measured in this run"
 TRAFFIC_BYTES = {
-    "config2": 1307.6e6,    # per launch, averaged over the four launches of a ring step (one diagonal + three full)
-    "config3": 5195.2e6,    # stage 1 of the fused call
-    "config1": 108.6e6,
+    "config2": 1294.7e6,    # per launch, averaged over the four launches of a ring step (one diagonal + three full)
+    "config3": 5195.5e6,    # stage 1 of the fused call
+    "config1": 108.7e6,
     "config4": 8596.5e6,    # stage 1 over one instance's 4 x 131072 tokens
-    "config5": 105164e6,    # the attention launch
+    "config5": 106016e6,    # the attention launch
+    "decode_8_1": 656.8e6,  # stage 1 of the large-group cases (matrix-pipe kernel)
+    "decode_16_2": 1308.5e6,
+    "decode_64_8": 5218.5e6,
 }
 PEAK_MFMA_TFLOPS = 2500.0  # dense fp16/bf16 MFMA, MI355X
 PEAK_HBM_GBS = 8000.0
@@ -517,6 +520,40 @@ def decode_latency():
             "cases": rows}
 
 
+def decode_large_groups(steps):
+    """Token-indexed decode for GQA groups of eight and more query heads per KV head (outside the five baseline configs:
+    Llama-3-70B is 64/8, 8/1 per GPU under 8-way tensor parallelism): batch 64, ctx U[4096,32768], scattered pool, fused
+    call and stage 1 alone, through the library's own choice of stage-1 kernel (the matrix-pipe one for these shapes) and
+    with LSATTN_DECODE_MFMA=0 (the lane kernel every smaller group runs on)."""
+    rows = []
+    saved = os.environ.get("LSATTN_DECODE_MFMA")
+    try:
+        for Hq, Hkv in ((8, 1), (16, 2), (64, 8)):
+            d = TokenDecode(Hq=Hq, Hkv=Hkv, seed=3300 + Hq)
+            row = {"q_heads": Hq, "kv_heads": Hkv, "algorithmic_gb_per_step": d.bytes / 1e9}
+            for key, env in (("matrix_pipe", None), ("lane_kernel", "0")):
+                if env is None:
+                    os.environ.pop("LSATTN_DECODE_MFMA", None)
+                else:
+                    os.environ["LSATTN_DECODE_MFMA"] = env
+                # (device time per call from a HIP graph of 20 of them: the shortest of these launches takes 0.12 ms)
+                fused = _time_graph(d.step, launches=20, reps=max(3, steps // 2))
+                s1 = _time_graph(d.stage1_only, launches=20, reps=max(3, steps // 2))
+                row[key] = {"fused_ms": fused, "fused_gbs": d.bytes / (fused * 1e-3) / 1e9, "stage1_ms": s1,
+                            "stage1_gbs": d.bytes / (s1 * 1e-3) / 1e9}
+            row["roofline"] = _roof("decode_stage1_mfma_kernel<F16>", "hbm", row["matrix_pipe"]["stage1_gbs"], row["matrix_pipe"]["stage1_ms"],
+                                    "decode_%d_%d" % (Hq, Hkv))
+            rows.append(row)
+            del d
+            torch.cuda.empty_cache()
+    finally:
+        if saved is None:
+            os.environ.pop("LSATTN_DECODE_MFMA", None)
+        else:
+            os.environ["LSATTN_DECODE_MFMA"] = saved
+    return {"what": " ".join(x.strip() for x in decode_large_groups.__doc__.split("\n")), "cases": rows}
+
+
 def other_steps(steps):
     """The steps around attention (not part of the five baseline configs)."""
     import loongserve_amd as lsa
@@ -726,6 +763,7 @@ def main():
     if args.only is None:
         line["workloads"] = workloads(max(3, min(args.steps, 10)))
         line["decode_latency"] = decode_latency()
+        line["decode_large_groups"] = decode_large_groups(max(5, min(args.steps, 10)))
     if args.all:
         line["other"] = other_steps(max(3, min(args.steps, 10)))
     print(json.dumps(line))
