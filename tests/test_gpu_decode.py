@@ -346,3 +346,48 @@ def test_one_request_of_a_million_tokens(lsa):
     o_ref = torch.einsum("hn,nhd->hd", torch.softmax(s.double(), dim=-1), kv[perm.long(), Hkv:].double()).float().repeat_interleave(Hq // Hkv, 0)
     assert_lse_close(lse2[0], lse_ref.cpu(), "peaked lse")
     assert_o_close(o2[0], o_ref.cpu(), "peaked o")
+
+
+@pytest.mark.parametrize("seed", [3, 11, 42])
+def test_random_decode_shapes_on_both_stage1_kernels(lsa, monkeypatch, seed):
+    """Seeded random sweep of stage 1 + stage 2 against the oracle, once with the library's own choice of stage-1 kernel
+    and once through the matrix-pipe kernel wherever its conditions hold: ragged batches with requests of a single token,
+    of exactly a block, and of a block plus one; groups of 1 to 20 query heads per KV head; blocks of 32 to 512 tokens;
+    per-block partials and merged groups of blocks; both dtypes; unused rows and requests in the table."""
+    import random
+    rng = random.Random(seed)
+    for case in range(10):
+        dtype = rng.choice([torch.float16, torch.bfloat16])
+        Hkv = rng.choice([1, 2, 3, 8])
+        group = rng.choice([1, 2, 4, 5, 7, 8, 9, 12, 16, 17, 20])
+        Hq = Hkv * group
+        BS = rng.choice([32, 64, 96, 128, 256, 512])
+        B = rng.choice([1, 2, 5, 9])
+        lens = [rng.choice([1, 2, 31, 32, 33, BS - 1, BS, BS + 1, 2 * BS, 3 * BS + 7, 700, 1500, 2600]) for _ in range(B)]
+        lens = [max(n, 1) for n in lens]
+        merge = rng.choice([1, 1, 2, 4, 16])
+        print("case", seed, case, dtype, Hq, Hkv, BS, lens, merge, flush=True)
+        D = 128
+        q, kv, table, b_req, b_len = decode_case(9000 + 100 * seed + case, B, Hq, Hkv, D, lens, sum(lens) + 200, dtype)
+        k, v = kv[:, :Hkv], kv[:, Hkv:]
+        o_ref, l_ref = orc.decode_full(q, k, v, table, b_req, b_len)
+        kvd, qd, td, rd, ld = kv.to(DEV), q.to(DEV), table.to(DEV), b_req.to(DEV), b_len.to(DEV)
+        nblk = (max(lens) + BS - 1) // BS
+        for forced in (False, True):
+            if forced:
+                monkeypatch.setenv("LSATTN_DECODE_MFMA", "1")
+            else:
+                monkeypatch.delenv("LSATTN_DECODE_MFMA", raising=False)
+            mo_d = torch.full((nblk, B, Hq, D), float("nan"), device=DEV)
+            ml_d = torch.full((nblk, B, Hq), float("nan"), device=DEV)
+            lsa.longserve_cuda_kernels.flash_decoding_stage1(mo_d, ml_d, qd, kvd[:, :Hkv], kvd[:, Hkv:], td, rd, ld, max(lens), BS, merge)
+            o_d = torch.empty(B, Hq, D, device=DEV)
+            l_d = torch.empty(B, Hq, device=DEV)
+            lsa.longserve_flash_decode_stage2(mo_d, ml_d, ld, o_d, l_d, BS)
+            torch.cuda.synchronize()
+            what = "seed %d case %d%s" % (seed, case, ", matrix pipe" if forced else "")
+            reach = torch.tensor([(n + BS - 1) // BS for n in lens])
+            untouched = (torch.arange(nblk)[:, None] >= reach[None, :])[:, :, None].expand(nblk, B, Hq)
+            assert torch.equal(torch.isnan(ml_d.cpu()), untouched), "rows written, " + what
+            assert_o_close(o_d, o_ref, "o, " + what)
+            assert_lse_close(l_d, l_ref, "lse, " + what)
