@@ -450,7 +450,7 @@ def workloads(steps):
         "value": e.bytes / (st["median_ms"] * 1e-3) / 1e9, "unit": "GB/s", "ms_per_step": st["median_ms"],
         "pct_of_hbm_peak": 100 * e.bytes / (st["median_ms"] * 1e-3) / 1e9 / PEAK_HBM_GBS, "algorithmic_gb_per_step": e.bytes / 1e9,
         "step_stats": st,
-        "roofline": _roof("decode_stage1_kernel<F16,1,4,false,true,1> (one instance: 4 x 131072 tokens x 32 KV heads)", "hbm",
+        "roofline": _roof("decode_stage1_mfma_kernel<F16> (one instance: 4 x 131072 tokens x 32 KV heads)", "hbm",
                           nbytes1 / (s1["median_ms"] * 1e-3) / 1e9, s1["median_ms"], "config4", algorithmic_gb_per_launch=nbytes1 / 1e9)}
     del e
     torch.cuda.empty_cache()
@@ -748,7 +748,7 @@ def main():
                                            "merged_blocks": {"what": "the same two calls with decoding.STAGE1_MERGES_BLOCKS = True (opt-in, "
                                                                      "not the reference's layout): one partial per group of blocks",
                                                              "ms_per_step": sepm["mean_ms"], "value": d.bytes / (sepm["mean_ms"] * 1e-3) / 1e9}}},
-            "roofline": _roof("decode_stage1_kernel<F16,4,4,false,true,1>", "hbm", ach, s1, "config3"),
+            "roofline": _roof("decode_stage1_mfma_kernel<F16>", "hbm", ach, s1, "config3"),
         }
         if not args.no_cpu:
             dec["cpu_baseline"] = d.cpu_baseline()

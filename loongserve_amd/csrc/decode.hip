@@ -372,9 +372,10 @@ __global__ __launch_bounds__(NW * 64) void decode_stage1_kernel(Stage1Params p) 
 }
 
 // ------------------------------------------------------------------------------------
-// Stage 1 for large GQA groups (five or more query heads per KV head, large launches): both products on the matrix pipe.
+// Stage 1 for large launches (any group size): both products on the matrix pipe.
 // One wave64 = one KV head, up to 16 query heads of its group (the 16 columns of a 16x16x32 MFMA) and a run of
-// consecutive blocks; the waves of a workgroup are independent (no barrier).  A batch is 32 tokens:
+// consecutive blocks; the waves of a workgroup are independent (no barrier) and take neighbouring KV heads over the same
+// tokens, whose rows lie side by side in memory.  A batch is 32 tokens:
 //   the K and V rows are loaded the way the other stage-1 kernels load them, a whole 256-byte row per 16 lanes (loading the
 //     MFMA operand layout straight from memory, 16 rows x 64 bytes per instruction, ran 20 % slower), double-buffered in
 //     registers so that the rows of batch j + 1 are in flight while batch j is computed;
@@ -420,7 +421,13 @@ __global__ __launch_bounds__(kMfmaWaves * 64, 2) void decode_stage1_mfma_kernel(
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int n = lane & 15, g = lane >> 4;  // query head (column) or 16-byte chunk of a row / token group or row of four
   const int64_t b = blockIdx.z;
-  const int task = blockIdx.y;
+  // The waves of a workgroup: tw of them on neighbouring tasks (KV heads: their rows of a token lie side by side in memory
+  // and are then fetched at about the same time), the rest on consecutive chunks of tokens.
+  const int tw = p.tasks_on_x & 7, cw = kMfmaWaves / tw;
+  const bool tasks_first = (p.tasks_on_x & 8) != 0;  // grid = (task groups, chunk groups, batch): a chunk's task groups are dispatched together
+  const unsigned bid_t = tasks_first ? blockIdx.x : blockIdx.y, bid_c = tasks_first ? blockIdx.y : blockIdx.x;
+  const int task = bid_t * tw + (wave & (tw - 1));
+  if (task >= p.tasks) return;
   const int group = (int)(p.hq / p.hkv);
   const int sub_groups = (group + 15) / 16;
   const int kvh = task / sub_groups;
@@ -434,8 +441,8 @@ __global__ __launch_bounds__(kMfmaWaves * 64, 2) void decode_stage1_mfma_kernel(
   if (nblk > (p.num_blocks + p.row_mul - 1) / p.row_mul) nblk = (p.num_blocks + p.row_mul - 1) / p.row_mul;
   int64_t fine_nblk = len <= 0 ? 0 : ((int64_t)len + p.fine_block_seq - 1) / p.fine_block_seq;
   if (fine_nblk > p.num_blocks) fine_nblk = p.num_blocks;
-  const unsigned n_chunks = gridDim.x * kMfmaWaves;
-  const unsigned chunk = (blockIdx.x * kMfmaWaves + wave + (unsigned)b) % n_chunks;  // (rotated by the request, as above)
+  const unsigned n_chunks = (tasks_first ? gridDim.y : gridDim.x) * cw;
+  const unsigned chunk = (bid_c * cw + (wave >> (tw == 4 ? 2 : tw == 2 ? 1 : 0)) + (unsigned)b) % n_chunks;  // (rotated by the request, as above)
   const int64_t blk_begin = (int64_t)chunk * p.blocks_per_wg;
   int64_t blk_end = blk_begin + p.blocks_per_wg;
   if (blk_end > nblk) blk_end = nblk;
@@ -804,7 +811,7 @@ static int launch_stage1(const lsattn_decode_stage1_args* a, hipStream_t st) {
   return check_launch();
 }
 
-// Large groups: the matrix-pipe kernel, when its conditions hold (blocks a multiple of 32 tokens, enough waves to fill
+// Large launches: the matrix-pipe kernel, when its conditions hold (blocks a multiple of 32 tokens, enough waves to fill
 // the chip); LSATTN_DECODE_MFMA = 0 / 1 in the environment forces the choice where the conditions allow it (tuning, tests).
 template <typename T> static int launch_stage1_mfma(const lsattn_decode_stage1_args* a, hipStream_t st, bool* taken) {
   *taken = false;
@@ -841,18 +848,26 @@ template <typename T> static int launch_stage1_mfma(const lsattn_decode_stage1_a
   if (nblk < 1) return LSATTN_OK;
   p.blocks_per_wg = (int32_t)per_wave;
   const int64_t chunks = (nblk + per_wave - 1) / per_wave;
-  const int64_t wgs_x = (chunks + kMfmaWaves - 1) / kMfmaWaves;
-  if (wgs_x > 0x7fffffff || a->batch > 65535 || p.tasks > 65535) return LSATTN_OK;
-  bool use = group >= 5 && chunks * p.tasks * a->batch >= 1024;
+  const int tw = p.tasks >= 4 ? 4 : p.tasks >= 2 ? 2 : 1, cw = kMfmaWaves / tw;
+  const int64_t wgs_x = (chunks + cw - 1) / cw, wgs_y = (p.tasks + tw - 1) / tw;
+  if (wgs_x > 0x7fffffff || a->batch > 65535 || wgs_y > 65535) return LSATTN_OK;
+  // Launches of enough waves to fill the chip (measured against the lane kernel, whose small-launch variant splits a
+  // block over the waves of a workgroup): from 512 waves for groups of five and more query heads on four or more KV
+  // heads, 1024 on fewer KV heads, 768 for smaller groups.
+  const int64_t min_waves = group >= 5 ? (p.tasks >= 4 ? 512 : 1024) : 768;
+  bool use = chunks * p.tasks * a->batch >= min_waves;
   if (const char* e = getenv("LSATTN_DECODE_MFMA")) {
     if (e[0] == '0' && !e[1]) use = false;
     if (e[0] == '1' && !e[1]) use = true;
   }
   if (!use) return LSATTN_OK;
   *taken = true;
-  p.tasks_on_x = 0;
-  hipLaunchKernelGGL((decode_stage1_mfma_kernel<T>), dim3((unsigned)wgs_x, (unsigned)p.tasks, (unsigned)a->batch), dim3(kMfmaWaves * 64), 0,
-                     st, p);
+  // The task groups of a chunk are dispatched one after the other (x runs fastest), so that all KV heads of a token are
+  // fetched at about the same time: config 3's shape 6.03 -> 6.17 TB/s, 32 KV heads 6.0 -> 6.5.
+  const bool tasks_first = wgs_y > 1 && wgs_x <= 65535;
+  p.tasks_on_x = tw | (tasks_first ? 8 : 0);  // (this kernel: waves of a workgroup on neighbouring tasks; the grid's order)
+  const dim3 grid = tasks_first ? dim3((unsigned)wgs_y, (unsigned)wgs_x, (unsigned)a->batch) : dim3((unsigned)wgs_x, (unsigned)wgs_y, (unsigned)a->batch);
+  hipLaunchKernelGGL((decode_stage1_mfma_kernel<T>), grid, dim3(kMfmaWaves * 64), 0, st, p);
   return check_launch();
 }
 
