@@ -83,6 +83,12 @@ typedef struct lsattn_prefill_args {
   float* m;           /* step_merge: [Tq,Hq] running max, log2 domain       */
   float* l;           /* step_merge: [Tq,Hq] running sum                    */
   int64_t ml_stride_t, ml_stride_h; /* strides of m and l (RING:274-275)     */
+  /* Optional (NULL: q_b_start_loc, the reference's layout): per sequence, the first row of o / lse / m / l that the
+   * sequence's results go to.  No counterpart in the reference: it lets one launch compute several partials of the same
+   * query rows over different slices of a long KV chunk (the sequence entered once per slice, with that slice's
+   * kv_b_start_loc / kv_b_seq_len / kv_first_token_global_idx and its own output rows), which lsattn_lse_merge then
+   * joins: short query chunks against long KV fill the chip that way.  Zero the struct before filling it in. */
+  const int32_t* o_b_start_loc;
 } lsattn_prefill_args;
 
 /* Partial of one step from the empty state: o = normalised fp32 output, lse = natural-log

@@ -34,6 +34,7 @@ class PrefillArgs(C.Structure):
         ("o_dtype", _i32), ("v_is_f16", _i32),
         ("lse", _vp), ("m", _vp), ("l", _vp),
         ("ml_stride_t", _i64), ("ml_stride_h", _i64),
+        ("o_b_start_loc", _vp),
     ]
 
 

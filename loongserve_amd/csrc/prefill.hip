@@ -63,6 +63,7 @@ struct PrefillParams {
   const int32_t* kv_start;
   const int32_t* kv_len;
   const int32_t* kv_first;
+  const int32_t* o_start;  // first output row per sequence (null: q_start)
   int32_t batch, hq, hkv, peers, nz, kv_slots, slices, units_per_slice, group;
   FastDiv d_peers, d_kv_slots, d_slices, d_units, d_group;
   float scale_log2;
@@ -246,8 +247,9 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
   // the way to the first tile load; a workgroup's start-up is what a short launch is made of).
   const int q_len = p.q_len[b], kv_len = p.kv_len[b], qf = p.q_first[b], kf = p.kv_first[b];
   const int q_start32 = p.q_start[b], kv_start32 = p.kv_start[b];
-  asm volatile("" ::"s"(q_len), "s"(kv_len), "s"(qf), "s"(kf), "s"(q_start32), "s"(kv_start32));
-  const int64_t q_start = q_start32, kv_start = kv_start32;
+  const int o_start32 = p.o_start ? p.o_start[b] : q_start32;
+  asm volatile("" ::"s"(q_len), "s"(kv_len), "s"(qf), "s"(kf), "s"(q_start32), "s"(kv_start32), "s"(o_start32));
+  const int64_t q_start = q_start32, kv_start = kv_start32, o_start = o_start32;
   const int vh = xcd + 8 * slot;  // (KV head, slice) pair: always < hkv * slices
   const int kvh = (int)div_by((uint32_t)vh, p.d_slices);
   const int u = up * p.slices + (vh - kvh * p.slices);
@@ -752,7 +754,7 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
 #pragma unroll
     for (int qb = 0; qb < 2; qb++) {
       const int m = m_w0 + 16 * qb + qc;
-      const int64_t tok = q_start + (m < q_len ? m : 0);
+      const int64_t tok = o_start + (m < q_len ? m : 0);
       if (MODE == 1) {
         st_a[qb] = p.m[tok * p.ml_st + (int64_t)h * p.ml_sh];
         st_b[qb] = p.l[tok * p.ml_st + (int64_t)h * p.ml_sh];
@@ -817,7 +819,7 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
         const int m = m_w0 + 16 * qb + qc;
         const float l_tot = column_sum(l_run[qb]);
         if (m < q_len) {
-          const int64_t tok = q_start + m;
+          const int64_t tok = o_start + m;
           const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
           float* orow = (float*)p.o + tok * p.o_st + (int64_t)h * p.o_sh;
 #pragma unroll
@@ -840,7 +842,7 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
           const int m = m_w0 + 16 * qb + qc;
           l_tot[i] = column_sum(l_run[qb]);
           in_range[i] = m < q_len;
-          const int64_t tok = q_start + (in_range[i] ? m : 0);
+          const int64_t tok = o_start + (in_range[i] ? m : 0);
           const uint16_t* orow = (const uint16_t*)p.o + tok * p.o_st + (int64_t)h * p.o_sh;
 #pragma unroll
           for (int d = 0; d < NDB; d++) old[i][d] = *(const u32x2*)(orow + (DB0 + d) * 16 + 4 * g);
@@ -851,7 +853,7 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
           const float m_old = st_a[qb], l_old = st_b[qb];
           const float M = fmaxf(m_run[qb], m_old);
           if (!in_range[i] || M == -INFINITY || !(l_tot[i] > 0.f)) continue;
-          const int64_t tok = q_start + m_w0 + 16 * qb + qc;
+          const int64_t tok = o_start + m_w0 + 16 * qb + qc;
           const float w_old = l_old * exp2_diff(m_old, M);
           const float w_new = exp2_diff(m_run[qb], M);
           const float L = w_old + l_tot[i] * w_new;
@@ -898,7 +900,7 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
           const int m = m_w0 + 16 * qb + qc;
           l_tot[i] = column_sum(l_run[qb]);
           live[i] = m < q_len && l_tot[i] > 0.f;
-          const int64_t tok = q_start + (m < q_len ? m : 0);
+          const int64_t tok = o_start + (m < q_len ? m : 0);
           const float* orow = (const float*)p.o + tok * p.o_st + (int64_t)h * p.o_sh;
 #pragma unroll
           for (int d = 0; d < NDB; d++) old[i][d] = *(const f32x4*)(orow + (DB0 + d) * 16 + 4 * g);
@@ -907,7 +909,7 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
         for (int i = 0; i < NB; i++) {
           if (!live[i]) continue;
           const int qb = qb0 + i;
-          const int64_t tok = q_start + m_w0 + 16 * qb + qc;
+          const int64_t tok = o_start + m_w0 + 16 * qb + qc;
           const float a_old = st_a[qb];
           const float a_new = m_run[qb] + __builtin_amdgcn_logf(l_tot[i]);
           const float top = fmaxf(a_old, a_new);
@@ -960,6 +962,7 @@ template <typename T, int MODE, bool DV, bool SPLIT> static int launch_prefill_r
   p.kv_start = a->kv_b_start_loc;
   p.kv_len = a->kv_b_seq_len;
   p.kv_first = a->kv_first_token_global_idx;
+  p.o_start = a->o_b_start_loc;
   p.batch = a->batch;
   p.hq = a->num_q_heads;
   p.hkv = a->num_kv_heads;

@@ -99,7 +99,7 @@ def _pad_head_dim(t: torch.Tensor) -> torch.Tensor:
 
 def _prefill_args(q, k, v, o, q_b_start_loc, q_b_seq_len, q_first, kv_b_start_loc, kv_b_seq_len, kv_first,
                   peers: int, max_q_len: int, sm_scale: Optional[float], v_f16: Optional[torch.Tensor] = None,
-                  v_f16_valid: bool = False) -> _lib.PrefillArgs:
+                  v_f16_valid: bool = False, o_b_start_loc: Optional[torch.Tensor] = None) -> _lib.PrefillArgs:
     for t, n in ((q, "q"), (k, "k"), (v, "v"), (o, "o")):
         _dev(t, n)
         if t.dim() != 3:
@@ -114,8 +114,10 @@ def _prefill_args(q, k, v, o, q_b_start_loc, q_b_seq_len, q_first, kv_b_start_lo
         raise ValueError("q, k, v must share dtype float16 or bfloat16")
     if k.shape[1] != v.shape[1] or q.shape[1] % k.shape[1] != 0:
         raise ValueError("bad head counts: Hq=%d Hkv=%d" % (q.shape[1], k.shape[1]))
-    if o.shape != q.shape:
+    if o_b_start_loc is None and o.shape != q.shape:
         raise ValueError("o must have the shape of q")
+    if o_b_start_loc is not None and o.shape[1:] != q.shape[1:]:
+        raise ValueError("o must have q's heads and head_dim")
     B = q_b_seq_len.shape[0]
     for t, n in ((q_b_start_loc, "q_b_start_loc"), (q_b_seq_len, "q_b_seq_len"), (q_first, "q_first_token_global_idx"),
                  (kv_b_start_loc, "kv_b_start_loc"), (kv_b_seq_len, "kv_b_seq_len"), (kv_first, "kv_first_token_global_idx")):
@@ -144,6 +146,9 @@ def _prefill_args(q, k, v, o, q_b_start_loc, q_b_seq_len, q_first, kv_b_start_lo
     a.o = o.data_ptr()
     a.o_stride_t, a.o_stride_h = o.stride(0), o.stride(1)
     a.o_dtype = _DT[o.dtype]
+    if o_b_start_loc is not None:
+        _i32vec(o_b_start_loc, "o_b_start_loc", B)
+        a.o_b_start_loc = o_b_start_loc.data_ptr()
     return a
 
 
@@ -188,15 +193,36 @@ def context_attention_fwd(q, k, v, o, q_b_start_loc, q_b_seq_len, q_first_token_
         o_user.copy_(o[..., :D])
 
 
+# Launches below this many 128-row workgroups (batch x query heads x ceil(max_q / 128)) are cut along the keys when the
+# KV buffer holds at least KV_SPLIT_MIN_KEYS rows: 256 CUs run one workgroup each.
+KV_SPLIT_BELOW_WORKGROUPS = 192
+KV_SPLIT_MIN_KEYS = 8192
+
+
+def kv_split_count(batch: int, num_q_heads: int, max_q_len: int, kv_rows: int) -> int:
+    """KV slices prefill_attention_step uses by itself: enough for about two workgroups per CU, slices of at least 2048
+    keys (kv_rows, the rows of the k buffer, bounds every sequence's chunk: the lengths themselves live on the device)."""
+    wgs = batch * num_q_heads * ((max_q_len + 127) // 128)
+    if wgs <= 0 or wgs >= KV_SPLIT_BELOW_WORKGROUPS or kv_rows < KV_SPLIT_MIN_KEYS:
+        return 1
+    return max(1, min(_lib.LSATTN_MAX_PARTS - 1, 512 // wgs, kv_rows // 2048))
+
+
 @torch.inference_mode()
 def prefill_attention_step(q, k, v, q_b_start_loc, q_b_seq_len, q_first_token_global_idx,
                            kv_b_start_loc, kv_b_seq_len, kv_first_token_global_idx,
                            logical_sp_peers_num: int, max_q_b_seq_len: int,
                            out: Optional[torch.Tensor] = None, lse: Optional[torch.Tensor] = None,
                            sm_scale: Optional[float] = None, accumulate: bool = False, v_f16: Optional[torch.Tensor] = None,
-                           v_f16_valid: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
+                           v_f16_valid: bool = False, kv_splits: Optional[int] = None,
+                           kv_split_workspace: Optional[Tuple[torch.Tensor, torch.Tensor]] = None) -> Tuple[torch.Tensor, torch.Tensor]:
     """One step as a mergeable partial: (O fp32 [Tq,Hq,D] normalised, LSE fp32 [Tq,Hq]).
     v_f16 / v_f16_valid: as in context_attention_fwd (the caller's buffer for the fp16 copy of a bfloat16 v).
+    kv_splits: short query chunks against a long KV chunk give the launch too few workgroups for the chip (one per 128
+    query rows and head); with kv_splits = S > 1 every sequence's KV chunk is cut into S slices, one launch computes the S
+    partials of every row (the sequence entered once per slice, lsattn_prefill_args.o_b_start_loc) and lsattn_lse_merge
+    joins them.  None chooses S from the shapes (kv_split_count), 1 switches it off.  The partials take S times the
+    size of (out, lse): kv_split_workspace = (float32 [S*Tq,Hq,D], float32 [S*Tq,Hq]) passes the caller's buffers for them.
 
     Same inputs as context_attention_fwd; rows that see no key get O = 0, LSE = -inf.
     With accumulate=True the step is LSE-merged into the (out, lse) passed in (a running partial of earlier steps over
@@ -219,6 +245,41 @@ def prefill_attention_step(q, k, v, q_b_start_loc, q_b_seq_len, q_first_token_gl
         q, k, v = _pad_head_dim(q), _pad_head_dim(k), _pad_head_dim(v)
         if sm_scale is None:
             sm_scale = 1.0 / (D ** 0.5)
+    S = kv_split_count(q_b_seq_len.shape[0], q.shape[1], int(max_q_b_seq_len), k.shape[0]) if kv_splits is None else int(kv_splits)
+    if S > 1:
+        if S + (1 if accumulate else 0) > _lib.LSATTN_MAX_PARTS:
+            raise ValueError("at most %d KV slices" % (_lib.LSATTN_MAX_PARTS - 1))
+        Tq, P = q.shape[0], int(logical_sp_peers_num)
+        L = -(-(-(-k.shape[0] // S)) // 64) * 64  # keys per slice: a multiple of the kernel's 64-key tile
+        if kv_split_workspace is None:
+            po = torch.empty((S * Tq,) + tuple(q.shape[1:]), dtype=torch.float32, device=q.device)
+            pl = torch.empty((S * Tq, q.shape[1]), dtype=torch.float32, device=q.device)
+        else:
+            po, pl = kv_split_workspace
+            if (po.dtype != torch.float32 or pl.dtype != torch.float32 or tuple(po.shape) != (S * Tq,) + tuple(q.shape[1:])
+                    or tuple(pl.shape) != (S * Tq, q.shape[1]) or not po.is_contiguous() or not pl.is_contiguous()):
+                raise ValueError("kv_split_workspace: contiguous float32 [S*Tq,Hq,D] and [S*Tq,Hq]")
+        # slice s of a sequence: keys [s L, (s+1) L) of its chunk; key n of the chunk has global position kv_first + n P
+        step = torch.arange(S, dtype=torch.int32, device=q.device)[:, None]
+        kv_start_x = (kv_b_start_loc[None, :] + step * L).reshape(-1)
+        kv_len_x = (kv_b_seq_len[None, :] - step * L).clamp_(0, L).reshape(-1)
+        kv_first_x = (kv_first_token_global_idx[None, :] + step * (L * P)).reshape(-1)
+        o_start_x = (q_b_start_loc[None, :] + step * Tq).reshape(-1)
+        a = _prefill_args(q, k, v, po, q_b_start_loc.repeat(S), q_b_seq_len.repeat(S), q_first_token_global_idx.repeat(S),
+                          kv_start_x, kv_len_x, kv_first_x, P, max_q_b_seq_len, sm_scale,
+                          v_f16 if out_user is None else None, v_f16_valid and out_user is None, o_b_start_loc=o_start_x)
+        a.lse = pl.data_ptr()
+        _lib.check(_lib.load().lsattn_prefill_step(C.byref(a), _stream()), "lsattn_prefill_step")
+        parts = [(po[s * Tq:(s + 1) * Tq], pl[s * Tq:(s + 1) * Tq]) for s in range(S)]
+        if accumulate:
+            parts.append((out, lse))  # (the merge reads a row of every part before it writes that row)
+        if not out.is_contiguous():
+            raise ValueError("kv_splits needs a contiguous out")
+        lse_merge(parts, out=out, lse=lse)
+        if out_user is not None:
+            out_user.copy_(out[..., :D])
+            out = out_user
+        return out, lse
     a = _prefill_args(q, k, v, out, q_b_start_loc, q_b_seq_len, q_first_token_global_idx, kv_b_start_loc,
                       kv_b_seq_len, kv_first_token_global_idx, logical_sp_peers_num, max_q_b_seq_len, sm_scale,
                       v_f16 if out_user is None else None, v_f16_valid and out_user is None)

@@ -182,3 +182,15 @@ def test_extension_module_resolves_by_its_reference_name():
     for name in ("flash_decoding_stage1", "flash_decoding_stage2", "rms_norm", "silu_and_mul_inplace", "rotary_emb", "ffn_block",
                  "hello_world"):
         assert getattr(m, name) is getattr(real, name)
+
+
+def test_kv_split_count_from_shapes():
+    """The split of a short-query step along the keys is chosen from shapes alone (no device read-back)."""
+    from loongserve_amd.ops import kv_split_count
+    assert kv_split_count(1, 32, 16384, 16384) == 1          # config 2: 4096 workgroups
+    assert kv_split_count(1, 32, 2048, 2048) == 1            # config 1: enough workgroups, few keys
+    assert kv_split_count(1, 32, 100, 131072) == 15          # one 100-row chunk against 131072 keys
+    assert kv_split_count(1, 8, 100, 20000) == 9             # slices of at least 2048 keys
+    assert kv_split_count(4, 32, 128, 100000) == 4           # 128 workgroups: four slices fill two rounds
+    assert kv_split_count(1, 32, 100, 4096) == 1             # short KV
+    assert kv_split_count(0, 32, 100, 100000) == 1

@@ -370,3 +370,44 @@ def test_peaked_softmax_keeps_the_bars(lsa, dtype, scale):
     o_ref, lse_ref = orc.attn_step(q, k, v, *m, *m, 1)
     assert_o_close(o, o_ref, "O")
     assert_lse_close(lse, lse_ref, "LSE")
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("P", [1, 3])
+def test_short_queries_against_long_kv_split_along_the_keys(lsa, dtype, P):
+    """kv_splits of prefill_attention_step: three sequences of 1 to 200 query rows against KV chunks of 0 to 20000 keys
+    (causal boundary inside the chunk, before it, and past its end), GQA 8/2: the slices' partials merged by the library
+    equal the unsplit step and the oracle; the library's own choice of the split; accumulate on top of a running partial;
+    the caller's workspace."""
+    from loongserve_amd import ops
+    Hq, Hkv, D = 8, 2, 128
+    qlens, klens = [200, 1, 77], [20000, 0, 9000]
+    qf = [19000 * P + 1, 5, 30000 * P]          # boundary inside the chunk / nothing to see / everything visible
+    kf = [0, 0, 2]
+    q = rand_t((sum(qlens), Hq, D), 4100 + P, dtype)
+    k = rand_t((sum(klens), Hkv, D), 4200 + P, dtype)
+    v = rand_t((sum(klens), Hkv, D), 4300 + P, dtype)
+    qm, km = meta(qlens, qf), meta(klens, kf)
+    o_ref, lse_ref = orc.attn_step(q, k, v, *qm, *km, P)
+    dq, dk, dv = q.to(DEV), k.to(DEV), v.to(DEV)
+    dqm, dkm = [t.to(DEV) for t in qm], [t.to(DEV) for t in km]
+    assert ops.kv_split_count(len(qlens), Hq, max(qlens), k.shape[0]) > 1
+    o1, l1 = lsa.prefill_attention_step(dq, dk, dv, *dqm, *dkm, P, max(qlens), kv_splits=1)
+    for S in (None, 2, 7, 15):
+        o, l = lsa.prefill_attention_step(dq, dk, dv, *dqm, *dkm, P, max(qlens), kv_splits=S)
+        torch.cuda.synchronize()
+        assert_o_close(o, o_ref, "O, %s slices" % S)
+        assert_lse_close(l, lse_ref, "LSE, %s slices" % S)
+        assert_o_close(o, o1.cpu(), "O against the unsplit step, %s slices" % S, max_abs=5e-4, rel=1e-3)
+    # accumulate: a running partial over other keys (here: the same chunk once more, so the merge of the two is the chunk's
+    # own result with LSE + ln 2), into the caller's workspace
+    S = 5
+    ws = (torch.empty((S * q.shape[0], Hq, D), device=DEV), torch.empty((S * q.shape[0], Hq), device=DEV))
+    o_run, l_run = o1.clone(), l1.clone()
+    lsa.prefill_attention_step(dq, dk, dv, *dqm, *dkm, P, max(qlens), out=o_run, lse=l_run, accumulate=True, kv_splits=S,
+                               kv_split_workspace=ws)
+    torch.cuda.synchronize()
+    assert_o_close(o_run, o_ref, "O, accumulated")
+    seen = torch.isfinite(lse_ref)
+    assert_lse_close(l_run.cpu()[seen], lse_ref[seen] + math.log(2.0), "LSE, accumulated")
+    assert bool((l_run.cpu()[~seen] == float("-inf")).all())
