@@ -512,9 +512,10 @@ __global__ __launch_bounds__(kMfmaWaves * 64, 2) void decode_stage1_mfma_kernel(
                    : "=v"(vr[i]), "=&v"(addr) : "v"(sl.v[i]), "s"(vrb), "v"(vbase) : "vcc", "memory");
     }
   };
-  // waits until at most 16 loads (the next batch's rows) are outstanding and makes kr / vr usable
+  // waits until at most 24 loads (the slot numbers requested last and the next batch's rows) are outstanding and makes
+  // kr / vr usable
   auto wait_rows = [&](u32x4 (&kr)[8], u32x4 (&vr)[8]) __attribute__((always_inline)) {
-    asm volatile("s_waitcnt vmcnt(16)"
+    asm volatile("s_waitcnt vmcnt(24)"
                  : "+v"(kr[0]), "+v"(kr[1]), "+v"(kr[2]), "+v"(kr[3]), "+v"(kr[4]), "+v"(kr[5]), "+v"(kr[6]), "+v"(kr[7]), "+v"(vr[0]),
                    "+v"(vr[1]), "+v"(vr[2]), "+v"(vr[3]), "+v"(vr[4]), "+v"(vr[5]), "+v"(vr[6]), "+v"(vr[7])
                  :
@@ -624,9 +625,10 @@ __global__ __launch_bounds__(kMfmaWaves * 64, 2) void decode_stage1_mfma_kernel(
     }
   };
 
-  // Order of the loads, oldest first, when batch j is about to be computed:  rows(j) | slots(j+2) | rows(j+1).  The wait for
-  // vmcnt(16) then leaves exactly rows(j+1) in flight; slots(j+1), which rows(j+1) were addressed with, were complete one
-  // wait earlier (the vmcnt(24) in front of an issue is a no-op except in the first trip).
+  // Order of the loads, oldest first, when batch j is about to be computed:  rows(j) | slots(j+2) | rows(j+1).  Loads return
+  // in order, so the wait for vmcnt(24) ends when rows(j) have landed and leaves the other two groups in flight (a partial's
+  // stores in between count too and only make a wait longer); slots(j+1), which rows(j+1) were addressed with, were the
+  // oldest group one wait earlier (that vmcnt(24), in front of an issue, is a no-op except in the first trip).
   u32x4 kr0[8], vr0[8], kr1[8], vr1[8];
   Slots s_even, s_odd;
   load_slots(t_begin, s_even);
