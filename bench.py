@@ -32,14 +32,14 @@ if ROOT not in sys.path:
 # which is regenerated with the kernels (the JSON line says so in "traffic_source").
 TRAFFIC_SOURCE = "profiles/bench_default_hbm_traffic.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this command, scaled by a 1 GiB copy); a constant of bench.py, not measured in this run"
 TRAFFIC_BYTES = {
-    "config2": 1294.9e6,    # per launch, averaged over the four launches of a ring step (one diagonal + three full)
-    "config3": 5203.1e6,    # stage 1 of the fused call
-    "config1": 108.7e6,
-    "config4": 8618.7e6,    # stage 1 over one instance's 4 x 131072 tokens
-    "config5": 106013e6,    # the attention launch
+    "config2": 1307.0e6,    # per launch, averaged over the four launches of a ring step (one diagonal + three full)
+    "config3": 5203.0e6,    # stage 1 of the fused call
+    "config1": 108.8e6,
+    "config4": 8618.5e6,    # stage 1 over one instance's 4 x 131072 tokens
+    "config5": 111159e6,    # the attention launch (K/V re-fetched from HBM about 25 times: 106-111 GB from run to run)
     "decode_8_1": 656.8e6,  # stage 1 of the large-group cases
     "decode_16_2": 1308.9e6,
-    "decode_64_8": 5222.5e6,
+    "decode_64_8": 5222.4e6,
 }
 PEAK_MFMA_TFLOPS = 2500.0  # dense fp16/bf16 MFMA, MI355X
 PEAK_HBM_GBS = 8000.0
