@@ -411,3 +411,23 @@ def test_short_queries_against_long_kv_split_along_the_keys(lsa, dtype, P):
     seen = torch.isfinite(lse_ref)
     assert_lse_close(l_run.cpu()[seen], lse_ref[seen] + math.log(2.0), "LSE, accumulated")
     assert bool((l_run.cpu()[~seen] == float("-inf")).all())
+
+
+@pytest.mark.parametrize("Hq,Hkv", [(3, 3), (12, 6), (24, 12), (40, 40), (35, 5), (21, 7), (18, 2), (9, 1)])
+@pytest.mark.parametrize("P", [5, 7, 13, 64])
+def test_launch_geometry_with_divisors_that_are_not_powers_of_two(lsa, Hq, Hkv, P):
+    """The kernel derives a workgroup's (sequence, KV head, query head, query tile) and every row's visible keys with
+    multiply-high divisions by launch constants (sp_peers, query heads per KV head, KV heads per XCD slot, slices, units per
+    slice): head counts and stripe widths that make every one of those divisors a non-power of two, two ragged sequences."""
+    D = 128
+    qlens, klens = [300, 129], [257, 700]
+    qf, kf = [3 * P + 2, 0], [1, 4]                  # striped positions: row m of q at qf + m P, key n at kf + n P
+    q = rand_t((sum(qlens), Hq, D), 5100 + Hq + P, torch.float16)
+    k = rand_t((sum(klens), Hkv, D), 5200 + Hq + P, torch.float16)
+    v = rand_t((sum(klens), Hkv, D), 5300 + Hq + P, torch.float16)
+    qm, km = meta(qlens, qf), meta(klens, kf)
+    o_ref, lse_ref = orc.attn_step(q, k, v, *qm, *km, P)
+    o, lse = lsa.prefill_attention_step(q.to(DEV), k.to(DEV), v.to(DEV), *[t.to(DEV) for t in qm], *[t.to(DEV) for t in km], P, max(qlens))
+    torch.cuda.synchronize()
+    assert_o_close(o, o_ref, "O")
+    assert_lse_close(lse, lse_ref, "LSE")
