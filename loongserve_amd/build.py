@@ -56,5 +56,23 @@ def build_all(verbose: bool = False, extra_flags=(), out: str = LIB_PATH) -> str
     return out
 
 
+C_ABI_EXAMPLE_SRC = os.path.join(ROOT, "tests", "c_abi", "decode_from_c.cpp")
+C_ABI_EXAMPLE_BIN = os.path.join(ROOT, "tests", "c_abi", "decode_from_c")
+
+
+def build_c_abi_example(verbose: bool = False) -> str:
+    """The C ABI's consumer without Python or PyTorch (tests/c_abi/decode_from_c.cpp), linked against the in-tree library
+    and finding it relative to its own place; tests/test_gpu_c_abi.py runs it."""
+    cmd = [HIPCC, "--offload-arch=gfx950", "-O2", "-std=c++17", "-I" + os.path.join(ROOT, "include"), C_ABI_EXAMPLE_SRC,
+           "-L" + PKG_DIR, "-llsattn", "-Wl,-rpath,$ORIGIN/../../loongserve_amd", "-o", C_ABI_EXAMPLE_BIN]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("hipcc failed for the C ABI example:\n%s\n%s" % (" ".join(cmd), r.stderr[-6000:]))
+    if verbose:
+        print("built", C_ABI_EXAMPLE_BIN)
+    return C_ABI_EXAMPLE_BIN
+
+
 if __name__ == "__main__":
     build_all(verbose=True, extra_flags=sys.argv[1:])
+    build_c_abi_example(verbose=True)
