@@ -56,21 +56,21 @@ def build_all(verbose: bool = False, extra_flags=(), out: str = LIB_PATH) -> str
     return out
 
 
-C_ABI_EXAMPLE_SRC = os.path.join(ROOT, "tests", "c_abi", "decode_from_c.cpp")
-C_ABI_EXAMPLE_BIN = os.path.join(ROOT, "tests", "c_abi", "decode_from_c")
+C_ABI_EXAMPLES = [os.path.join(ROOT, "tests", "c_abi", n) for n in ("decode_from_c", "prefill_from_c")]
 
 
-def build_c_abi_example(verbose: bool = False) -> str:
-    """The C ABI's consumer without Python or PyTorch (tests/c_abi/decode_from_c.cpp), linked against the in-tree library
-    and finding it relative to its own place; tests/test_gpu_c_abi.py runs it."""
-    cmd = [HIPCC, "--offload-arch=gfx950", "-O2", "-std=c++17", "-I" + os.path.join(ROOT, "include"), C_ABI_EXAMPLE_SRC,
-           "-L" + PKG_DIR, "-llsattn", "-Wl,-rpath,$ORIGIN/../../loongserve_amd", "-o", C_ABI_EXAMPLE_BIN]
-    r = subprocess.run(cmd, capture_output=True, text=True)
-    if r.returncode != 0:
-        raise RuntimeError("hipcc failed for the C ABI example:\n%s\n%s" % (" ".join(cmd), r.stderr[-6000:]))
-    if verbose:
-        print("built", C_ABI_EXAMPLE_BIN)
-    return C_ABI_EXAMPLE_BIN
+def build_c_abi_example(verbose: bool = False):
+    """The C ABI's consumers without Python or PyTorch (tests/c_abi/*.cpp), linked against the in-tree library and
+    finding it relative to their own place; tests/test_gpu_c_abi.py runs them."""
+    for out in C_ABI_EXAMPLES:
+        cmd = [HIPCC, "--offload-arch=gfx950", "-O2", "-std=c++17", "-I" + os.path.join(ROOT, "include"), out + ".cpp",
+               "-L" + PKG_DIR, "-llsattn", "-Wl,-rpath,$ORIGIN/../../loongserve_amd", "-o", out]
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError("hipcc failed for the C ABI example:\n%s\n%s" % (" ".join(cmd), r.stderr[-6000:]))
+        if verbose:
+            print("built", out)
+    return C_ABI_EXAMPLES
 
 
 if __name__ == "__main__":
