@@ -491,15 +491,16 @@ def workloads(steps):
 
 
 def decode_latency():
-    """Small-batch decode: the host's cost of a call against the device's.  GQA 32/8, head_dim 128, fp16, scattered slots,
+    """Small-batch decode: the host's cost of a call against the device's.  GQA 32/8 (and 8/1: Llama-3-70B's heads per GPU
+    under 8-way tensor parallelism), head_dim 128, fp16, scattered slots,
     fused stage 1 + stage 2 call (the operator a decode step of the layer makes, longserve_transformer_layer_infer.py:293-308).
     eager_us: wall clock per call over 200 back-to-back calls and one synchronize (host-bound when the host is slower
     than the kernels); graph_us: the same call replayed from a HIP graph of 20 of them, per call (device time)."""
     import loongserve_amd as lsa
     rows = []
-    for B in (1, 4, 16):
-        for ctx in (2048, 8192, 32768):
-            d = TokenDecode(B=B, lens=[ctx] * B, pool=B * ctx + 1024, seed=3100 + B)
+    for Hq, Hkv, B, ctx in [(32, 8, B, ctx) for B in (1, 4, 16) for ctx in (2048, 8192, 32768)] + [(8, 1, 1, 8192), (8, 1, 8, 8192), (8, 1, 16, 32768)]:
+        if True:
+            d = TokenDecode(B=B, Hq=Hq, Hkv=Hkv, lens=[ctx] * B, pool=B * ctx + 1024, seed=3100 + B)
             for _ in range(5):
                 d.step()
             torch.cuda.synchronize()
@@ -510,7 +511,7 @@ def decode_latency():
             torch.cuda.synchronize()
             eager = (time.perf_counter() - t0) / n * 1e6
             graph = _time_graph(d.step, launches=20, reps=10) * 1e3
-            rows.append({"batch": B, "ctx": ctx, "eager_us": round(eager, 2), "graph_us": round(graph, 2),
+            rows.append({"q_heads": Hq, "kv_heads": Hkv, "batch": B, "ctx": ctx, "eager_us": round(eager, 2), "graph_us": round(graph, 2),
                          "kv_gbs_at_graph_rate": round(d.bytes / (graph * 1e-6) / 1e9, 1)})
             del d
     torch.cuda.empty_cache()

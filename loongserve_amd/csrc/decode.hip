@@ -414,7 +414,9 @@ constexpr int kMfmaBatch = 32;       // tokens per batch
 constexpr int kMfmaKRow = 272, kMfmaVRow = 288;  // padded row lengths in LDS (bytes)
 constexpr int kMfmaStage = kMfmaBatch * (kMfmaKRow + kMfmaVRow);  // LDS bytes per wave: the K rows and the V rows of one batch
 
-template <typename T>
+// WS (small launches with fewer than four tasks): the four waves of a workgroup share one task and one block, take every
+// fourth batch of its tokens and merge their partials through LDS: four times the waves of the plain shape, each short.
+template <typename T, bool WS>
 __global__ __launch_bounds__(kMfmaWaves * 64, 2) void decode_stage1_mfma_kernel(Stage1Params p) {
   __shared__ __attribute__((aligned(1024))) char lds[kMfmaWaves * kMfmaStage];
   const int lane = threadIdx.x & 63;
@@ -423,10 +425,10 @@ __global__ __launch_bounds__(kMfmaWaves * 64, 2) void decode_stage1_mfma_kernel(
   const int64_t b = blockIdx.z;
   // The waves of a workgroup: tw of them on neighbouring tasks (KV heads: their rows of a token lie side by side in memory
   // and are then fetched at about the same time), the rest on consecutive chunks of tokens.
-  const int tw = p.tasks_on_x & 7, cw = kMfmaWaves / tw;
-  const bool tasks_first = (p.tasks_on_x & 8) != 0;  // grid = (task groups, chunk groups, batch): a chunk's task groups are dispatched together
+  const int tw = WS ? 1 : (p.tasks_on_x & 7), cw = WS ? 1 : kMfmaWaves / tw;
+  const bool tasks_first = !WS && (p.tasks_on_x & 8) != 0;  // grid = (task groups, chunk groups, batch): a chunk's task groups are dispatched together
   const unsigned bid_t = tasks_first ? blockIdx.x : blockIdx.y, bid_c = tasks_first ? blockIdx.y : blockIdx.x;
-  const int task = bid_t * tw + (wave & (tw - 1));
+  const int task = WS ? (int)bid_t : bid_t * tw + (wave & (tw - 1));
   if (task >= p.tasks) return;
   const int group = (int)(p.hq / p.hkv);
   const int sub_groups = (group + 15) / 16;
@@ -442,16 +444,17 @@ __global__ __launch_bounds__(kMfmaWaves * 64, 2) void decode_stage1_mfma_kernel(
   int64_t fine_nblk = len <= 0 ? 0 : ((int64_t)len + p.fine_block_seq - 1) / p.fine_block_seq;
   if (fine_nblk > p.num_blocks) fine_nblk = p.num_blocks;
   const unsigned n_chunks = (tasks_first ? gridDim.y : gridDim.x) * cw;
-  const unsigned chunk = (bid_c * cw + (wave >> (tw == 4 ? 2 : tw == 2 ? 1 : 0)) + (unsigned)b) % n_chunks;  // (rotated by the request, as above)
-  const int64_t blk_begin = (int64_t)chunk * p.blocks_per_wg;
+  const unsigned chunk = (bid_c * cw + (WS ? 0 : wave >> (tw == 4 ? 2 : tw == 2 ? 1 : 0)) + (unsigned)b) % n_chunks;  // (rotated by the request, as above)
+  const int64_t blk_begin = (int64_t)chunk * p.blocks_per_wg;  // (WS: one block per workgroup)
   int64_t blk_end = blk_begin + p.blocks_per_wg;
   if (blk_end > nblk) blk_end = nblk;
-  if (blk_begin >= blk_end) return;
+  if (blk_begin >= blk_end) return;  // (WS: the same for the four waves, which meet at a barrier below)
   const int bs = (int)p.block_seq;                    // a multiple of 32 (checked on the host)
-  const int t_begin = (int)(blk_begin * bs);
+  constexpr int kStep = WS ? kMfmaWaves * kMfmaBatch : kMfmaBatch;  // tokens from one of the wave's batches to its next
+  const int t_begin = (int)(blk_begin * bs) + (WS ? wave * kMfmaBatch : 0);
   const int t_end = blk_end * bs > len ? len : (int)(blk_end * bs);
   const int t_last = t_end - 1;
-  const int n_batches = (t_end - t_begin + kMfmaBatch - 1) / kMfmaBatch;
+  const int n_batches = t_begin < t_end ? (t_end - t_begin + kStep - 1) / kStep : 0;
 
   const int32_t* table = p.req_to_tokens + (int64_t)p.b_req_idx[b] * p.max_seq_len;
   const char* kbase = (const char*)p.k + ((int64_t)kvh * p.k_s1) * 2 + n * 16;
@@ -619,6 +622,7 @@ __global__ __launch_bounds__(kMfmaWaves * 64, 2) void decode_stage1_mfma_kernel(
     }
   };
   auto finish_batch = [&](int t0) __attribute__((always_inline)) {
+    if (WS) return;  // (the block's partial is merged from the four waves after the loop)
     if ((t0 + kMfmaBatch - t_begin) % bs == 0 || t0 + kMfmaBatch >= t_end) {
       flush(blk_begin + (t0 - t_begin) / bs);
       reset();
@@ -632,28 +636,72 @@ __global__ __launch_bounds__(kMfmaWaves * 64, 2) void decode_stage1_mfma_kernel(
   u32x4 kr0[8], vr0[8], kr1[8], vr1[8];
   Slots s_even, s_odd;
   load_slots(t_begin, s_even);
-  load_slots(t_begin + kMfmaBatch, s_odd);
+  load_slots(t_begin + kStep, s_odd);
   wait_slots(std::integral_constant<int, 8>{}, s_even);
   issue(s_even, kr0, vr0);
   // two batches per trip, so that the register set of a batch is a compile-time choice
   for (int j = 0; j < n_batches; j += 2) {
-    const int t0 = t_begin + j * kMfmaBatch;
-    load_slots(t0 + 2 * kMfmaBatch, s_even);                // slots(j+2): rows(j) have been addressed
+    const int t0 = t_begin + j * kStep;
+    load_slots(t0 + 2 * kStep, s_even);                     // slots(j+2): rows(j) have been addressed
     wait_slots(std::integral_constant<int, 24>{}, s_odd);   // slots(j+1) usable
     issue(s_odd, kr1, vr1);                                 // rows(j+1) (past the end: the last row again, never used)
     wait_rows(kr0, vr0);
     compute(t0, kr0, vr0);
     finish_batch(t0);
-    load_slots(t0 + 3 * kMfmaBatch, s_odd);                 // slots(j+3)
+    load_slots(t0 + 3 * kStep, s_odd);                      // slots(j+3)
     wait_slots(std::integral_constant<int, 24>{}, s_even);  // slots(j+2) usable
     issue(s_even, kr0, vr0);                                // rows(j+2)
     wait_rows(kr1, vr1);
     if (j + 1 < n_batches) {
-      compute(t0 + kMfmaBatch, kr1, vr1);
-      finish_batch(t0 + kMfmaBatch);
+      compute(t0 + kStep, kr1, vr1);
+      finish_batch(t0 + kStep);
     }
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // (rows requested past the end land before the registers are given back)
+  if constexpr (WS) {
+    // The four partials of the block meet in LDS (each wave's own 17.5 KB: its last batch's operands have been consumed);
+    // every wave then finishes two of the eight d-blocks.  A wave without a batch of its own brings m = -inf, l = 0.
+    float lt = l + xlane16(l);
+    lt += xlane32(lt);
+    f32x4* mine = (f32x4*)(lds + wave * kMfmaStage);
+#pragma unroll
+    for (int db = 0; db < 8; db++) mine[db * 64 + lane] = oacc[db];
+    typedef float f32x2 __attribute__((ext_vector_type(2)));
+    *(f32x2*)(lds + wave * kMfmaStage + 8192 + lane * 8) = f32x2{m, lt};
+    __syncthreads();
+    float mi[kMfmaWaves], li[kMfmaWaves], M = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < kMfmaWaves; w++) {
+      const f32x2 ml = *(const f32x2*)(lds + w * kMfmaStage + 8192 + lane * 8);
+      mi[w] = ml[0];
+      li[w] = ml[1];
+      M = fmaxf(M, mi[w]);
+    }
+    float L = 0.f;
+#pragma unroll
+    for (int w = 0; w < kMfmaWaves; w++) {
+      mi[w] = exp2_diff(mi[w], M);  // (the weight of wave w's partial; 0 for one that saw no token)
+      L += li[w] * mi[w];
+    }
+    if (n < nh) {
+      const float inv = 1.f / L;  // a block holds at least one token
+      const int64_t row = (blk_begin * p.row_mul * p.batch + b) * p.hq + qh0 + n;
+      float* dst = p.mid_o + row * 128 + 4 * g;
+#pragma unroll
+      for (int d = 0; d < 2; d++) {
+        const int db = 2 * wave + d;
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int w = 0; w < kMfmaWaves; w++) acc += ((const f32x4*)(lds + w * kMfmaStage))[db * 64 + lane] * mi[w];
+        *(f32x4*)(dst + 16 * db) = acc * inv;
+      }
+      if (wave == 0) {
+        if (g == 0) p.mid_lse[row] = (M + __builtin_amdgcn_logf(L)) * kLn2;
+        for (int r = 1 + g; r < p.row_mul; r += 4)
+          if (blk_begin * p.row_mul + r < fine_nblk) p.mid_lse[((blk_begin * p.row_mul + r) * p.batch + b) * p.hq + qh0 + n] = -INFINITY;
+      }
+    }
+  }
 }
 
 // ------------------------------------------------------------------------------------
@@ -853,14 +901,27 @@ template <typename T> static int launch_stage1_mfma(const lsattn_decode_stage1_a
   const int tw = p.tasks >= 4 ? 4 : p.tasks >= 2 ? 2 : 1, cw = kMfmaWaves / tw;
   const int64_t wgs_x = (chunks + cw - 1) / cw, wgs_y = (p.tasks + tw - 1) / tw;
   if (wgs_x > 0x7fffffff || a->batch > 65535 || wgs_y > 65535) return LSATTN_OK;
-  // Launches of enough waves to fill the chip (measured against the lane kernel, whose small-launch variant splits a
-  // block over the waves of a workgroup): from 512 waves for groups of five and more query heads on four or more KV
-  // heads, 1024 on fewer KV heads, 768 for smaller groups.
-  const int64_t min_waves = group >= 5 ? (p.tasks >= 4 ? 512 : 1024) : 768;
-  bool use = chunks * p.tasks * a->batch >= min_waves;
-  if (const char* e = getenv("LSATTN_DECODE_MFMA")) {
-    if (e[0] == '0' && !e[1]) use = false;
-    if (e[0] == '1' && !e[1]) use = true;
+  // Which shape, by the launch's size in waves of the plain shape (256 tokens x task x request; measured):
+  //   groups of four and more query heads per KV head: up to 512 waves (3072 on fewer than four KV heads, where the plain
+  //     shape has no neighbouring heads to put side by side) the shape whose four waves split a block (a launch of 8 to 512
+  //     plain waves runs 30-45 % shorter with it than with either other kernel), above that the plain shape;
+  //   smaller groups (most of an MFMA's sixteen columns idle): the plain shape from 768 waves, below that the lane kernel.
+  const int64_t waves = chunks * p.tasks * a->batch;
+  const bool can_split = p.block_seq % (kMfmaWaves * kMfmaBatch) == 0 && nblk <= 0x7fffffff;
+  bool split_waves = group >= 4 && can_split && waves <= (p.tasks < 4 ? 3072 : 512);
+  bool use = !split_waves && waves >= (group >= 4 ? 513 : 768);
+  if (const char* e = getenv("LSATTN_DECODE_MFMA")) {  // 0: the lane kernel, 1: the plain shape, 2: the split shape
+    if (e[0] == '0' && !e[1]) use = split_waves = false;
+    if (e[0] == '1' && !e[1]) use = true, split_waves = false;
+    if (e[0] == '2' && !e[1] && can_split) use = false, split_waves = true;
+  }
+  if (split_waves) {
+    *taken = true;
+    p.blocks_per_wg = 1;
+    p.tasks_on_x = 1;
+    hipLaunchKernelGGL((decode_stage1_mfma_kernel<T, true>), dim3((unsigned)nblk, (unsigned)p.tasks, (unsigned)a->batch), dim3(kMfmaWaves * 64),
+                       0, st, p);
+    return check_launch();
   }
   if (!use) return LSATTN_OK;
   *taken = true;
@@ -869,7 +930,7 @@ template <typename T> static int launch_stage1_mfma(const lsattn_decode_stage1_a
   const bool tasks_first = wgs_y > 1 && wgs_x <= 65535;
   p.tasks_on_x = tw | (tasks_first ? 8 : 0);  // (this kernel: waves of a workgroup on neighbouring tasks; the grid's order)
   const dim3 grid = tasks_first ? dim3((unsigned)wgs_y, (unsigned)wgs_x, (unsigned)a->batch) : dim3((unsigned)wgs_x, (unsigned)wgs_y, (unsigned)a->batch);
-  hipLaunchKernelGGL((decode_stage1_mfma_kernel<T>), grid, dim3(kMfmaWaves * 64), 0, st, p);
+  hipLaunchKernelGGL((decode_stage1_mfma_kernel<T, false>), grid, dim3(kMfmaWaves * 64), 0, st, p);
   return check_launch();
 }
 

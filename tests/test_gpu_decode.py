@@ -130,12 +130,12 @@ def _check_merge_blocks(lsa, dtype, merge, Hq, Hkv, BS, lens):
     assert_lse_close(l_d, l_ref, "lse")
 
 
-@pytest.fixture
-def matrix_pipe(monkeypatch):
-    """Stage 1 through the matrix-pipe kernel wherever its conditions hold (blocks a multiple of 32 tokens), whatever the
-    launch's size: by itself the library takes it for groups of five or more query heads per KV head in launches of
-    1024 waves or more."""
-    monkeypatch.setenv("LSATTN_DECODE_MFMA", "1")
+@pytest.fixture(params=["1", "2"], ids=["plain", "split"])
+def matrix_pipe(monkeypatch, request):
+    """Stage 1 through the matrix-pipe kernel wherever its conditions hold, whatever the launch's size: its plain shape
+    (a wave per 256 tokens; blocks a multiple of 32 tokens; by itself the library takes it for large launches) and the
+    shape whose four waves split a block (blocks a multiple of 128 tokens; small launches of groups of four and more)."""
+    monkeypatch.setenv("LSATTN_DECODE_MFMA", request.param)
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
@@ -361,7 +361,7 @@ def test_random_decode_shapes_on_both_stage1_kernels(lsa, monkeypatch, seed):
         Hkv = rng.choice([1, 2, 3, 8])
         group = rng.choice([1, 2, 4, 5, 7, 8, 9, 12, 16, 17, 20])
         Hq = Hkv * group
-        BS = rng.choice([32, 64, 96, 128, 256, 512])
+        BS = rng.choice([32, 64, 96, 128, 256, 384, 512])
         B = rng.choice([1, 2, 5, 9])
         lens = [rng.choice([1, 2, 31, 32, 33, BS - 1, BS, BS + 1, 2 * BS, 3 * BS + 7, 700, 1500, 2600]) for _ in range(B)]
         lens = [max(n, 1) for n in lens]
@@ -373,9 +373,9 @@ def test_random_decode_shapes_on_both_stage1_kernels(lsa, monkeypatch, seed):
         o_ref, l_ref = orc.decode_full(q, k, v, table, b_req, b_len)
         kvd, qd, td, rd, ld = kv.to(DEV), q.to(DEV), table.to(DEV), b_req.to(DEV), b_len.to(DEV)
         nblk = (max(lens) + BS - 1) // BS
-        for forced in (False, True):
+        for forced in (False, "1", "2"):
             if forced:
-                monkeypatch.setenv("LSATTN_DECODE_MFMA", "1")
+                monkeypatch.setenv("LSATTN_DECODE_MFMA", forced)
             else:
                 monkeypatch.delenv("LSATTN_DECODE_MFMA", raising=False)
             mo_d = torch.full((nblk, B, Hq, D), float("nan"), device=DEV)
@@ -385,7 +385,7 @@ def test_random_decode_shapes_on_both_stage1_kernels(lsa, monkeypatch, seed):
             l_d = torch.empty(B, Hq, device=DEV)
             lsa.longserve_flash_decode_stage2(mo_d, ml_d, ld, o_d, l_d, BS)
             torch.cuda.synchronize()
-            what = "seed %d case %d%s" % (seed, case, ", matrix pipe" if forced else "")
+            what = "seed %d case %d%s" % (seed, case, ", matrix pipe shape " + forced if forced else "")
             reach = torch.tensor([(n + BS - 1) // BS for n in lens])
             untouched = (torch.arange(nblk)[:, None] >= reach[None, :])[:, :, None].expand(nblk, B, Hq)
             assert torch.equal(torch.isnan(ml_d.cpu()), untouched), "rows written, " + what
