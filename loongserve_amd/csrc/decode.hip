@@ -666,6 +666,8 @@ __global__ __launch_bounds__(kMfmaWaves * 64, 2) void decode_stage1_mfma_kernel(
     f32x4* mine = (f32x4*)(lds + wave * kMfmaStage);
 #pragma unroll
     for (int db = 0; db < 8; db++) mine[db * 64 + lane] = oacc[db];
+    // (as a float vector: __builtin_bit_cast applied to an element of an integer vector, bit_cast(float, v[1]), compiled to a
+    // read of element 0 with this compiler)
     typedef float f32x2 __attribute__((ext_vector_type(2)));
     *(f32x2*)(lds + wave * kMfmaStage + 8192 + lane * 8) = f32x2{m, lt};
     __syncthreads();
