@@ -32,12 +32,12 @@ if ROOT not in sys.path:
 # which is regenerated with the kernels (the JSON line says so in "traffic_source").
 TRAFFIC_SOURCE = "profiles/bench_default_hbm_traffic.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this command, scaled by a 1 GiB copy); a constant of bench.py, not measured in this run"
 TRAFFIC_BYTES = {
-    "config2": 1307.0e6,    # per launch, averaged over the four launches of a ring step (one diagonal + three full)
+    "config2": 1306.8e6,    # per launch, averaged over the four launches of a ring step (one diagonal + three full)
     "config3": 5203.0e6,    # stage 1 of the fused call
-    "config1": 108.8e6,
-    "config4": 8618.5e6,    # stage 1 over one instance's 4 x 131072 tokens
-    "config5": 111159e6,    # the attention launch (K/V re-fetched from HBM about 25 times: 106-111 GB from run to run)
-    "decode_8_1": 656.8e6,  # stage 1 of the large-group cases
+    "config1": 108.7e6,
+    "config4": 8618.6e6,    # stage 1 over one instance's 4 x 131072 tokens
+    "config5": 106677e6,    # the attention launch (K/V re-fetched from HBM about 25 times: 106-111 GB from run to run)
+    "decode_8_1": 657.6e6,  # stage 1 of the large-group cases
     "decode_16_2": 1308.9e6,
     "decode_64_8": 5222.4e6,
 }
@@ -450,7 +450,7 @@ def workloads(steps):
         "value": e.bytes / (st["median_ms"] * 1e-3) / 1e9, "unit": "GB/s", "ms_per_step": st["median_ms"],
         "pct_of_hbm_peak": 100 * e.bytes / (st["median_ms"] * 1e-3) / 1e9 / PEAK_HBM_GBS, "algorithmic_gb_per_step": e.bytes / 1e9,
         "step_stats": st,
-        "roofline": _roof("decode_stage1_mfma_kernel<F16> (one instance: 4 x 131072 tokens x 32 KV heads)", "hbm",
+        "roofline": _roof("decode_stage1_mfma_kernel<F16,false> (one instance: 4 x 131072 tokens x 32 KV heads)", "hbm",
                           nbytes1 / (s1["median_ms"] * 1e-3) / 1e9, s1["median_ms"], "config4", algorithmic_gb_per_launch=nbytes1 / 1e9)}
     del e
     torch.cuda.empty_cache()
@@ -542,7 +542,7 @@ def decode_large_groups(steps):
                 s1 = _time_graph(d.stage1_only, launches=20, reps=max(3, steps // 2))
                 row[key] = {"fused_ms": fused, "fused_gbs": d.bytes / (fused * 1e-3) / 1e9, "stage1_ms": s1,
                             "stage1_gbs": d.bytes / (s1 * 1e-3) / 1e9}
-            row["roofline"] = _roof("decode_stage1_mfma_kernel<F16>", "hbm", row["matrix_pipe"]["stage1_gbs"], row["matrix_pipe"]["stage1_ms"],
+            row["roofline"] = _roof("decode_stage1_mfma_kernel<F16,false|true> (the shape the library chooses)", "hbm", row["matrix_pipe"]["stage1_gbs"], row["matrix_pipe"]["stage1_ms"],
                                     "decode_%d_%d" % (Hq, Hkv))
             rows.append(row)
             del d
@@ -749,7 +749,7 @@ def main():
                                            "merged_blocks": {"what": "the same two calls with decoding.STAGE1_MERGES_BLOCKS = True (opt-in, "
                                                                      "not the reference's layout): one partial per group of blocks",
                                                              "ms_per_step": sepm["mean_ms"], "value": d.bytes / (sepm["mean_ms"] * 1e-3) / 1e9}}},
-            "roofline": _roof("decode_stage1_mfma_kernel<F16>", "hbm", ach, s1, "config3"),
+            "roofline": _roof("decode_stage1_mfma_kernel<F16,false>", "hbm", ach, s1, "config3"),
         }
         if not args.no_cpu:
             dec["cpu_baseline"] = d.cpu_baseline()
