@@ -65,6 +65,7 @@ struct PrefillParams {
   const int32_t* kv_first;
   const int32_t* o_start;  // first output row per sequence (null: q_start)
   int32_t batch, hq, hkv, peers, nz, kv_slots, slices, units_per_slice, group;
+  int32_t tile_major;  // order of the workgroups in the grid: heaviest query tiles of the whole launch first
   FastDiv d_peers, d_kv_slots, d_slices, d_units, d_group;
   float scale_log2;
   void* o;
@@ -79,7 +80,8 @@ constexpr int BM = 256;   // query rows per workgroup (32 per wave)
 constexpr int BN = 64;    // keys per LDS tile
 constexpr int SUB = 32;   // keys per pipeline step (the contraction length of one P V MFMA)
 constexpr int NWAVE = 8;  // two per SIMD
-constexpr int64_t kSplitBelowWorkgroups = 1024;  // 256-row workgroups in a launch below which the 128-row variant runs
+constexpr int64_t kCUs = 256;  // compute units of the MI355X (one workgroup of this kernel each)
+constexpr int64_t kTileMajorBelowWorkgroups = 2048;  // 256-row workgroups in a launch below which the grid runs the heaviest tiles of all KV heads first
 constexpr float kLazyRescale = 8.f;  // log2 units the running max may lag before O is rescaled
 
 template <typename T> struct Mfma;
@@ -227,22 +229,24 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
   const int group = p.group;
   uint32_t j = blockIdx.x >> 3;
   const int xcd = blockIdx.x & 7;
-  int up, slot;
-  if (SPLIT) {
-    // Small launches: the heaviest query tiles of all KV heads first, so that a CU that has finished a light tile of the
-    // first round takes a heavy one of the rest and the other way round.
+  int up, slot, b;
+  if (SPLIT || p.tile_major) {
+    // Launches of a few workgroups per CU: the heaviest query tiles of all KV heads first (under causal
+    // masking tile z walks z + 1 key blocks), so that a CU that has finished a light tile of the first round takes a
+    // heavy one of the rest and the other way round, and the last round is made of the lightest tiles.
     const uint32_t j1 = div_by(j, p.d_kv_slots);
     slot = (int)(j - j1 * p.kv_slots);
     j = div_by(j1, p.d_units);
     up = (int)(j1 - j * p.units_per_slice);
+    b = (int)j;  // < batch for every workgroup of the grid (one request after the other: its K/V stays in the L2s)
   } else {
     // Large launches: one KV head at a time per XCD, whose K/V then serves all the workgroups the XCD runs.
     const uint32_t j1 = div_by(j, p.d_units);
     up = (int)(j - j1 * p.units_per_slice);
     j = div_by(j1, p.d_kv_slots);
     slot = (int)(j1 - j * p.kv_slots);
+    b = (int)j;  // < batch for every workgroup of the grid
   }
-  const int b = (int)j;  // < batch for every workgroup of the grid
   // The request's six numbers, all requested before the first of them is used (one memory latency instead of three on
   // the way to the first tile load; a workgroup's start-up is what a short launch is made of).
   const int q_len = p.q_len[b], kv_len = p.kv_len[b], qf = p.q_first[b], kf = p.kv_first[b];
@@ -944,7 +948,8 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
   }
 }
 
-template <typename T, int MODE, bool DV, bool SPLIT> static int launch_prefill_rows(const lsattn_prefill_args* a, hipStream_t st) {
+template <typename T, int MODE, bool DV, bool SPLIT>
+static int launch_prefill_rows(const lsattn_prefill_args* a, bool tile_major, hipStream_t st) {
   constexpr int BMW = SPLIT ? BM / 2 : BM;
   PrefillParams p;
   p.q = a->q;
@@ -990,6 +995,7 @@ template <typename T, int MODE, bool DV, bool SPLIT> static int launch_prefill_r
   p.d_group = fast_div((uint32_t)group);
   p.d_slices = fast_div((uint32_t)p.slices);
   p.d_kv_slots = fast_div((uint32_t)p.kv_slots);
+  p.tile_major = tile_major;
   p.d_units = fast_div((uint32_t)p.units_per_slice);
   const int64_t wgs = (int64_t)8 * p.units_per_slice * p.kv_slots * a->batch;
   if (wgs > 0x7fffffff) return LSATTN_ERR_INVALID_ARG;
@@ -997,21 +1003,36 @@ template <typename T, int MODE, bool DV, bool SPLIT> static int launch_prefill_r
   return check_launch();
 }
 
-// Rows per workgroup.  256 is the efficient shape (each staged K/V tile serves twice the rows); 128 (the split variant)
-// when 256-row workgroups would be too few for the chip: under causal masking their work runs from 1 to nz tiles of
-// rows, and with less than a few of them per CU the heaviest one is the launch's duration.  LSATTN_PREFILL_ROWS = 128
-// or 256 in the environment overrides the choice (tuning and tests).
+// Rows per workgroup and the order of the grid, both from the launch's size in 256-row workgroups (the host knows the
+// batch, the head count and the longest query chunk, not the requests' lengths).
+// 256 rows is the efficient shape (each staged K/V tile serves twice the rows at 1.57 us per 64 keys against 0.86 us
+// for 128 rows, and a workgroup's fixed start and end cost comes once per 256 rows).  128 rows (the split variant) when
+// 256-row workgroups cannot fill the chip: at most half a round of them, or at most one round whose heaviest workgroup
+// walks five or more tiles of rows under the causal mask (its duration is the launch's; two rounds of 128-row
+// workgroups, heaviest first, end sooner).  Above one round the 256-row shape measured faster on every shape tried
+// (16 to 64 heads, 1 to 32 requests of 256 to 16384 tokens), provided the grid is in the order below.
+// Grid order: launches under kTileMajorBelowWorkgroups run the heaviest tiles of all KV heads first; larger ones one KV
+// head at a time per XCD (the order that keeps K/V in the L2s when every workgroup walks all keys).  With 32 KV heads
+// and 4096 tokens the head-by-head order leaves a CU with tiles 9 and 16 of 16 and takes 160 us where the other takes 128.
+// LSATTN_PREFILL_ROWS = 128 or 256 and LSATTN_PREFILL_ORDER = tile or head in the environment override the choices
+// (tuning and tests).
 template <typename T, int MODE, bool DV> static int launch_prefill(const lsattn_prefill_args* a, hipStream_t st) {
+  const int64_t nz256 = (a->max_q_len + BM - 1) / BM;
+  const int64_t wgs256 = (int64_t)a->batch * a->num_q_heads * nz256;
+  bool tile_major = wgs256 < kTileMajorBelowWorkgroups;
+  if (const char* e = getenv("LSATTN_PREFILL_ORDER")) {
+    if (e[0] == 't') tile_major = true;
+    if (e[0] == 'h') tile_major = false;
+  }
   if constexpr (!DV) {
-    return launch_prefill_rows<T, MODE, false, false>(a, st);
+    return launch_prefill_rows<T, MODE, false, false>(a, tile_major, st);
   } else {
-    const int64_t wgs256 = (int64_t)a->batch * a->num_q_heads * ((a->max_q_len + BM - 1) / BM);
-    bool split = wgs256 < kSplitBelowWorkgroups;
+    bool split = wgs256 <= kCUs / 2 || (wgs256 <= kCUs && nz256 >= 5);
     if (const char* e = getenv("LSATTN_PREFILL_ROWS")) {
       if (e[0] == '1' && e[1] == '2' && e[2] == '8' && !e[3]) split = true;
       if (e[0] == '2' && e[1] == '5' && e[2] == '6' && !e[3]) split = false;
     }
-    return split ? launch_prefill_rows<T, MODE, true, true>(a, st) : launch_prefill_rows<T, MODE, true, false>(a, st);
+    return split ? launch_prefill_rows<T, MODE, true, true>(a, true, st) : launch_prefill_rows<T, MODE, true, false>(a, tile_major, st);
   }
 }
 

@@ -20,3 +20,23 @@ def lsa():
         pytest.skip("no GPU")
     import loongserve_amd
     return loongserve_amd
+
+
+PREFILL_GEOMETRIES = {
+    "library-choice": {},
+    "rows128": {"LSATTN_PREFILL_ROWS": "128"},
+    "rows256-head-major": {"LSATTN_PREFILL_ROWS": "256", "LSATTN_PREFILL_ORDER": "head"},
+    "rows256-tile-major": {"LSATTN_PREFILL_ROWS": "256", "LSATTN_PREFILL_ORDER": "tile"},
+}
+
+
+@pytest.fixture(params=list(PREFILL_GEOMETRIES))
+def prefill_geometry(request, monkeypatch):
+    """Runs a prefill test once per workgroup shape (128 or 256 query rows) and grid order (one KV head at a time per
+    XCD, or the heaviest query tiles of all KV heads first) of the prefill kernel.  The library picks both from the size
+    of the launch; the test shapes alone would leave most combinations to the few large cases."""
+    for name in ("LSATTN_PREFILL_ROWS", "LSATTN_PREFILL_ORDER"):
+        monkeypatch.delenv(name, raising=False)
+    for name, value in PREFILL_GEOMETRIES[request.param].items():
+        monkeypatch.setenv(name, value)
+    return request.param

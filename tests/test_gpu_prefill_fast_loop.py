@@ -8,7 +8,7 @@ import torch
 from oracle import attn_oracle as orc
 from tests.helpers import assert_inplace_o_close, assert_lse_close, assert_o_close, meta, rand_t
 
-pytestmark = pytest.mark.gpu
+pytestmark = [pytest.mark.gpu, pytest.mark.usefixtures("prefill_geometry")]
 DEV = "cuda:0"
 
 
