@@ -65,8 +65,9 @@ struct PrefillParams {
   const int32_t* kv_first;
   const int32_t* o_start;  // first output row per sequence (null: q_start)
   int32_t batch, hq, hkv, peers, nz, kv_slots, slices, units_per_slice, group;
-  int32_t tile_major;  // order of the workgroups in the grid: heaviest query tiles of the whole launch first
-  FastDiv d_peers, d_kv_slots, d_slices, d_units, d_group;
+  int32_t tile_major;  // order of the workgroups in the grid: heaviest query tiles of all KV heads first
+  int32_t n_first, n_second;  // the fastest and the second index of the grid: (kv_slots, units_per_slice) if tile_major, else swapped
+  FastDiv d_peers, d_first, d_second, d_slices, d_group;
   float scale_log2;
   void* o;
   int64_t o_st, o_sh;
@@ -229,24 +230,17 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
   const int group = p.group;
   uint32_t j = blockIdx.x >> 3;
   const int xcd = blockIdx.x & 7;
-  int up, slot, b;
-  if (SPLIT || p.tile_major) {
-    // Launches of a few workgroups per CU: the heaviest query tiles of all KV heads first (under causal
-    // masking tile z walks z + 1 key blocks), so that a CU that has finished a light tile of the first round takes a
-    // heavy one of the rest and the other way round, and the last round is made of the lightest tiles.
-    const uint32_t j1 = div_by(j, p.d_kv_slots);
-    slot = (int)(j - j1 * p.kv_slots);
-    j = div_by(j1, p.d_units);
-    up = (int)(j1 - j * p.units_per_slice);
-    b = (int)j;  // < batch for every workgroup of the grid (one request after the other: its K/V stays in the L2s)
-  } else {
-    // Large launches: one KV head at a time per XCD, whose K/V then serves all the workgroups the XCD runs.
-    const uint32_t j1 = div_by(j, p.d_units);
-    up = (int)(j - j1 * p.units_per_slice);
-    j = div_by(j1, p.d_kv_slots);
-    slot = (int)(j1 - j * p.kv_slots);
-    b = (int)j;  // < batch for every workgroup of the grid
-  }
+  // Two orders of the grid within a request, by which of the two indices runs fastest (the host sets d_first / d_second):
+  // launches of a few workgroups per CU deal the heaviest query tiles of all KV heads first (under causal masking tile z
+  // walks z + 1 key blocks), so that a CU that has finished a light tile of the first round takes a heavy one of the rest
+  // and the last round is made of the lightest tiles; large launches take one KV head at a time per XCD, whose K/V then
+  // serves all the workgroups the XCD runs.  One request after the other in both (its K/V stays in the L2s).
+  const uint32_t j1 = div_by(j, p.d_first);
+  const int r1 = (int)(j - j1 * p.n_first);
+  j = div_by(j1, p.d_second);
+  const int r2 = (int)(j1 - j * p.n_second);
+  const int up = p.tile_major ? r2 : r1, slot = p.tile_major ? r1 : r2;
+  const int b = (int)j;  // < batch for every workgroup of the grid
   // The request's six numbers, all requested before the first of them is used (one memory latency instead of three on
   // the way to the first tile load; a workgroup's start-up is what a short launch is made of).
   const int q_len = p.q_len[b], kv_len = p.kv_len[b], qf = p.q_first[b], kf = p.kv_first[b];
@@ -572,7 +566,7 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
       const uint32_t any = (pk[0][0] | pk[0][1] | pk[0][2]) | (pk[0][3] | pk[1][0] | pk[1][1]) | (pk[1][2] | pk[1][3]);
       over = (any & 0x40004000u) != 0;
     }
-    if (__builtin_amdgcn_ballot_w64(over) != 0) {
+    if (__builtin_expect(__builtin_amdgcn_ballot_w64(over) != 0, 0)) {
       // rare: some score is above the lazy threshold (always so for the first key a row sees); raise the running maxima
       // and redo the sub-tile (the accumulators' last MFMAs were issued before this phase's barrier and the whole of
       // compute_p lies between them and these multiplies)
@@ -994,9 +988,11 @@ static int launch_prefill_rows(const lsattn_prefill_args* a, bool tile_major, hi
   p.units_per_slice = (int32_t)(((int64_t)group * p.nz + p.slices - 1) / p.slices);
   p.d_group = fast_div((uint32_t)group);
   p.d_slices = fast_div((uint32_t)p.slices);
-  p.d_kv_slots = fast_div((uint32_t)p.kv_slots);
-  p.tile_major = tile_major;
-  p.d_units = fast_div((uint32_t)p.units_per_slice);
+  p.tile_major = tile_major || SPLIT;
+  p.n_first = p.tile_major ? p.kv_slots : p.units_per_slice;
+  p.n_second = p.tile_major ? p.units_per_slice : p.kv_slots;
+  p.d_first = fast_div((uint32_t)p.n_first);
+  p.d_second = fast_div((uint32_t)p.n_second);
   const int64_t wgs = (int64_t)8 * p.units_per_slice * p.kv_slots * a->batch;
   if (wgs > 0x7fffffff) return LSATTN_ERR_INVALID_ARG;
   hipLaunchKernelGGL((prefill_kernel<T, MODE, DV, SPLIT>), dim3((unsigned)wgs), dim3(NWAVE * 64), 0, st, p);
