@@ -44,6 +44,7 @@ TRAFFIC_BYTES = {
 PEAK_MFMA_TFLOPS = 2500.0  # dense fp16/bf16 MFMA, MI355X
 PEAK_HBM_GBS = 8000.0
 DEV = "cuda:0"
+D = 128  # head_dim of every workload here
 
 
 def _randn_half(shape, seed, dtype=torch.float16, chunk_rows=1 << 18):
@@ -490,6 +491,48 @@ def workloads(steps):
     return out
 
 
+def prefill_launch_sizes():
+    """Causal prefill launches from a quarter of a round of workgroups to a few rounds (outside the five baseline configs):
+    fp16, head_dim 128, fp32 (O, LSE) out, device time per launch from a HIP graph of 5 launches.  chosen_us is the
+    library's own choice of workgroup height and grid order; the other columns force 128-row workgroups, 256-row
+    workgroups one KV head at a time per XCD, and 256-row workgroups with the heaviest query tiles of all heads first
+    (LSATTN_PREFILL_ROWS / LSATTN_PREFILL_ORDER)."""
+    import loongserve_amd as lsa
+    rows = []
+    saved = {k: os.environ.get(k) for k in ("LSATTN_PREFILL_ROWS", "LSATTN_PREFILL_ORDER")}
+    try:
+        for N, Hq, Hkv, B in ((1024, 32, 8, 1), (2048, 32, 32, 1), (512, 32, 8, 8), (4096, 32, 32, 1), (2048, 32, 8, 8), (8192, 32, 8, 1)):
+            q = _randn_half((B * N, Hq, D), 4100 + N + B)
+            kv = _randn_half((B * N, 2 * Hkv, D), 4200 + N + B)
+            st = torch.arange(B, dtype=torch.int32, device=DEV) * N
+            ln = torch.full((B,), N, dtype=torch.int32, device=DEV)
+            z = torch.zeros(B, dtype=torch.int32, device=DEV)
+            o = torch.empty((B * N, Hq, D), dtype=torch.float32, device=DEV)
+            lse = torch.empty((B * N, Hq), dtype=torch.float32, device=DEV)
+            fn = lambda: lsa.prefill_attention_step(q, kv[:, :Hkv], kv[:, Hkv:], st, ln, z, st, ln, z, 1, N, out=o, lse=lse, kv_splits=1)
+            fl = 4.0 * D * Hq * B * N * (N + 1) / 2
+            row = {"tokens": N, "requests": B, "q_heads": Hq, "kv_heads": Hkv, "workgroups_of_256_rows": B * Hq * ((N + 255) // 256)}
+            _time_graph(fn, launches=5, reps=2)  # first touch of the new buffers
+            for key, env in (("chosen_us", {}), ("rows128_us", {"LSATTN_PREFILL_ROWS": "128"}),
+                             ("rows256_head_major_us", {"LSATTN_PREFILL_ROWS": "256", "LSATTN_PREFILL_ORDER": "head"}),
+                             ("rows256_tile_major_us", {"LSATTN_PREFILL_ROWS": "256", "LSATTN_PREFILL_ORDER": "tile"})):
+                for k in saved:
+                    os.environ.pop(k, None)
+                os.environ.update(env)
+                row[key] = round(_time_graph(fn, launches=5, reps=5) * 1e3, 1)
+            row["chosen_tflops"] = round(fl / (row["chosen_us"] * 1e-6) / 1e12, 1)
+            rows.append(row)
+            del q, kv, o, lse
+    finally:
+        for k, v in saved.items():
+            if v is None:
+                os.environ.pop(k, None)
+            else:
+                os.environ[k] = v
+    torch.cuda.empty_cache()
+    return {"what": " ".join(x.strip() for x in prefill_launch_sizes.__doc__.split("\n")), "cases": rows}
+
+
 def decode_latency():
     """Small-batch decode: the host's cost of a call against the device's.  GQA 32/8 (and 8/1: Llama-3-70B's heads per GPU
     under 8-way tensor parallelism), head_dim 128, fp16, scattered slots,
@@ -763,6 +806,7 @@ def main():
         torch.cuda.empty_cache()
     if args.only is None:
         line["workloads"] = workloads(max(3, min(args.steps, 10)))
+        line["prefill_launch_sizes"] = prefill_launch_sizes()
         line["decode_latency"] = decode_latency()
         line["decode_large_groups"] = decode_large_groups(max(5, min(args.steps, 10)))
     if args.all:
