@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the per-GPU attention hot path on one MI355X.
 
-A step is one pass of the ring-prefill workload (BASELINE config 2): the 16384 queries of
+A step is one pass of the ring-prefill workload (baseline configuration 2 of five): the 16384 queries of
 shard 3 of a 131072-token sequence attend to KV shards 3 (causal), 0, 1, 2 (full), one
 kernel launch per shard, each later launch LSE-merging its partial into the running result.
 The same run times the token-indexed decode workload (config 3, under "decode"), the other

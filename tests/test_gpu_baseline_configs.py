@@ -1,4 +1,4 @@
-"""The five BASELINE configurations at full size on the GPU.
+"""The five baseline configurations (the shapes the reference's headline figures are quoted on) at full size on the GPU.
 
 Where the whole result is too large for the CPU oracle in seconds, the oracle checks a
 seeded sample of rows / requests / heads (it receives exactly the rows it reads) and the

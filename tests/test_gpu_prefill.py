@@ -38,7 +38,7 @@ def test_causal_step_vs_oracle(lsa, dtype, lens, Hq, Hkv):
 
 
 def test_cfg1_single_causal_2048(lsa):
-    # BASELINE config 1: 1 x 2048 tokens, 32/32 heads, D=128, fp16, one step
+    # baseline configuration 1: 1 x 2048 tokens, 32/32 heads, D=128, fp16, one step
     T, H, D = 2048, 32, 128
     q, k, v = rand_t((T, H, D), 1001), rand_t((T, H, D), 1002), rand_t((T, H, D), 1003)
     m = meta([T])
