@@ -416,18 +416,15 @@ constexpr int kMfmaStage = kMfmaBatch * (kMfmaKRow + kMfmaVRow);  // LDS bytes p
 
 // WS (small launches with fewer than four tasks): the four waves of a workgroup share one task and one block, take every
 // fourth batch of its tokens and merge their partials through LDS: four times the waves of the plain shape, each short.
-template <typename T, bool WS>
-__global__ __launch_bounds__(kMfmaWaves * 64, 2) void decode_stage1_mfma_kernel(Stage1Params p) {
-  __shared__ __attribute__((aligned(1024))) char lds[kMfmaWaves * kMfmaStage];
-  const int lane = threadIdx.x & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+// One unit of work of a workgroup: request b, task group bid_t, chunk group bid_c (of n_cgroups in the grid; LISTED: the
+// unit comes from a list of the units that exist, and its chunk group is taken as it is).
+template <typename T, bool WS, bool LISTED>
+__device__ __forceinline__ void stage1_mfma_unit(const Stage1Params& p, char* lds, const int lane, const int wave, const int64_t b,
+                                                 const unsigned bid_t, const unsigned bid_c, const unsigned n_cgroups) {
   const int n = lane & 15, g = lane >> 4;  // query head (column) or 16-byte chunk of a row / token group or row of four
-  const int64_t b = blockIdx.z;
   // The waves of a workgroup: tw of them on neighbouring tasks (KV heads: their rows of a token lie side by side in memory
   // and are then fetched at about the same time), the rest on consecutive chunks of tokens.
   const int tw = WS ? 1 : (p.tasks_on_x & 7), cw = WS ? 1 : kMfmaWaves / tw;
-  const bool tasks_first = !WS && (p.tasks_on_x & 8) != 0;  // grid = (task groups, chunk groups, batch): a chunk's task groups are dispatched together
-  const unsigned bid_t = tasks_first ? blockIdx.x : blockIdx.y, bid_c = tasks_first ? blockIdx.y : blockIdx.x;
   const int task = WS ? (int)bid_t : bid_t * tw + (wave & (tw - 1));
   if (task >= p.tasks) return;
   const int group = (int)(p.hq / p.hkv);
@@ -443,8 +440,9 @@ __global__ __launch_bounds__(kMfmaWaves * 64, 2) void decode_stage1_mfma_kernel(
   if (nblk > (p.num_blocks + p.row_mul - 1) / p.row_mul) nblk = (p.num_blocks + p.row_mul - 1) / p.row_mul;
   int64_t fine_nblk = len <= 0 ? 0 : ((int64_t)len + p.fine_block_seq - 1) / p.fine_block_seq;
   if (fine_nblk > p.num_blocks) fine_nblk = p.num_blocks;
-  const unsigned n_chunks = (tasks_first ? gridDim.y : gridDim.x) * cw;
-  const unsigned chunk = (bid_c * cw + (WS ? 0 : wave >> (tw == 4 ? 2 : tw == 2 ? 1 : 0)) + (unsigned)b) % n_chunks;  // (rotated by the request, as above)
+  const unsigned n_chunks = n_cgroups * cw;
+  const unsigned wave_chunk = bid_c * cw + (WS ? 0 : wave >> (tw == 4 ? 2 : tw == 2 ? 1 : 0));
+  const unsigned chunk = LISTED ? wave_chunk : (wave_chunk + (unsigned)b) % n_chunks;  // (rotated by the request, as above)
   const int64_t blk_begin = (int64_t)chunk * p.blocks_per_wg;  // (WS: one block per workgroup)
   int64_t blk_end = blk_begin + p.blocks_per_wg;
   if (blk_end > nblk) blk_end = nblk;
@@ -706,6 +704,78 @@ __global__ __launch_bounds__(kMfmaWaves * 64, 2) void decode_stage1_mfma_kernel(
   }
 }
 
+template <typename T, bool WS>
+__global__ __launch_bounds__(kMfmaWaves * 64, 2) void decode_stage1_mfma_kernel(Stage1Params p) {
+  __shared__ __attribute__((aligned(1024))) char lds[kMfmaWaves * kMfmaStage];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const bool tasks_first = !WS && (p.tasks_on_x & 8) != 0;  // grid = (task groups, chunk groups, batch): a chunk's task groups are dispatched together
+  stage1_mfma_unit<T, WS, false>(p, lds, lane, wave, blockIdx.z, tasks_first ? blockIdx.x : blockIdx.y, tasks_first ? blockIdx.y : blockIdx.x,
+                                 tasks_first ? gridDim.y : gridDim.x);
+}
+
+// The plain shape over a list of the units that exist.  The grid above has a workgroup for every (chunk group, task group)
+// of the longest request times the batch, and the host does not know the lengths: a batch of one long request and many
+// short ones is mostly workgroups that find nothing to do (one request of 131072 tokens with 255 of 512, 256 tokens per
+// partial: a million workgroups for 5000 units; starting and ending them takes three times as long as the reads).  Here
+// a fixed grid of two workgroups per CU walks the units: every workgroup first numbers the units of all requests (the
+// first unit of each request, a prefix sum over the batch, in LDS), then takes units blockIdx.x, blockIdx.x + gridDim.x,
+// ...; the request of a unit is found by bisection.  Within a request the task groups of a chunk group are
+// neighbouring units, which run at the same time on neighbouring workgroups (all KV heads of a token are fetched together).
+constexpr int kListedMaxBatch = 1024;
+constexpr int64_t kListedFromWorkgroups = 32768;  // launches of the plain grid from which the list is walked instead
+constexpr int64_t kCUs = 256;                     // compute units of the MI355X
+template <typename T>
+__global__ __launch_bounds__(kMfmaWaves * 64, 2) void decode_stage1_mfma_listed_kernel(Stage1Params p) {
+  __shared__ __attribute__((aligned(1024))) char lds[kMfmaWaves * kMfmaStage];
+  __shared__ uint32_t first_unit[kListedMaxBatch + 1];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int tw = p.tasks_on_x & 7, cw = kMfmaWaves / tw;
+  const uint32_t task_groups = (uint32_t)((p.tasks + tw - 1) / tw);
+  const int batch = (int)p.batch;  // <= kListedMaxBatch (checked on the host)
+  if (wave == 0) {
+    const int64_t rows_avail = (p.num_blocks + p.row_mul - 1) / p.row_mul;
+    uint32_t carry = 0;
+    for (int b0 = 0; b0 < batch; b0 += 64) {
+      const int bb = b0 + lane;
+      uint32_t units = 0;
+      if (bb < batch) {
+        const int len = p.b_seqlen[bb];
+        int64_t nblk = len <= 0 ? 0 : ((int64_t)len + p.block_seq - 1) / p.block_seq;  // (the same clamps as in the unit)
+        if (nblk > p.grid_blocks) nblk = p.grid_blocks;
+        if (nblk > rows_avail) nblk = rows_avail;
+        const int64_t per_group = (int64_t)p.blocks_per_wg * cw;
+        units = (uint32_t)((nblk + per_group - 1) / per_group) * task_groups;
+      }
+      uint32_t incl = units;  // inclusive prefix sum over the 64 lanes
+#pragma unroll
+      for (int d = 1; d < 64; d <<= 1) {
+        const uint32_t up = __shfl_up(incl, d, 64);
+        if (lane >= d) incl += up;
+      }
+      if (bb < batch) first_unit[bb] = carry + incl - units;
+      carry += __builtin_amdgcn_readlane(incl, 63);
+    }
+    if (lane == 0) first_unit[batch] = carry;
+  }
+  __syncthreads();
+  const uint32_t total = first_unit[batch];
+  for (uint32_t unit = blockIdx.x; unit < total; unit += gridDim.x) {
+    // the request that holds the unit: first_unit[lo] <= unit < first_unit[hi] throughout (requests without units are skipped)
+    int lo = 0, hi = batch;
+    while (hi - lo > 1) {
+      const int mid = (lo + hi) >> 1;
+      const uint32_t f = __builtin_amdgcn_readfirstlane(first_unit[mid]);
+      if (f <= unit) lo = mid;
+      else hi = mid;
+    }
+    const uint32_t local = unit - __builtin_amdgcn_readfirstlane(first_unit[lo]);
+    const uint32_t cgroup = local / task_groups;
+    stage1_mfma_unit<T, false, true>(p, lds, lane, wave, lo, local - cgroup * task_groups, cgroup, 0);
+  }
+}
+
 // ------------------------------------------------------------------------------------
 // Stage 2: grid (batch, heads); SL slices of D/4 lanes walk the block axis in parallel
 // (the reference walks it serially, flash_decoding_stage2.cu:38-48), then merge through LDS.
@@ -734,7 +804,7 @@ template <typename OT, int D, int NT>
 __global__ __launch_bounds__(NT) void decode_stage2_kernel(Stage2Params p) {
   constexpr int LPR = D / 4;      // lanes per row (float4 each)
   constexpr int SL = NT / LPR;    // slices walking the block axis
-  constexpr int U = 4;            // rows a slice has in flight
+  constexpr int U = 8;            // rows a slice has in flight
   const int64_t b = blockIdx.x, h = blockIdx.y;
   const int slice = threadIdx.x / LPR, c = threadIdx.x % LPR;
   const int64_t len = p.b_seqlen[b];
@@ -754,26 +824,24 @@ __global__ __launch_bounds__(NT) void decode_stage2_kernel(Stage2Params p) {
     L = L * so + sn;
     M = Mn;
   };
-  int64_t i = slice;
-  for (; i + (U - 1) * SL < n; i += U * SL) {
+  // U rows and their log-sum-exps requested together, none waiting for another: with many requests in the batch the
+  // partials of one request lie batch x heads rows apart (a megabyte and more) and every load pays the full latency; a
+  // long request's merge is a chain of them.  Positions past the request's last block repeat that block and are
+  // dropped; an empty partial's row is loaded like any other (it may hold anything: stage 1 leaves the rows it merged
+  // into another one untouched) and dropped by its log-sum-exp.
+  for (int64_t i = slice; i < n; i += U * SL) {
     float lse[U];
     f32x4 tv[U];
 #pragma unroll
-    for (int u = 0; u < U; u++) lse[u] = p.mid_lse[(i + u * SL) * row_stride + row0];
-    // an empty partial's row of mid_o is not read (stage 1 leaves the rows it merged into another one untouched)
-#pragma unroll
     for (int u = 0; u < U; u++) {
-      const int64_t row = (i + u * SL) * row_stride + row0;
-      tv[u] = f32x4{0.f, 0.f, 0.f, 0.f};
-      if (lse[u] != -INFINITY) tv[u] = *(const f32x4*)(p.mid_o + row * D + c * 4);
+      const int64_t blk = i + u * SL < n ? i + u * SL : n - 1;
+      const int64_t row = blk * row_stride + row0;
+      lse[u] = p.mid_lse[row];
+      tv[u] = *(const f32x4*)(p.mid_o + row * D + c * 4);
     }
 #pragma unroll
-    for (int u = 0; u < U; u++) fold(lse[u], tv[u]);
-  }
-  for (; i < n; i += SL) {
-    const int64_t row = i * row_stride + row0;
-    const float lse = p.mid_lse[row];
-    if (lse != -INFINITY) fold(lse, *(const f32x4*)(p.mid_o + row * D + c * 4));
+    for (int u = 0; u < U; u++)
+      if (i + u * SL < n) fold(lse[u], tv[u]);
   }
   __shared__ float sM[SL], sL[SL];
   __shared__ f32x4 sAcc[SL][LPR];
@@ -931,6 +999,21 @@ template <typename T> static int launch_stage1_mfma(const lsattn_decode_stage1_a
   // fetched at about the same time: config 3's shape 6.03 -> 6.17 TB/s, 32 KV heads 6.0 -> 6.5.
   const bool tasks_first = wgs_y > 1 && wgs_x <= 65535;
   p.tasks_on_x = tw | (tasks_first ? 8 : 0);  // (this kernel: waves of a workgroup on neighbouring tasks; the grid's order)
+  // Launches of very many workgroups walk a list of the units that exist instead (see the kernel): most of such a grid
+  // is empty whenever the batch mixes long and short requests, which the host cannot see.
+  // LSATTN_DECODE_LISTED = 0 or 1 in the environment overrides the choice (tuning and tests).
+  const int64_t wgs_total = wgs_x * wgs_y * a->batch;
+  bool listed = wgs_total >= kListedFromWorkgroups;
+  if (const char* e = getenv("LSATTN_DECODE_LISTED")) {
+    if (e[0] == '0' && !e[1]) listed = false;
+    if (e[0] == '1' && !e[1]) listed = true;
+  }
+  if (listed && a->batch <= kListedMaxBatch && wgs_total <= 0x7fffffff) {
+    const int64_t resident = 2 * kCUs;  // two workgroups of this kernel per CU
+    hipLaunchKernelGGL((decode_stage1_mfma_listed_kernel<T>), dim3((unsigned)(wgs_total < resident ? wgs_total : resident)),
+                       dim3(kMfmaWaves * 64), 0, st, p);
+    return check_launch();
+  }
   const dim3 grid = tasks_first ? dim3((unsigned)wgs_y, (unsigned)wgs_x, (unsigned)a->batch) : dim3((unsigned)wgs_x, (unsigned)wgs_y, (unsigned)a->batch);
   hipLaunchKernelGGL((decode_stage1_mfma_kernel<T, false>), grid, dim3(kMfmaWaves * 64), 0, st, p);
   return check_launch();

@@ -130,12 +130,14 @@ def _check_merge_blocks(lsa, dtype, merge, Hq, Hkv, BS, lens):
     assert_lse_close(l_d, l_ref, "lse")
 
 
-@pytest.fixture(params=["1", "2"], ids=["plain", "split"])
+@pytest.fixture(params=["1", "2", "1 listed"], ids=["plain", "split", "listed"])
 def matrix_pipe(monkeypatch, request):
     """Stage 1 through the matrix-pipe kernel wherever its conditions hold, whatever the launch's size: its plain shape
-    (a wave per 256 tokens; blocks a multiple of 32 tokens; by itself the library takes it for large launches) and the
-    shape whose four waves split a block (blocks a multiple of 128 tokens; small launches of groups of four and more)."""
-    monkeypatch.setenv("LSATTN_DECODE_MFMA", request.param)
+    (a wave per 256 tokens; blocks a multiple of 32 tokens; by itself the library takes it for large launches), the
+    shape whose four waves split a block (blocks a multiple of 128 tokens; small launches of groups of four and more),
+    and the plain shape over a list of the units that exist (by itself: launches of very many workgroups)."""
+    monkeypatch.setenv("LSATTN_DECODE_MFMA", request.param[0])
+    monkeypatch.setenv("LSATTN_DECODE_LISTED", "1" if "listed" in request.param else "0")
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
@@ -190,6 +192,41 @@ def test_large_group_launch_that_takes_the_matrix_pipe_by_itself(lsa, dtype):
     assert torch.equal(torch.isnan(ml_d.cpu()), (torch.arange(nblk)[:, None] >= reach[None, :])[:, :, None].expand(nblk, B, Hq))
     assert_o_close(o_d, o_ref, "o, two stages")
     assert_lse_close(l_d, l_ref, "lse, two stages")
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_skewed_batch_that_walks_the_unit_list_by_itself(lsa, dtype):
+    """One request of 40000 tokens among 127 of 1 to 300 (and two of none), 64 tokens per partial: the plain grid would
+    be 157 x 2 x 130 = 40820 workgroups, nearly all of them without work, so the library walks the list of the units
+    that exist (its own choice: no environment override).  Two stages, per-block partials; rows no request reaches stay
+    untouched."""
+    env = __import__("os").environ
+    assert "LSATTN_DECODE_MFMA" not in env and "LSATTN_DECODE_LISTED" not in env
+    import random
+    rng = random.Random(5)
+    B, Hq, Hkv, D, BS = 130, 32, 8, 128, 64
+    lens = [rng.randint(1, 300) for _ in range(B)]
+    lens[37] = 40000
+    lens[0] = lens[129] = lens[64] = 0
+    lens[1] = 64
+    q, kv, table, b_req, b_len = decode_case(78, B, Hq, Hkv, D, lens, sum(lens) + 1000, dtype)
+    k, v = kv[:, :Hkv], kv[:, Hkv:]
+    live = [b for b in range(B) if lens[b] > 0]
+    o_ref, l_ref = orc.decode_full(q[live], k, v, table, b_req[live], b_len[live])
+    kvd = kv.to(DEV)
+    nblk = (max(lens) + BS - 1) // BS
+    mo_d = torch.full((nblk, B, Hq, D), float("nan"), device=DEV)
+    ml_d = torch.full((nblk, B, Hq), float("nan"), device=DEV)
+    o_d = torch.empty(B, Hq, D, device=DEV)
+    l_d = torch.empty(B, Hq, device=DEV)
+    lsa.longserve_flash_decode_stage1(q.to(DEV), kvd[:, :Hkv], kvd[:, Hkv:], table.to(DEV), b_req.to(DEV), b_len.to(DEV), max(lens),
+                                      mo_d, ml_d, BS)
+    lsa.longserve_flash_decode_stage2(mo_d, ml_d, b_len.to(DEV), o_d, l_d, BS)
+    torch.cuda.synchronize()
+    reach = torch.tensor([(n + BS - 1) // BS for n in lens])
+    assert torch.equal(torch.isnan(ml_d.cpu()), (torch.arange(nblk)[:, None] >= reach[None, :])[:, :, None].expand(nblk, B, Hq))
+    assert_o_close(o_d[live], o_ref, "o, two stages")
+    assert_lse_close(l_d[live], l_ref, "lse, two stages")
 
 
 def test_gather_indices_bit_exact(lsa):
@@ -351,7 +388,8 @@ def test_one_request_of_a_million_tokens(lsa):
 @pytest.mark.parametrize("seed", [3, 11, 42])
 def test_random_decode_shapes_on_both_stage1_kernels(lsa, monkeypatch, seed):
     """Seeded random sweep of stage 1 + stage 2 against the oracle, once with the library's own choice of stage-1 kernel
-    and once through the matrix-pipe kernel wherever its conditions hold: ragged batches with requests of a single token,
+    and once through each shape of the matrix-pipe kernel wherever its conditions hold (plain grid, split waves, listed
+    units): ragged batches with requests of a single token,
     of exactly a block, and of a block plus one; groups of 1 to 20 query heads per KV head; blocks of 32 to 512 tokens;
     per-block partials and merged groups of blocks; both dtypes; unused rows and requests in the table."""
     import random
@@ -373,9 +411,11 @@ def test_random_decode_shapes_on_both_stage1_kernels(lsa, monkeypatch, seed):
         o_ref, l_ref = orc.decode_full(q, k, v, table, b_req, b_len)
         kvd, qd, td, rd, ld = kv.to(DEV), q.to(DEV), table.to(DEV), b_req.to(DEV), b_len.to(DEV)
         nblk = (max(lens) + BS - 1) // BS
-        for forced in (False, "1", "2"):
+        for forced in (False, "1", "2", "1 listed"):
+            monkeypatch.delenv("LSATTN_DECODE_LISTED", raising=False)
             if forced:
-                monkeypatch.setenv("LSATTN_DECODE_MFMA", forced)
+                monkeypatch.setenv("LSATTN_DECODE_MFMA", forced[0])
+                monkeypatch.setenv("LSATTN_DECODE_LISTED", "1" if "listed" in forced else "0")
             else:
                 monkeypatch.delenv("LSATTN_DECODE_MFMA", raising=False)
             mo_d = torch.full((nblk, B, Hq, D), float("nan"), device=DEV)
