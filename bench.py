@@ -513,9 +513,10 @@ def prefill_launch_sizes():
             fl = 4.0 * D * Hq * B * N * (N + 1) / 2
             row = {"tokens": N, "requests": B, "q_heads": Hq, "kv_heads": Hkv, "workgroups_of_256_rows": B * Hq * ((N + 255) // 256)}
             _time_graph(fn, launches=5, reps=2)  # first touch of the new buffers
-            for key, env in (("chosen_us", {}), ("rows128_us", {"LSATTN_PREFILL_ROWS": "128"}),
+            # (the library's choice is timed last: the first timing after new buffers reads a few per cent long)
+            for key, env in (("rows128_us", {"LSATTN_PREFILL_ROWS": "128"}),
                              ("rows256_head_major_us", {"LSATTN_PREFILL_ROWS": "256", "LSATTN_PREFILL_ORDER": "head"}),
-                             ("rows256_tile_major_us", {"LSATTN_PREFILL_ROWS": "256", "LSATTN_PREFILL_ORDER": "tile"})):
+                             ("rows256_tile_major_us", {"LSATTN_PREFILL_ROWS": "256", "LSATTN_PREFILL_ORDER": "tile"}), ("chosen_us", {})):
                 for k in saved:
                     os.environ.pop(k, None)
                 os.environ.update(env)
@@ -596,6 +597,38 @@ def decode_large_groups(steps):
         else:
             os.environ["LSATTN_DECODE_MFMA"] = saved
     return {"what": " ".join(x.strip() for x in decode_large_groups.__doc__.split("\n")), "cases": rows}
+
+
+def decode_mixed_lengths():
+    """Token-indexed decode of batches that mix one long request with many short ones (outside the five baseline
+    configs), GQA 32/8, scattered pool: the two stages as the master of a decode step calls them (BLOCK_SEQ 256, one
+    partial per block) and the fused call, through the library's own choice (stage 1 walks a list of the units of work
+    that exist when the plain grid would have 32768 workgroups and more) and with LSATTN_DECODE_LISTED=0 (the grid
+    sized by the longest request, as the reference's).  Device time per call from a HIP graph of 5 calls."""
+    rows = []
+    saved = os.environ.get("LSATTN_DECODE_LISTED")
+    try:
+        for lens, name in (([131072] + [512] * 255, "1 x 131072 + 255 x 512 tokens"), ([524288] + [2048] * 63, "1 x 524288 + 63 x 2048 tokens")):
+            d = TokenDecode(B=len(lens), lens=lens, pool=sum(lens) + 1024, seed=3400 + len(lens))
+            row = {"batch": name, "algorithmic_gb_per_step": d.bytes / 1e9}
+            for key, env in (("chosen", None), ("grid_by_longest_request", "0")):
+                if env is None:
+                    os.environ.pop("LSATTN_DECODE_LISTED", None)
+                else:
+                    os.environ["LSATTN_DECODE_LISTED"] = env
+                two = _time_graph(d.step_separate_stages, launches=5, reps=5)
+                fused = _time_graph(d.step, launches=5, reps=5)
+                row[key] = {"two_stages_ms": two, "two_stages_gbs": d.bytes / (two * 1e-3) / 1e9, "fused_ms": fused,
+                            "fused_gbs": d.bytes / (fused * 1e-3) / 1e9}
+            rows.append(row)
+            del d
+            torch.cuda.empty_cache()
+    finally:
+        if saved is None:
+            os.environ.pop("LSATTN_DECODE_LISTED", None)
+        else:
+            os.environ["LSATTN_DECODE_LISTED"] = saved
+    return {"what": " ".join(x.strip() for x in decode_mixed_lengths.__doc__.split("\n")), "cases": rows}
 
 
 def other_steps(steps):
@@ -809,6 +842,7 @@ def main():
         line["prefill_launch_sizes"] = prefill_launch_sizes()
         line["decode_latency"] = decode_latency()
         line["decode_large_groups"] = decode_large_groups(max(5, min(args.steps, 10)))
+        line["decode_mixed_lengths"] = decode_mixed_lengths()
     if args.all:
         line["other"] = other_steps(max(3, min(args.steps, 10)))
     print(json.dumps(line))
