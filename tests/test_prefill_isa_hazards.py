@@ -98,19 +98,29 @@ def test_scanner_flags_the_patterns_it_is_meant_to():
     assert len(bad) == 2 and "written by v_mov_b64_e32" in bad[0] and "touched by v_mul_f32_e32" in bad[1], bad
 
 
+_DEVICE_ASM = {}
+
+
+def _device_asm(source):
+    """The device assembly of a file of loongserve_amd/csrc under the library's own compile flags, from the build recipe
+    (loaded by path: it does not need the built library); compiled once per session."""
+    if source not in _DEVICE_ASM:
+        import importlib.util
+        spec = importlib.util.spec_from_file_location("_lsattn_build_flags", os.path.join(REPO, "loongserve_amd", "build.py"))
+        recipe = importlib.util.module_from_spec(spec)
+        spec.loader.exec_module(recipe)
+        src = os.path.join(REPO, "loongserve_amd", "csrc", source)
+        with tempfile.TemporaryDirectory() as tmp:
+            out = os.path.join(tmp, source + ".s")
+            cmd = [recipe.HIPCC, *recipe.FLAGS, *recipe.FILE_FLAGS.get(source, []), "-S", "--cuda-device-only", src, "-o", out]
+            subprocess.run(cmd, check=True, stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)
+            _DEVICE_ASM[source] = open(out).read()
+    return _DEVICE_ASM[source]
+
+
 @pytest.mark.skipif(shutil.which(HIPCC) is None, reason="hipcc not available")
 def test_no_vector_write_next_to_an_inline_assembly_mfma():
-    # the library's own compile flags, from the build recipe (loaded by path: it does not need the built library)
-    import importlib.util
-    spec = importlib.util.spec_from_file_location("_lsattn_build_flags", os.path.join(REPO, "loongserve_amd", "build.py"))
-    recipe = importlib.util.module_from_spec(spec)
-    spec.loader.exec_module(recipe)
-    src = os.path.join(REPO, "loongserve_amd", "csrc", "prefill.hip")
-    with tempfile.TemporaryDirectory() as tmp:
-        out = os.path.join(tmp, "prefill.s")
-        cmd = [recipe.HIPCC, *recipe.FLAGS, *recipe.FILE_FLAGS.get("prefill.hip", []), "-S", "--cuda-device-only", src, "-o", out]
-        subprocess.run(cmd, check=True, stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)
-        text = open(out).read()
+    text = _device_asm("prefill.hip")
     ins, bad = find_hazards(text)
     n_asm_mfma = sum(1 for _, op, _, in_asm in ins if in_asm and op.startswith("v_mfma"))
     # fifteen kernels (dtype / V route / rows per workgroup x three epilogues); the 256-row ones hold eight unrolled
@@ -273,23 +283,9 @@ def test_dpp_scanner_flags_a_close_write():
     assert len(bad) == 1 and "written by v_mov_b32_e32" in bad[0], bad
 
 
-_DECODE_ASM = []
-
-
 def _decode_asm():
     """The device assembly of decode.hip under the library's own flags (compiled once per session)."""
-    if not _DECODE_ASM:
-        import importlib.util
-        spec = importlib.util.spec_from_file_location("_lsattn_build_flags", os.path.join(REPO, "loongserve_amd", "build.py"))
-        recipe = importlib.util.module_from_spec(spec)
-        spec.loader.exec_module(recipe)
-        src = os.path.join(REPO, "loongserve_amd", "csrc", "decode.hip")
-        with tempfile.TemporaryDirectory() as tmp:
-            out = os.path.join(tmp, "decode.s")
-            cmd = [recipe.HIPCC, *recipe.FLAGS, *recipe.FILE_FLAGS.get("decode.hip", []), "-S", "--cuda-device-only", src, "-o", out]
-            subprocess.run(cmd, check=True, stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)
-            _DECODE_ASM.append(open(out).read())
-    return _DECODE_ASM[0]
+    return _device_asm("decode.hip")
 
 
 @pytest.mark.skipif(shutil.which(HIPCC) is None, reason="hipcc not available")
@@ -337,10 +333,16 @@ def loads_in_flight_violations(text, kernel_pattern):
                 m = re.search(r"vmcnt\((\d+)\)", ins)
                 if m:
                     n = int(m.group(1))
-                    keep = set(sorted(set(pending.values()))[-n:]) if n > 0 else set()
-                    pending = {r: v for r, v in pending.items() if v in keep}
+                    pending = {r: v for r, v in pending.items() if v > nload - n}  # (v: the load's number in issue order)
                 continue
             touched = set().union(*[_regs(t) for t in ops]) if ops else set()
+            if in_asm and op.startswith("global_load_lds_dword"):
+                # a load into LDS: it counts for vmcnt like any other and writes no register
+                nload += 1
+                hit = touched & set(pending)
+                if hit:
+                    bad.append("line %d: %s addresses with v%s, which a load in flight writes" % (ln, ins, sorted(hit)))
+                continue
             if in_asm and op.startswith("global_load_dword"):
                 nload += 1
                 hit = set().union(*[_regs(t) for t in ops[1:]]) & set(pending) if len(ops) > 1 else set()
