@@ -162,6 +162,10 @@ typedef struct lsattn_decode_stage1_args {
                               merge over the rows (stage 2 with the same seq_block_size, or with block_seq = 1 and the
                               block count as length, longserve_model.py:514-516) gives the same result with a quarter
                               (m = 4) of the partial bytes written while the gather runs */
+  int64_t partials_by_request; /* 0: mid_o is [num_blocks, batch, Hq, D], the reference's buffers (S1H:7-20).  1 (not in the
+                              reference): [batch, num_blocks, Hq, D], the partials of a request side by side, for callers to
+                              whom mid_o is scratch (the fused call): in a batch the rows of one request lie batch x Hq
+                              rows apart in the reference's layout, a page of their own each */
 } lsattn_decode_stage1_args;
 int lsattn_decode_stage1(const lsattn_decode_stage1_args* a, void* stream);
 
@@ -184,13 +188,14 @@ typedef struct lsattn_decode_stage2_args {
   int64_t num_seq_blocks;
   int64_t head_dim;        /* 32, 64 or 128 */
   int64_t block_seq;
+  int64_t partials_by_request; /* as in lsattn_decode_stage1_args: 1 reads mid_o as [batch, num_seq_blocks, H, D] */
 } lsattn_decode_stage2_args;
 int lsattn_decode_stage2(const lsattn_decode_stage2_args* a, void* stream);
 
 /*
  * Stage 1 and stage 2 over the same partials from one call: the two launches of
  * longserve_token_decode_attention_flash_decoding (FDPY:12-27) back to back on `stream`.  Both argument blocks must name
- * the same mid_o, mid_o_logexpsum, b_seqlen, batch, heads, block count, head_dim and block size (else
+ * the same mid_o, mid_o_logexpsum, b_seqlen, batch, heads, block count, head_dim, block size and layout of the partials (else
  * LSATTN_ERR_INVALID_ARG); everything else as in the two calls it stands for.
  */
 int lsattn_decode_attention(const lsattn_decode_stage1_args* s1, const lsattn_decode_stage2_args* s2, void* stream);

@@ -54,7 +54,7 @@ class DecodeStage1Args(C.Structure):
         ("req_to_tokens", _vp), ("b_req_idx", _vp), ("b_seqlen", _vp),
         ("batch", _i64), ("num_q_heads", _i64), ("num_kv_heads", _i64), ("num_blocks", _i64),
         ("head_dim", _i64), ("max_seq_len", _i64), ("seq_block_size", _i64), ("max_len_in_batch", _i64),
-        ("merge_blocks", _i64),
+        ("merge_blocks", _i64), ("partials_by_request", _i64),
     ]
 
 
@@ -63,6 +63,7 @@ class DecodeStage2Args(C.Structure):
         ("o", _vp), ("o_dtype", _i32), ("reserved", _i32), ("out_logexpsum", _vp), ("b_seqlen", _vp),
         ("mid_o", _vp), ("mid_o_logexpsum", _vp),
         ("batch", _i64), ("num_heads", _i64), ("num_seq_blocks", _i64), ("head_dim", _i64), ("block_seq", _i64),
+        ("partials_by_request", _i64),
     ]
 
 

@@ -34,6 +34,7 @@ struct Stage1Params {
   const int32_t* b_seqlen;
   int64_t batch, hq, hkv, num_blocks, max_seq_len, block_seq, grid_blocks;  // block_seq: tokens per partial computed
   int64_t row_mul, fine_block_seq;  // partial of coarse block i goes to row i * row_mul; rows in between are marked empty
+  int64_t blk_rows, req_rows;       // rows of mid_o between consecutive blocks / requests: (batch * hq, hq) in the reference's layout
   int32_t blocks_per_wg;  // consecutive blocks walked by one workgroup
   int32_t tasks;          // hkv * (group / GT) wave tasks
   int32_t tasks_on_x;     // grid = (task groups, chunks, batch) instead of (chunks, task groups, batch)
@@ -309,14 +310,14 @@ __global__ __launch_bounds__(NW * 64) void decode_stage1_kernel(Stage1Params p) 
     auto write_partial = [&](int h, float M, float L, const float (&ov)[8]) {
       if (h >= nh) return;
       const float inv = 1.f / L;
-      const int64_t row = (blk * p.row_mul * p.batch + b) * p.hq + qh0 + h;
+      const int64_t row = blk * p.row_mul * p.blk_rows + b * p.req_rows + qh0 + h;
       f32x4* dst = (f32x4*)(p.mid_o + row * 128 + sub * 8);
       dst[0] = f32x4{ov[0] * inv, ov[1] * inv, ov[2] * inv, ov[3] * inv};
       dst[1] = f32x4{ov[4] * inv, ov[5] * inv, ov[6] * inv, ov[7] * inv};
       if (sub == 0) p.mid_lse[row] = (M + __builtin_amdgcn_logf(L)) * kLn2;
       // the rows of the blocks merged into this partial (row_mul <= 16: lane `sub` takes the sub-th of them)
       if (sub >= 1 && sub < p.row_mul && blk * p.row_mul + sub < fine_nblk)
-        p.mid_lse[((blk * p.row_mul + sub) * p.batch + b) * p.hq + qh0 + h] = -INFINITY;
+        p.mid_lse[(blk * p.row_mul + sub) * p.blk_rows + b * p.req_rows + qh0 + h] = -INFINITY;
     };
 #pragma unroll
     for (int h = 0; h < GH; h++) {
@@ -537,14 +538,14 @@ __device__ __forceinline__ void stage1_mfma_unit(const Stage1Params& p, char* ld
     lt += xlane32(lt);
     if (n < nh) {
       const float inv = 1.f / lt;  // a block holds at least one token
-      const int64_t row = (blk * p.row_mul * p.batch + b) * p.hq + qh0 + n;
+      const int64_t row = blk * p.row_mul * p.blk_rows + b * p.req_rows + qh0 + n;
       float* dst = p.mid_o + row * 128 + 4 * g;
 #pragma unroll
       for (int db = 0; db < 8; db++) *(f32x4*)(dst + 16 * db) = oacc[db] * inv;
       if (g == 0) p.mid_lse[row] = (m + __builtin_amdgcn_logf(lt)) * kLn2;
       // the rows of the blocks merged into this partial (row_mul <= 16: lane group g takes every fourth of them)
       for (int r = 1 + g; r < p.row_mul; r += 4)
-        if (blk * p.row_mul + r < fine_nblk) p.mid_lse[((blk * p.row_mul + r) * p.batch + b) * p.hq + qh0 + n] = -INFINITY;
+        if (blk * p.row_mul + r < fine_nblk) p.mid_lse[(blk * p.row_mul + r) * p.blk_rows + b * p.req_rows + qh0 + n] = -INFINITY;
     }
   };
   // one batch whose rows have arrived in kr / vr
@@ -685,7 +686,7 @@ __device__ __forceinline__ void stage1_mfma_unit(const Stage1Params& p, char* ld
     }
     if (n < nh) {
       const float inv = 1.f / L;  // a block holds at least one token
-      const int64_t row = (blk_begin * p.row_mul * p.batch + b) * p.hq + qh0 + n;
+      const int64_t row = blk_begin * p.row_mul * p.blk_rows + b * p.req_rows + qh0 + n;
       float* dst = p.mid_o + row * 128 + 4 * g;
 #pragma unroll
       for (int d = 0; d < 2; d++) {
@@ -698,7 +699,7 @@ __device__ __forceinline__ void stage1_mfma_unit(const Stage1Params& p, char* ld
       if (wave == 0) {
         if (g == 0) p.mid_lse[row] = (M + __builtin_amdgcn_logf(L)) * kLn2;
         for (int r = 1 + g; r < p.row_mul; r += 4)
-          if (blk_begin * p.row_mul + r < fine_nblk) p.mid_lse[((blk_begin * p.row_mul + r) * p.batch + b) * p.hq + qh0 + n] = -INFINITY;
+          if (blk_begin * p.row_mul + r < fine_nblk) p.mid_lse[(blk_begin * p.row_mul + r) * p.blk_rows + b * p.req_rows + qh0 + n] = -INFINITY;
       }
     }
   }
@@ -787,6 +788,7 @@ struct Stage2Params {
   const float* mid_o;
   const float* mid_lse;
   int64_t batch, heads, num_seq_blocks, block_seq;
+  int64_t blk_rows, req_rows;  // rows of mid_o between consecutive blocks / requests
 };
 
 template <typename OT> __device__ __forceinline__ void store4(void* base, int64_t elem, const f32x4& v);
@@ -810,8 +812,9 @@ __global__ __launch_bounds__(NT) void decode_stage2_kernel(Stage2Params p) {
   const int64_t len = p.b_seqlen[b];
   int64_t n = len <= 0 ? 0 : (len + p.block_seq - 1) / p.block_seq;
   if (n > p.num_seq_blocks) n = p.num_seq_blocks;
-  const int64_t row_stride = p.batch * p.heads;
-  const int64_t row0 = b * p.heads + h;
+  const int64_t row_stride = p.blk_rows;
+  const int64_t row0 = b * p.req_rows + h;
+  const int64_t out_row = b * p.heads + h;
 
   float M = -INFINITY, L = 0.f;
   f32x4 acc = {0.f, 0.f, 0.f, 0.f};
@@ -864,8 +867,8 @@ __global__ __launch_bounds__(NT) void decode_stage2_kernel(Stage2Params p) {
       a += sAcc[s][c] * w;
     }
     const float inv = Lt > 0.f ? 1.f / Lt : 0.f;
-    store4<OT>(p.o, row0 * D + c * 4, a * inv);
-    if (c == 0) p.out_lse[row0] = Lt > 0.f ? Mt + __builtin_amdgcn_logf(Lt) * kLn2 : -INFINITY;
+    store4<OT>(p.o, out_row * D + c * 4, a * inv);
+    if (c == 0) p.out_lse[out_row] = Lt > 0.f ? Mt + __builtin_amdgcn_logf(Lt) * kLn2 : -INFINITY;
   }
 }
 
@@ -890,6 +893,8 @@ static int launch_stage1(const lsattn_decode_stage1_args* a, hipStream_t st) {
   p.hq = a->num_q_heads;
   p.hkv = a->num_kv_heads;
   p.num_blocks = a->num_blocks;
+  p.blk_rows = a->partials_by_request ? a->num_q_heads : a->batch * a->num_q_heads;
+  p.req_rows = a->partials_by_request ? a->num_blocks * a->num_q_heads : a->num_q_heads;
   p.max_seq_len = a->max_seq_len;
   p.row_mul = a->merge_blocks > 1 ? a->merge_blocks : 1;
   p.fine_block_seq = a->seq_block_size;
@@ -954,6 +959,8 @@ template <typename T> static int launch_stage1_mfma(const lsattn_decode_stage1_a
   p.hq = a->num_q_heads;
   p.hkv = a->num_kv_heads;
   p.num_blocks = a->num_blocks;
+  p.blk_rows = a->partials_by_request ? a->num_q_heads : a->batch * a->num_q_heads;
+  p.req_rows = a->partials_by_request ? a->num_blocks * a->num_q_heads : a->num_q_heads;
   p.max_seq_len = a->max_seq_len;
   p.row_mul = a->merge_blocks > 1 ? a->merge_blocks : 1;
   p.fine_block_seq = a->seq_block_size;
@@ -1084,7 +1091,9 @@ extern "C" int lsattn_decode_stage2(const lsattn_decode_stage2_args* a, void* st
   if (a->batch == 0) return LSATTN_OK;
   if (a->num_heads > 65535) return LSATTN_ERR_INVALID_ARG;
   Stage2Params p{a->o, a->out_logexpsum, a->b_seqlen, a->mid_o, a->mid_o_logexpsum,
-                 a->batch, a->num_heads, a->num_seq_blocks, a->block_seq};
+                 a->batch, a->num_heads, a->num_seq_blocks, a->block_seq,
+                 a->partials_by_request ? a->num_heads : a->batch * a->num_heads,
+                 a->partials_by_request ? a->num_seq_blocks * a->num_heads : a->num_heads};
   dim3 grid((unsigned)a->batch, (unsigned)a->num_heads);
   hipStream_t st = (hipStream_t)stream;
   switch (a->o_dtype) {
@@ -1100,7 +1109,7 @@ extern "C" int lsattn_decode_attention(const lsattn_decode_stage1_args* s1, cons
   // the two stages must describe the same partials
   if (s1->mid_o != s2->mid_o || s1->mid_o_logexpsum != s2->mid_o_logexpsum || s1->b_seqlen != s2->b_seqlen ||
       s1->batch != s2->batch || s1->num_q_heads != s2->num_heads || s1->num_blocks != s2->num_seq_blocks ||
-      s1->head_dim != s2->head_dim || s1->seq_block_size != s2->block_seq)
+      s1->head_dim != s2->head_dim || s1->seq_block_size != s2->block_seq || !s1->partials_by_request != !s2->partials_by_request)
     return LSATTN_ERR_INVALID_ARG;
   const int rc = lsattn_decode_stage1(s1, stream);
   if (rc != LSATTN_OK) return rc;
@@ -1162,6 +1171,7 @@ extern "C" int lsattn_decode_attention_static(const lsattn_decode_stage1_args* s
   a1.mid_o = base;
   a1.mid_o_logexpsum = base + o_floats;
   a1.num_blocks = rows;
+  a1.partials_by_request = a2.partials_by_request = 1;  // (the layout is nobody's but the library's here)
   a2.mid_o = a1.mid_o;
   a2.mid_o_logexpsum = a1.mid_o_logexpsum;
   a2.num_seq_blocks = rows;

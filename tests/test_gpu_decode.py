@@ -229,6 +229,37 @@ def test_skewed_batch_that_walks_the_unit_list_by_itself(lsa, dtype):
     assert_lse_close(l_d[live], l_ref, "lse, two stages")
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_fused_call_gives_the_same_bits_with_either_layout_of_its_partials(lsa, monkeypatch, dtype):
+    """The fused call keeps the partials of a request side by side in mid_o; with the reference's layout (a block of all
+    requests after the other, what the two stage functions use) it must return the same bits."""
+    B, Hq, Hkv, D, BS = 5, 16, 4, 128, 64
+    lens = [700, 1, 64, 2049, 333]
+    q, kv, table, b_req, b_len = decode_case(91, B, Hq, Hkv, D, lens, sum(lens) + 100, dtype)
+    o_ref, l_ref = orc.decode_full(q, kv[:, :Hkv], kv[:, Hkv:], table, b_req, b_len)
+    kvd = kv.to(DEV)
+    nblk = (max(lens) + BS - 1) // BS
+    res = []
+    for by_request in (True, False):
+        monkeypatch.setattr(lsa.longserve_cuda_kernels, "FUSED_PARTIALS_BY_REQUEST", by_request)
+        mo_d = torch.full((nblk, B, Hq, D), float("nan"), device=DEV)
+        ml_d = torch.full((nblk, B, Hq), float("nan"), device=DEV)
+        o_d = torch.empty(B, Hq, D, device=DEV)
+        l_d = torch.empty(B, Hq, device=DEV)
+        lsa.longserve_cuda_kernels.flash_decoding(mo_d, ml_d, q.to(DEV), kvd[:, :Hkv], kvd[:, Hkv:], table.to(DEV), b_req.to(DEV),
+                                                  b_len.to(DEV), max(lens), o_d, l_d, BS)
+        torch.cuda.synchronize()
+        assert_o_close(o_d, o_ref, "o, partials by request %s" % by_request)
+        assert_lse_close(l_d, l_ref, "lse, partials by request %s" % by_request)
+        res.append((o_d.cpu(), l_d.cpu(), ml_d.cpu()))
+    assert torch.equal(res[0][0], res[1][0]) and torch.equal(res[0][1], res[1][1])
+    # the same partials, in the other order: request b's block i is row (b, i) of the one and row (i, b) of the other
+    by_req = res[0][2].reshape(B, nblk, Hq)
+    for b, n in enumerate(lens):
+        for i in range((n + BS - 1) // BS):
+            assert torch.equal(by_req[b, i], res[1][2][i, b]), (b, i)
+
+
 def test_gather_indices_bit_exact(lsa):
     # q = 0 and V[slot] = ordinal code of the slot: the set of gathered slots is read back from O*len
     B, H, D = 3, 2, 128
