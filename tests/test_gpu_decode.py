@@ -260,6 +260,36 @@ def test_fused_call_gives_the_same_bits_with_either_layout_of_its_partials(lsa, 
             assert torch.equal(by_req[b, i], res[1][2][i, b]), (b, i)
 
 
+@pytest.mark.parametrize("B", [1024, 1025])
+def test_unit_list_at_its_largest_batch_and_past_it(lsa, monkeypatch, B):
+    """The list of units is numbered in LDS for up to 1024 requests; a larger batch takes the plain grid whatever the
+    environment asks for.  Requests of 0 to 120 tokens and one of 9000, 64 tokens per partial."""
+    import random
+    monkeypatch.setenv("LSATTN_DECODE_MFMA", "1")
+    monkeypatch.setenv("LSATTN_DECODE_LISTED", "1")
+    rng = random.Random(B)
+    Hq, Hkv, D, BS = 8, 2, 128, 64
+    lens = [rng.randint(0, 120) for _ in range(B)]
+    lens[B // 3] = 9000
+    q, kv, table, b_req, b_len = decode_case(500 + B, B, Hq, Hkv, D, lens, sum(lens) + 300)
+    o_ref, l_ref = orc.decode_full(q, kv[:, :Hkv], kv[:, Hkv:], table, b_req, b_len)
+    kvd = kv.to(DEV)
+    nblk = (max(lens) + BS - 1) // BS
+    mo_d = torch.full((nblk, B, Hq, D), float("nan"), device=DEV)
+    ml_d = torch.full((nblk, B, Hq), float("nan"), device=DEV)
+    lsa.longserve_flash_decode_stage1(q.to(DEV), kvd[:, :Hkv], kvd[:, Hkv:], table.to(DEV), b_req.to(DEV), b_len.to(DEV), max(lens),
+                                      mo_d, ml_d, BS)
+    o_d = torch.empty(B, Hq, D, device=DEV)
+    l_d = torch.empty(B, Hq, device=DEV)
+    lsa.longserve_flash_decode_stage2(mo_d, ml_d, b_len.to(DEV), o_d, l_d, BS)
+    torch.cuda.synchronize()
+    live = [b for b in range(B) if lens[b] > 0]
+    reach = torch.tensor([(n + BS - 1) // BS for n in lens])
+    assert torch.equal(torch.isnan(ml_d.cpu()), (torch.arange(nblk)[:, None] >= reach[None, :])[:, :, None].expand(nblk, B, Hq))
+    assert_o_close(o_d[live], o_ref[live], "o")
+    assert_lse_close(l_d[live], l_ref[live], "lse")
+
+
 def test_gather_indices_bit_exact(lsa):
     # q = 0 and V[slot] = ordinal code of the slot: the set of gathered slots is read back from O*len
     B, H, D = 3, 2, 128
