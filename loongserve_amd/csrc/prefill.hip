@@ -67,6 +67,7 @@ struct PrefillParams {
   int32_t batch, hq, hkv, peers, nz, kv_slots, slices, units_per_slice, group;
   int32_t tile_major;  // order of the workgroups in the grid: heaviest query tiles of all KV heads first
   int32_t n_first, n_second;  // the fastest and the second index of the grid: (kv_slots, units_per_slice) if tile_major, else swapped
+  int32_t pack_shift, heads_per_kv;  // 1 << pack_shift query heads of a KV head side by side in a workgroup; query heads per KV head
   FastDiv d_peers, d_first, d_second, d_slices, d_group;
   float scale_log2;
   void* o;
@@ -253,10 +254,14 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
   const int u = up * p.slices + (vh - kvh * p.slices);
   if (u >= group * p.nz) return;
   const int zr = (int)div_by((uint32_t)u, p.d_group), gq = u - zr * group;
-  const int h = kvh * group + gq;
   const int z = p.nz - 1 - zr;
 
-  const int m_lo = z * BMW;
+  // The workgroup's rows: 1 << pack_shift query heads of the KV head side by side, BMW >> pack_shift query positions of
+  // each (grouped-query attention: the heads of a group read the same K/V, so a workgroup of several of them walks the
+  // same tiles as one of a single head with as many rows, but its positions end sooner: a quarter of the diagonal with
+  // four heads, one masked tile instead of four and a sixteenth of the scores computed for nothing).
+  const int rows_wg = BMW >> p.pack_shift;  // query positions of this workgroup
+  const int m_lo = z * rows_wg;
   if (m_lo >= q_len) return;
   const int P = p.peers;
 
@@ -265,6 +270,8 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
   const int qc = lane & 15, g = lane >> 4;  // query column within a 16-row block, lane group
   const int wrow = SPLIT ? (wave & 3) : wave;  // which 32 rows of the workgroup
   const int kp = SPLIT ? (wave >> 2) : 0;      // SPLIT: parity of the sub-tiles this wave takes
+  const int wph_shift = (SPLIT ? 2 : 3) - p.pack_shift;  // log2 of the 32-row groups per head
+  const int h = kvh * p.heads_per_kv + (gq << p.pack_shift) + (wrow >> wph_shift);  // the wave's query head
 
   // keys of this KV chunk visible to global query position qpos (RING:156-159)
   auto visible_keys = [&](int qpos) -> int {
@@ -272,10 +279,10 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
     const int n = dq >= 0 ? (int)div_by((uint32_t)dq, p.d_peers) + 1 : 0;
     return n > kv_len ? kv_len : n;
   };
-  const int m_hi = (m_lo + BMW < q_len ? m_lo + BMW : q_len) - 1;
+  const int m_hi = (m_lo + rows_wg < q_len ? m_lo + rows_wg : q_len) - 1;
   const int nt = (visible_keys(qf + m_hi * P) + BN - 1) / BN;  // tiles the workgroup walks
 
-  const int m_w0 = m_lo + wrow * 32;
+  const int m_w0 = m_lo + (wrow & ((1 << wph_shift) - 1)) * 32;
 
   // Q as B operands: qreg[qb][ks] = Q[row 16 qb + qc][32 ks + 8g .. +7]; cnt[qb] = keys that row sees (0 past the end)
   u32x4 qreg[2][4];
@@ -942,6 +949,17 @@ __global__ __launch_bounds__(NWAVE * 64, 1) void prefill_kernel(PrefillParams p)
   }
 }
 
+// log2 of the query heads of a KV head that share a workgroup: as many as the workgroup has 32-row groups and the group
+// size divides by (a power of two), unless LSATTN_PREFILL_PACK=0 in the environment (tuning and tests)
+static int pack_shift_for(const lsattn_prefill_args* a, bool split) {
+  if (const char* e = getenv("LSATTN_PREFILL_PACK"))
+    if (e[0] == '0' && !e[1]) return 0;
+  const int64_t group = a->num_q_heads / a->num_kv_heads;
+  int s = 0;
+  while (s < (split ? 2 : 3) && group % (2 << s) == 0) s++;
+  return s;
+}
+
 template <typename T, int MODE, bool DV, bool SPLIT>
 static int launch_prefill_rows(const lsattn_prefill_args* a, bool tile_major, hipStream_t st) {
   constexpr int BMW = SPLIT ? BM / 2 : BM;
@@ -967,7 +985,8 @@ static int launch_prefill_rows(const lsattn_prefill_args* a, bool tile_major, hi
   p.hkv = a->num_kv_heads;
   p.peers = a->sp_peers;
   p.d_peers = fast_div((uint32_t)a->sp_peers);
-  p.nz = (a->max_q_len + BMW - 1) / BMW;
+  p.pack_shift = pack_shift_for(a, SPLIT);
+  p.nz = (a->max_q_len + (BMW >> p.pack_shift) - 1) / (BMW >> p.pack_shift);
   {
     int g8 = 8;  // gcd(num_kv_heads, 8)
     while (a->num_kv_heads % g8) g8 >>= 1;
@@ -983,7 +1002,8 @@ static int launch_prefill_rows(const lsattn_prefill_args* a, bool tile_major, hi
   p.l = a->l;
   p.ml_st = a->ml_stride_t;
   p.ml_sh = a->ml_stride_h;
-  const int group = a->num_q_heads / a->num_kv_heads;
+  p.heads_per_kv = a->num_q_heads / a->num_kv_heads;
+  const int group = p.heads_per_kv >> p.pack_shift;  // workgroups side by side over the heads of a KV head
   p.group = group;
   p.units_per_slice = (int32_t)(((int64_t)group * p.nz + p.slices - 1) / p.slices);
   p.d_group = fast_div((uint32_t)group);
@@ -1011,10 +1031,12 @@ static int launch_prefill_rows(const lsattn_prefill_args* a, bool tile_major, hi
 // head at a time per XCD (the order that keeps K/V in the L2s when every workgroup walks all keys).  With 32 KV heads
 // and 4096 tokens the head-by-head order leaves a CU with tiles 9 and 16 of 16 and takes 160 us where the other takes 128.
 // LSATTN_PREFILL_ROWS = 128 or 256 and LSATTN_PREFILL_ORDER = tile or head in the environment override the choices
-// (tuning and tests).
+// (tuning and tests).  The size counts workgroups as they are launched: with the query heads of a KV head side by side
+// (pack_shift_for) a workgroup covers 256 >> pack_shift positions of 1 << pack_shift heads.
 template <typename T, int MODE, bool DV> static int launch_prefill(const lsattn_prefill_args* a, hipStream_t st) {
   const int64_t nz256 = (a->max_q_len + BM - 1) / BM;
-  const int64_t wgs256 = (int64_t)a->batch * a->num_q_heads * nz256;
+  const int ps = pack_shift_for(a, false);  // (the workgroups of several heads are shorter: less padding past a short chunk)
+  const int64_t wgs256 = (int64_t)a->batch * (a->num_q_heads >> ps) * ((a->max_q_len + (BM >> ps) - 1) / (BM >> ps));
   bool tile_major = wgs256 < kTileMajorBelowWorkgroups;
   if (const char* e = getenv("LSATTN_PREFILL_ORDER")) {
     if (e[0] == 't') tile_major = true;

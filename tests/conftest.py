@@ -27,15 +27,18 @@ PREFILL_GEOMETRIES = {
     "rows128": {"LSATTN_PREFILL_ROWS": "128"},
     "rows256-head-major": {"LSATTN_PREFILL_ROWS": "256", "LSATTN_PREFILL_ORDER": "head"},
     "rows256-tile-major": {"LSATTN_PREFILL_ROWS": "256", "LSATTN_PREFILL_ORDER": "tile"},
+    "rows256-one-head": {"LSATTN_PREFILL_ROWS": "256", "LSATTN_PREFILL_PACK": "0"},
+    "rows128-one-head": {"LSATTN_PREFILL_ROWS": "128", "LSATTN_PREFILL_PACK": "0"},
 }
 
 
 @pytest.fixture(params=list(PREFILL_GEOMETRIES))
 def prefill_geometry(request, monkeypatch):
-    """Runs a prefill test once per workgroup shape (128 or 256 query rows) and grid order (one KV head at a time per
-    XCD, or the heaviest query tiles of all KV heads first) of the prefill kernel.  The library picks both from the size
+    """Runs a prefill test once per workgroup shape (128 or 256 query rows; the query heads of a KV head side by side in
+    a workgroup, the library's way wherever the group size allows, or one head per workgroup) and grid order (one KV head
+    at a time per XCD, or the heaviest query tiles of all KV heads first) of the prefill kernel.  The library picks both from the size
     of the launch; the test shapes alone would leave most combinations to the few large cases."""
-    for name in ("LSATTN_PREFILL_ROWS", "LSATTN_PREFILL_ORDER"):
+    for name in ("LSATTN_PREFILL_ROWS", "LSATTN_PREFILL_ORDER", "LSATTN_PREFILL_PACK"):
         monkeypatch.delenv(name, raising=False)
     for name, value in PREFILL_GEOMETRIES[request.param].items():
         monkeypatch.setenv(name, value)
