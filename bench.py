@@ -32,11 +32,11 @@ if ROOT not in sys.path:
 # which is regenerated with the kernels (the JSON line says so in "traffic_source").
 TRAFFIC_SOURCE = "profiles/bench_default_hbm_traffic.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this command, scaled by a 1 GiB copy); a constant of bench.py, not measured in this run"
 TRAFFIC_BYTES = {
-    "config2": 1307.2e6,    # per launch, averaged over the four launches of a ring step (one diagonal + three full)
+    "config2": 1305.1e6,    # per launch, averaged over the four launches of a ring step (one diagonal + three full)
     "config3": 5203.0e6,    # stage 1 of the fused call
     "config1": 108.7e6,
     "config4": 8618.6e6,    # stage 1 over one instance's 4 x 131072 tokens
-    "config5": 105999.7e6,    # the attention launch (K/V re-fetched from HBM about 25 times: 106-111 GB from run to run)
+    "config5": 104951.1e6,    # the attention launch (K/V re-fetched from HBM about 25 times: 106-111 GB from run to run)
     "decode_8_1": 657.6e6,  # stage 1 of the large-group cases
     "decode_16_2": 1308.9e6,
     "decode_64_8": 5222.4e6,
