@@ -150,12 +150,18 @@ int main(int argc, char** argv) {
     }
 
   int bad = 0;
-  for (int pass = 0; pass < 2; pass++) {
+  for (int pass = 0; pass < 3; pass++) {
     HIP_OK(hipMemsetAsync(dout, 0xff, (size_t)B * Hq * D * 4, stream));
     HIP_OK(hipMemsetAsync(dlse, 0xff, (size_t)B * Hq * 4, stream));
     int rc;
     if (pass == 0) {
       rc = lsattn_decode_attention(&s1, &s2, stream);
+    } else if (pass == 2) {
+      // the same buffers with a request's partials side by side ([batch, blocks, heads, head_dim])
+      lsattn_decode_stage1_args t1 = s1;
+      lsattn_decode_stage2_args t2 = s2;
+      t1.partials_by_request = t2.partials_by_request = 1;
+      rc = lsattn_decode_attention(&t1, &t2, stream);
     } else {
       // the entry point that allocates nothing keeps the partials in the library: the caller names none
       lsattn_decode_stage1_args t1 = s1;
@@ -184,7 +190,8 @@ int main(int argc, char** argv) {
       max_lse = e > max_lse ? e : max_lse;
     }
     printf("%s: heads %d/%d, max |O - ref| = %.3e (bar 2e-3), max rel LSE error = %.3e (bar 1e-4)\n",
-           pass == 0 ? "lsattn_decode_attention" : "lsattn_decode_attention_static", Hq, Hkv, max_abs, max_lse);
+           pass == 0 ? "lsattn_decode_attention" : pass == 1 ? "lsattn_decode_attention_static" : "lsattn_decode_attention, partials by request", Hq, Hkv,
+           max_abs, max_lse);
   }
   printf(bad ? "FAILED: %d values outside the bars\n" : "ok\n", bad);
   return bad ? 1 : 0;
