@@ -32,7 +32,7 @@ if ROOT not in sys.path:
 # which is regenerated with the kernels (the JSON line says so in "traffic_source").
 TRAFFIC_SOURCE = "profiles/bench_default_hbm_traffic.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this command, scaled by a 1 GiB copy); a constant of bench.py, not measured in this run"
 TRAFFIC_BYTES = {
-    "config2": 1305.1e6,    # per launch, averaged over the four launches of a ring step (one diagonal + three full)
+    "config2": 1305.0e6,    # per launch, averaged over the four launches of a ring step (one diagonal + three full)
     "config3": 5203.0e6,    # stage 1 of the fused call
     "config1": 108.7e6,
     "config4": 8618.6e6,    # stage 1 over one instance's 4 x 131072 tokens
@@ -495,13 +495,14 @@ def prefill_launch_sizes():
     """Causal prefill launches from a quarter of a round of workgroups to a few rounds (outside the five baseline configs):
     fp16, head_dim 128, fp32 (O, LSE) out, device time per launch from a HIP graph of 5 launches.  chosen_us is the
     library's own choice of workgroup height and grid order; the other columns force 128-row workgroups, 256-row
-    workgroups one KV head at a time per XCD, and 256-row workgroups with the heaviest query tiles of all heads first
-    (LSATTN_PREFILL_ROWS / LSATTN_PREFILL_ORDER)."""
+    workgroups one KV head at a time per XCD, 256-row workgroups with the heaviest query tiles of all heads first
+    (LSATTN_PREFILL_ROWS / LSATTN_PREFILL_ORDER), and one query head per workgroup instead of the heads of a KV head side
+    by side (LSATTN_PREFILL_PACK=0; the same thing for the 32/32 cases)."""
     import loongserve_amd as lsa
     rows = []
-    saved = {k: os.environ.get(k) for k in ("LSATTN_PREFILL_ROWS", "LSATTN_PREFILL_ORDER")}
+    saved = {k: os.environ.get(k) for k in ("LSATTN_PREFILL_ROWS", "LSATTN_PREFILL_ORDER", "LSATTN_PREFILL_PACK")}
     try:
-        for N, Hq, Hkv, B in ((1024, 32, 8, 1), (2048, 32, 32, 1), (512, 32, 8, 8), (4096, 32, 32, 1), (2048, 32, 8, 6), (8192, 32, 8, 1)):
+        for N, Hq, Hkv, B in ((1024, 32, 8, 1), (2048, 32, 32, 1), (512, 32, 8, 8), (4096, 32, 32, 1), (2048, 32, 8, 6), (1024, 32, 8, 32), (8192, 32, 8, 1)):
             q = _randn_half((B * N, Hq, D), 4100 + N + B)
             kv = _randn_half((B * N, 2 * Hkv, D), 4200 + N + B)
             st = torch.arange(B, dtype=torch.int32, device=DEV) * N
@@ -516,7 +517,8 @@ def prefill_launch_sizes():
             # (the library's choice is timed last: the first timing after new buffers reads a few per cent long)
             for key, env in (("rows128_us", {"LSATTN_PREFILL_ROWS": "128"}),
                              ("rows256_head_major_us", {"LSATTN_PREFILL_ROWS": "256", "LSATTN_PREFILL_ORDER": "head"}),
-                             ("rows256_tile_major_us", {"LSATTN_PREFILL_ROWS": "256", "LSATTN_PREFILL_ORDER": "tile"}), ("chosen_us", {})):
+                             ("rows256_tile_major_us", {"LSATTN_PREFILL_ROWS": "256", "LSATTN_PREFILL_ORDER": "tile"}),
+                             ("one_head_per_workgroup_us", {"LSATTN_PREFILL_PACK": "0"}), ("chosen_us", {})):
                 for k in saved:
                     os.environ.pop(k, None)
                 os.environ.update(env)
