@@ -442,6 +442,10 @@ int lsattn_bf16_to_f16_rows(const void* src, int64_t src_stride, void* dst, int6
                             int64_t row_elems, void* stream);
 
 const char* lsattn_strerror(int code);
+/* Version of this interface.  It grows when an argument block gains a field (always at its end, zero meaning the
+ * behaviour before the field existed): 2 = o_b_start_loc in lsattn_prefill_args, partials_by_request in both decode
+ * argument blocks.  A caller built against version n runs against any library of version >= n if it zeroes its blocks. */
+#define LSATTN_VERSION 2
 int lsattn_version(void);
 
 #ifdef __cplusplus

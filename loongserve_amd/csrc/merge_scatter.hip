@@ -394,4 +394,4 @@ extern "C" const char* lsattn_strerror(int code) {
   }
 }
 
-extern "C" int lsattn_version(void) { return 1; }
+extern "C" int lsattn_version(void) { return LSATTN_VERSION; }

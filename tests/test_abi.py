@@ -24,7 +24,7 @@ def test_library_exports_every_declared_symbol():
     assert set(names) == set(_lib.EXPORTS), (names, sorted(_lib.EXPORTS))
     for n in names:
         assert getattr(lib, n) is not None
-    assert lib.lsattn_version() >= 1
+    assert lib.lsattn_version() == 2  # LSATTN_VERSION of include/lsattn.h: the argument blocks as _lib.py declares them
     assert lib.lsattn_strerror(0) == b"ok"
     assert b"invalid" in lib.lsattn_strerror(-1)
 
