@@ -29,6 +29,8 @@ PREFILL_GEOMETRIES = {
     "rows256-tile-major": {"LSATTN_PREFILL_ROWS": "256", "LSATTN_PREFILL_ORDER": "tile"},
     "rows256-one-head": {"LSATTN_PREFILL_ROWS": "256", "LSATTN_PREFILL_PACK": "0"},
     "rows128-one-head": {"LSATTN_PREFILL_ROWS": "128", "LSATTN_PREFILL_PACK": "0"},
+    "rows128-four-waves": {"LSATTN_PREFILL_ROWS": "half"},
+    "rows128-four-waves-one-head": {"LSATTN_PREFILL_ROWS": "half", "LSATTN_PREFILL_PACK": "0"},
 }
 
 
