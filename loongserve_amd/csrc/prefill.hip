@@ -1141,13 +1141,15 @@ template <typename T, int MODE, bool DV> static int launch_prefill(const lsattn_
     return launch_prefill_rows<T, MODE, false, false>(a, tile_major, st);
   } else {
     bool split = wgs256 <= kCUs / 2 || (wgs256 <= kCUs && nz256 >= 5);
-    // The four-wave shape (two workgroups per CU) for chunks of up to 1536 rows, whose workgroups walk a few tiles each
-    // and spend as long starting and ending as working: 3 to 27 % shorter launches on 60 shapes of 2 to 32 requests of
-    // 128 to 1536 tokens, except around one workgroup pair per CU (384 to 768 workgroups: within +-3 %), which keep the
-    // shapes above.  Not for launches that write their rows elsewhere (the step cut along the keys: few, long workgroups).
+    // The four-wave shape (two workgroups per CU) for chunks of up to 1024 rows (1536 with one head per workgroup),
+    // whose workgroups walk a few tiles each and spend as long starting and ending as working, from three workgroups
+    // per CU on: 3 to 17 % shorter launches on batches of 4 to 32 requests of 128 to 1536 tokens.  Smaller launches keep
+    // the shapes above: with at most a pair of these workgroups per CU a launch of short chunks would gain as much, but
+    // one of short chunks against long K/V (which the host cannot tell apart) would run on half the CUs.  Not for
+    // launches that write their rows elsewhere either (the step cut along the keys: few, long workgroups).
     const int ph = pack_shift_for(a, true);
     const int64_t wgs128 = (int64_t)a->batch * (a->num_q_heads >> ph) * ((a->max_q_len + (BM / 2 >> ph) - 1) / (BM / 2 >> ph));
-    bool half = a->max_q_len <= 1536 && !a->o_b_start_loc && (wgs128 <= 384 || wgs128 >= 768);
+    bool half = a->max_q_len <= (ph ? 1024 : 1536) && !a->o_b_start_loc && wgs128 >= 3 * kCUs;
     if (const char* e = getenv("LSATTN_PREFILL_ROWS")) {
       if (e[0] == '1' && e[1] == '2' && e[2] == '8' && !e[3]) split = true, half = false;
       if (e[0] == '2' && e[1] == '5' && e[2] == '6' && !e[3]) split = false, half = false;
