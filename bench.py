@@ -32,11 +32,11 @@ if ROOT not in sys.path:
 # which is regenerated with the kernels (the JSON line says so in "traffic_source").
 TRAFFIC_SOURCE = "profiles/bench_default_hbm_traffic.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this command, scaled by a 1 GiB copy); a constant of bench.py, not measured in this run"
 TRAFFIC_BYTES = {
-    "config2": 1305.0e6,    # per launch, averaged over the four launches of a ring step (one diagonal + three full)
+    "config2": 1304.9e6,    # per launch, averaged over the four launches of a ring step (one diagonal + three full)
     "config3": 5203.0e6,    # stage 1 of the fused call
     "config1": 108.7e6,
     "config4": 8618.6e6,    # stage 1 over one instance's 4 x 131072 tokens
-    "config5": 104951.1e6,    # the attention launch (K/V re-fetched from HBM about 25 times: 106-111 GB from run to run)
+    "config5": 104949.1e6,    # the attention launch (K/V re-fetched from HBM about 25 times: 106-111 GB from run to run)
     "decode_8_1": 657.6e6,  # stage 1 of the large-group cases
     "decode_16_2": 1308.9e6,
     "decode_64_8": 5222.4e6,
@@ -495,14 +495,14 @@ def prefill_launch_sizes():
     """Causal prefill launches from a quarter of a round of workgroups to a few rounds (outside the five baseline configs):
     fp16, head_dim 128, fp32 (O, LSE) out, device time per launch from a HIP graph of 5 launches.  chosen_us is the
     library's own choice of workgroup height and grid order; the other columns force 128-row workgroups, 256-row
-    workgroups one KV head at a time per XCD, 256-row workgroups with the heaviest query tiles of all heads first
-    (LSATTN_PREFILL_ROWS / LSATTN_PREFILL_ORDER), and one query head per workgroup instead of the heads of a KV head side
+    workgroups one KV head at a time per XCD, 256-row workgroups with the heaviest query tiles of all heads first, the
+    four-wave shape of which two workgroups share a CU (LSATTN_PREFILL_ROWS / LSATTN_PREFILL_ORDER), and one query head per workgroup instead of the heads of a KV head side
     by side (LSATTN_PREFILL_PACK=0; the same thing for the 32/32 cases)."""
     import loongserve_amd as lsa
     rows = []
     saved = {k: os.environ.get(k) for k in ("LSATTN_PREFILL_ROWS", "LSATTN_PREFILL_ORDER", "LSATTN_PREFILL_PACK")}
     try:
-        for N, Hq, Hkv, B in ((1024, 32, 8, 1), (2048, 32, 32, 1), (512, 32, 8, 8), (4096, 32, 32, 1), (2048, 32, 8, 6), (1024, 32, 8, 32), (8192, 32, 8, 1)):
+        for N, Hq, Hkv, B in ((1024, 32, 8, 1), (2048, 32, 32, 1), (512, 32, 8, 8), (4096, 32, 32, 1), (2048, 32, 8, 6), (1024, 32, 8, 32), (256, 32, 32, 16), (8192, 32, 8, 1)):
             q = _randn_half((B * N, Hq, D), 4100 + N + B)
             kv = _randn_half((B * N, 2 * Hkv, D), 4200 + N + B)
             st = torch.arange(B, dtype=torch.int32, device=DEV) * N
@@ -518,6 +518,7 @@ def prefill_launch_sizes():
             for key, env in (("rows128_us", {"LSATTN_PREFILL_ROWS": "128"}),
                              ("rows256_head_major_us", {"LSATTN_PREFILL_ROWS": "256", "LSATTN_PREFILL_ORDER": "head"}),
                              ("rows256_tile_major_us", {"LSATTN_PREFILL_ROWS": "256", "LSATTN_PREFILL_ORDER": "tile"}),
+                             ("four_waves_us", {"LSATTN_PREFILL_ROWS": "half"}),
                              ("one_head_per_workgroup_us", {"LSATTN_PREFILL_PACK": "0"}), ("chosen_us", {})):
                 for k in saved:
                     os.environ.pop(k, None)
