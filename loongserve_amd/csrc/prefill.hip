@@ -4,9 +4,12 @@
 // (loongserve/models/llama/triton_kernel/ring_context_flashattention_nopad.py:13-284).
 //
 // Shape of the computation (head_dim 128):
-//   * a workgroup of 8 waves owns 256 consecutive local query rows of one (sequence, q head);
-//     each wave owns 32 of them and keeps their Q as MFMA B operands in registers; waves w and
-//     w + 4 share a SIMD;
+//   * a workgroup of 8 waves owns 256 query rows of one sequence: consecutive local rows of one query head, or, with
+//     grouped-query attention, as many rows of each of the (up to eight) query heads of a KV head; each wave owns 32 of
+//     them and keeps their Q as MFMA B operands in registers; waves w and w + 4 share a SIMD.  Two smaller shapes of
+//     128 rows serve small launches: SPLIT (eight waves, two per 32 rows, each taking every other 32-key step) when
+//     256-row workgroups would not fill the chip, HALF (four waves, rings of two tiles, two workgroups per CU) for
+//     short chunks, whose workgroups spend as long starting and ending as working;
 //   * K/V tiles of 64 keys are staged through LDS (rings of four tiles, filled by global->LDS DMA,
 //     XOR-swizzled 16-byte chunks so that both the row-wise K reads and the transposing V reads
 //     use all 64 banks);
