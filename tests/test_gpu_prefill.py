@@ -37,6 +37,20 @@ def test_causal_step_vs_oracle(lsa, dtype, lens, Hq, Hkv):
     assert_lse_close(lse, lse_ref, "LSE")
 
 
+@pytest.mark.parametrize("Hq,Hkv", [(16, 16), (32, 8)])
+def test_batch_of_short_prompts(lsa, Hq, Hkv):
+    """24 requests of 1 to 1000 tokens: a launch of more than three workgroups per CU whose chunks are short, the kind the
+    library gives the four-wave shape (two workgroups per CU) by itself; with grouped heads, four of them per workgroup."""
+    lens = [300, 17, 512, 1000, 64, 700, 129, 1] * 3
+    T, D = sum(lens), 128
+    q, k, v = rand_t((T, Hq, D), 41), rand_t((T, Hkv, D), 42), rand_t((T, Hkv, D), 43)
+    m = meta(lens)
+    o, lse = _run_step(lsa, q, k, v, m, m, 1, max(lens))
+    o_ref, lse_ref = orc.attn_step(q, k, v, *m, *m, 1)
+    assert_o_close(o, o_ref, "O")
+    assert_lse_close(lse, lse_ref, "LSE")
+
+
 def test_cfg1_single_causal_2048(lsa):
     # baseline configuration 1: 1 x 2048 tokens, 32/32 heads, D=128, fp16, one step
     T, H, D = 2048, 32, 128
