@@ -5,7 +5,9 @@
  * (a hipStream_t is passed as `void*`; NULL means the default stream).  Every entry point
  *   - launches asynchronously on the given stream and returns without a host sync,
  *   - allocates nothing and keeps no pointer after it returns (the caller owns every
- *     buffer, scratch included),
+ *     buffer, scratch included); the only state the library keeps between calls is the
+ *     block of launch choices that lsattn_set_tuning stores (and the scratch array of
+ *     lsattn_decode_attention_static),
  *   - returns LSATTN_OK or a negative LSATTN_ERR_* code and never aborts or throws.
  *
  * Citations name the reference interface each entry point replaces, relative to the
@@ -89,6 +91,16 @@ typedef struct lsattn_prefill_args {
    * kv_b_start_loc / kv_b_seq_len / kv_first_token_global_idx and its own output rows), which lsattn_lse_merge then
    * joins: short query chunks against long KV fill the chip that way.  Zero the struct before filling it in. */
   const int32_t* o_b_start_loc;
+  /* Optional (0 or 1: off), lsattn_prefill_step only; no counterpart in the reference.  kv_cuts = S in 2..LSATTN_MAX_PARTS
+   * enters every sequence S times into the launch: entry c attends to keys [c * kv_cut_len, (c + 1) * kv_cut_len) of the
+   * sequence's KV chunk (kv_cut_len a multiple of 64) and writes the partial (o, lse) of its rows o_cut_rows * c rows
+   * further down than entry 0 does, so o and lse hold S * o_cut_rows rows (o_cut_rows >= the rows of q).  A short query
+   * chunk against a long KV chunk fills the chip that way (one workgroup per 128 query rows and head otherwise);
+   * lsattn_prefill_merge_cuts joins the S partials.  The slices are computed in the kernel from the six vectors above:
+   * nothing is prepared on the host or in other launches. */
+  int32_t kv_cuts;
+  int32_t kv_cut_len;
+  int64_t o_cut_rows;
 } lsattn_prefill_args;
 
 /* Partial of one step from the empty state: o = normalised fp32 output, lse = natural-log
@@ -126,6 +138,42 @@ typedef struct lsattn_merge_args {
   float* lse;      /* [rows] */
 } lsattn_merge_args;
 int lsattn_lse_merge(const lsattn_merge_args* a, void* stream);
+
+/*
+ * Joins the partials that lsattn_prefill_step wrote with kv_cuts = n_parts (part c of row r at row c * part_rows + r of
+ * o_parts [n_parts * part_rows, Hq, D] / lse_parts [n_parts * part_rows, Hq], fp32 contiguous) for the rows of the
+ * sequences only (rows q_b_start_loc[b] .. + q_b_seq_len[b]; other rows of the outputs are left alone), into one of the
+ * three forms the step itself can produce:
+ *   mode 0: (o fp32, lse) written: the partial of the whole step, as lsattn_prefill_step without cuts;
+ *   mode 1: folded into the running (o, m, l) in place by the update of RING:171-188, as lsattn_prefill_step_merge
+ *           (o in o_dtype F16 / BF16; the step enters with m_i = its LSE in the log2 domain, l_i = 1);
+ *   mode 2: LSE-merged into the running (o fp32, lse), as lsattn_prefill_step_accumulate.
+ * Rows whose cuts all saw no key: mode 0 writes o = 0, lse = -inf; modes 1 and 2 leave the state as it is.
+ * o strides in elements; lse is [rows of q, Hq] contiguous; m, l with their own strides (RING:274-275).
+ * No counterpart in the reference, whose grid is one program per 128 query rows and head whatever the KV length (RING:262).
+ */
+typedef struct lsattn_merge_cuts_args {
+  const float* o_parts;
+  const float* lse_parts;
+  int64_t part_rows;
+  int32_t n_parts;     /* 1..LSATTN_MAX_PARTS */
+  int32_t mode;        /* 0, 1, 2 as above */
+  int32_t batch;
+  int32_t num_q_heads;
+  int32_t head_dim;    /* 128 */
+  int32_t max_q_len;   /* max over q_b_seq_len (sizes the launch) */
+  const int32_t* q_b_start_loc;
+  const int32_t* q_b_seq_len;
+  void* o;
+  int64_t o_stride_t, o_stride_h;
+  int32_t o_dtype;     /* modes 0, 2: LSATTN_F32; mode 1: LSATTN_F16 or LSATTN_BF16 */
+  int32_t reserved;
+  float* lse;          /* modes 0, 2 */
+  float* m;            /* mode 1 */
+  float* l;            /* mode 1 */
+  int64_t ml_stride_t, ml_stride_h;
+} lsattn_merge_cuts_args;
+int lsattn_prefill_merge_cuts(const lsattn_merge_cuts_args* a, void* stream);
 
 /*
  * Flash-decoding stage 1 over a token-indexed KV pool.  Replaces
@@ -441,11 +489,42 @@ int lsattn_pool_update_refs(int32_t* mem_state, int64_t pool_size, const int64_t
 int lsattn_bf16_to_f16_rows(const void* src, int64_t src_stride, void* dst, int64_t dst_stride, int64_t n_rows,
                             int64_t row_elems, void* stream);
 
+/*
+ * Launch choices that the library otherwise makes from the size of a launch, forced process-wide (tuning, and tests that
+ * must reach every kernel shape whatever the size of their inputs).  No counterpart in the reference.  Every field 0 means
+ * "the library's choice"; a NULL argument restores that for all of them.  The block is copied; launches made after the
+ * call returns see it (calls from several threads: each field is stored and read atomically, a launch may see a mix
+ * while a store is under way).  The library reads no environment variable.  Returns LSATTN_ERR_INVALID_ARG for a value
+ * not listed here.
+ */
+#define LSATTN_PREFILL_ROWS_128 1   /* eight waves, 128 query rows, two waves per 32 rows                          */
+#define LSATTN_PREFILL_ROWS_256 2   /* eight waves, 256 query rows                                                */
+#define LSATTN_PREFILL_ROWS_HALF 3  /* four waves, 128 query rows, two workgroups per CU                          */
+#define LSATTN_PREFILL_ORDER_TILE 1 /* heaviest query tiles of all KV heads first                                  */
+#define LSATTN_PREFILL_ORDER_HEAD 2 /* one KV head at a time per XCD                                               */
+#define LSATTN_PREFILL_PACK_OFF 1   /* one query head per workgroup instead of the heads of a KV head side by side */
+#define LSATTN_DECODE_STAGE1_LANE 1  /* the lane kernel                                                            */
+#define LSATTN_DECODE_STAGE1_MFMA 2  /* the matrix-pipe kernel, one wave per block (where its conditions hold)      */
+#define LSATTN_DECODE_STAGE1_SPLIT 3 /* the matrix-pipe kernel, the four waves of a workgroup on one block          */
+#define LSATTN_DECODE_LISTED_OFF 1   /* stage 1's grid sized by the longest request                                */
+#define LSATTN_DECODE_LISTED_ON 2    /* a fixed grid walks the list of units that exist                            */
+typedef struct lsattn_tuning {
+  int32_t prefill_rows;
+  int32_t prefill_order;
+  int32_t prefill_pack;
+  int32_t decode_stage1;
+  int32_t decode_listed;
+  int32_t reserved[3];  /* 0 */
+} lsattn_tuning;
+int lsattn_set_tuning(const lsattn_tuning* t);
+
 const char* lsattn_strerror(int code);
-/* Version of this interface.  It grows when an argument block gains a field (always at its end, zero meaning the
- * behaviour before the field existed): 2 = o_b_start_loc in lsattn_prefill_args, partials_by_request in both decode
- * argument blocks.  A caller built against version n runs against any library of version >= n if it zeroes its blocks. */
-#define LSATTN_VERSION 2
+/* Version of this interface.  It changes whenever an argument block or an entry point changes.  The argument blocks
+ * carry no size field, so a caller must be compiled against the header of the library it loads: check
+ * lsattn_version() == LSATTN_VERSION once after loading and refuse to run otherwise.
+ * 2 = o_b_start_loc in lsattn_prefill_args, partials_by_request in both decode argument blocks; 3 = lsattn_set_tuning,
+ * kv_cuts / kv_cut_len / o_cut_rows in lsattn_prefill_args, lsattn_prefill_merge_cuts. */
+#define LSATTN_VERSION 3
 int lsattn_version(void);
 
 #ifdef __cplusplus

@@ -17,6 +17,7 @@ _building = len(getattr(_sys, "orig_argv", [])) >= 3 and _sys.orig_argv[1:3] == 
 if not _building:
     _lib.load()  # fail loudly at import time if the HIP library is missing or stale
 
+from ._lib import set_tuning  # noqa: E402
 from . import longserve_cuda_kernels  # noqa: E402
 from .kv_pool import LongServeMemoryManager, LongServeReqManager  # noqa: E402
 from .decoding import (longserve_flash_decode_stage1, longserve_flash_decode_stage2,  # noqa: E402
@@ -33,5 +34,5 @@ __all__ = [
     "decoding_stage_migration_sender_kernel", "decoding_stage_migration_receiver_kernel",
     "longserve_flash_decode_stage1", "longserve_flash_decode_stage2",
     "longserve_token_decode_attention_flash_decoding", "longserve_cuda_kernels",
-    "LongServeMemoryManager", "LongServeReqManager",
+    "LongServeMemoryManager", "LongServeReqManager", "set_tuning",
 ]

@@ -35,6 +35,7 @@ class PrefillArgs(C.Structure):
         ("lse", _vp), ("m", _vp), ("l", _vp),
         ("ml_stride_t", _i64), ("ml_stride_h", _i64),
         ("o_b_start_loc", _vp),
+        ("kv_cuts", _i32), ("kv_cut_len", _i32), ("o_cut_rows", _i64),
     ]
 
 
@@ -43,6 +44,16 @@ class MergeArgs(C.Structure):
         ("n_parts", _i32), ("head_dim", _i32), ("rows", _i64),
         ("o_parts", _vp * LSATTN_MAX_PARTS), ("lse_parts", _vp * LSATTN_MAX_PARTS),
         ("o", _vp), ("o_dtype", _i32), ("reserved", _i32), ("lse", _vp),
+    ]
+
+
+class MergeCutsArgs(C.Structure):  # mirrors lsattn_merge_cuts_args
+    _fields_ = [
+        ("o_parts", _vp), ("lse_parts", _vp), ("part_rows", _i64), ("n_parts", _i32), ("mode", _i32),
+        ("batch", _i32), ("num_q_heads", _i32), ("head_dim", _i32), ("max_q_len", _i32),
+        ("q_b_start_loc", _vp), ("q_b_seq_len", _vp),
+        ("o", _vp), ("o_stride_t", _i64), ("o_stride_h", _i64), ("o_dtype", _i32), ("reserved", _i32),
+        ("lse", _vp), ("m", _vp), ("l", _vp), ("ml_stride_t", _i64), ("ml_stride_h", _i64),
     ]
 
 
@@ -65,6 +76,22 @@ class DecodeStage2Args(C.Structure):
         ("batch", _i64), ("num_heads", _i64), ("num_seq_blocks", _i64), ("head_dim", _i64), ("block_seq", _i64),
         ("partials_by_request", _i64),
     ]
+
+
+class Tuning(C.Structure):  # mirrors lsattn_tuning
+    _fields_ = [("prefill_rows", _i32), ("prefill_order", _i32), ("prefill_pack", _i32), ("decode_stage1", _i32),
+                ("decode_listed", _i32), ("reserved", _i32 * 3)]
+
+
+# the values of lsattn_tuning's fields by name (0 / None = the library's own choice)
+TUNING_VALUES = {
+    "prefill_rows": {None: 0, "128": 1, "256": 2, "half": 3},
+    "prefill_order": {None: 0, "tile": 1, "head": 2},
+    "prefill_pack": {None: 0, "off": 1},
+    "decode_stage1": {None: 0, "lane": 1, "mfma": 2, "split": 3},
+    "decode_listed": {None: 0, "off": 1, "on": 2},
+}
+LSATTN_VERSION = 3  # of include/lsattn.h, which the argument blocks above mirror
 
 
 # every symbol include/lsattn.h declares: name -> (restype, argtypes)
@@ -100,6 +127,7 @@ EXPORTS = {
     "lsattn_prefill_step_merge": (C.c_int, [C.POINTER(PrefillArgs), _vp]),
     "lsattn_prefill_step_accumulate": (C.c_int, [C.POINTER(PrefillArgs), _vp]),
     "lsattn_lse_merge": (C.c_int, [C.POINTER(MergeArgs), _vp]),
+    "lsattn_prefill_merge_cuts": (C.c_int, [C.POINTER(MergeCutsArgs), _vp]),
     "lsattn_decode_stage1": (C.c_int, [C.POINTER(DecodeStage1Args), _vp]),
     "lsattn_decode_stage2": (C.c_int, [C.POINTER(DecodeStage2Args), _vp]),
     "lsattn_decode_attention": (C.c_int, [C.POINTER(DecodeStage1Args), C.POINTER(DecodeStage2Args), _vp]),
@@ -121,6 +149,7 @@ EXPORTS = {
     "lsattn_pool_refs_workspace_bytes": (C.c_size_t, [_i64]),
     "lsattn_pool_update_refs": (C.c_int, [_vp, _i64, _vp, _i64, C.c_int, _vp, _vp, C.c_size_t, _vp]),
     "lsattn_bf16_to_f16_rows": (C.c_int, [_vp, _i64, _vp, _i64, _i64, _i64, _vp]),
+    "lsattn_set_tuning": (C.c_int, [C.POINTER(Tuning)]),
     "lsattn_strerror": (C.c_char_p, [C.c_int]),
     "lsattn_version": (C.c_int, []),
 }
@@ -142,8 +171,24 @@ def load():
         fn = getattr(lib, name)  # AttributeError if the symbol is not exported
         fn.restype = res
         fn.argtypes = args
+    # the argument blocks carry no size field: a library of another interface version would read them wrongly
+    if lib.lsattn_version() != LSATTN_VERSION:
+        raise ImportError("loongserve_amd: %s has interface version %d, this package is written against %d; rebuild it with "
+                          "`python -m loongserve_amd.build`" % (LIB_PATH, lib.lsattn_version(), LSATTN_VERSION))
     _lib = lib
     return lib
+
+
+def set_tuning(**choices) -> None:
+    """Force launch choices of the library process-wide (lsattn_set_tuning): prefill_rows "128" | "256" | "half",
+    prefill_order "tile" | "head", prefill_pack "off", decode_stage1 "lane" | "mfma" | "split", decode_listed "off" | "on";
+    fields not named (or None) go back to the library's own choice, so set_tuning() restores all of them."""
+    t = Tuning()
+    for name, value in choices.items():
+        if name not in TUNING_VALUES or value not in TUNING_VALUES[name]:
+            raise ValueError("unknown tuning choice %s=%r" % (name, value))
+        setattr(t, name, TUNING_VALUES[name][value])
+    check(load().lsattn_set_tuning(C.byref(t)), "lsattn_set_tuning")
 
 
 def check(rc: int, what: str) -> None:

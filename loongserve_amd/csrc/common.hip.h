@@ -73,6 +73,12 @@ __device__ __forceinline__ float exp2_diff(float a, float b) {
   return (a == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(a - b);
 }
 
+// The launch choices of lsattn_set_tuning (0 = the library's own); defined in merge_scatter.hip.
+struct Tuning {
+  int prefill_rows, prefill_order, prefill_pack, decode_stage1, decode_listed;
+};
+Tuning tuning();
+
 inline int check_launch() { return hipGetLastError() == hipSuccess ? LSATTN_OK : LSATTN_ERR_LAUNCH; }
 
 }  // namespace lsattn

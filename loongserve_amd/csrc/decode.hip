@@ -14,7 +14,6 @@
 //   * a workgroup walks several consecutive blocks, so the launch is sized for the chip
 //     and not for block_seq.
 #include <atomic>
-#include <cstdlib>
 #include <type_traits>
 
 #include "common.hip.h"
@@ -937,7 +936,7 @@ static int launch_stage1(const lsattn_decode_stage1_args* a, hipStream_t st) {
 }
 
 // Large launches: the matrix-pipe kernel, when its conditions hold (blocks a multiple of 32 tokens, enough waves to fill
-// the chip); LSATTN_DECODE_MFMA = 0 / 1 in the environment forces the choice where the conditions allow it (tuning, tests).
+// the chip); lsattn_set_tuning forces the choice where the conditions allow it (tuning, tests).
 template <typename T> static int launch_stage1_mfma(const lsattn_decode_stage1_args* a, hipStream_t st, bool* taken) {
   *taken = false;
   const int group = (int)(a->num_q_heads / a->num_kv_heads);
@@ -987,11 +986,10 @@ template <typename T> static int launch_stage1_mfma(const lsattn_decode_stage1_a
   const bool can_split = p.block_seq % (kMfmaWaves * kMfmaBatch) == 0 && nblk <= 0x7fffffff;
   bool split_waves = group >= 4 && can_split && waves <= (p.tasks < 4 ? 3072 : 512);
   bool use = !split_waves && waves >= (group >= 4 ? 513 : 768);
-  if (const char* e = getenv("LSATTN_DECODE_MFMA")) {  // 0: the lane kernel, 1: the plain shape, 2: the split shape
-    if (e[0] == '0' && !e[1]) use = split_waves = false;
-    if (e[0] == '1' && !e[1]) use = true, split_waves = false;
-    if (e[0] == '2' && !e[1] && can_split) use = false, split_waves = true;
-  }
+  const Tuning tn = tuning();  // (lsattn_set_tuning: tuning and tests)
+  if (tn.decode_stage1 == LSATTN_DECODE_STAGE1_LANE) use = split_waves = false;
+  if (tn.decode_stage1 == LSATTN_DECODE_STAGE1_MFMA) use = true, split_waves = false;
+  if (tn.decode_stage1 == LSATTN_DECODE_STAGE1_SPLIT && can_split) use = false, split_waves = true;
   if (split_waves) {
     *taken = true;
     p.blocks_per_wg = 1;
@@ -1008,13 +1006,11 @@ template <typename T> static int launch_stage1_mfma(const lsattn_decode_stage1_a
   p.tasks_on_x = tw | (tasks_first ? 8 : 0);  // (this kernel: waves of a workgroup on neighbouring tasks; the grid's order)
   // Launches of very many workgroups walk a list of the units that exist instead (see the kernel): most of such a grid
   // is empty whenever the batch mixes long and short requests, which the host cannot see.
-  // LSATTN_DECODE_LISTED = 0 or 1 in the environment overrides the choice (tuning and tests).
+  // lsattn_set_tuning overrides the choice (tuning and tests).
   const int64_t wgs_total = wgs_x * wgs_y * a->batch;
   bool listed = wgs_total >= kListedFromWorkgroups;
-  if (const char* e = getenv("LSATTN_DECODE_LISTED")) {
-    if (e[0] == '0' && !e[1]) listed = false;
-    if (e[0] == '1' && !e[1]) listed = true;
-  }
+  if (tn.decode_listed == LSATTN_DECODE_LISTED_OFF) listed = false;
+  if (tn.decode_listed == LSATTN_DECODE_LISTED_ON) listed = true;
   if (listed && a->batch <= kListedMaxBatch && wgs_total <= 0x7fffffff) {
     const int64_t resident = 2 * kCUs;  // two workgroups of this kernel per CU
     hipLaunchKernelGGL((decode_stage1_mfma_listed_kernel<T>), dim3((unsigned)(wgs_total < resident ? wgs_total : resident)),
@@ -1067,10 +1063,12 @@ extern "C" int lsattn_decode_stage1(const lsattn_decode_stage1_args* a, void* st
   return LSATTN_ERR_UNSUPPORTED;
 }
 
-template <typename OT> static int dispatch_stage2(const Stage2Params& p, int64_t D, dim3 grid, hipStream_t st) {
+// `live_blocks`: an upper bound of the partial rows any request has (the rows of the buffer, or fewer when the caller
+// knows the longest request); it picks the shape of the merge, which decides the order of its additions.
+template <typename OT> static int dispatch_stage2(const Stage2Params& p, int64_t D, dim3 grid, int64_t live_blocks, hipStream_t st) {
   // few (batch, head) pairs with many partials each (long contexts at small batch): 1024 threads walk the block axis in 32
   // slices instead of 8, or the merge takes a fifth of the time of the gather it follows
-  const bool wide = D == 128 && p.num_seq_blocks >= 64 && (int64_t)grid.x * grid.y < 2048;
+  const bool wide = D == 128 && live_blocks >= 64 && (int64_t)grid.x * grid.y < 2048;
   switch (D) {
     case 32: hipLaunchKernelGGL((decode_stage2_kernel<OT, 32, 256>), grid, dim3(256), 0, st, p); break;
     case 64: hipLaunchKernelGGL((decode_stage2_kernel<OT, 64, 256>), grid, dim3(256), 0, st, p); break;
@@ -1083,7 +1081,7 @@ template <typename OT> static int dispatch_stage2(const Stage2Params& p, int64_t
   return check_launch();
 }
 
-extern "C" int lsattn_decode_stage2(const lsattn_decode_stage2_args* a, void* stream) {
+static int decode_stage2(const lsattn_decode_stage2_args* a, int64_t live_blocks, void* stream) {
   if (!a || !a->o || !a->out_logexpsum || !a->b_seqlen || !a->mid_o || !a->mid_o_logexpsum) return LSATTN_ERR_INVALID_ARG;
   if (a->batch < 0 || a->num_heads <= 0 || a->num_seq_blocks < 0 || a->block_seq < 1) return LSATTN_ERR_INVALID_ARG;
   if (((uintptr_t)a->o | (uintptr_t)a->mid_o) & 15) return LSATTN_ERR_INVALID_ARG;
@@ -1097,11 +1095,15 @@ extern "C" int lsattn_decode_stage2(const lsattn_decode_stage2_args* a, void* st
   dim3 grid((unsigned)a->batch, (unsigned)a->num_heads);
   hipStream_t st = (hipStream_t)stream;
   switch (a->o_dtype) {
-    case LSATTN_F32: return dispatch_stage2<float>(p, a->head_dim, grid, st);
-    case LSATTN_F16: return dispatch_stage2<F16>(p, a->head_dim, grid, st);
-    case LSATTN_BF16: return dispatch_stage2<BF16>(p, a->head_dim, grid, st);
+    case LSATTN_F32: return dispatch_stage2<float>(p, a->head_dim, grid, live_blocks, st);
+    case LSATTN_F16: return dispatch_stage2<F16>(p, a->head_dim, grid, live_blocks, st);
+    case LSATTN_BF16: return dispatch_stage2<BF16>(p, a->head_dim, grid, live_blocks, st);
     default: return LSATTN_ERR_UNSUPPORTED;
   }
+}
+
+extern "C" int lsattn_decode_stage2(const lsattn_decode_stage2_args* a, void* stream) {
+  return decode_stage2(a, a ? a->num_seq_blocks : 0, stream);
 }
 
 extern "C" int lsattn_decode_attention(const lsattn_decode_stage1_args* s1, const lsattn_decode_stage2_args* s2, void* stream) {
@@ -1113,7 +1115,11 @@ extern "C" int lsattn_decode_attention(const lsattn_decode_stage1_args* s1, cons
     return LSATTN_ERR_INVALID_ARG;
   const int rc = lsattn_decode_stage1(s1, stream);
   if (rc != LSATTN_OK) return rc;
-  return lsattn_decode_stage2(s2, stream);
+  // the merge's shape from the rows the longest request can reach, not from the rows the buffer happens to have: the
+  // same call gives the same bits whatever the buffer's height (lsattn_decode_attention_static passes its own)
+  int64_t live = s1->seq_block_size > 0 ? (s1->max_len_in_batch + s1->seq_block_size - 1) / s1->seq_block_size : 0;
+  if (live > s2->num_seq_blocks) live = s2->num_seq_blocks;
+  return decode_stage2(s2, live, stream);
 }
 
 // ------------------------------------------------------------------------------------

@@ -1,5 +1,7 @@
 // HBM-bound helpers around the attention kernels: LSE merge of separately allocated
 // prefill partials, KV-pool row scatter, and prefill slot registration.
+#include <atomic>
+
 #include "common.hip.h"
 
 namespace lsattn {
@@ -48,6 +50,96 @@ __global__ __launch_bounds__(256) void lse_merge_kernel(MergeParams p) {
   const float inv = L > 0.f ? 1.f / L : 0.f;
   put4<OT>(p.out, row * D + c * 4, acc * inv);
   if (c == 0) p.out_lse[row] = L > 0.f ? M + __builtin_amdgcn_logf(L) * kLn2 : -INFINITY;
+}
+
+// The partials of a step cut along the keys, joined for the rows of the sequences: one thread per (row of a sequence,
+// head, 4 consecutive elements); the workgroup's 256 threads cover 8 (row, head) pairs.  MODE as the prefill kernel's
+// epilogues: 0 writes (o fp32, lse), 1 folds into (o, m, l) (ring_context_flashattention_nopad.py:171-188), 2 merges into
+// a running (o fp32, lse).
+struct MergeCutsParams {
+  const float* o_parts;
+  const float* lse_parts;
+  int64_t part_rows;
+  int32_t n, hq;
+  const int32_t* q_start;
+  const int32_t* q_len;
+  void* o;
+  int64_t o_st, o_sh;
+  float* lse;
+  float* m;
+  float* l;
+  int64_t ml_st, ml_sh;
+};
+template <typename OT, int MODE> __global__ __launch_bounds__(256) void merge_cuts_kernel(MergeCutsParams p) {
+  constexpr int D = 128, LPR = D / 4;
+  const int b = blockIdx.y;
+  const int64_t pair = (int64_t)blockIdx.x * (256 / LPR) + threadIdx.x / LPR;  // (row of the sequence, head)
+  const int c = threadIdx.x % LPR;
+  const int64_t r = pair / p.hq;
+  const int h = (int)(pair - r * p.hq);
+  if (r >= p.q_len[b]) return;
+  const int64_t row = (int64_t)p.q_start[b] + r;
+  float M = -INFINITY;
+  for (int i = 0; i < p.n; i++) M = fmaxf(M, p.lse_parts[(i * p.part_rows + row) * p.hq + h]);
+  float L = 0.f;
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  if (M != -INFINITY) {
+    for (int i = 0; i < p.n; i++) {
+      const int64_t pr = (i * p.part_rows + row) * p.hq + h;
+      const float w = __builtin_amdgcn_exp2f((p.lse_parts[pr] - M) * kLog2e);
+      if (w == 0.f) continue;
+      L += w;
+      acc += *(const f32x4*)(p.o_parts + pr * D + c * 4) * w;
+    }
+  }
+  // the step's partial for this row: acc / L, natural LSE = M + ln L (L >= 1 whenever any cut saw a key)
+  const int64_t o_at = row * p.o_st + (int64_t)h * p.o_sh + c * 4;
+  if constexpr (MODE == 0) {
+    const float inv = L > 0.f ? 1.f / L : 0.f;
+    put4<OT>(p.o, o_at, acc * inv);
+    if (c == 0) p.lse[row * p.hq + h] = L > 0.f ? M + __builtin_amdgcn_logf(L) * kLn2 : -INFINITY;
+    return;
+  }
+  if (!(L > 0.f)) return;  // no key in any cut: the state stays
+  if constexpr (MODE == 2) {
+    const float a_old = p.lse[row * p.hq + h], a_new = M + __builtin_amdgcn_logf(L) * kLn2;
+    const float top = fmaxf(a_old, a_new);
+    const float w_old = a_old == -INFINITY ? 0.f : __builtin_amdgcn_exp2f((a_old - top) * kLog2e);
+    const float w_new = __builtin_amdgcn_exp2f((a_new - top) * kLog2e);
+    const float W = w_old + w_new;
+    // (an empty row may hold anything: its old values are dropped, not multiplied by zero)
+    const f32x4 old = w_old != 0.f ? *(const f32x4*)((const float*)p.o + o_at) : f32x4{0.f, 0.f, 0.f, 0.f};
+    *(f32x4*)((float*)p.o + o_at) = old * (w_old / W) + acc * (w_new / (W * L));
+    // (the 32 threads of a row are half a wave: the load of the old lse has returned for all of them before the one
+    // store that depends on it is issued)
+    if (c == 0) p.lse[row * p.hq + h] = top + __builtin_amdgcn_logf(W) * kLn2;
+    return;
+  }
+  if constexpr (MODE == 1) {
+    // the step as (m_i, l_i, acc_i) = (log2-domain LSE, 1, normalised output) into the running state
+    const int64_t ml_at = row * p.ml_st + (int64_t)h * p.ml_sh;
+    const float m_old = p.m[ml_at], l_old = p.l[ml_at];
+    const float m_i = (M + __builtin_amdgcn_logf(L) * kLn2) * kLog2e;
+    const float Mx = fmaxf(m_i, m_old);
+    const float w_old = l_old * exp2_diff(m_old, Mx);
+    const float w_new = __builtin_amdgcn_exp2f(m_i - Mx);
+    const float Ln = w_old + w_new;
+    const float inv = 1.f / Ln;
+    float o0 = 0.f, o1 = 0.f, o2 = 0.f, o3 = 0.f;
+    uint16_t* optr = (uint16_t*)p.o + o_at;
+    if (w_old != 0.f) {  // a row in its start state (m = -inf, l = 0) may hold anything in o
+      const u32x2 old = *(const u32x2*)optr;
+      unpack2<OT>(old[0], o0, o1);
+      unpack2<OT>(old[1], o2, o3);
+    }
+    const float cn = w_new / L;
+    *(u32x2*)optr = u32x2{pack2<OT>((o0 * w_old + acc[0] * cn) * inv, (o1 * w_old + acc[1] * cn) * inv),
+                          pack2<OT>((o2 * w_old + acc[2] * cn) * inv, (o3 * w_old + acc[3] * cn) * inv)};
+    if (c == 0) {
+      p.m[ml_at] = Mx;
+      p.l[ml_at] = Ln;
+    }
+  }
 }
 
 // dst[dest_index[i]] = src[i]; 16 bytes per lane, consecutive lanes cover one row
@@ -275,6 +367,31 @@ extern "C" int lsattn_lse_merge(const lsattn_merge_args* a, void* stream) {
   }
 }
 
+extern "C" int lsattn_prefill_merge_cuts(const lsattn_merge_cuts_args* a, void* stream) {
+  if (!a || !a->o_parts || !a->lse_parts || !a->q_b_start_loc || !a->q_b_seq_len || !a->o) return LSATTN_ERR_INVALID_ARG;
+  if (a->n_parts < 1 || a->n_parts > LSATTN_MAX_PARTS || a->part_rows < 0 || a->batch < 0 || a->num_q_heads <= 0 || a->max_q_len < 0)
+    return LSATTN_ERR_INVALID_ARG;
+  if (a->head_dim != 128) return LSATTN_ERR_UNSUPPORTED;
+  if (a->mode < 0 || a->mode > 2) return LSATTN_ERR_INVALID_ARG;
+  if (a->mode == 1 ? (!a->m || !a->l || (a->o_dtype != LSATTN_F16 && a->o_dtype != LSATTN_BF16)) : (!a->lse || a->o_dtype != LSATTN_F32))
+    return LSATTN_ERR_INVALID_ARG;
+  if (a->o_stride_t % 4 || a->o_stride_h % 4 || (((uintptr_t)a->o | (uintptr_t)a->o_parts) & 15)) return LSATTN_ERR_INVALID_ARG;
+  if (a->batch == 0 || a->max_q_len == 0) return LSATTN_OK;
+  if (a->batch > 65535) return LSATTN_ERR_INVALID_ARG;
+  MergeCutsParams p{a->o_parts, a->lse_parts, a->part_rows, a->n_parts, a->num_q_heads, a->q_b_start_loc, a->q_b_seq_len, a->o,
+                    a->o_stride_t, a->o_stride_h, a->lse, a->m, a->l, a->ml_stride_t, a->ml_stride_h};
+  const int64_t pairs = (int64_t)a->max_q_len * a->num_q_heads;
+  const int64_t blocks = (pairs + 7) / 8;
+  if (blocks > 0x7fffffff) return LSATTN_ERR_INVALID_ARG;
+  const dim3 grid((unsigned)blocks, (unsigned)a->batch);
+  hipStream_t st = (hipStream_t)stream;
+  if (a->mode == 0) hipLaunchKernelGGL((merge_cuts_kernel<float, 0>), grid, dim3(256), 0, st, p);
+  else if (a->mode == 2) hipLaunchKernelGGL((merge_cuts_kernel<float, 2>), grid, dim3(256), 0, st, p);
+  else if (a->o_dtype == LSATTN_F16) hipLaunchKernelGGL((merge_cuts_kernel<F16, 1>), grid, dim3(256), 0, st, p);
+  else hipLaunchKernelGGL((merge_cuts_kernel<BF16, 1>), grid, dim3(256), 0, st, p);
+  return check_launch();
+}
+
 extern "C" int lsattn_kv_scatter(const void* src, int64_t src_stride_bytes, void* dst, int64_t dst_stride_bytes,
                                  const int32_t* dest_index, int64_t n_rows, int64_t row_bytes, void* stream) {
   if (!src || !dst || !dest_index || n_rows < 0 || row_bytes <= 0) return LSATTN_ERR_INVALID_ARG;
@@ -381,6 +498,31 @@ extern "C" int lsattn_decode_migration_send(const lsattn_decode_migration_args* 
 }
 extern "C" int lsattn_decode_migration_recv(const lsattn_decode_migration_args* a, void* stream) {
   return launch_migration<false>(a, (hipStream_t)stream);
+}
+
+namespace lsattn {
+static std::atomic<int32_t> g_tuning[5];
+Tuning tuning() {
+  Tuning t;
+  t.prefill_rows = g_tuning[0].load(std::memory_order_relaxed);
+  t.prefill_order = g_tuning[1].load(std::memory_order_relaxed);
+  t.prefill_pack = g_tuning[2].load(std::memory_order_relaxed);
+  t.decode_stage1 = g_tuning[3].load(std::memory_order_relaxed);
+  t.decode_listed = g_tuning[4].load(std::memory_order_relaxed);
+  return t;
+}
+}  // namespace lsattn
+
+extern "C" int lsattn_set_tuning(const lsattn_tuning* t) {
+  lsattn_tuning z = {};
+  if (!t) t = &z;
+  if (t->prefill_rows < 0 || t->prefill_rows > LSATTN_PREFILL_ROWS_HALF || t->prefill_order < 0 || t->prefill_order > LSATTN_PREFILL_ORDER_HEAD ||
+      t->prefill_pack < 0 || t->prefill_pack > LSATTN_PREFILL_PACK_OFF || t->decode_stage1 < 0 || t->decode_stage1 > LSATTN_DECODE_STAGE1_SPLIT ||
+      t->decode_listed < 0 || t->decode_listed > LSATTN_DECODE_LISTED_ON || t->reserved[0] || t->reserved[1] || t->reserved[2])
+    return LSATTN_ERR_INVALID_ARG;
+  const int32_t v[5] = {t->prefill_rows, t->prefill_order, t->prefill_pack, t->decode_stage1, t->decode_listed};
+  for (int i = 0; i < 5; i++) lsattn::g_tuning[i].store(v[i], std::memory_order_relaxed);
+  return LSATTN_OK;
 }
 
 extern "C" const char* lsattn_strerror(int code) {

@@ -26,15 +26,15 @@
 //     therefore runs as alternating phases: one wave of the SIMD issues the thirty-four MFMAs of a
 //     32-key step (scores, P V, and the row sums of P as a product with a matrix of ones) while the
 //     other does the exponentials of its own step, a workgroup barrier ends each phase;
-//   * tiles that straddle the diagonal or the end of the KV chunk take a general, masked,
-//     bounds-checked step; causal work is skipped per wave;
+//   * tiles that straddle the diagonal or the end of the KV chunk run the same pipeline with a masked softmax phase
+//     (scores past a row's limit become -inf, loads clamp to the chunk's last row); tiles no row of the workgroup sees
+//     are not walked;
 //   * workgroup ids are mapped so that the workgroups sharing one KV head run on one XCD (ids are dealt
 //     round-robin to the 8 XCDs; with fewer KV heads than XCDs a head's work is dealt to several of them)
 //     and heavy (late) query tiles start first.
 //   * one kernel, three epilogues (MODE): 0 writes the step's fp32 partial (O, LSE) from the empty state, 1 folds the
 //     step into the reference's in-place (o, m, l) state (ring_context_flashattention_nopad.py:171-188), 2 LSE-merges it
 //     into a running fp32 (O, LSE); the folding ones read the old state of both row blocks of a wave at once.
-#include <cstdlib>
 #include <type_traits>
 
 #include "common.hip.h"
@@ -71,7 +71,9 @@ struct PrefillParams {
   int32_t tile_major;  // order of the workgroups in the grid: heaviest query tiles of all KV heads first
   int32_t n_first, n_second;  // the fastest and the second index of the grid: (kv_slots, units_per_slice) if tile_major, else swapped
   int32_t pack_shift, heads_per_kv;  // 1 << pack_shift query heads of a KV head side by side in a workgroup; query heads per KV head
-  FastDiv d_peers, d_first, d_second, d_slices, d_group;
+  int32_t kv_cuts, kv_cut_len;       // every sequence entered kv_cuts times, entry c taking keys [c, c + 1) * kv_cut_len of its chunk
+  int64_t o_cut_rows;                // and writing its rows o_cut_rows * c further down
+  FastDiv d_peers, d_first, d_second, d_slices, d_group, d_cuts;
   float scale_log2;
   void* o;
   int64_t o_st, o_sh;
@@ -254,14 +256,21 @@ __global__ __launch_bounds__(HALF ? NWAVE * 32 : NWAVE * 64, HALF ? 2 : 1) void 
   j = div_by(j1, p.d_second);
   const int r2 = (int)(j1 - j * p.n_second);
   const int up = p.tile_major ? r2 : r1, slot = p.tile_major ? r1 : r2;
-  const int b = (int)j;  // < batch for every workgroup of the grid
+  // (sequence, cut of its KV chunk): j < batch * kv_cuts for every workgroup of the grid
+  const int b = (int)div_by(j, p.d_cuts);
+  const int cut = (int)j - b * p.kv_cuts;
   // The request's six numbers, all requested before the first of them is used (one memory latency instead of three on
   // the way to the first tile load; a workgroup's start-up is what a short launch is made of).
-  const int q_len = p.q_len[b], kv_len = p.kv_len[b], qf = p.q_first[b], kf = p.kv_first[b];
+  const int q_len = p.q_len[b], kv_len_all = p.kv_len[b], qf = p.q_first[b], kf_all = p.kv_first[b];
   const int q_start32 = p.q_start[b], kv_start32 = p.kv_start[b];
   const int o_start32 = p.o_start ? p.o_start[b] : q_start32;
-  asm volatile("" ::"s"(q_len), "s"(kv_len), "s"(qf), "s"(kf), "s"(q_start32), "s"(kv_start32), "s"(o_start32));
-  const int64_t q_start = q_start32, kv_start = kv_start32, o_start = o_start32;
+  asm volatile("" ::"s"(q_len), "s"(kv_len_all), "s"(qf), "s"(kf_all), "s"(q_start32), "s"(kv_start32), "s"(o_start32));
+  // the cut's share of the chunk: keys [cut, cut + 1) * kv_cut_len, key n of the chunk at global position kv_first + n * peers
+  const int key0 = cut * p.kv_cut_len;
+  const int kv_rest = kv_len_all - key0;
+  const int kv_len = kv_rest < 0 ? 0 : (kv_rest < p.kv_cut_len ? kv_rest : p.kv_cut_len);
+  const int kf = kf_all + key0 * p.peers;
+  const int64_t q_start = q_start32, kv_start = (int64_t)kv_start32 + key0, o_start = o_start32 + (int64_t)cut * p.o_cut_rows;
   const int vh = xcd + 8 * slot;  // (KV head, slice) pair: always < hkv * slices
   const int kvh = (int)div_by((uint32_t)vh, p.d_slices);
   const int u = up * p.slices + (vh - kvh * p.slices);
@@ -1048,10 +1057,9 @@ __global__ __launch_bounds__(HALF ? NWAVE * 32 : NWAVE * 64, HALF ? 2 : 1) void 
 }
 
 // log2 of the query heads of a KV head that share a workgroup: as many as the workgroup has 32-row groups and the group
-// size divides by (a power of two), unless LSATTN_PREFILL_PACK=0 in the environment (tuning and tests)
-static int pack_shift_for(const lsattn_prefill_args* a, bool split) {
-  if (const char* e = getenv("LSATTN_PREFILL_PACK"))
-    if (e[0] == '0' && !e[1]) return 0;
+// size divides by (a power of two), unless lsattn_set_tuning asked for one head per workgroup
+static int pack_shift_for(const lsattn_prefill_args* a, bool split, const Tuning& tn) {
+  if (tn.prefill_pack == LSATTN_PREFILL_PACK_OFF) return 0;
   const int64_t group = a->num_q_heads / a->num_kv_heads;
   int s = 0;
   while (s < (split ? 2 : 3) && group % (2 << s) == 0) s++;
@@ -1059,7 +1067,7 @@ static int pack_shift_for(const lsattn_prefill_args* a, bool split) {
 }
 
 template <typename T, int MODE, bool DV, bool SPLIT, bool HALF = false>
-static int launch_prefill_rows(const lsattn_prefill_args* a, bool tile_major, hipStream_t st) {
+static int launch_prefill_rows(const lsattn_prefill_args* a, bool tile_major, const Tuning& tn, hipStream_t st) {
   constexpr int BMW = SPLIT || HALF ? BM / 2 : BM;
   PrefillParams p;
   p.q = a->q;
@@ -1083,7 +1091,7 @@ static int launch_prefill_rows(const lsattn_prefill_args* a, bool tile_major, hi
   p.hkv = a->num_kv_heads;
   p.peers = a->sp_peers;
   p.d_peers = fast_div((uint32_t)a->sp_peers);
-  p.pack_shift = pack_shift_for(a, SPLIT || HALF);
+  p.pack_shift = pack_shift_for(a, SPLIT || HALF, tn);
   p.nz = (a->max_q_len + (BMW >> p.pack_shift) - 1) / (BMW >> p.pack_shift);
   {
     int g8 = 8;  // gcd(num_kv_heads, 8)
@@ -1106,12 +1114,16 @@ static int launch_prefill_rows(const lsattn_prefill_args* a, bool tile_major, hi
   p.units_per_slice = (int32_t)(((int64_t)group * p.nz + p.slices - 1) / p.slices);
   p.d_group = fast_div((uint32_t)group);
   p.d_slices = fast_div((uint32_t)p.slices);
+  p.kv_cuts = a->kv_cuts > 1 ? a->kv_cuts : 1;
+  p.kv_cut_len = a->kv_cuts > 1 ? a->kv_cut_len : 0x7fffffff;
+  p.o_cut_rows = a->kv_cuts > 1 ? a->o_cut_rows : 0;
+  p.d_cuts = fast_div((uint32_t)p.kv_cuts);
   p.tile_major = tile_major || SPLIT || HALF;
   p.n_first = p.tile_major ? p.kv_slots : p.units_per_slice;
   p.n_second = p.tile_major ? p.units_per_slice : p.kv_slots;
   p.d_first = fast_div((uint32_t)p.n_first);
   p.d_second = fast_div((uint32_t)p.n_second);
-  const int64_t wgs = (int64_t)8 * p.units_per_slice * p.kv_slots * a->batch;
+  const int64_t wgs = (int64_t)8 * p.units_per_slice * p.kv_slots * a->batch * p.kv_cuts;
   if (wgs > 0x7fffffff) return LSATTN_ERR_INVALID_ARG;
   hipLaunchKernelGGL((prefill_kernel<T, MODE, DV, SPLIT, HALF>), dim3((unsigned)wgs), dim3(HALF ? NWAVE * 32 : NWAVE * 64), 0, st, p);
   return check_launch();
@@ -1128,20 +1140,19 @@ static int launch_prefill_rows(const lsattn_prefill_args* a, bool tile_major, hi
 // Grid order: launches under kTileMajorBelowWorkgroups run the heaviest tiles of all KV heads first; larger ones one KV
 // head at a time per XCD (the order that keeps K/V in the L2s when every workgroup walks all keys).  With 32 KV heads
 // and 4096 tokens the head-by-head order leaves a CU with tiles 9 and 16 of 16 and takes 160 us where the other takes 128.
-// LSATTN_PREFILL_ROWS = 128 or 256 and LSATTN_PREFILL_ORDER = tile or head in the environment override the choices
-// (tuning and tests).  The size counts workgroups as they are launched: with the query heads of a KV head side by side
+// lsattn_set_tuning overrides both choices (tuning and tests).  The size counts workgroups as they are launched: with the query heads of a KV head side by side
 // (pack_shift_for) a workgroup covers 256 >> pack_shift positions of 1 << pack_shift heads.
 template <typename T, int MODE, bool DV> static int launch_prefill(const lsattn_prefill_args* a, hipStream_t st) {
+  const Tuning tn = tuning();
   const int64_t nz256 = (a->max_q_len + BM - 1) / BM;
-  const int ps = pack_shift_for(a, false);  // (the workgroups of several heads are shorter: less padding past a short chunk)
-  const int64_t wgs256 = (int64_t)a->batch * (a->num_q_heads >> ps) * ((a->max_q_len + (BM >> ps) - 1) / (BM >> ps));
+  const int ps = pack_shift_for(a, false, tn);  // (the workgroups of several heads are shorter: less padding past a short chunk)
+  const int64_t cuts = a->kv_cuts > 1 ? a->kv_cuts : 1;
+  const int64_t wgs256 = cuts * a->batch * (a->num_q_heads >> ps) * ((a->max_q_len + (BM >> ps) - 1) / (BM >> ps));
   bool tile_major = wgs256 < kTileMajorBelowWorkgroups;
-  if (const char* e = getenv("LSATTN_PREFILL_ORDER")) {
-    if (e[0] == 't') tile_major = true;
-    if (e[0] == 'h') tile_major = false;
-  }
+  if (tn.prefill_order == LSATTN_PREFILL_ORDER_TILE) tile_major = true;
+  if (tn.prefill_order == LSATTN_PREFILL_ORDER_HEAD) tile_major = false;
   if constexpr (!DV) {
-    return launch_prefill_rows<T, MODE, false, false>(a, tile_major, st);
+    return launch_prefill_rows<T, MODE, false, false>(a, tile_major, tn, st);
   } else {
     bool split = wgs256 <= kCUs / 2 || (wgs256 <= kCUs && nz256 >= 5);
     // The four-wave shape (two workgroups per CU) for chunks of up to 1024 rows (1536 with one head per workgroup),
@@ -1150,16 +1161,14 @@ template <typename T, int MODE, bool DV> static int launch_prefill(const lsattn_
     // the shapes above: with at most a pair of these workgroups per CU a launch of short chunks would gain as much, but
     // one of short chunks against long K/V (which the host cannot tell apart) would run on half the CUs.  Not for
     // launches that write their rows elsewhere either (the step cut along the keys: few, long workgroups).
-    const int ph = pack_shift_for(a, true);
-    const int64_t wgs128 = (int64_t)a->batch * (a->num_q_heads >> ph) * ((a->max_q_len + (BM / 2 >> ph) - 1) / (BM / 2 >> ph));
-    bool half = a->max_q_len <= (ph ? 1024 : 1536) && !a->o_b_start_loc && wgs128 >= 3 * kCUs;
-    if (const char* e = getenv("LSATTN_PREFILL_ROWS")) {
-      if (e[0] == '1' && e[1] == '2' && e[2] == '8' && !e[3]) split = true, half = false;
-      if (e[0] == '2' && e[1] == '5' && e[2] == '6' && !e[3]) split = false, half = false;
-      if (e[0] == 'h') half = true;  // "half": four waves, 128 rows, two workgroups per CU
-    }
-    if (half) return launch_prefill_rows<T, MODE, true, false, true>(a, true, st);
-    return split ? launch_prefill_rows<T, MODE, true, true>(a, true, st) : launch_prefill_rows<T, MODE, true, false>(a, tile_major, st);
+    const int ph = pack_shift_for(a, true, tn);
+    const int64_t wgs128 = cuts * a->batch * (a->num_q_heads >> ph) * ((a->max_q_len + (BM / 2 >> ph) - 1) / (BM / 2 >> ph));
+    bool half = a->max_q_len <= (ph ? 1024 : 1536) && !a->o_b_start_loc && a->kv_cuts <= 1 && wgs128 >= 3 * kCUs;
+    if (tn.prefill_rows == LSATTN_PREFILL_ROWS_128) split = true, half = false;
+    if (tn.prefill_rows == LSATTN_PREFILL_ROWS_256) split = false, half = false;
+    if (tn.prefill_rows == LSATTN_PREFILL_ROWS_HALF) half = true;
+    if (half) return launch_prefill_rows<T, MODE, true, false, true>(a, true, tn, st);
+    return split ? launch_prefill_rows<T, MODE, true, true>(a, true, tn, st) : launch_prefill_rows<T, MODE, true, false>(a, tile_major, tn, st);
   }
 }
 
@@ -1174,6 +1183,12 @@ static int validate(const lsattn_prefill_args* a, int mode) {
   if (a->head_dim != 128) return LSATTN_ERR_UNSUPPORTED;
   if (a->dtype != LSATTN_F16 && a->dtype != LSATTN_BF16) return LSATTN_ERR_UNSUPPORTED;
   if (a->v_is_f16 != 0 && (a->v_is_f16 != 1 || a->dtype != LSATTN_BF16)) return LSATTN_ERR_INVALID_ARG;
+  // the chunk cut along the keys: a multiple of the 64-key tile per cut, the cuts' outputs apart (fp32 partials only),
+  // and key positions that stay within 31 bits
+  if (a->kv_cuts < 0 || a->kv_cuts > LSATTN_MAX_PARTS) return LSATTN_ERR_INVALID_ARG;
+  if (a->kv_cuts > 1 && (mode != 0 || a->kv_cut_len < 64 || a->kv_cut_len % 64 || a->o_cut_rows <= 0 ||
+                         (int64_t)a->kv_cut_len * a->kv_cuts > 0x7fffffff))
+    return LSATTN_ERR_INVALID_ARG;
   // 16-byte operand loads / 8- or 16-byte output stores
   if (a->q_stride_t % 8 || a->q_stride_h % 8 || a->k_stride_t % 8 || a->k_stride_h % 8 || a->v_stride_t % 8 || a->v_stride_h % 8)
     return LSATTN_ERR_INVALID_ARG;

@@ -133,7 +133,7 @@ _FUSED_CACHE_MAX = 64
 
 
 def _meta(t):
-    return (t.data_ptr(), t.shape, t.stride(), t.dtype)
+    return (t.data_ptr(), t.shape, t.stride(), t.dtype, t.device.index)
 
 
 # The fused call keeps the partials of a request side by side in mid_o ([batch, blocks, heads, head_dim] in the same
@@ -147,15 +147,14 @@ def flash_decoding(mid_o, mid_o_logexpsum, q, k, v, req_to_tokens, b_req_idx, b_
     """Stage 1 and stage 2 with the same block size from one library call (what FDPY:12-27 does with two): the checks of
     both, one argument pass, the two launches back to back."""
     key = (_meta(mid_o), _meta(mid_o_logexpsum), _meta(q), _meta(k), _meta(v), _meta(req_to_tokens), _meta(b_req_idx),
-           _meta(b_seqlen), _meta(o), _meta(out_logexpsum), max_len_in_batch, block_seq, q.device.index,
-           FUSED_PARTIALS_BY_REQUEST)
+           _meta(b_seqlen), _meta(o), _meta(out_logexpsum), max_len_in_batch, block_seq, FUSED_PARTIALS_BY_REQUEST)
     blocks = _FUSED_CACHE.get(key)
     if blocks is None:
         a1 = _stage1_args(mid_o, mid_o_logexpsum, q, k, v, req_to_tokens, b_req_idx, b_seqlen, max_len_in_batch, block_seq)
         a2 = _stage2_args(o, out_logexpsum, b_seqlen, mid_o, mid_o_logexpsum, block_seq)
         a1.partials_by_request = a2.partials_by_request = 1 if FUSED_PARTIALS_BY_REQUEST else 0
         if len(_FUSED_CACHE) >= _FUSED_CACHE_MAX:
-            _FUSED_CACHE.clear()
+            del _FUSED_CACHE[next(iter(_FUSED_CACHE))]  # the oldest entry (a caller that allocates new outputs every call never hits)
         blocks = _FUSED_CACHE[key] = (a1, a2, C.byref(a1), C.byref(a2), _lib.load().lsattn_decode_attention)
     rc = blocks[4](blocks[2], blocks[3], _stream())
     if rc:

@@ -99,7 +99,8 @@ def _pad_head_dim(t: torch.Tensor) -> torch.Tensor:
 
 def _prefill_args(q, k, v, o, q_b_start_loc, q_b_seq_len, q_first, kv_b_start_loc, kv_b_seq_len, kv_first,
                   peers: int, max_q_len: int, sm_scale: Optional[float], v_f16: Optional[torch.Tensor] = None,
-                  v_f16_valid: bool = False, o_b_start_loc: Optional[torch.Tensor] = None) -> _lib.PrefillArgs:
+                  v_f16_valid: bool = False, o_b_start_loc: Optional[torch.Tensor] = None,
+                  cuts: Optional[Tuple[int, int, int]] = None) -> _lib.PrefillArgs:
     for t, n in ((q, "q"), (k, "k"), (v, "v"), (o, "o")):
         _dev(t, n)
         if t.dim() != 3:
@@ -114,8 +115,10 @@ def _prefill_args(q, k, v, o, q_b_start_loc, q_b_seq_len, q_first, kv_b_start_lo
         raise ValueError("q, k, v must share dtype float16 or bfloat16")
     if k.shape[1] != v.shape[1] or q.shape[1] % k.shape[1] != 0:
         raise ValueError("bad head counts: Hq=%d Hkv=%d" % (q.shape[1], k.shape[1]))
-    if o_b_start_loc is None and o.shape != q.shape:
+    if o_b_start_loc is None and cuts is None and o.shape != q.shape:
         raise ValueError("o must have the shape of q")
+    if cuts is not None and (o.shape[1:] != q.shape[1:] or o.shape[0] < cuts[0] * cuts[2] or cuts[2] < q.shape[0]):
+        raise ValueError("o must hold kv_cuts * o_cut_rows rows of q's heads and head_dim")
     if o_b_start_loc is not None and o.shape[1:] != q.shape[1:]:
         raise ValueError("o must have q's heads and head_dim")
     B = q_b_seq_len.shape[0]
@@ -149,20 +152,94 @@ def _prefill_args(q, k, v, o, q_b_start_loc, q_b_seq_len, q_first, kv_b_start_lo
     if o_b_start_loc is not None:
         _i32vec(o_b_start_loc, "o_b_start_loc", B)
         a.o_b_start_loc = o_b_start_loc.data_ptr()
+    if cuts is not None:
+        a.kv_cuts, a.kv_cut_len, a.o_cut_rows = int(cuts[0]), int(cuts[1]), int(cuts[2])
     return a
+
+
+def _cut_workspace(workspace, S: int, Tq: int, Hq: int, D: int, device):
+    """(po [S*Tq,Hq,D], pl [S*Tq,Hq]) fp32 views for the partials of S cuts: of `workspace` (one contiguous float32 tensor
+    of at least S*Tq*Hq*(D+1) elements, or a pair of tensors of exactly those shapes), or new tensors if it is None."""
+    n_o, n_l = S * Tq * Hq * D, S * Tq * Hq
+    if workspace is None:
+        return (torch.empty((S * Tq, Hq, D), dtype=torch.float32, device=device),
+                torch.empty((S * Tq, Hq), dtype=torch.float32, device=device))
+    if isinstance(workspace, (tuple, list)):
+        po, pl = workspace
+        if (po.dtype != torch.float32 or pl.dtype != torch.float32 or tuple(po.shape) != (S * Tq, Hq, D)
+                or tuple(pl.shape) != (S * Tq, Hq) or not po.is_contiguous() or not pl.is_contiguous()):
+            raise ValueError("workspace pair: contiguous float32 [S*Tq,Hq,D] and [S*Tq,Hq]")
+        _dev(po, "workspace"); _dev(pl, "workspace")
+        return po, pl
+    _dev(workspace, "workspace")
+    if workspace.dtype != torch.float32 or not workspace.is_contiguous() or workspace.numel() < n_o + n_l:
+        raise ValueError("workspace: a contiguous float32 tensor of at least S*Tq*Hq*(D+1) = %d elements" % (n_o + n_l))
+    flat = workspace.view(-1)
+    return flat[:n_o].view(S * Tq, Hq, D), flat[n_o:n_o + n_l].view(S * Tq, Hq)
+
+
+def _workspace_cuts(workspace, Tq: int, Hq: int, D: int) -> int:
+    """How many cuts' partials a single-tensor workspace holds."""
+    if workspace is None or isinstance(workspace, (tuple, list)) or Tq == 0:
+        return _lib.LSATTN_MAX_PARTS
+    return workspace.numel() // (Tq * Hq * (D + 1))
+
+
+def _merge_cuts(po, pl, S: int, Tq: int, q_b_start_loc, q_b_seq_len, max_q_len: int, mode: int, o, lse=None, m=None, l=None):
+    a = _lib.MergeCutsArgs()
+    a.o_parts, a.lse_parts, a.part_rows, a.n_parts, a.mode = po.data_ptr(), pl.data_ptr(), Tq, S, mode
+    a.batch, a.num_q_heads, a.head_dim, a.max_q_len = q_b_seq_len.shape[0], po.shape[1], po.shape[2], int(max_q_len)
+    a.q_b_start_loc, a.q_b_seq_len = q_b_start_loc.data_ptr(), q_b_seq_len.data_ptr()
+    a.o, a.o_stride_t, a.o_stride_h, a.o_dtype = o.data_ptr(), o.stride(0), o.stride(1), _DT[o.dtype]
+    if mode == 1:
+        a.m, a.l, a.ml_stride_t, a.ml_stride_h = m.data_ptr(), l.data_ptr(), m.stride(0), m.stride(1)
+    else:
+        a.lse = lse.data_ptr()
+    _lib.check(_lib.load().lsattn_prefill_merge_cuts(C.byref(a), _stream()), "lsattn_prefill_merge_cuts")
+
+
+# Launches below this many 128-row workgroups (batch x query heads x ceil(max_q / 128)) are cut along the keys when the
+# KV chunks may hold at least KV_SPLIT_MIN_KEYS keys: 256 CUs run one workgroup each.
+KV_SPLIT_BELOW_WORKGROUPS = 192
+KV_SPLIT_MIN_KEYS = 8192
+
+
+def kv_split_count(batch: int, num_q_heads: int, max_q_len: int, kv_rows: int) -> int:
+    """KV cuts the prefill operators use by themselves: enough for about two workgroups per CU, cuts of at least 2048
+    keys (kv_rows bounds every sequence's chunk: max_kv_len where the caller gives it, else the rows of the k buffer;
+    the lengths themselves live on the device)."""
+    wgs = batch * num_q_heads * ((max_q_len + 127) // 128)
+    if wgs <= 0 or wgs >= KV_SPLIT_BELOW_WORKGROUPS or kv_rows < KV_SPLIT_MIN_KEYS:
+        return 1
+    return max(1, min(_lib.LSATTN_MAX_PARTS - 1, 512 // wgs, kv_rows // 2048))
+
+
+def _cut_len(kv_rows: int, S: int) -> int:
+    """Keys per cut: kv_rows over S cuts, rounded up to the kernel's 64-key tile."""
+    return -(-(-(-kv_rows // S)) // 64) * 64
 
 
 @torch.inference_mode()
 def context_attention_fwd(q, k, v, o, q_b_start_loc, q_b_seq_len, q_first_token_global_idx,
                           kv_b_start_loc, kv_b_seq_len, kv_first_token_global_idx,
                           logical_sp_peers_num: int, max_q_b_seq_len: int, m, l, *, v_f16: Optional[torch.Tensor] = None,
-                          v_f16_valid: bool = False) -> None:
+                          v_f16_valid: bool = False, workspace=None, max_kv_len: Optional[int] = None,
+                          kv_splits: Optional[int] = None) -> None:
     """One ring-attention step folded in place into (o, m, l); signature of RING:191-206.
 
     Keyword-only additions for bfloat16 inputs (the reference is fp16 only): the kernel multiplies P and V in fp16, so V is
     rewritten as fp16 first.  v_f16 is the caller's buffer for that copy (contiguous float16, v's shape): with it the call
     allocates nothing; v_f16_valid=True says it already holds the copy of this v (e.g. from an earlier step over the same
     chunk) and skips the conversion.
+
+    Keyword-only, for short query chunks against a long KV chunk (a chunked-prefill step of a long request): the launch has
+    one workgroup per 128 query rows and head, too few for the chip.  With workspace (a contiguous float32 tensor the caller
+    owns, S * Tq * Hq * (D + 1) elements for S cuts; or a pair of tensors [S*Tq,Hq,D], [S*Tq,Hq]) the KV chunks are cut
+    into S slices inside one launch that writes S fp32 partials per row to the workspace, and a second launch folds
+    them into (o, m, l) by the same update (RING:171-188).  S follows kv_split_count (from shapes alone; max_kv_len, an
+    upper bound of every chunk's length, replaces the rows of the k buffer there: in the layer k is a view of a buffer
+    sized for the longest batch), capped by what the workspace holds; kv_splits forces it.  Without a workspace the call
+    is the reference's: one launch, no scratch.  (m, l) stay opaque: a step folded this way enters as (its LSE, 1).
 
     Call it repeatedly with the same local q/o/m/l and a different kv chunk each time.
     Start from m = -inf, l = 0 (o need not be zeroed).  After k calls o is the
@@ -177,35 +254,37 @@ def context_attention_fwd(q, k, v, o, q_b_start_loc, q_b_seq_len, q_first_token_
         # (the step folds into it), and copy the first D columns back
         o_user, o = o, _pad_head_dim(o)
         q, k, v = _pad_head_dim(q), _pad_head_dim(k), _pad_head_dim(v)
-    a = _prefill_args(q, k, v, o, q_b_start_loc, q_b_seq_len, q_first_token_global_idx, kv_b_start_loc,
-                      kv_b_seq_len, kv_first_token_global_idx, logical_sp_peers_num, max_q_b_seq_len,
-                      1.0 / (D ** 0.5), v_f16 if o_user is None else None, v_f16_valid and o_user is None)
     for t, n in ((m, "m"), (l, "l")):
         _dev(t, n)
         if t.dtype != torch.float32 or t.dim() != 2 or tuple(t.shape) != (q.shape[0], q.shape[1]):
             raise ValueError("%s must be float32 [tokens, q_heads]" % n)
     if m.stride() != l.stride():
         raise ValueError("m and l must share strides")
+    S = 1
+    if workspace is not None and o_user is None and q.dim() == 3:
+        kv_rows = k.shape[0] if max_kv_len is None else int(max_kv_len)
+        S = kv_split_count(q_b_seq_len.shape[0], q.shape[1], int(max_q_b_seq_len), kv_rows) if kv_splits is None else int(kv_splits)
+        S = min(S, _workspace_cuts(workspace, q.shape[0], q.shape[1], D), _lib.LSATTN_MAX_PARTS)
+    if S > 1:
+        Tq = q.shape[0]
+        po, pl = _cut_workspace(workspace, S, Tq, q.shape[1], D, q.device)
+        a = _prefill_args(q, k, v, po, q_b_start_loc, q_b_seq_len, q_first_token_global_idx, kv_b_start_loc,
+                          kv_b_seq_len, kv_first_token_global_idx, logical_sp_peers_num, max_q_b_seq_len,
+                          1.0 / (D ** 0.5), v_f16, v_f16_valid, cuts=(S, _cut_len(kv_rows, S), Tq))
+        a.lse = pl.data_ptr()
+        if o.dim() != 3 or o.stride(2) != 1:
+            raise ValueError("o must be [tokens, heads, head_dim], contiguous in head_dim")
+        _lib.check(_lib.load().lsattn_prefill_step(C.byref(a), _stream()), "lsattn_prefill_step")
+        _merge_cuts(po, pl, S, Tq, q_b_start_loc, q_b_seq_len, max_q_b_seq_len, 1, o, m=m, l=l)
+        return
+    a = _prefill_args(q, k, v, o, q_b_start_loc, q_b_seq_len, q_first_token_global_idx, kv_b_start_loc,
+                      kv_b_seq_len, kv_first_token_global_idx, logical_sp_peers_num, max_q_b_seq_len,
+                      1.0 / (D ** 0.5), v_f16 if o_user is None else None, v_f16_valid and o_user is None)
     a.m, a.l = m.data_ptr(), l.data_ptr()
     a.ml_stride_t, a.ml_stride_h = m.stride(0), m.stride(1)
     _lib.check(_lib.load().lsattn_prefill_step_merge(C.byref(a), _stream()), "lsattn_prefill_step_merge")
     if o_user is not None:
         o_user.copy_(o[..., :D])
-
-
-# Launches below this many 128-row workgroups (batch x query heads x ceil(max_q / 128)) are cut along the keys when the
-# KV buffer holds at least KV_SPLIT_MIN_KEYS rows: 256 CUs run one workgroup each.
-KV_SPLIT_BELOW_WORKGROUPS = 192
-KV_SPLIT_MIN_KEYS = 8192
-
-
-def kv_split_count(batch: int, num_q_heads: int, max_q_len: int, kv_rows: int) -> int:
-    """KV slices prefill_attention_step uses by itself: enough for about two workgroups per CU, slices of at least 2048
-    keys (kv_rows, the rows of the k buffer, bounds every sequence's chunk: the lengths themselves live on the device)."""
-    wgs = batch * num_q_heads * ((max_q_len + 127) // 128)
-    if wgs <= 0 or wgs >= KV_SPLIT_BELOW_WORKGROUPS or kv_rows < KV_SPLIT_MIN_KEYS:
-        return 1
-    return max(1, min(_lib.LSATTN_MAX_PARTS - 1, 512 // wgs, kv_rows // 2048))
 
 
 @torch.inference_mode()
@@ -215,14 +294,15 @@ def prefill_attention_step(q, k, v, q_b_start_loc, q_b_seq_len, q_first_token_gl
                            out: Optional[torch.Tensor] = None, lse: Optional[torch.Tensor] = None,
                            sm_scale: Optional[float] = None, accumulate: bool = False, v_f16: Optional[torch.Tensor] = None,
                            v_f16_valid: bool = False, kv_splits: Optional[int] = None,
-                           kv_split_workspace: Optional[Tuple[torch.Tensor, torch.Tensor]] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+                           kv_split_workspace=None, max_kv_len: Optional[int] = None) -> Tuple[torch.Tensor, torch.Tensor]:
     """One step as a mergeable partial: (O fp32 [Tq,Hq,D] normalised, LSE fp32 [Tq,Hq]).
     v_f16 / v_f16_valid: as in context_attention_fwd (the caller's buffer for the fp16 copy of a bfloat16 v).
     kv_splits: short query chunks against a long KV chunk give the launch too few workgroups for the chip (one per 128
-    query rows and head); with kv_splits = S > 1 every sequence's KV chunk is cut into S slices, one launch computes the S
-    partials of every row (the sequence entered once per slice, lsattn_prefill_args.o_b_start_loc) and lsattn_lse_merge
-    joins them.  None chooses S from the shapes (kv_split_count), 1 switches it off.  The partials take S times the
-    size of (out, lse): kv_split_workspace = (float32 [S*Tq,Hq,D], float32 [S*Tq,Hq]) passes the caller's buffers for them.
+    query rows and head); with kv_splits = S > 1 every sequence's KV chunk is cut into S slices inside one launch, which
+    computes the S partials of every row (lsattn_prefill_args.kv_cuts), and lsattn_prefill_merge_cuts joins them for the
+    rows of the sequences.  None chooses S from the shapes (kv_split_count over max_kv_len, an upper bound of every
+    chunk's length; the rows of the k buffer if not given), 1 switches it off.  The partials take S times the size of
+    (out, lse): kv_split_workspace passes the caller's memory for them (as context_attention_fwd's workspace).
 
     Same inputs as context_attention_fwd; rows that see no key get O = 0, LSE = -inf.
     With accumulate=True the step is LSE-merged into the (out, lse) passed in (a running partial of earlier steps over
@@ -245,37 +325,21 @@ def prefill_attention_step(q, k, v, q_b_start_loc, q_b_seq_len, q_first_token_gl
         q, k, v = _pad_head_dim(q), _pad_head_dim(k), _pad_head_dim(v)
         if sm_scale is None:
             sm_scale = 1.0 / (D ** 0.5)
-    S = kv_split_count(q_b_seq_len.shape[0], q.shape[1], int(max_q_b_seq_len), k.shape[0]) if kv_splits is None else int(kv_splits)
+    kv_rows = k.shape[0] if max_kv_len is None else int(max_kv_len)
+    S = kv_split_count(q_b_seq_len.shape[0], q.shape[1], int(max_q_b_seq_len), kv_rows) if kv_splits is None else int(kv_splits)
     if S > 1:
-        if S + (1 if accumulate else 0) > _lib.LSATTN_MAX_PARTS:
-            raise ValueError("at most %d KV slices" % (_lib.LSATTN_MAX_PARTS - 1))
-        Tq, P = q.shape[0], int(logical_sp_peers_num)
-        L = -(-(-(-k.shape[0] // S)) // 64) * 64  # keys per slice: a multiple of the kernel's 64-key tile
-        if kv_split_workspace is None:
-            po = torch.empty((S * Tq,) + tuple(q.shape[1:]), dtype=torch.float32, device=q.device)
-            pl = torch.empty((S * Tq, q.shape[1]), dtype=torch.float32, device=q.device)
-        else:
-            po, pl = kv_split_workspace
-            if (po.dtype != torch.float32 or pl.dtype != torch.float32 or tuple(po.shape) != (S * Tq,) + tuple(q.shape[1:])
-                    or tuple(pl.shape) != (S * Tq, q.shape[1]) or not po.is_contiguous() or not pl.is_contiguous()):
-                raise ValueError("kv_split_workspace: contiguous float32 [S*Tq,Hq,D] and [S*Tq,Hq]")
-        # slice s of a sequence: keys [s L, (s+1) L) of its chunk; key n of the chunk has global position kv_first + n P
-        step = torch.arange(S, dtype=torch.int32, device=q.device)[:, None]
-        kv_start_x = (kv_b_start_loc[None, :] + step * L).reshape(-1)
-        kv_len_x = (kv_b_seq_len[None, :] - step * L).clamp_(0, L).reshape(-1)
-        kv_first_x = (kv_first_token_global_idx[None, :] + step * (L * P)).reshape(-1)
-        o_start_x = (q_b_start_loc[None, :] + step * Tq).reshape(-1)
-        a = _prefill_args(q, k, v, po, q_b_start_loc.repeat(S), q_b_seq_len.repeat(S), q_first_token_global_idx.repeat(S),
-                          kv_start_x, kv_len_x, kv_first_x, P, max_q_b_seq_len, sm_scale,
-                          v_f16 if out_user is None else None, v_f16_valid and out_user is None, o_b_start_loc=o_start_x)
+        if S > _lib.LSATTN_MAX_PARTS:
+            raise ValueError("at most %d KV slices" % _lib.LSATTN_MAX_PARTS)
+        if out.dim() != 3 or out.stride(2) != 1 or tuple(out.shape) != tuple(q.shape):
+            raise ValueError("out must have q's shape and be contiguous in head_dim")
+        Tq = q.shape[0]
+        po, pl = _cut_workspace(kv_split_workspace, S, Tq, q.shape[1], q.shape[2], q.device)
+        a = _prefill_args(q, k, v, po, q_b_start_loc, q_b_seq_len, q_first_token_global_idx, kv_b_start_loc, kv_b_seq_len,
+                          kv_first_token_global_idx, logical_sp_peers_num, max_q_b_seq_len, sm_scale,
+                          v_f16 if out_user is None else None, v_f16_valid and out_user is None, cuts=(S, _cut_len(kv_rows, S), Tq))
         a.lse = pl.data_ptr()
         _lib.check(_lib.load().lsattn_prefill_step(C.byref(a), _stream()), "lsattn_prefill_step")
-        parts = [(po[s * Tq:(s + 1) * Tq], pl[s * Tq:(s + 1) * Tq]) for s in range(S)]
-        if accumulate:
-            parts.append((out, lse))  # (the merge reads a row of every part before it writes that row)
-        if not out.is_contiguous():
-            raise ValueError("kv_splits needs a contiguous out")
-        lse_merge(parts, out=out, lse=lse)
+        _merge_cuts(po, pl, S, Tq, q_b_start_loc, q_b_seq_len, max_q_b_seq_len, 2 if accumulate else 0, out, lse=lse)
         if out_user is not None:
             out_user.copy_(out[..., :D])
             out = out_user

@@ -24,24 +24,29 @@ def lsa():
 
 PREFILL_GEOMETRIES = {
     "library-choice": {},
-    "rows128": {"LSATTN_PREFILL_ROWS": "128"},
-    "rows256-head-major": {"LSATTN_PREFILL_ROWS": "256", "LSATTN_PREFILL_ORDER": "head"},
-    "rows256-tile-major": {"LSATTN_PREFILL_ROWS": "256", "LSATTN_PREFILL_ORDER": "tile"},
-    "rows256-one-head": {"LSATTN_PREFILL_ROWS": "256", "LSATTN_PREFILL_PACK": "0"},
-    "rows128-one-head": {"LSATTN_PREFILL_ROWS": "128", "LSATTN_PREFILL_PACK": "0"},
-    "rows128-four-waves": {"LSATTN_PREFILL_ROWS": "half"},
-    "rows128-four-waves-one-head": {"LSATTN_PREFILL_ROWS": "half", "LSATTN_PREFILL_PACK": "0"},
+    "rows128": {"prefill_rows": "128"},
+    "rows256-head-major": {"prefill_rows": "256", "prefill_order": "head"},
+    "rows256-tile-major": {"prefill_rows": "256", "prefill_order": "tile"},
+    "rows256-one-head": {"prefill_rows": "256", "prefill_pack": "off"},
+    "rows128-one-head": {"prefill_rows": "128", "prefill_pack": "off"},
+    "rows128-four-waves": {"prefill_rows": "half"},
+    "rows128-four-waves-one-head": {"prefill_rows": "half", "prefill_pack": "off"},
 }
 
 
+@pytest.fixture
+def tuning(lsa):
+    """set_tuning of the library for the length of a test: call it with the choices to force; the library's own choices
+    come back when the test ends."""
+    yield lsa.set_tuning
+    lsa.set_tuning()
+
+
 @pytest.fixture(params=list(PREFILL_GEOMETRIES))
-def prefill_geometry(request, monkeypatch):
+def prefill_geometry(request, tuning):
     """Runs a prefill test once per workgroup shape (128 or 256 query rows; the query heads of a KV head side by side in
     a workgroup, the library's way wherever the group size allows, or one head per workgroup) and grid order (one KV head
     at a time per XCD, or the heaviest query tiles of all KV heads first) of the prefill kernel.  The library picks both from the size
     of the launch; the test shapes alone would leave most combinations to the few large cases."""
-    for name in ("LSATTN_PREFILL_ROWS", "LSATTN_PREFILL_ORDER", "LSATTN_PREFILL_PACK"):
-        monkeypatch.delenv(name, raising=False)
-    for name, value in PREFILL_GEOMETRIES[request.param].items():
-        monkeypatch.setenv(name, value)
+    tuning(**PREFILL_GEOMETRIES[request.param])
     return request.param

@@ -24,7 +24,9 @@ def test_library_exports_every_declared_symbol():
     assert set(names) == set(_lib.EXPORTS), (names, sorted(_lib.EXPORTS))
     for n in names:
         assert getattr(lib, n) is not None
-    assert lib.lsattn_version() == 2  # LSATTN_VERSION of include/lsattn.h: the argument blocks as _lib.py declares them
+    # LSATTN_VERSION of include/lsattn.h: the argument blocks as _lib.py declares them
+    header = open(os.path.join(ROOT, "include", "lsattn.h")).read()
+    assert lib.lsattn_version() == _lib.LSATTN_VERSION == int(re.search(r"#define LSATTN_VERSION (\d+)", header).group(1))
     assert lib.lsattn_strerror(0) == b"ok"
     assert b"invalid" in lib.lsattn_strerror(-1)
 
@@ -43,6 +45,8 @@ int main(void) {
          sizeof(lsattn_decode_stage1_args), sizeof(lsattn_decode_stage2_args), sizeof(lsattn_kv_copy_register_args));
   printf("%zu %zu\n", sizeof(lsattn_decode_migration_args), offsetof(lsattn_decode_migration_args, b_seq_len));
   printf("%zu %zu\n", sizeof(lsattn_rotary_kv_write_args), offsetof(lsattn_rotary_kv_write_args, register_mode));
+  printf("%zu %zu\n", sizeof(lsattn_tuning), offsetof(lsattn_tuning, decode_listed));
+  printf("%zu %zu %zu\n", sizeof(lsattn_merge_cuts_args), offsetof(lsattn_merge_cuts_args, ml_stride_h), offsetof(lsattn_prefill_args, o_cut_rows));
   printf("%zu %zu %zu %zu %zu %zu\n", offsetof(lsattn_prefill_args, sm_scale), offsetof(lsattn_prefill_args, ml_stride_h),
          offsetof(lsattn_decode_stage1_args, req_to_tokens), offsetof(lsattn_decode_stage2_args, block_seq),
          offsetof(lsattn_kv_copy_register_args, req_to_tokens), offsetof(lsattn_kv_copy_register_args, should_register));
@@ -57,7 +61,11 @@ int main(void) {
     sizes = [int(x) for x in out[:5]]
     mig = [int(x) for x in out[5:7]]
     rot = [int(x) for x in out[7:9]]
-    offs = [int(x) for x in out[9:]]
+    tun = [int(x) for x in out[9:11]]
+    cuts = [int(x) for x in out[11:14]]
+    offs = [int(x) for x in out[14:]]
+    assert cuts == [C.sizeof(_lib.MergeCutsArgs), _lib.MergeCutsArgs.ml_stride_h.offset, _lib.PrefillArgs.o_cut_rows.offset]
+    assert tun == [C.sizeof(_lib.Tuning), _lib.Tuning.decode_listed.offset]
     assert rot == [C.sizeof(_lib.RotaryKvWriteArgs), _lib.RotaryKvWriteArgs.register_mode.offset]
     assert mig == [C.sizeof(_lib.DecodeMigrationArgs), _lib.DecodeMigrationArgs.b_seq_len.offset]
     assert sizes == [C.sizeof(_lib.PrefillArgs), C.sizeof(_lib.MergeArgs), C.sizeof(_lib.DecodeStage1Args),
@@ -122,6 +130,28 @@ def test_validation_rejects_bad_arguments_without_gpu():
     for ks, vs in ((0, 256), (256, -256), ((1 << 24) + 8, 256), (256, 1 << 25)):
         a.k_stride_t, a.v_stride_t = ks, vs
         assert lib.lsattn_prefill_step(C.byref(a), None) == -1, (ks, vs)
+    # the chunk cut along the keys: fp32 partials only, whole 64-key tiles per cut, the cuts' rows apart
+    a.k_stride_t = a.v_stride_t = 256
+    a.kv_cuts, a.kv_cut_len, a.o_cut_rows = 4, 100, 8
+    assert lib.lsattn_prefill_step(C.byref(a), None) == -1          # not a multiple of 64 keys
+    a.kv_cut_len, a.o_cut_rows = 128, 0
+    assert lib.lsattn_prefill_step(C.byref(a), None) == -1          # no room between the cuts' outputs
+    a.o_cut_rows, a.kv_cuts = 8, 17
+    assert lib.lsattn_prefill_step(C.byref(a), None) == -1          # more cuts than LSATTN_MAX_PARTS
+    a.kv_cuts = 4
+    assert lib.lsattn_prefill_step_accumulate(C.byref(a), None) == -1  # the folding steps take no cuts
+    mc = _lib.MergeCutsArgs()
+    assert lib.lsattn_prefill_merge_cuts(C.byref(mc), None) == -1
+    assert lib.lsattn_prefill_merge_cuts(None, None) == -1
+    for f in ("o_parts", "lse_parts", "q_b_start_loc", "q_b_seq_len", "o", "lse"):
+        setattr(mc, f, fake)
+    mc.n_parts, mc.batch, mc.num_q_heads, mc.head_dim, mc.max_q_len, mc.part_rows = 2, 1, 4, 64, 8, 8
+    mc.o_stride_t, mc.o_stride_h, mc.o_dtype = 512, 128, _lib.LSATTN_F32
+    assert lib.lsattn_prefill_merge_cuts(C.byref(mc), None) == -2   # head_dim
+    mc.head_dim, mc.mode = 128, 1
+    assert lib.lsattn_prefill_merge_cuts(C.byref(mc), None) == -1   # mode 1 needs m, l and a 16-bit o
+    mc.mode, mc.n_parts = 0, 17
+    assert lib.lsattn_prefill_merge_cuts(C.byref(mc), None) == -1
     # the fused decode call refuses argument blocks that do not describe the same partials
     s1, s2 = _lib.DecodeStage1Args(), _lib.DecodeStage2Args()
     assert lib.lsattn_decode_attention(None, C.byref(s2), None) == -1
@@ -141,6 +171,52 @@ def test_validation_rejects_bad_arguments_without_gpu():
     for bad in (-1, 17):
         s3.merge_blocks = bad
         assert lib.lsattn_decode_stage1(C.byref(s3), None) == -1, bad
+
+
+def test_tuning_block_is_validated_and_named_values_match_the_header():
+    """lsattn_set_tuning takes the values include/lsattn.h names, refuses others, and NULL restores the library's choices;
+    the names the Python side uses stand for the header's numbers."""
+    from loongserve_amd import _lib
+    lib = _lib.load()
+    header = open(os.path.join(ROOT, "include", "lsattn.h")).read()
+    num = {k: int(v) for k, v in re.findall(r"#define (LSATTN_(?:PREFILL|DECODE)_[A-Z0-9_]+) (\d+)", header)}
+    want = {("prefill_rows", "128"): "LSATTN_PREFILL_ROWS_128", ("prefill_rows", "256"): "LSATTN_PREFILL_ROWS_256",
+            ("prefill_rows", "half"): "LSATTN_PREFILL_ROWS_HALF", ("prefill_order", "tile"): "LSATTN_PREFILL_ORDER_TILE",
+            ("prefill_order", "head"): "LSATTN_PREFILL_ORDER_HEAD", ("prefill_pack", "off"): "LSATTN_PREFILL_PACK_OFF",
+            ("decode_stage1", "lane"): "LSATTN_DECODE_STAGE1_LANE", ("decode_stage1", "mfma"): "LSATTN_DECODE_STAGE1_MFMA",
+            ("decode_stage1", "split"): "LSATTN_DECODE_STAGE1_SPLIT", ("decode_listed", "off"): "LSATTN_DECODE_LISTED_OFF",
+            ("decode_listed", "on"): "LSATTN_DECODE_LISTED_ON"}
+    assert len(num) == len(want)
+    for (field, name), macro in want.items():
+        assert _lib.TUNING_VALUES[field][name] == num[macro]
+        assert _lib.TUNING_VALUES[field][None] == 0
+    try:
+        t = _lib.Tuning()
+        for field, top in (("prefill_rows", 3), ("prefill_order", 2), ("prefill_pack", 1), ("decode_stage1", 3), ("decode_listed", 2)):
+            for bad in (-1, top + 1):
+                t = _lib.Tuning()
+                setattr(t, field, bad)
+                assert lib.lsattn_set_tuning(C.byref(t)) == -1, (field, bad)
+            t = _lib.Tuning()
+            setattr(t, field, top)
+            assert lib.lsattn_set_tuning(C.byref(t)) == 0
+        t = _lib.Tuning()
+        t.reserved[1] = 1
+        assert lib.lsattn_set_tuning(C.byref(t)) == -1
+        with pytest.raises(ValueError):
+            _lib.set_tuning(prefill_rows="512")
+        with pytest.raises(ValueError):
+            _lib.set_tuning(no_such_choice="x")
+    finally:
+        assert lib.lsattn_set_tuning(None) == 0
+
+
+def test_library_reads_no_environment_variable():
+    """The launch choices come from lsattn_set_tuning alone: no source of the library calls getenv."""
+    csrc = os.path.join(ROOT, "loongserve_amd", "csrc")
+    for name in os.listdir(csrc):
+        if name.endswith((".hip", ".h")):
+            assert "getenv" not in open(os.path.join(csrc, name)).read(), name
 
 
 def test_python_wrappers_reject_cpu_tensors():

@@ -130,14 +130,13 @@ def _check_merge_blocks(lsa, dtype, merge, Hq, Hkv, BS, lens):
     assert_lse_close(l_d, l_ref, "lse")
 
 
-@pytest.fixture(params=["1", "2", "1 listed"], ids=["plain", "split", "listed"])
-def matrix_pipe(monkeypatch, request):
+@pytest.fixture(params=["mfma", "split", "mfma listed"], ids=["plain", "split", "listed"])
+def matrix_pipe(tuning, request):
     """Stage 1 through the matrix-pipe kernel wherever its conditions hold, whatever the launch's size: its plain shape
     (a wave per 256 tokens; blocks a multiple of 32 tokens; by itself the library takes it for large launches), the
     shape whose four waves split a block (blocks a multiple of 128 tokens; small launches of groups of four and more),
     and the plain shape over a list of the units that exist (by itself: launches of very many workgroups)."""
-    monkeypatch.setenv("LSATTN_DECODE_MFMA", request.param[0])
-    monkeypatch.setenv("LSATTN_DECODE_LISTED", "1" if "listed" in request.param else "0")
+    tuning(decode_stage1=request.param.split()[0], decode_listed="on" if "listed" in request.param else "off")
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
@@ -164,8 +163,8 @@ def test_matrix_pipe_stage1_forced_merge_blocks(lsa, matrix_pipe, dtype, merge, 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_large_group_launch_that_takes_the_matrix_pipe_by_itself(lsa, dtype):
     """64 query heads over 8 KV heads, 2 requests of about 17000 tokens: 2 x 8 x 67 waves of the matrix-pipe kernel, the
-    library's own choice (no environment override), through the fused call and through the two stages."""
-    assert "LSATTN_DECODE_MFMA" not in __import__("os").environ
+    library's own choice (nothing forced), through the fused call and through the two stages."""
+    lsa.set_tuning()
     B, Hq, Hkv, D, BS = 2, 64, 8, 128, 256
     lens = [17000, 16411]
     q, kv, table, b_req, b_len = decode_case(77, B, Hq, Hkv, D, lens, sum(lens) + 1000, dtype)
@@ -198,10 +197,9 @@ def test_large_group_launch_that_takes_the_matrix_pipe_by_itself(lsa, dtype):
 def test_skewed_batch_that_walks_the_unit_list_by_itself(lsa, dtype):
     """One request of 40000 tokens among 127 of 1 to 300 (and two of none), 64 tokens per partial: the plain grid would
     be 157 x 2 x 130 = 40820 workgroups, nearly all of them without work, so the library walks the list of the units
-    that exist (its own choice: no environment override).  Two stages, per-block partials; rows no request reaches stay
+    that exist (its own choice: nothing forced).  Two stages, per-block partials; rows no request reaches stay
     untouched."""
-    env = __import__("os").environ
-    assert "LSATTN_DECODE_MFMA" not in env and "LSATTN_DECODE_LISTED" not in env
+    lsa.set_tuning()
     import random
     rng = random.Random(5)
     B, Hq, Hkv, D, BS = 130, 32, 8, 128, 64
@@ -261,12 +259,11 @@ def test_fused_call_gives_the_same_bits_with_either_layout_of_its_partials(lsa, 
 
 
 @pytest.mark.parametrize("B", [1024, 1025])
-def test_unit_list_at_its_largest_batch_and_past_it(lsa, monkeypatch, B):
+def test_unit_list_at_its_largest_batch_and_past_it(lsa, tuning, B):
     """The list of units is numbered in LDS for up to 1024 requests; a larger batch takes the plain grid whatever the
-    environment asks for.  Requests of 0 to 120 tokens and one of 9000, 64 tokens per partial."""
+    tuning block asks for.  Requests of 0 to 120 tokens and one of 9000, 64 tokens per partial."""
     import random
-    monkeypatch.setenv("LSATTN_DECODE_MFMA", "1")
-    monkeypatch.setenv("LSATTN_DECODE_LISTED", "1")
+    tuning(decode_stage1="mfma", decode_listed="on")
     rng = random.Random(B)
     Hq, Hkv, D, BS = 8, 2, 128, 64
     lens = [rng.randint(0, 120) for _ in range(B)]
@@ -447,7 +444,7 @@ def test_one_request_of_a_million_tokens(lsa):
 
 
 @pytest.mark.parametrize("seed", [3, 11, 42])
-def test_random_decode_shapes_on_both_stage1_kernels(lsa, monkeypatch, seed):
+def test_random_decode_shapes_on_both_stage1_kernels(lsa, tuning, seed):
     """Seeded random sweep of stage 1 + stage 2 against the oracle, once with the library's own choice of stage-1 kernel
     and once through each shape of the matrix-pipe kernel wherever its conditions hold (plain grid, split waves, listed
     units): ragged batches with requests of a single token,
@@ -472,13 +469,11 @@ def test_random_decode_shapes_on_both_stage1_kernels(lsa, monkeypatch, seed):
         o_ref, l_ref = orc.decode_full(q, k, v, table, b_req, b_len)
         kvd, qd, td, rd, ld = kv.to(DEV), q.to(DEV), table.to(DEV), b_req.to(DEV), b_len.to(DEV)
         nblk = (max(lens) + BS - 1) // BS
-        for forced in (False, "1", "2", "1 listed"):
-            monkeypatch.delenv("LSATTN_DECODE_LISTED", raising=False)
+        for forced in (False, "mfma", "split", "mfma listed"):
             if forced:
-                monkeypatch.setenv("LSATTN_DECODE_MFMA", forced[0])
-                monkeypatch.setenv("LSATTN_DECODE_LISTED", "1" if "listed" in forced else "0")
+                tuning(decode_stage1=forced.split()[0], decode_listed="on" if "listed" in forced else "off")
             else:
-                monkeypatch.delenv("LSATTN_DECODE_MFMA", raising=False)
+                tuning()
             mo_d = torch.full((nblk, B, Hq, D), float("nan"), device=DEV)
             ml_d = torch.full((nblk, B, Hq), float("nan"), device=DEV)
             lsa.longserve_cuda_kernels.flash_decoding_stage1(mo_d, ml_d, qd, kvd[:, :Hkv], kvd[:, Hkv:], td, rd, ld, max(lens), BS, merge)

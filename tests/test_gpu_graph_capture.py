@@ -12,9 +12,9 @@ DEV = "cuda:0"
 
 
 @pytest.mark.parametrize("kernel", ["the library's choice", "matrix pipe"])
-def test_decode_step_replays_match_eager(lsa, monkeypatch, kernel):
+def test_decode_step_replays_match_eager(lsa, tuning, kernel):
     if kernel == "matrix pipe":  # (a launch this small takes the lane kernel by itself)
-        monkeypatch.setenv("LSATTN_DECODE_MFMA", "1")
+        tuning(decode_stage1="mfma")
     B, Hq, Hkv, D, BS = 4, 8, 2, 128, 64
     pool, max_len = 4000, 900
     _, kv, _, _, _ = decode_case(300, B, Hq, Hkv, D, [1] * B, pool)

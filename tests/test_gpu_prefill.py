@@ -427,6 +427,92 @@ def test_short_queries_against_long_kv_split_along_the_keys(lsa, dtype, P):
     assert bool((l_run.cpu()[~seen] == float("-inf")).all())
 
 
+def test_kv_cuts_leave_rows_outside_the_sequences_alone(lsa):
+    """Rows of q / out that belong to no sequence (a gap between two sequences and a tail) keep what they hold on the
+    route cut along the keys, as on the unsplit one, with and without accumulate; the partials' workspace starts as NaN.
+    One tensor as workspace, max_kv_len as the bound the cuts are sized by (the k buffer is much taller than the chunks)."""
+    Hq, Hkv, D, P = 8, 2, 128, 1
+    qlens, klens = [130, 40], [9000, 12000]
+    q = rand_t((200, Hq, D), 4401)                       # rows 130..139 and 180..199 belong to no sequence
+    k = rand_t((40000, Hkv, D), 4402)                    # chunks at rows 100 and 20000 of a tall buffer
+    v = rand_t((40000, Hkv, D), 4403)
+    qm = (torch.tensor([0, 140], dtype=torch.int32), torch.tensor(qlens, dtype=torch.int32), torch.tensor([50000, 11000], dtype=torch.int32))
+    km = (torch.tensor([100, 20000], dtype=torch.int32), torch.tensor(klens, dtype=torch.int32), torch.tensor([0, 0], dtype=torch.int32))
+    o_ref, lse_ref = orc.attn_step(q, k, v, *qm, *km, P)
+    covered = torch.zeros(200, dtype=torch.bool)
+    covered[0:130] = True
+    covered[140:180] = True
+    dq, dk, dv = q.to(DEV), k.to(DEV), v.to(DEV)
+    dqm, dkm = [t.to(DEV) for t in qm], [t.to(DEV) for t in km]
+    from loongserve_amd import ops
+    assert ops.kv_split_count(2, Hq, max(qlens), max(klens)) > 1
+    S = 6
+    ws = torch.full((S * 200 * Hq * (D + 1) + 7,), float("nan"), device=DEV)
+    out = torch.full((200, Hq, D), 7.0, device=DEV)
+    lse = torch.full((200, Hq), 7.0, device=DEV)
+    lsa.prefill_attention_step(dq, dk, dv, *dqm, *dkm, P, max(qlens), out=out, lse=lse, kv_splits=S, kv_split_workspace=ws,
+                               max_kv_len=max(klens))
+    torch.cuda.synchronize()
+    assert_o_close(out.cpu()[covered], o_ref[covered], "O")
+    assert_lse_close(lse.cpu()[covered], lse_ref[covered], "LSE")
+    assert bool((out.cpu()[~covered] == 7.0).all()) and bool((lse.cpu()[~covered] == 7.0).all())
+    # accumulate onto an empty running partial whose rows outside the sequences hold a sentinel
+    out2 = torch.full((200, Hq, D), float("nan"), device=DEV)
+    lse2 = torch.full((200, Hq), float("-inf"), device=DEV)
+    out2[~covered.to(DEV)] = 3.0
+    lse2[~covered.to(DEV)] = 3.0
+    lsa.prefill_attention_step(dq, dk, dv, *dqm, *dkm, P, max(qlens), out=out2, lse=lse2, accumulate=True, max_kv_len=max(klens))
+    torch.cuda.synchronize()
+    assert_o_close(out2.cpu()[covered], o_ref[covered], "O, accumulated onto empty rows")
+    assert_lse_close(lse2.cpu()[covered], lse_ref[covered], "LSE, accumulated onto empty rows")
+    assert bool((out2.cpu()[~covered] == 3.0).all()) and bool((lse2.cpu()[~covered] == 3.0).all())
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("P", [1, 3])
+def test_context_attention_fwd_with_a_workspace_cuts_the_kv_chunk(lsa, dtype, P):
+    """The reference's operator with workspace=: short query chunks (a chunked-prefill step) against KV chunks of up to
+    20000 keys, GQA 8/2.  Three steps into one (o, m, l): from the start state through the cut route, an ordinary step,
+    and a cut step on top of the running state; against the oracle's restatement of the same update after every step, and
+    the final result against one exact step over all keys.  o, m, l strided views (RING:270-275 pass their strides)."""
+    Hq, Hkv, D = 8, 2, 128
+    qlens = [100, 7, 64]
+    Tq = sum(qlens)
+    q = rand_t((Tq, Hq, D), 4500 + P, dtype)
+    chunks = []
+    for j, klens in enumerate(([20000, 3000, 0], [500, 200, 300], [9000, 11000, 8200])):
+        k = rand_t((sum(klens), Hkv, D), 4510 + 10 * j + P, dtype)
+        v = rand_t((sum(klens), Hkv, D), 4511 + 10 * j + P, dtype)
+        kf = [j, 100000 * P + j, 40000 * P + j] if P > 1 else [30000 * j, 300000 + 20000 * j, 100000 + 20000 * j]
+        chunks.append((k, v, meta(klens, kf), klens))
+    qf = [59990 * P + 1, 390000 * P, 150000 * P]  # sequence 0 ends inside chunk 2's first KV range when P = 1
+    qm = meta(qlens, qf)
+    o_big = torch.zeros((Tq, Hq + 2, D), dtype=dtype, device=DEV)
+    ml_big = torch.zeros((2, Tq, Hq + 1), device=DEV)
+    o, m, l = o_big[:, 1:Hq + 1], ml_big[0, :, :Hq], ml_big[1, :, :Hq]
+    m.fill_(float("-inf"))
+    o_st = torch.zeros((Tq, Hq, D), dtype=dtype)
+    m_st, l_st = torch.full((Tq, Hq), float("-inf")), torch.zeros(Tq, Hq)
+    ws = torch.full((6 * Tq * Hq * (D + 1),), float("nan"), device=DEV)
+    dq, dqm = q.to(DEV), [t.to(DEV) for t in qm]
+    parts = []
+    for j, (k, v, km, klens) in enumerate(chunks):
+        dkm = [t.to(DEV) for t in km]
+        kw = dict(workspace=ws, max_kv_len=max(klens), kv_splits=None if j == 0 else 5) if j != 1 else {}
+        lsa.context_attention_fwd(dq, k.to(DEV), v.to(DEV), o, *dqm, *dkm, P, max(qlens), m, l, **kw)
+        torch.cuda.synchronize()
+        orc.context_attention_fwd(q, k, v, o_st, *qm, *km, P, max(qlens), m_st, l_st)
+        parts.append(orc.attn_step(q, k, v, *qm, *km, P))
+        o_exact, lse_exact = orc.lse_merge(parts)
+        seen = torch.isfinite(lse_exact)
+        assert_inplace_o_close(o.cpu()[seen], o_st[seen], o_exact[seen], "o after step %d" % j)
+        assert_lse_close(orc.state_lse(m.cpu(), l.cpu()).float(), lse_exact, "state LSE after step %d" % j)
+    assert bool((o_big[:, 0] == 0).all()) and bool((o_big[:, Hq + 1] == 0).all()) and bool((ml_big[:, :, Hq] == 0).all())
+    # without max_kv_len the bound is the k buffer's height; a workspace that holds one cut only: the ordinary launch
+    from loongserve_amd import ops
+    assert ops._workspace_cuts(ws[:Tq * Hq * (D + 1)], Tq, Hq, D) == 1
+
+
 @pytest.mark.parametrize("Hq,Hkv", [(3, 3), (12, 6), (24, 12), (40, 40), (35, 5), (21, 7), (18, 2), (9, 1)])
 @pytest.mark.parametrize("P", [5, 7, 13, 64])
 def test_launch_geometry_with_divisors_that_are_not_powers_of_two(lsa, Hq, Hkv, P):
