@@ -4,17 +4,21 @@
 A step is one pass of the ring-prefill workload (baseline configuration 2 of five): the 16384 queries of
 shard 3 of a 131072-token sequence attend to KV shards 3 (causal), 0, 1, 2 (full), one
 kernel launch per shard, each later launch LSE-merging its partial into the running result.
-The same run times the token-indexed decode workload (config 3, under "decode"), the other
-three baseline configs (1, 4, 5, under "workloads", each with its own roofline block) and
-small-batch decode latency against the host's call overhead ("decode_latency").
+The same run times the token-indexed decode workload (config 3), the other three baseline configs (1, 4, 5), a
+few batches of short prompts, and what the box sustains with nothing in the way (a stream of fp16 MFMAs on random
+operands, a streaming read of 4 GiB: libls_ceiling.so), so that every fraction of the nominal peak stands beside the
+fraction of what this box delivered in this run.
 Inputs are synthetic (seeded N(0,1)*0.5) and resident in HBM before the timed region.
 
-One JSON line goes to stdout; `--all` adds the steps around attention (element-wise kernels,
-migration, allocator) under `other`.
+One compact JSON line goes to stdout: the headline (config 2) with `roofline` and `cpu_baseline`, which also carry the
+scalar figures of decode and of configs 1, 4, 5, and a `summary` of all five configs as the last key.
+`--sweeps` also times the launch-size, decode-latency, large-group and mixed-length sweeps and `--all` the steps around
+attention; both go to the file `--details-out` names (default gpurun_out/bench_details.json), not into the line.
 """
 from __future__ import annotations
 
 import argparse
+import ctypes
 import json
 import math
 import os
@@ -30,7 +34,7 @@ if ROOT not in sys.path:
 # HBM bytes per launch of each workload's dominant kernel: rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled by what the same
 # counter reads for a plain copy of 1 GiB.  Not measured by this run: taken from profiles/bench_default_hbm_traffic.txt,
 # which is regenerated with the kernels (the JSON line says so in "traffic_source").
-TRAFFIC_SOURCE = "profiles/bench_default_hbm_traffic.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this command, scaled by a 1 GiB copy); a constant of bench.py, not measured in this run"
+TRAFFIC_SOURCE = "profiles/bench_default_hbm_traffic.txt (rocprofv3 --pmc, scaled by a 1 GiB copy); constants of bench.py, not measured in this run"
 TRAFFIC_BYTES = {
     "config2": 1304.9e6,    # per launch, averaged over the four launches of a ring step (one diagonal + three full)
     "config3": 5203.0e6,    # stage 1 of the fused call
@@ -76,9 +80,10 @@ def _time_events(fn, steps, warmup):
     return [a.elapsed_time(b) for a, b in evs]
 
 
-def _time_graph(fn, launches=20, reps=10):
+def _time_graph(fn, launches=20, reps=10, warm_reps=2, every=False):
     """Device time (ms) of one call of `fn`, for calls too short to time from the host: `launches` calls are recorded
-    into one HIP graph, whose replays are timed with HIP events; the median over `reps` replays, per call."""
+    into one HIP graph, whose replays are timed with HIP events; `warm_reps` replays are thrown away, then the median
+    over `reps` replays, per call (every=True: the list of all of them)."""
     for _ in range(3):
         fn()
     torch.cuda.synchronize()
@@ -86,7 +91,8 @@ def _time_graph(fn, launches=20, reps=10):
     with torch.cuda.graph(g):
         for _ in range(launches):
             fn()
-    g.replay()
+    for _ in range(max(1, warm_reps)):
+        g.replay()
     torch.cuda.synchronize()
     ts = []
     for _ in range(reps):
@@ -96,7 +102,59 @@ def _time_graph(fn, launches=20, reps=10):
         b.record()
         torch.cuda.synchronize()
         ts.append(a.elapsed_time(b) / launches)
-    return sorted(ts)[len(ts) // 2]
+    return ts if every else sorted(ts)[len(ts) // 2]
+
+
+def _r(x, nd=4):
+    return None if x is None else round(float(x), nd)
+
+
+class Ceiling:
+    """What this box sustains with nothing in the way (libls_ceiling.so, include/ls_ceiling.h)."""
+
+    def __init__(self):
+        path = os.path.join(ROOT, "loongserve_amd", "libls_ceiling.so")
+        if not os.path.exists(path):
+            raise RuntimeError("bench.py: %s is missing; build it with `python -m loongserve_amd.build`" % path)
+        self.lib = ctypes.CDLL(path)
+        vp = ctypes.c_void_p
+        self.lib.ls_ceiling_mfma_f16.restype = ctypes.c_int
+        self.lib.ls_ceiling_mfma_f16.argtypes = [vp, vp, ctypes.c_int, ctypes.c_int, vp]
+        self.lib.ls_ceiling_mfma_f16_flop.restype = ctypes.c_double
+        self.lib.ls_ceiling_mfma_f16_flop.argtypes = [ctypes.c_int, ctypes.c_int]
+        self.lib.ls_ceiling_read.restype = ctypes.c_int
+        self.lib.ls_ceiling_read.argtypes = [vp, ctypes.c_uint64, vp, vp]
+
+    def mfma_tflops(self, iters=60000, workgroups=256, launches=24, warm=8):
+        """A stream of v_mfma_f32_16x16x32_f16 on random fp16 operands, one wave per SIMD, nothing else; launches of
+        about 10 ms back to back, the first `warm` thrown away (the clock settles under the power limit), the median."""
+        ops = _randn_half((1024, 128), 8001)  # 256 KiB of N(0,1)*0.5 fp16 values
+        sink = torch.zeros(256 * workgroups, dtype=torch.float32, device=DEV)
+        st = torch.cuda.current_stream().cuda_stream
+
+        def call():
+            if self.lib.ls_ceiling_mfma_f16(ops.data_ptr(), sink.data_ptr(), iters, workgroups, st) != 0:
+                raise RuntimeError("ls_ceiling_mfma_f16 failed")
+        ms = _time_events(call, launches, warm)
+        flop = self.lib.ls_ceiling_mfma_f16_flop(iters, workgroups)
+        med = sorted(ms)[len(ms) // 2]
+        return flop / (med * 1e-3) / 1e12, med
+
+    def read_gbs(self, nbytes=4 << 30, launches=20, warm=5):
+        """A plain streaming read of 4 GiB (16 bytes per lane and load, non-temporal), the median launch."""
+        src = torch.empty(nbytes, dtype=torch.uint8, device=DEV)
+        src.view(torch.int32).random_(0, 1 << 30)
+        sink = torch.zeros(256, dtype=torch.int32, device=DEV)
+        st = torch.cuda.current_stream().cuda_stream
+
+        def call():
+            if self.lib.ls_ceiling_read(src.data_ptr(), nbytes, sink.data_ptr(), st) != 0:
+                raise RuntimeError("ls_ceiling_read failed")
+        ms = _time_events(call, launches, warm)
+        med = sorted(ms)[len(ms) // 2]
+        del src
+        torch.cuda.empty_cache()
+        return nbytes / (med * 1e-3) / 1e9, med
 
 
 def _roof(kernel, bound, achieved, per_launch_ms, traffic_key, **extra):
@@ -416,125 +474,145 @@ def _stats(ms):
     return {"median_ms": s[n // 2], "p10_ms": s[int(0.1 * (n - 1))], "p90_ms": s[int(math.ceil(0.9 * (n - 1)))], "mean_ms": sum(s) / n}
 
 
-def workloads(steps):
-    """Configs 1, 4 and 5 of the baseline: each timed as a whole and with the launch duration of its dominant kernel."""
+def config1():
+    """Config 1: single causal prefill, 2048 tokens, 32/32 heads, fp16, one ring step, one launch."""
     import loongserve_amd as lsa
-    out = {}
-    # ---- config 1: single causal prefill, 2048 tokens, 32/32 heads, fp16, one ring step
-    T, H, D = 2048, 32, 128
+    T, H = 2048, 32
     q, kv = _randn_half((T, H, D), 1001), _randn_half((T, 2 * H, D), 1002)
     s0, ln, f0 = _i32([0]), _i32([T]), _i32([0])
     ob = torch.empty((T, H, D), dtype=torch.float32, device=DEV)
     lb = torch.empty((T, H), dtype=torch.float32, device=DEV)
     call = lambda: lsa.prefill_attention_step(q, kv[:, :H], kv[:, H:], s0, ln, f0, s0, ln, f0, 1, T, ob, lb)  # noqa: E731
-    st = _stats(_time_events(call, 50, 10))
-    dev_ms = _time_graph(call, launches=20, reps=10)
+    eager = _stats(_time_events(call, 50, 10))
+    # device time per launch: 20 launches recorded in one HIP graph (the launch is shorter than the host's call), 12 replays
+    st = _stats(_time_graph(call, launches=20, reps=12, warm_reps=3, every=True))
     fl = 4 * D * H * (T * (T + 1) // 2)
-    out["config1"] = {
-        "workload": "config 1: 1 x 2048 tokens causal, 32/32 heads, head_dim 128, fp16, fp32 (O, LSE) out, one launch",
-        "value": fl / (dev_ms * 1e-3) / 1e12, "unit": "TFLOP/s", "ms_per_step": dev_ms, "pct_of_mfma_peak": 100 * fl / (dev_ms * 1e-3) / 1e12 / PEAK_MFMA_TFLOPS,
-        "algorithmic_tflop_per_step": fl / 1e12,
-        "timing": "device time per launch: 20 launches recorded in one HIP graph, replays timed with HIP events (the launch "
-                  "is shorter than the host's call overhead); eager_call_ms is one call bracketed by HIP events, host overhead included",
-        "eager_call_ms": st["median_ms"],
-        "roofline": _roof("prefill_kernel<F16,0,true,true> (128-row workgroups: 512 of them)", "mfma", fl / (dev_ms * 1e-3) / 1e12, dev_ms, "config1",
-                          algorithmic_tflop_per_launch=fl / 1e12)}
-    del q, kv, ob, lb
-    # ---- config 4: long-context elastic decode, 4 x 524288, MHA 32, four instances, merge at the master
+    ms = st["median_ms"]
+    return {"workload": "config 1: 1 x 2048 tokens causal, MHA 32, fp16, fp32 (O, LSE) out, one launch",
+            "value": fl / (ms * 1e-3) / 1e12, "unit": "TFLOP/s", "ms": ms, "p10_ms": st["p10_ms"], "p90_ms": st["p90_ms"],
+            "frac": fl / (ms * 1e-3) / 1e12 / PEAK_MFMA_TFLOPS, "kernel": "prefill_kernel<F16,0,true,true> (128-row workgroups)",
+            "timing": "per launch, 20 launches in a HIP graph x 12 replays", "eager_call_ms": eager["median_ms"],
+            "algorithmic_tflop": fl / 1e12, "traffic": TRAFFIC_BYTES["config1"]}
+
+
+def config4():
+    """Config 4: long-context elastic decode, 4 x 524288, MHA 32, four instances, merge at the master."""
     e = ElasticDecode()
-    st = _stats(_time_events(e.step, steps, 2))
+    st = _stats(_time_events(e.step, 50, 10))
     nbytes1 = e.stage1_of_one_instance()
-    s1 = _stats(_time_events(e.stage1_of_one_instance, max(steps, 5), 2))
-    out["config4"] = {
-        "workload": "config 4: decode 4 x 524288 tokens, MHA 32 heads, head_dim 128, fp16, scattered pool; four simulated instances "
-                    "(three peers through the fused call, the master through stage 1 + the block_seq = 1 merge of all partials)",
-        "value": e.bytes / (st["median_ms"] * 1e-3) / 1e9, "unit": "GB/s", "ms_per_step": st["median_ms"],
-        "pct_of_hbm_peak": 100 * e.bytes / (st["median_ms"] * 1e-3) / 1e9 / PEAK_HBM_GBS, "algorithmic_gb_per_step": e.bytes / 1e9,
-        "step_stats": st,
-        "roofline": _roof("decode_stage1_mfma_kernel<F16,false> (one instance: 4 x 131072 tokens x 32 KV heads)", "hbm",
-                          nbytes1 / (s1["median_ms"] * 1e-3) / 1e9, s1["median_ms"], "config4", algorithmic_gb_per_launch=nbytes1 / 1e9)}
+    s1 = _stats(_time_events(e.stage1_of_one_instance, 50, 10))
+    gbs1 = nbytes1 / (s1["median_ms"] * 1e-3) / 1e9
+    out = {"workload": "config 4: decode 4 x 524288 tokens, MHA 32, fp16, scattered pool; 4 simulated instances (3 peers fused, "
+                       "master stage 1 + block_seq=1 merge of all partials)",
+           "value": e.bytes / (st["median_ms"] * 1e-3) / 1e9, "unit": "GB/s", "ms": st["median_ms"], "p10_ms": st["p10_ms"],
+           "p90_ms": st["p90_ms"], "frac": e.bytes / (st["median_ms"] * 1e-3) / 1e9 / PEAK_HBM_GBS,
+           "kernel": "decode_stage1_mfma_kernel<F16,false>", "kernel_ms": s1["median_ms"], "kernel_gbs": gbs1,
+           "kernel_frac": gbs1 / PEAK_HBM_GBS, "algorithmic_gb": e.bytes / 1e9, "kernel_algorithmic_gb": nbytes1 / 1e9,
+           "traffic": TRAFFIC_BYTES["config4"]}
     del e
     torch.cuda.empty_cache()
-    # ---- config 5: mixed varlen prefill, bf16, GQA 32/8, K/V rows written to pool slots and registered
+    return out
+
+
+def config5(details=None):
+    """Config 5: mixed varlen prefill, bf16, GQA 32/8, K/V rows written to pool slots and registered."""
     v = VarlenPrefill()
-    sa = _stats(_time_events(v.attention, 3, 1))
-    sk = _stats(_time_events(v.attention_kernel_only, 3, 0))
-    sp = _stats(_time_events(v.persist, 5, 1))
-    sm = _stats(_time_events(v.migrate, 5, 1))
-    v.write_back_setup()
-    wsep = _stats(_time_events(v.write_back_separate, 5, 1))
-    wfus = _stats(_time_events(v.write_back_fused, 5, 1))
+    sa = _stats(_time_events(v.attention, 5, 1))
+    sk = _stats(_time_events(v.attention_kernel_only, 5, 1))
+    sp = _stats(_time_events(v.persist, 20, 3))
     whole_ms = sa["median_ms"] + sp["median_ms"]
-    out["config5"] = {
-        "workload": "config 5: 24 packed sequences, lengths log-uniform in [1024, 200000], %d tokens, GQA 32/8, head_dim 128, bf16, "
-                    "causal, through context_attention_fwd ((m, l) reset, fp16 copy of V into the caller's buffer, one attention "
-                    "launch), then the K/V rows scattered to pool slots and registered" % v.T,
-        "value": v.flops / (whole_ms * 1e-3) / 1e12, "unit": "TFLOP/s", "ms_per_step": whole_ms,
-        "pct_of_mfma_peak": 100 * v.flops / (whole_ms * 1e-3) / 1e12 / PEAK_MFMA_TFLOPS, "algorithmic_tflop_per_step": v.flops / 1e12,
-        "attention_ms": sa["median_ms"], "attention_tflops": v.flops / (sa["median_ms"] * 1e-3) / 1e12,
-        "kv_write": {"what": "lsattn_kv_scatter + lsattn_register_tokens: every K/V row (4096 B) read and written once",
-                     "ms": sp["median_ms"], "gbs": v.scatter_bytes / (sp["median_ms"] * 1e-3) / 1e9,
-                     "pct_of_hbm_peak": 100 * v.scatter_bytes / (sp["median_ms"] * 1e-3) / 1e9 / PEAK_HBM_GBS},
-        "write_back_with_rotary": {
-            "what": "rotary embedding of q and k + K/V rows to their pool slots + registration, on the same buffers read as fp16 "
-                    "(the reference's rotary kernel is fp16 only): the four launches the layer makes (rotary of q, rotary of k, "
-                    "scatter, registration) against the one launch of lsattn_rotary_kv_write; GB/s on the bytes the fused launch moves",
+    tf = v.flops / (sk["median_ms"] * 1e-3) / 1e12
+    out = {"workload": "config 5: 24 packed sequences, lengths log-uniform in [1024, 200000], %d tokens, GQA 32/8, bf16, causal, "
+                       "context_attention_fwd ((m, l) reset, fp16 copy of V, one launch) + K/V rows to pool slots + registration" % v.T,
+           "value": v.flops / (whole_ms * 1e-3) / 1e12, "unit": "TFLOP/s", "ms": whole_ms,
+           "frac": v.flops / (whole_ms * 1e-3) / 1e12 / PEAK_MFMA_TFLOPS, "kernel": "prefill_kernel<BF16,1,true,false>",
+           "kernel_ms": sk["median_ms"], "kernel_p10_ms": sk["p10_ms"], "kernel_p90_ms": sk["p90_ms"], "kernel_tflops": tf,
+           "kernel_frac": tf / PEAK_MFMA_TFLOPS, "kv_write_ms": sp["median_ms"],
+           "kv_write_gbs": v.scatter_bytes / (sp["median_ms"] * 1e-3) / 1e9, "algorithmic_tflop": v.flops / 1e12,
+           "traffic": TRAFFIC_BYTES["config5"]}
+    if details is not None:
+        sm = _stats(_time_events(v.migrate, 10, 2))
+        v.write_back_setup()
+        wsep = _stats(_time_events(v.write_back_separate, 10, 2))
+        wfus = _stats(_time_events(v.write_back_fused, 10, 2))
+        details["config5_write_back"] = {
+            "what": "rotary of q and k + K/V rows to their pool slots + registration on the same buffers read as fp16: the "
+                    "layer's four launches against lsattn_rotary_kv_write; the rows through lsattn_kv_copy_register",
             "separate_ms": wsep["median_ms"], "fused_ms": wfus["median_ms"], "bytes": v.write_back_bytes,
-            "separate_gbs": v.write_back_bytes / (wsep["median_ms"] * 1e-3) / 1e9, "fused_gbs": v.write_back_bytes / (wfus["median_ms"] * 1e-3) / 1e9,
-            "fused_pct_of_hbm_peak": 100 * v.write_back_bytes / (wfus["median_ms"] * 1e-3) / 1e9 / PEAK_HBM_GBS},
-        "migration_copy_register": {"what": "the same rows through lsattn_kv_copy_register (copy + registration in one launch)",
-                                    "ms": sm["median_ms"], "gbs": v.scatter_bytes / (sm["median_ms"] * 1e-3) / 1e9},
-        "roofline": _roof("prefill_kernel<BF16,1,true,false>", "mfma", v.flops / (sk["median_ms"] * 1e-3) / 1e12, sk["median_ms"], "config5",
-                          algorithmic_tflop_per_launch=v.flops / 1e12)}
+            "fused_gbs": v.write_back_bytes / (wfus["median_ms"] * 1e-3) / 1e9,
+            "migration_copy_register_ms": sm["median_ms"], "migration_copy_register_gbs": v.scatter_bytes / (sm["median_ms"] * 1e-3) / 1e9}
     del v
     torch.cuda.empty_cache()
     return out
 
 
-def prefill_launch_sizes():
+def _causal_case(N, Hq, Hkv, B):
+    q = _randn_half((B * N, Hq, D), 4100 + N + B)
+    kv = _randn_half((B * N, 2 * Hkv, D), 4200 + N + B)
+    st = torch.arange(B, dtype=torch.int32, device=DEV) * N
+    ln = torch.full((B,), N, dtype=torch.int32, device=DEV)
+    z = torch.zeros(B, dtype=torch.int32, device=DEV)
+    o = torch.empty((B * N, Hq, D), dtype=torch.float32, device=DEV)
+    lse = torch.empty((B * N, Hq), dtype=torch.float32, device=DEV)
+    import loongserve_amd as lsa
+    fn = lambda: lsa.prefill_attention_step(q, kv[:, :Hkv], kv[:, Hkv:], st, ln, z, st, ln, z, 1, N, out=o, lse=lse, kv_splits=1)  # noqa: E731
+    return fn, 4.0 * D * Hq * B * N * (N + 1) / 2
+
+
+def short_prompts():
+    """Batches of short prompts (outside the five configs; the regime of the reference's published 1 x 100 / 1 x 1000
+    token rows): causal, fp16, device time per launch from a HIP graph of 20 launches, median of 10 replays."""
+    rows = {}
+    for name, (N, Hq, Hkv, B) in (("16x256_mha", (256, 32, 32, 16)), ("8x512_gqa", (512, 32, 8, 8)), ("32x1024_gqa", (1024, 32, 8, 32)),
+                                  ("6x2048_gqa", (2048, 32, 8, 6)), ("1x4096_mha", (4096, 32, 32, 1)), ("1x8192_gqa", (8192, 32, 8, 1))):
+        fn, fl = _causal_case(N, Hq, Hkv, B)
+        ms = _time_graph(fn, launches=20, reps=10, warm_reps=3)
+        rows[name] = {"us": _r(ms * 1e3, 1), "frac": _r(fl / (ms * 1e-3) / 1e12 / PEAK_MFMA_TFLOPS)}
+        torch.cuda.empty_cache()
+    return rows
+
+
+def _tiles_256x64(N, Hq, B, pack=1):
+    """64-key tiles that 256-row workgroups walk for B causal sequences of N tokens (pack query heads side by side)."""
+    rows = 256 // pack
+    nz = (N + rows - 1) // rows
+    return B * (Hq // pack) * sum(min((z + 1) * rows, N) // 64 + (1 if min((z + 1) * rows, N) % 64 else 0) for z in range(nz))
+
+
+def prefill_launch_sizes(tile_us):
     """Causal prefill launches from a quarter of a round of workgroups to a few rounds (outside the five baseline configs):
-    fp16, head_dim 128, fp32 (O, LSE) out, device time per launch from a HIP graph of 5 launches.  chosen_us is the
-    library's own choice of workgroup height and grid order; the other columns force 128-row workgroups, 256-row
-    workgroups one KV head at a time per XCD, 256-row workgroups with the heaviest query tiles of all heads first, the
-    four-wave shape of which two workgroups share a CU (LSATTN_PREFILL_ROWS / LSATTN_PREFILL_ORDER), and one query head per workgroup instead of the heads of a KV head side
-    by side (LSATTN_PREFILL_PACK=0; the same thing for the 32/32 cases)."""
+    fp16, head_dim 128, fp32 (O, LSE) out, device time per launch from a HIP graph of 20 launches, median of 10 replays.
+    chosen_us is the library's own choice of workgroup height and grid order; the other columns force 128-row workgroups,
+    256-row workgroups one KV head at a time per XCD, 256-row workgroups with the heaviest query tiles of all heads
+    first, the four-wave shape of which two workgroups share a CU, and one query head per workgroup instead of the heads
+    of a KV head side by side (lsattn_set_tuning).  tiles_only_floor_us: the 64-key tiles that 256-row workgroups walk,
+    spread evenly over 256 CUs, at the rate per tile that config 2's full launches ran at in this run: what the launch
+    would take if workgroups cost nothing besides their tiles."""
     import loongserve_amd as lsa
     rows = []
-    saved = {k: os.environ.get(k) for k in ("LSATTN_PREFILL_ROWS", "LSATTN_PREFILL_ORDER", "LSATTN_PREFILL_PACK")}
     try:
-        for N, Hq, Hkv, B in ((1024, 32, 8, 1), (2048, 32, 32, 1), (512, 32, 8, 8), (4096, 32, 32, 1), (2048, 32, 8, 6), (1024, 32, 8, 32), (256, 32, 32, 16), (8192, 32, 8, 1)):
-            q = _randn_half((B * N, Hq, D), 4100 + N + B)
-            kv = _randn_half((B * N, 2 * Hkv, D), 4200 + N + B)
-            st = torch.arange(B, dtype=torch.int32, device=DEV) * N
-            ln = torch.full((B,), N, dtype=torch.int32, device=DEV)
-            z = torch.zeros(B, dtype=torch.int32, device=DEV)
-            o = torch.empty((B * N, Hq, D), dtype=torch.float32, device=DEV)
-            lse = torch.empty((B * N, Hq), dtype=torch.float32, device=DEV)
-            fn = lambda: lsa.prefill_attention_step(q, kv[:, :Hkv], kv[:, Hkv:], st, ln, z, st, ln, z, 1, N, out=o, lse=lse, kv_splits=1)
-            fl = 4.0 * D * Hq * B * N * (N + 1) / 2
+        for N, Hq, Hkv, B in ((1024, 32, 8, 1), (2048, 32, 32, 1), (512, 32, 8, 8), (4096, 32, 32, 1), (2048, 32, 8, 6), (1024, 32, 8, 32),
+                              (256, 32, 32, 16), (8192, 32, 8, 1)):
+            fn, fl = _causal_case(N, Hq, Hkv, B)
             row = {"tokens": N, "requests": B, "q_heads": Hq, "kv_heads": Hkv, "workgroups_of_256_rows": B * Hq * ((N + 255) // 256)}
             _time_graph(fn, launches=5, reps=2)  # first touch of the new buffers
             # (the library's choice is timed last: the first timing after new buffers reads a few per cent long)
-            for key, env in (("rows128_us", {"LSATTN_PREFILL_ROWS": "128"}),
-                             ("rows256_head_major_us", {"LSATTN_PREFILL_ROWS": "256", "LSATTN_PREFILL_ORDER": "head"}),
-                             ("rows256_tile_major_us", {"LSATTN_PREFILL_ROWS": "256", "LSATTN_PREFILL_ORDER": "tile"}),
-                             ("four_waves_us", {"LSATTN_PREFILL_ROWS": "half"}),
-                             ("one_head_per_workgroup_us", {"LSATTN_PREFILL_PACK": "0"}), ("chosen_us", {})):
-                for k in saved:
-                    os.environ.pop(k, None)
-                os.environ.update(env)
-                row[key] = round(_time_graph(fn, launches=5, reps=5) * 1e3, 1)
+            for key, choice in (("rows128_us", dict(prefill_rows="128")),
+                                ("rows256_head_major_us", dict(prefill_rows="256", prefill_order="head")),
+                                ("rows256_tile_major_us", dict(prefill_rows="256", prefill_order="tile")),
+                                ("four_waves_us", dict(prefill_rows="half")),
+                                ("one_head_per_workgroup_us", dict(prefill_pack="off")), ("chosen_us", {})):
+                lsa.set_tuning(**choice)
+                row[key] = round(_time_graph(fn, launches=20, reps=10, warm_reps=2) * 1e3, 1)
             row["chosen_tflops"] = round(fl / (row["chosen_us"] * 1e-6) / 1e12, 1)
+            group = Hq // Hkv
+            pack = 8 if group % 8 == 0 else 4 if group % 4 == 0 else 2 if group % 2 == 0 else 1
+            row["tiles_only_floor_us"] = round(_tiles_256x64(N, Hq, B, pack) / 256.0 * tile_us, 1)
             rows.append(row)
-            del q, kv, o, lse
     finally:
-        for k, v in saved.items():
-            if v is None:
-                os.environ.pop(k, None)
-            else:
-                os.environ[k] = v
+        lsa.set_tuning()
     torch.cuda.empty_cache()
-    return {"what": " ".join(x.strip() for x in prefill_launch_sizes.__doc__.split("\n")), "cases": rows}
+    return {"what": " ".join(x.strip() for x in prefill_launch_sizes.__doc__.split("\n")), "tile_us": tile_us, "cases": rows}
 
 
 def decode_latency():
@@ -542,51 +620,48 @@ def decode_latency():
     under 8-way tensor parallelism), head_dim 128, fp16, scattered slots,
     fused stage 1 + stage 2 call (the operator a decode step of the layer makes, longserve_transformer_layer_infer.py:293-308).
     eager_us: wall clock per call over 200 back-to-back calls and one synchronize (host-bound when the host is slower
-    than the kernels); graph_us: the same call replayed from a HIP graph of 20 of them, per call (device time)."""
-    import loongserve_amd as lsa
+    than the kernels); graph_us: the same call replayed from a HIP graph of 20 of them, per call (device time; for the
+    cases of a few megabytes the replays read the same K/V out of the caches, so no bandwidth is quoted for them)."""
     rows = []
     for Hq, Hkv, B, ctx in [(32, 8, B, ctx) for B in (1, 4, 16) for ctx in (2048, 8192, 32768)] + [(8, 1, 1, 8192), (8, 1, 8, 8192), (8, 1, 16, 32768)]:
-        if True:
-            d = TokenDecode(B=B, Hq=Hq, Hkv=Hkv, lens=[ctx] * B, pool=B * ctx + 1024, seed=3100 + B)
-            for _ in range(5):
-                d.step()
-            torch.cuda.synchronize()
-            n = 200
-            t0 = time.perf_counter()
-            for _ in range(n):
-                d.step()
-            torch.cuda.synchronize()
-            eager = (time.perf_counter() - t0) / n * 1e6
-            graph = _time_graph(d.step, launches=20, reps=10) * 1e3
-            rows.append({"q_heads": Hq, "kv_heads": Hkv, "batch": B, "ctx": ctx, "eager_us": round(eager, 2), "graph_us": round(graph, 2),
-                         "kv_gbs_at_graph_rate": round(d.bytes / (graph * 1e-6) / 1e9, 1)})
-            del d
+        d = TokenDecode(B=B, Hq=Hq, Hkv=Hkv, lens=[ctx] * B, pool=B * ctx + 1024, seed=3100 + B)
+        for _ in range(10):
+            d.step()
+        torch.cuda.synchronize()
+        n = 200
+        t0 = time.perf_counter()
+        for _ in range(n):
+            d.step()
+        torch.cuda.synchronize()
+        eager = (time.perf_counter() - t0) / n * 1e6
+        graph = _time_graph(d.step, launches=20, reps=10) * 1e3
+        row = {"q_heads": Hq, "kv_heads": Hkv, "batch": B, "ctx": ctx, "eager_us": round(eager, 2), "graph_us": round(graph, 2)}
+        if d.bytes > 512e6:  # beyond what the 256 MB last-level cache can serve on replays
+            row["kv_gbs_at_graph_rate"] = round(d.bytes / (graph * 1e-6) / 1e9, 1)
+        rows.append(row)
+        del d
     torch.cuda.empty_cache()
-    return {"what": decode_latency.__doc__.split("\n")[0].strip() + " eager_us = wall clock per call over 200 back-to-back calls + one "
-                    "synchronize; graph_us = per call when 20 calls are replayed from one HIP graph (device time)",
+    return {"what": " ".join(x.strip() for x in decode_latency.__doc__.split("\n")),
             "reference_launch_overhead_us": "100-400 (Triton launch overhead the reference reports, longserve_cuda_kernels/README.md:7-9)",
             "cases": rows}
 
 
-def decode_large_groups(steps):
+def decode_large_groups():
     """Token-indexed decode for GQA groups of eight and more query heads per KV head (outside the five baseline configs:
     Llama-3-70B is 64/8, 8/1 per GPU under 8-way tensor parallelism): batch 64, ctx U[4096,32768], scattered pool, fused
     call and stage 1 alone, through the library's own choice of stage-1 kernel (the matrix-pipe one for these shapes) and
-    with LSATTN_DECODE_MFMA=0 (the lane kernel every smaller group runs on)."""
+    with the lane kernel forced (lsattn_set_tuning), which every smaller group runs on.  Device time per call from a HIP
+    graph of 20 calls, median of 10 replays."""
+    import loongserve_amd as lsa
     rows = []
-    saved = os.environ.get("LSATTN_DECODE_MFMA")
     try:
         for Hq, Hkv in ((8, 1), (16, 2), (64, 8)):
             d = TokenDecode(Hq=Hq, Hkv=Hkv, seed=3300 + Hq)
             row = {"q_heads": Hq, "kv_heads": Hkv, "algorithmic_gb_per_step": d.bytes / 1e9}
-            for key, env in (("matrix_pipe", None), ("lane_kernel", "0")):
-                if env is None:
-                    os.environ.pop("LSATTN_DECODE_MFMA", None)
-                else:
-                    os.environ["LSATTN_DECODE_MFMA"] = env
-                # (device time per call from a HIP graph of 20 of them: the shortest of these launches takes 0.12 ms)
-                fused = _time_graph(d.step, launches=20, reps=max(3, steps // 2))
-                s1 = _time_graph(d.stage1_only, launches=20, reps=max(3, steps // 2))
+            for key, choice in (("matrix_pipe", {}), ("lane_kernel", dict(decode_stage1="lane"))):
+                lsa.set_tuning(**choice)
+                fused = _time_graph(d.step, launches=20, reps=10)
+                s1 = _time_graph(d.stage1_only, launches=20, reps=10)
                 row[key] = {"fused_ms": fused, "fused_gbs": d.bytes / (fused * 1e-3) / 1e9, "stage1_ms": s1,
                             "stage1_gbs": d.bytes / (s1 * 1e-3) / 1e9}
             row["roofline"] = _roof("decode_stage1_mfma_kernel<F16,false|true> (the shape the library chooses)", "hbm", row["matrix_pipe"]["stage1_gbs"], row["matrix_pipe"]["stage1_ms"],
@@ -595,42 +670,33 @@ def decode_large_groups(steps):
             del d
             torch.cuda.empty_cache()
     finally:
-        if saved is None:
-            os.environ.pop("LSATTN_DECODE_MFMA", None)
-        else:
-            os.environ["LSATTN_DECODE_MFMA"] = saved
+        lsa.set_tuning()
     return {"what": " ".join(x.strip() for x in decode_large_groups.__doc__.split("\n")), "cases": rows}
 
 
-def decode_mixed_lengths():
+def decode_mixed_lengths(full=True):
     """Token-indexed decode of batches that mix one long request with many short ones (outside the five baseline
     configs), GQA 32/8, scattered pool: the two stages as the master of a decode step calls them (BLOCK_SEQ 256, one
     partial per block) and the fused call, through the library's own choice (stage 1 walks a list of the units of work
-    that exist when the plain grid would have 32768 workgroups and more) and with LSATTN_DECODE_LISTED=0 (the grid
-    sized by the longest request, as the reference's).  Device time per call from a HIP graph of 5 calls."""
+    that exist when the plain grid would have 32768 workgroups and more) and with the grid sized by the longest request
+    forced (lsattn_set_tuning), as the reference's.  Device time per call from a HIP graph of 10 calls, median of 10 replays."""
+    import loongserve_amd as lsa
     rows = []
-    saved = os.environ.get("LSATTN_DECODE_LISTED")
     try:
         for lens, name in (([131072] + [512] * 255, "1 x 131072 + 255 x 512 tokens"), ([524288] + [2048] * 63, "1 x 524288 + 63 x 2048 tokens")):
             d = TokenDecode(B=len(lens), lens=lens, pool=sum(lens) + 1024, seed=3400 + len(lens))
             row = {"batch": name, "algorithmic_gb_per_step": d.bytes / 1e9}
-            for key, env in (("chosen", None), ("grid_by_longest_request", "0")):
-                if env is None:
-                    os.environ.pop("LSATTN_DECODE_LISTED", None)
-                else:
-                    os.environ["LSATTN_DECODE_LISTED"] = env
-                two = _time_graph(d.step_separate_stages, launches=5, reps=5)
-                fused = _time_graph(d.step, launches=5, reps=5)
+            for key, choice in (("chosen", {}), ("grid_by_longest_request", dict(decode_listed="off")))[:2 if full else 1]:
+                lsa.set_tuning(**choice)
+                two = _time_graph(d.step_separate_stages, launches=10, reps=10)
+                fused = _time_graph(d.step, launches=10, reps=10)
                 row[key] = {"two_stages_ms": two, "two_stages_gbs": d.bytes / (two * 1e-3) / 1e9, "fused_ms": fused,
                             "fused_gbs": d.bytes / (fused * 1e-3) / 1e9}
             rows.append(row)
             del d
             torch.cuda.empty_cache()
     finally:
-        if saved is None:
-            os.environ.pop("LSATTN_DECODE_LISTED", None)
-        else:
-            os.environ["LSATTN_DECODE_LISTED"] = saved
+        lsa.set_tuning()
     return {"what": " ".join(x.strip() for x in decode_mixed_lengths.__doc__.split("\n")), "cases": rows}
 
 
@@ -735,12 +801,16 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
-    ap.add_argument("--only", choices=["prefill", "decode"], default=None, help="time one workload only (profiling aid)")
+    ap.add_argument("--only", choices=["prefill", "decode", "config1", "config4", "config5", "ceiling"], default=None,
+                    help="time one workload only (profiling aid)")
     ap.add_argument("--calib-copy", action="store_true",
                     help="only run three plain 1 GiB device-to-device copies (known traffic, for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE)")
-    ap.add_argument("--all", action="store_true", help="also time the steps around attention: element-wise kernels, migration, allocator (under 'other')")
+    ap.add_argument("--sweeps", action="store_true", help="also time the launch-size, decode-latency, large-group and mixed-length sweeps (to --details-out)")
+    ap.add_argument("--all", action="store_true", help="also time the steps around attention: element-wise kernels, migration, allocator (to --details-out)")
+    ap.add_argument("--details-out", default=os.path.join(ROOT, "gpurun_out", "bench_details.json"),
+                    help="file for everything that is not in the JSON line (written when there is something to write)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU (no collectives, no second GPU); --gpus %d is not supported" % args.gpus,
@@ -765,8 +835,11 @@ def main():
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f16", "data": "synthetic",
     }
+    details, summary, roof, cpu = {}, {}, {}, {}
+    ceil = Ceiling()
+    only = args.only
 
-    if args.only != "decode":
+    if only in (None, "prefill"):
         w = RingPrefill()
         torch.cuda.synchronize()
         step_ms = _time_events(w.step, args.steps, args.warmup)
@@ -782,72 +855,111 @@ def main():
         # a step is nothing but its four launches: the average launch duration is the step's HIP-event time / 4
         per_launch_ms = st["mean_ms"] / w.launches
         ach = (w.flops / w.launches) / (per_launch_ms * 1e-3) / 1e12
+        # the box's ceiling right behind the timed steps (same thermal state): an MFMA stream and nothing else
+        mfma_peak, _ = ceil.mfma_tflops()
         sep = _stats(_time_events(w.step_separate_merge, max(5, args.steps // 2), 2))
         inp = _stats(_time_events(w.step_in_place, max(5, args.steps // 2), 2))
         line.update({
             "value": tflops, "unit": "TFLOP/s", "ms_per_step": wall_ms,
-            "pct_of_mfma_peak": 100.0 * tflops / PEAK_MFMA_TFLOPS,
-            "config": {"workload": "config 2: ring prefill on one GPU, queries of shard 3 (16384 rows) of a 131072-token sequence vs KV "
-                                   "shards 3 (causal), 0, 1, 2 (full), in that order; 32 heads MHA, head_dim 128, fp16; fp32 partial "
-                                   "(O, LSE) per step, LSE-merged into the running result in the epilogue of the launch that produces it",
-                       "algorithmic_tflop_per_step": w.flops / 1e12, "launches_per_step": w.launches, "step_stats": st,
-                       "separate_merge": {"what": "the same steps as four separate fp32 partials + one lsattn_lse_merge pass",
-                                          "ms_per_step": sep["mean_ms"], "value": w.flops / (sep["mean_ms"] * 1e-3) / 1e12,
-                                          "launches_per_step": w.launches + 1},
-                       "in_place": {"what": "the same steps through context_attention_fwd: (o fp16, m, l) reset and updated in place",
-                                    "ms_per_step": inp["mean_ms"], "value": w.flops / (inp["mean_ms"] * 1e-3) / 1e12}},
-            "roofline": _roof("prefill_kernel<F16,0,true,false> (diagonal launch) + prefill_kernel<F16,2,true,false> (three full launches)",
-                              "mfma", ach, per_launch_ms, "config2", algorithmic_tflop_per_launch=w.flops / w.launches / 1e12),
+            "config": {"workload": "config 2: ring prefill on one GPU, 16384 queries of shard 3 of a 131072-token sequence vs KV shards 3 "
+                                   "(causal), 0, 1, 2 (full); MHA 32, head_dim 128, fp16; fp32 (O, LSE), each later launch merging its "
+                                   "partial into the running result in its epilogue",
+                       "algorithmic_tflop_per_step": w.flops / 1e12, "launches_per_step": w.launches,
+                       "median_ms": st["median_ms"], "p10_ms": st["p10_ms"], "p90_ms": st["p90_ms"],
+                       "separate_merge_ms": sep["median_ms"], "in_place_ms": inp["median_ms"]},
         })
+        roof = _roof("prefill_kernel<F16,0,true,false> (diagonal) + prefill_kernel<F16,2,true,false> (three full launches)",
+                     "mfma", ach, per_launch_ms, "config2", algorithmic_tflop_per_launch=w.flops / w.launches / 1e12,
+                     sustained_peak=mfma_peak, frac_of_sustained=ach / mfma_peak,
+                     sustained_peak_what="v_mfma_f32_16x16x32_f16 stream on random fp16 operands, one wave per SIMD, measured in this run (libls_ceiling.so)")
+        summary["config2"] = {"value": _r(tflops, 1), "unit": "TFLOP/s", "frac": _r(tflops / PEAK_MFMA_TFLOPS), "ms": _r(wall_ms),
+                              "kernel": "prefill_kernel<F16,0|2,true,false>", "frac_of_sustained": _r(ach / mfma_peak)}
+        # the rate per 256-row x 64-key tile that the full launches run at, for the tiles-only floors of the sweeps
+        tile_us = per_launch_ms * 1e3 * w.launches / ((3 * 256 + 130) * 8.0)  # tiles a CU walks per step: 8 workgroups x (3 x 256 + 130 average on the diagonal)
         if not args.no_cpu:
-            line["cpu_baseline"] = w.cpu_baseline()
+            cpu = w.cpu_baseline()
         del w
         torch.cuda.empty_cache()
+    else:
+        tile_us = 1.5
 
-    if args.only != "prefill":
+    if only in (None, "decode"):
         d = TokenDecode()
         torch.cuda.synchronize()
-        dsteps = max(args.steps, 10)
-        d_ms = _time_events(d.step, dsteps, max(args.warmup, 2))
-        s1_ms = _time_events(d.stage1_only, dsteps, 1)
-        sep = _stats(_time_events(d.step_separate_stages, dsteps, 2))
-        sepm = _stats(_time_events(d.step_separate_stages_merged, dsteps, 2))
-        st = _stats(d_ms)
-        gbs = d.bytes / (st["mean_ms"] * 1e-3) / 1e9
-        s1 = sum(s1_ms) / len(s1_ms)
-        ach = d.bytes / (s1 * 1e-3) / 1e9
-        dec = {
-            "value": gbs, "unit": "GB/s", "ms_per_step": st["mean_ms"], "pct_of_hbm_peak": 100.0 * gbs / PEAK_HBM_GBS,
-            "config": {"workload": "config 3: token-indexed decode, batch 64, ctx U[4096,32768], GQA 32/8, head_dim 128, fp16, "
-                                   "2.5M-slot scattered pool; fused stage1 + stage2 call with BLOCK_SEQ %d (mid_o is scratch there: "
-                                   "split-K at %d tokens between the stages)" % (d.BS, d.split),
-                       "tokens": d.tokens, "algorithmic_gb_per_step": d.bytes / 1e9, "step_stats": st,
-                       "separate_stages": {"what": "stage 1 and stage 2 as two calls at BLOCK_SEQ %d (the master path of a decode "
-                                                   "step), one partial per block: the reference's buffers" % d.BS,
-                                           "ms_per_step": sep["mean_ms"], "value": d.bytes / (sep["mean_ms"] * 1e-3) / 1e9,
-                                           "merged_blocks": {"what": "the same two calls with decoding.STAGE1_MERGES_BLOCKS = True (opt-in, "
-                                                                     "not the reference's layout): one partial per group of blocks",
-                                                             "ms_per_step": sepm["mean_ms"], "value": d.bytes / (sepm["mean_ms"] * 1e-3) / 1e9}}},
-            "roofline": _roof("decode_stage1_mfma_kernel<F16,false>", "hbm", ach, s1, "config3"),
-        }
-        if not args.no_cpu:
-            dec["cpu_baseline"] = d.cpu_baseline()
-        if args.only == "decode":
-            line.update({"value": gbs, "unit": "GB/s", "ms_per_step": st["mean_ms"], "config": dec["config"], "roofline": dec["roofline"]})
-            if "cpu_baseline" in dec:
-                line["cpu_baseline"] = dec["cpu_baseline"]
+        st = _stats(_time_events(d.step, 50, 10))
+        s1 = _stats(_time_events(d.stage1_only, 50, 10))
+        sep = _stats(_time_events(d.step_separate_stages, 50, 10))
+        sepm = _stats(_time_events(d.step_separate_stages_merged, 30, 5))
+        read_peak, _ = ceil.read_gbs()
+        gbs = d.bytes / (st["median_ms"] * 1e-3) / 1e9
+        ach = d.bytes / (s1["median_ms"] * 1e-3) / 1e9
+        droof = {"decode_kernel": "decode_stage1_mfma_kernel<F16,false>", "decode_achieved_gbs": ach, "decode_frac": ach / PEAK_HBM_GBS,
+                 "decode_per_launch_ms": s1["median_ms"], "decode_traffic": TRAFFIC_BYTES["config3"], "decode_algorithmic_gb": d.bytes / 1e9,
+                 "decode_sustained_peak_gbs": read_peak, "decode_frac_of_sustained": ach / read_peak}
+        summary["config3"] = {"value": _r(gbs, 1), "unit": "GB/s", "frac": _r(gbs / PEAK_HBM_GBS), "ms": _r(st["median_ms"]),
+                              "p10_ms": _r(st["p10_ms"]), "p90_ms": _r(st["p90_ms"]), "kernel": "decode_stage1_mfma_kernel<F16,false> + decode_stage2_kernel",
+                              "stage1_frac": _r(ach / PEAK_HBM_GBS), "frac_of_sustained": _r(gbs / read_peak),
+                              "two_stages_reference_buffers_ms": _r(sep["median_ms"]),
+                              "two_stages_reference_buffers_frac": _r(d.bytes / (sep["median_ms"] * 1e-3) / 1e9 / PEAK_HBM_GBS),
+                              "two_stages_merged_blocks_frac": _r(d.bytes / (sepm["median_ms"] * 1e-3) / 1e9 / PEAK_HBM_GBS),
+                              "workload": "config 3: batch 64, ctx U[4096,32768], GQA 32/8, fp16, 2.5M-slot scattered pool; fused call, BLOCK_SEQ %d, split at %d" % (d.BS, d.split)}
+        if only == "decode":
+            line.update({"value": gbs, "unit": "GB/s", "ms_per_step": st["median_ms"], "steps": 50, "warmup": 10,
+                         "config": {"workload": summary["config3"]["workload"]}})
+            roof = _roof(droof["decode_kernel"], "hbm", ach, s1["median_ms"], "config3", sustained_peak=read_peak, frac_of_sustained=ach / read_peak)
         else:
-            line["decode"] = dec
+            roof.update(droof)
+        if not args.no_cpu:
+            c = d.cpu_baseline()
+            if only == "decode":
+                cpu = c
+            else:
+                cpu.update({"decode_value_gbs": c["value"], "decode_sample": c["sample"]})
         del d
         torch.cuda.empty_cache()
-    if args.only is None:
-        line["workloads"] = workloads(max(3, min(args.steps, 10)))
-        line["prefill_launch_sizes"] = prefill_launch_sizes()
-        line["decode_latency"] = decode_latency()
-        line["decode_large_groups"] = decode_large_groups(max(5, min(args.steps, 10)))
-        line["decode_mixed_lengths"] = decode_mixed_lengths()
+
+    if only in (None, "config1"):
+        c1 = config1()
+        summary["config1"] = {k: (_r(v) if isinstance(v, float) else v) for k, v in c1.items() if k in ("value", "unit", "frac", "ms", "p10_ms", "p90_ms", "kernel")}
+        roof.update({"config1_frac": c1["frac"], "config1_per_launch_ms": c1["ms"], "config1_traffic": c1["traffic"]})
+        details["config1"] = c1
+    if only in (None, "config4"):
+        c4 = config4()
+        summary["config4"] = {k: (_r(v) if isinstance(v, float) else v) for k, v in c4.items() if k in ("value", "unit", "frac", "ms", "p10_ms", "p90_ms", "kernel", "kernel_frac")}
+        roof.update({"config4_frac": c4["kernel_frac"], "config4_per_launch_ms": c4["kernel_ms"], "config4_traffic": c4["traffic"]})
+        details["config4"] = c4
+    if only in (None, "config5"):
+        c5 = config5(details if (args.sweeps or args.all) else None)
+        summary["config5"] = {k: (_r(v) if isinstance(v, float) else v) for k, v in c5.items() if k in ("value", "unit", "frac", "ms", "kernel", "kernel_frac", "kernel_ms", "kv_write_gbs")}
+        roof.update({"config5_frac": c5["kernel_frac"], "config5_per_launch_ms": c5["kernel_ms"], "config5_traffic": c5["traffic"]})
+        details["config5"] = c5
+    if only == "ceiling":
+        mfma_peak, mfma_ms = ceil.mfma_tflops()
+        read_peak, read_ms = ceil.read_gbs()
+        line.update({"value": mfma_peak, "unit": "TFLOP/s", "ms_per_step": mfma_ms, "config": {"workload": "ceilings: MFMA stream, 4 GiB read"}})
+        summary["ceiling"] = {"mfma_tflops": _r(mfma_peak, 1), "mfma_ms": _r(mfma_ms), "read_gbs": _r(read_peak, 1), "read_ms": _r(read_ms)}
+    if only is None:
+        summary["short_prompts"] = short_prompts()
+        summary["ceiling"] = {"mfma_tflops": _r(roof.get("sustained_peak"), 1), "read_gbs": _r(roof.get("decode_sustained_peak_gbs"), 1)}
+    if args.sweeps:
+        details["prefill_launch_sizes"] = prefill_launch_sizes(tile_us)
+        details["decode_latency"] = decode_latency()
+        details["decode_large_groups"] = decode_large_groups()
+        details["decode_mixed_lengths"] = decode_mixed_lengths()
     if args.all:
-        line["other"] = other_steps(max(3, min(args.steps, 10)))
+        details["other"] = other_steps(10)
+    if roof:
+        line["roofline"] = {k: (_r(v, 5) if isinstance(v, float) else v) for k, v in roof.items()}
+    if cpu:
+        line["cpu_baseline"] = cpu
+    if "value" not in line and summary:  # --only config1/4/5: that workload is the line's value
+        k = next(iter(summary))
+        line.update({"value": summary[k]["value"], "unit": summary[k]["unit"], "ms_per_step": summary[k]["ms"], "config": {"workload": details[k]["workload"]}})
+    line["summary"] = summary  # (last: a reader that keeps the tail of the line keeps all five configs)
+    if (args.sweeps or args.all) and details:
+        os.makedirs(os.path.dirname(os.path.abspath(args.details_out)), exist_ok=True)
+        with open(args.details_out, "w") as f:
+            json.dump(details, f, indent=1)
     print(json.dumps(line))
 
 

@@ -14,6 +14,7 @@ PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(PKG_DIR)
 CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_PATH = os.path.join(PKG_DIR, "liblsattn.so")
+CEILING_LIB_PATH = os.path.join(PKG_DIR, "libls_ceiling.so")  # measurement aids of bench.py (include/ls_ceiling.h)
 SOURCES = ["prefill.hip", "decode.hip", "merge_scatter.hip", "elementwise.hip", "pool.hip"]
 # elementwise.hip reproduces the reference's half arithmetic operation by operation: no fused multiply-adds
 # other than the ones it writes
@@ -56,6 +57,18 @@ def build_all(verbose: bool = False, extra_flags=(), out: str = LIB_PATH) -> str
     return out
 
 
+def build_ceiling(verbose: bool = False, out: str = CEILING_LIB_PATH) -> str:
+    """libls_ceiling.so: the MFMA stream and the streaming read that bench.py measures a box's sustained ceilings with."""
+    obj = _compile("ceiling.hip", [])
+    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-fno-gpu-rdc", obj, "-o", out]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("link failed:\n%s\n%s" % (" ".join(cmd), r.stderr[-6000:]))
+    if verbose:
+        print("built", out)
+    return out
+
+
 C_ABI_EXAMPLES = [os.path.join(ROOT, "tests", "c_abi", n) for n in ("decode_from_c", "prefill_from_c")]
 
 
@@ -75,4 +88,5 @@ def build_c_abi_example(verbose: bool = False):
 
 if __name__ == "__main__":
     build_all(verbose=True, extra_flags=sys.argv[1:])
+    build_ceiling(verbose=True)
     build_c_abi_example(verbose=True)
