@@ -71,6 +71,7 @@ struct PrefillParams {
   int32_t tile_major;  // order of the workgroups in the grid: heaviest query tiles of all KV heads first
   int32_t n_first, n_second;  // the fastest and the second index of the grid: (kv_slots, units_per_slice) if tile_major, else swapped
   int32_t pack_shift, heads_per_kv;  // 1 << pack_shift query heads of a KV head side by side in a workgroup; query heads per KV head
+  int32_t fold_from, fold_sum;       // (ids >> 3) from fold_from on run backwards: j -> fold_sum - j (0: the whole grid runs forwards)
   int32_t kv_cuts, kv_cut_len;       // every sequence entered kv_cuts times, entry c taking keys [c, c + 1) * kv_cut_len of its chunk
   int64_t o_cut_rows;                // and writing its rows o_cut_rows * c further down
   FastDiv d_peers, d_first, d_second, d_slices, d_group, d_cuts;
@@ -246,6 +247,10 @@ __global__ __launch_bounds__(HALF ? NWAVE * 32 : NWAVE * 64, HALF ? 2 : 1) void 
   const int group = p.group;
   uint32_t j = blockIdx.x >> 3;
   const int xcd = blockIdx.x & 7;
+  // A launch of the four-wave shape that fits the chip at once (two workgroups per CU) is paired up by the hardware:
+  // workgroup id and id + 256 share a CU.  The second 256 then run from the lightest tile upwards, so that the heaviest
+  // meets the lightest and every CU gets the same work.
+  if (HALF && p.fold_from && j >= (uint32_t)p.fold_from) j = (uint32_t)p.fold_sum - j;
   // Two orders of the grid within a request, by which of the two indices runs fastest (the host sets d_first / d_second):
   // launches of a few workgroups per CU deal the heaviest query tiles of all KV heads first (under causal masking tile z
   // walks z + 1 key blocks), so that a CU that has finished a light tile of the first round takes a heavy one of the rest
@@ -1067,7 +1072,7 @@ static int pack_shift_for(const lsattn_prefill_args* a, bool split, const Tuning
 }
 
 template <typename T, int MODE, bool DV, bool SPLIT, bool HALF = false>
-static int launch_prefill_rows(const lsattn_prefill_args* a, bool tile_major, const Tuning& tn, hipStream_t st) {
+static int launch_prefill_rows(const lsattn_prefill_args* a, bool tile_major, const Tuning& tn, hipStream_t st, bool fold = false) {
   constexpr int BMW = SPLIT || HALF ? BM / 2 : BM;
   PrefillParams p;
   p.q = a->q;
@@ -1125,6 +1130,11 @@ static int launch_prefill_rows(const lsattn_prefill_args* a, bool tile_major, co
   p.d_second = fast_div((uint32_t)p.n_second);
   const int64_t wgs = (int64_t)8 * p.units_per_slice * p.kv_slots * a->batch * p.kv_cuts;
   if (wgs > 0x7fffffff) return LSATTN_ERR_INVALID_ARG;
+  p.fold_from = p.fold_sum = 0;
+  if (HALF && fold && wgs > 2 * kCUs / 2 && wgs <= 2 * kCUs) {
+    p.fold_from = (int32_t)(kCUs / 8);
+    p.fold_sum = p.fold_from + (int32_t)(wgs / 8) - 1;
+  }
   hipLaunchKernelGGL((prefill_kernel<T, MODE, DV, SPLIT, HALF>), dim3((unsigned)wgs), dim3(HALF ? NWAVE * 32 : NWAVE * 64), 0, st, p);
   return check_launch();
 }
@@ -1167,6 +1177,14 @@ template <typename T, int MODE, bool DV> static int launch_prefill(const lsattn_
     if (tn.prefill_rows == LSATTN_PREFILL_ROWS_128) split = true, half = false;
     if (tn.prefill_rows == LSATTN_PREFILL_ROWS_256) split = false, half = false;
     if (tn.prefill_rows == LSATTN_PREFILL_ROWS_HALF) half = true;
+    // One request whose four-wave workgroups all fit the chip at once, more than one and at most two per CU (a single
+    // sequence of up to 2048 tokens: 32 heads x sixteen 128-row tiles): the four-wave shape with the second half of the
+    // grid running backwards (see the kernel), each CU one heavy and one light workgroup side by side, instead of the
+    // split shape's two rounds.  Longer chunks keep the rules above (the pairs' work is then long against what a
+    // workgroup costs besides its tiles, and the shape's rings of two tiles are the slower ones per tile).
+    const bool fold = a->batch == 1 && cuts == 1 && !a->o_b_start_loc && a->max_q_len <= 2048 && wgs128 > kCUs && wgs128 <= 2 * kCUs &&
+                      tn.prefill_rows == 0;
+    if (fold) return launch_prefill_rows<T, MODE, true, false, true>(a, true, tn, st, true);
     if (half) return launch_prefill_rows<T, MODE, true, false, true>(a, true, tn, st);
     return split ? launch_prefill_rows<T, MODE, true, true>(a, true, tn, st) : launch_prefill_rows<T, MODE, true, false>(a, tile_major, tn, st);
   }

@@ -139,6 +139,12 @@ def test_config5_varlen_prefill_full_size(lsa):
     heads = [3, 30]
     kvh = [h // (v.Hq // v.Hkv) for h in heads]
     lse_state = (0.6931471805599453 * (v.m.double() + torch.log2(v.l.double()))).float()
+    # the same step on the fp32-partial route (bf16 in, fp32 (O, LSE) out), which is held to the stated bars
+    o32 = torch.empty((v.T, v.Hq, v.D), dtype=torch.float32, device=DEV)
+    l32 = torch.empty((v.T, v.Hq), dtype=torch.float32, device=DEV)
+    lsa.prefill_attention_step(v.q, v.kv[:, :v.Hkv], v.kv[:, v.Hkv:], v.start, v.len, v.first, v.start, v.len, v.first, 1, v.max_len,
+                               out=o32, lse=l32, v_f16=v.v_f16, v_f16_valid=True)
+    torch.cuda.synchronize()
     for i in (order[0], order[5], order[-2], order[-1]):
         n, s0 = lens[i], starts[i]
         rows = sorted(set([0, 1, 63, 64, n // 3, n - 2, n - 1]))
@@ -156,6 +162,8 @@ def test_config5_varlen_prefill_full_size(lsa):
         # o is stored in bfloat16 (8 significant bits): bar scaled to 2^-8
         assert_o_close(got, o_ref, "cfg5 o seq %d" % i, max_abs=8e-3, rel=4e-3)
         assert_lse_close(lse_state[[s0 + r for r in rows]][:, heads], l_ref, "cfg5 LSE seq %d" % i)
+        assert_o_close(o32[[s0 + r for r in rows]][:, heads], o_ref, "cfg5 fp32 partial O seq %d" % i)  # 2e-3 / 1e-3
+        assert_lse_close(l32[[s0 + r for r in rows]][:, heads], l_ref, "cfg5 fp32 partial LSE seq %d" % i)
     # KV persistence: every scattered row reads back bit-for-bit through the registered table
     for i in (order[0], order[-1]):
         n, s0 = lens[i], starts[i]

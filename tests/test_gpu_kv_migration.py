@@ -28,6 +28,20 @@ def test_kv_ranges_match_oracle(lsa):
     assert rb.numel() == 0
 
 
+def test_kv_ranges_of_a_window_that_starts_before_the_first_held_token(lsa):
+    """The ceil of a negative quotient, in the form the reference documents (Python floor division of x + P - 1,
+    copy_and_register_kv.py:42-45), in literal numbers: window [0, 3) or [4, 20) against a chunk whose first held token is
+    9, 5 or 8 with 4 peers.  The reference's own windows never start more than P - 1 before the first held token, where
+    every reading of the division agrees; for the others a C-style truncating division would give -1 / 0 / 0 here."""
+    begin, end, first = _i32([0, 0, 4]).to(DEV), _i32([3, 3, 20]).to(DEV), _i32([9, 5, 8]).to(DEV)
+    rb, re, nl = lsa.pre_copy_and_register_kv(begin, end, first, 4)
+    assert rb.tolist() == [-2, -1, -1]          # ceil(-9/4), ceil(-5/4), ceil(-4/4)
+    assert re.tolist() == [-1, 0, 3]            # ceil(-6/4), ceil(-2/4), ceil(12/4)
+    assert nl.tolist() == [1, 1, 4]
+    rb_o, re_o, nl_o = orc.kv_ranges([0, 0, 4], [3, 3, 20], [9, 5, 8], 4)
+    assert torch.equal(rb.cpu(), rb_o) and torch.equal(re.cpu(), re_o) and torch.equal(nl.cpu(), nl_o)
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("register", [True, False])
 def test_copy_and_register_matches_oracle(lsa, dtype, register):

@@ -257,6 +257,48 @@ def test_bf16_v_converted_inside_the_kernel_or_before_it(lsa):
         ops.PRECONVERT_BF16_V = True
 
 
+def test_bf16_step_whose_v_leaves_fp16s_range(lsa):
+    """A bfloat16 V with magnitudes beyond fp16's largest finite value and below its smallest normal one: the P V product
+    runs in fp16, so the step's result is that of the same step on V rewritten as fp16 toward zero (65504 for anything
+    larger, fp16's subnormal grid below 2^-14, zero below 2^-24), on both routes (V rewritten before the launch, and
+    inside the kernel).  The expected rewriting is spelled out value by value; the oracle runs on the rewritten V.
+    O reaches the hundreds here, so its max-abs bar is scaled by the largest |O| of the oracle."""
+    from loongserve_amd import ops
+    lens, Hq, Hkv, D = [900, 333], 8, 2, 128
+    T = sum(lens)
+    q = rand_t((T, Hq, D), 21, torch.bfloat16)
+    kv = rand_t((T, 2 * Hkv, D), 22, torch.bfloat16)
+    special = [(70000.0, 65504.0), (-70000.0, -65504.0), (1e38, 65504.0), (-3e20, -65504.0), (65504.0, 65504.0),
+               (2.0 ** -15, 2.0 ** -15), (3 * 2.0 ** -17, 3 * 2.0 ** -17), (-2.0 ** -20, -2.0 ** -20),
+               (2.0 ** -26, 0.0), (1.5 * 2.0 ** -25, 0.0), (-1.75 * 2.0 ** -24, -2.0 ** -24)]
+    g = torch.Generator().manual_seed(23)
+    v_expect = kv[:, Hkv:].float().clone()     # every other value of N(0, 1) * 0.5 in bfloat16 is exact in fp16 down to 2^-24
+    tiny = v_expect.abs() < 2.0 ** -14
+    v_expect[tiny] = torch.trunc(v_expect[tiny] * 2.0 ** 24) / 2.0 ** 24
+    for i in range(400):
+        t, h, d = int(torch.randint(0, T, (1,), generator=g)), int(torch.randint(0, Hkv, (1,), generator=g)), int(torch.randint(0, D, (1,), generator=g))
+        src, want = special[i % len(special)]
+        kv[t, Hkv + h, d] = src
+        assert float(kv[t, Hkv + h, d]) == float(torch.tensor(src).to(torch.bfloat16))
+        v_expect[t, h, d] = want
+    assert float(torch.tensor(1.5 * 2.0 ** -25).to(torch.bfloat16)) == 1.5 * 2.0 ** -25     # (the sources are exact in bfloat16)
+    m = meta(lens)
+    o_ref, lse_ref = orc.attn_step(q.float(), kv[:, :Hkv].float(), v_expect, *m, *m, 1)
+    scale = max(1.0, float(o_ref.abs().max()))
+    assert scale > 50
+    kvd, qd = kv.to(DEV), q.to(DEV)
+    qs, ql, qf = _dev(*m)
+    try:
+        for pre in (True, False):
+            ops.PRECONVERT_BF16_V = pre
+            o, lse = lsa.prefill_attention_step(qd, kvd[:, :Hkv], kvd[:, Hkv:], qs, ql, qf, qs, ql, qf, 1, max(lens))
+            torch.cuda.synchronize()
+            assert_o_close(o, o_ref, "O (pre-converted V: %s)" % pre, max_abs=2e-3 * scale)
+            assert_lse_close(lse, lse_ref, "LSE (pre-converted V: %s)" % pre)
+    finally:
+        ops.PRECONVERT_BF16_V = True
+
+
 def test_bf16_to_f16_rows_is_exact_in_range_and_saturates(lsa):
     from loongserve_amd import _lib
     lib = _lib.load()
