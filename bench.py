@@ -572,6 +572,38 @@ def short_prompts():
     return rows
 
 
+def chunked_prefill_step():
+    """A chunked-prefill step of a long request (outside the five configs): 100 query rows against a KV chunk of 131072
+    keys, GQA 32/8, fp16, all keys visible.  Through prefill_attention_step (fp32 partial, KV cut chosen by the library),
+    through the reference's operator context_attention_fwd with a caller workspace (the same cut, folded into (o, m, l)),
+    and through context_attention_fwd as the reference calls it (no workspace: one workgroup per 128 rows and head).
+    Device time per call from a HIP graph of 10 calls, median of 10 replays."""
+    import loongserve_amd as lsa
+    Tq, Tk, Hq, Hkv = 100, 131072, 32, 8
+    q = _randn_half((Tq, Hq, D), 4601)
+    kv = _randn_half((Tk, 2 * Hkv, D), 4602)
+    qm = (_i32([0]), _i32([Tq]), _i32([Tk]))
+    km = (_i32([0]), _i32([Tk]), _i32([0]))
+    o32 = torch.empty((Tq, Hq, D), dtype=torch.float32, device=DEV)
+    l32 = torch.empty((Tq, Hq), dtype=torch.float32, device=DEV)
+    o16 = torch.zeros((Tq, Hq, D), dtype=torch.float16, device=DEV)
+    m = torch.full((Tq, Hq), float("-inf"), device=DEV)
+    l = torch.zeros((Tq, Hq), device=DEV)
+    from loongserve_amd.ops import kv_split_count
+    S = kv_split_count(1, Hq, Tq, Tk)
+    ws = torch.empty(S * Tq * Hq * (D + 1), dtype=torch.float32, device=DEV)
+    step = lambda: lsa.prefill_attention_step(q, kv[:, :Hkv], kv[:, Hkv:], *qm, *km, 1, Tq, out=o32, lse=l32, kv_split_workspace=ws)  # noqa: E731
+    op_ws = lambda: lsa.context_attention_fwd(q, kv[:, :Hkv], kv[:, Hkv:], o16, *qm, *km, 1, Tq, m, l, workspace=ws)  # noqa: E731
+    op = lambda: lsa.context_attention_fwd(q, kv[:, :Hkv], kv[:, Hkv:], o16, *qm, *km, 1, Tq, m, l)  # noqa: E731
+    out = {"workload": "100 query rows x 131072 keys, GQA 32/8, fp16", "kv_cuts": S}
+    for key, fn in (("prefill_attention_step_us", step), ("context_attention_fwd_workspace_us", op_ws), ("context_attention_fwd_us", op)):
+        out[key] = _r(_time_graph(fn, launches=10, reps=10, warm_reps=2) * 1e3, 1)
+    gb = Tk * 2 * Hkv * D * 2 / 1e9
+    out["kv_gbs_workspace_route"] = _r(gb / (out["context_attention_fwd_workspace_us"] * 1e-6), 0)
+    torch.cuda.empty_cache()
+    return out
+
+
 def _tiles_256x64(N, Hq, B, pack=1):
     """64-key tiles that 256-row workgroups walk for B causal sequences of N tokens (pack query heads side by side)."""
     rows = 256 // pack
@@ -803,7 +835,7 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
-    ap.add_argument("--only", choices=["prefill", "decode", "config1", "config4", "config5", "ceiling"], default=None,
+    ap.add_argument("--only", choices=["prefill", "decode", "config1", "config4", "config5", "ceiling", "chunked"], default=None,
                     help="time one workload only (profiling aid)")
     ap.add_argument("--calib-copy", action="store_true",
                     help="only run three plain 1 GiB device-to-device copies (known traffic, for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE)")
@@ -938,8 +970,13 @@ def main():
         read_peak, read_ms = ceil.read_gbs()
         line.update({"value": mfma_peak, "unit": "TFLOP/s", "ms_per_step": mfma_ms, "config": {"workload": "ceilings: MFMA stream, 4 GiB read"}})
         summary["ceiling"] = {"mfma_tflops": _r(mfma_peak, 1), "mfma_ms": _r(mfma_ms), "read_gbs": _r(read_peak, 1), "read_ms": _r(read_ms)}
+    if only == "chunked":
+        summary["chunked_prefill_step"] = c = chunked_prefill_step()
+        line.update({"value": c["kv_gbs_workspace_route"], "unit": "GB/s", "ms_per_step": c["context_attention_fwd_workspace_us"] * 1e-3,
+                     "config": {"workload": c["workload"]}})
     if only is None:
         summary["short_prompts"] = short_prompts()
+        summary["chunked_prefill_step"] = chunked_prefill_step()
         summary["ceiling"] = {"mfma_tflops": _r(roof.get("sustained_peak"), 1), "read_gbs": _r(roof.get("decode_sustained_peak_gbs"), 1)}
     if args.sweeps:
         details["prefill_launch_sizes"] = prefill_launch_sizes(tile_us)

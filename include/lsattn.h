@@ -101,6 +101,12 @@ typedef struct lsattn_prefill_args {
   int32_t kv_cuts;
   int32_t kv_cut_len;
   int64_t o_cut_rows;
+  /* Optional (0: unknown); no counterpart in the reference.  An upper bound of the sum of q_b_seq_len over the batch (the
+   * rows of a packed q, for sequences that do not share rows).  The launch is sized by max_q_len times the batch (RING:262),
+   * all the host knows; in a batch of one long request and many short ones most of those workgroups find no rows.  With
+   * the bound the launch may be sized by the query tiles that can exist instead, each workgroup finding its request from
+   * q_b_seq_len.  A bound below the real sum leaves the rows beyond it uncomputed. */
+  int64_t total_q_rows;
 } lsattn_prefill_args;
 
 /* Partial of one step from the empty state: o = normalised fp32 output, lse = natural-log
@@ -523,7 +529,7 @@ const char* lsattn_strerror(int code);
  * carry no size field, so a caller must be compiled against the header of the library it loads: check
  * lsattn_version() == LSATTN_VERSION once after loading and refuse to run otherwise.
  * 2 = o_b_start_loc in lsattn_prefill_args, partials_by_request in both decode argument blocks; 3 = lsattn_set_tuning,
- * kv_cuts / kv_cut_len / o_cut_rows in lsattn_prefill_args, lsattn_prefill_merge_cuts. */
+ * kv_cuts / kv_cut_len / o_cut_rows / total_q_rows in lsattn_prefill_args, lsattn_prefill_merge_cuts. */
 #define LSATTN_VERSION 3
 int lsattn_version(void);
 

@@ -35,7 +35,7 @@ class PrefillArgs(C.Structure):
         ("lse", _vp), ("m", _vp), ("l", _vp),
         ("ml_stride_t", _i64), ("ml_stride_h", _i64),
         ("o_b_start_loc", _vp),
-        ("kv_cuts", _i32), ("kv_cut_len", _i32), ("o_cut_rows", _i64),
+        ("kv_cuts", _i32), ("kv_cut_len", _i32), ("o_cut_rows", _i64), ("total_q_rows", _i64),
     ]
 
 

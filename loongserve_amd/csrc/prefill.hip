@@ -72,6 +72,7 @@ struct PrefillParams {
   int32_t n_first, n_second;  // the fastest and the second index of the grid: (kv_slots, units_per_slice) if tile_major, else swapped
   int32_t pack_shift, heads_per_kv;  // 1 << pack_shift query heads of a KV head side by side in a workgroup; query heads per KV head
   int32_t fold_from, fold_sum;       // (ids >> 3) from fold_from on run backwards: j -> fold_sum - j (0: the whole grid runs forwards)
+  int32_t listed, rows_shift;        // the grid numbers the (request, query tile, head group) units that exist (see the kernel); log2 of a workgroup's query positions
   int32_t kv_cuts, kv_cut_len;       // every sequence entered kv_cuts times, entry c taking keys [c, c + 1) * kv_cut_len of its chunk
   int64_t o_cut_rows;                // and writing its rows o_cut_rows * c further down
   FastDiv d_peers, d_first, d_second, d_slices, d_group, d_cuts;
@@ -90,6 +91,8 @@ constexpr int SUB = 32;   // keys per pipeline step (the contraction length of o
 constexpr int NWAVE = 8;  // two per SIMD
 constexpr int64_t kCUs = 256;  // compute units of the MI355X (one workgroup of this kernel each)
 constexpr int64_t kTileMajorBelowWorkgroups = 2048;  // 256-row workgroups in a launch below which the grid runs the heaviest tiles of all KV heads first
+constexpr int64_t kListedFromWorkgroups = 4096;  // launches from which a caller's bound on the rows of all requests may shrink the grid
+constexpr int kListedMaxBatch = 4096;            // (every workgroup walks the batch's lengths once)
 constexpr float kLazyRescale = 8.f;  // log2 units the running max may lag before O is rescaled
 
 template <typename T> struct Mfma;
@@ -258,12 +261,53 @@ __global__ __launch_bounds__(HALF ? NWAVE * 32 : NWAVE * 64, HALF ? 2 : 1) void 
   // serves all the workgroups the XCD runs.  One request after the other in both (its K/V stays in the L2s).
   const uint32_t j1 = div_by(j, p.d_first);
   const int r1 = (int)(j - j1 * p.n_first);
-  j = div_by(j1, p.d_second);
-  const int r2 = (int)(j1 - j * p.n_second);
-  const int up = p.tile_major ? r2 : r1, slot = p.tile_major ? r1 : r2;
-  // (sequence, cut of its KV chunk): j < batch * kv_cuts for every workgroup of the grid
-  const int b = (int)div_by(j, p.d_cuts);
-  const int cut = (int)j - b * p.kv_cuts;
+  int up, slot, b, cut, nz = p.nz;
+  if (p.listed) {
+    // The grid above is sized by the longest request times the batch (the host knows max_q_len, not the lengths): a
+    // batch of one long request and many short ones is mostly workgroups without rows.  Here the grid has a workgroup
+    // per unit that can exist (from an upper bound of the rows of all requests together) and a workgroup finds its
+    // request by numbering the units of all requests: request b has (query heads per KV head / heads per workgroup) x
+    // ceil(q_len[b] / positions per workgroup) of them, heaviest tile first.  Every wave numbers them by itself, 64
+    // requests per step (an inclusive sum over the lanes); no LDS, no barrier.
+    slot = r1;
+    const uint32_t unit = j1;  // (KV head slots run fastest)
+    const int lane_id = threadIdx.x & 63;
+    uint32_t carry = 0;
+    b = -1;
+    up = 0;
+    for (int b0 = 0; b0 < p.batch; b0 += 64) {
+      const int bb = b0 + lane_id;
+      const int len = bb < p.batch ? p.q_len[bb] : 0;
+      const uint32_t tiles = len > 0 ? ((uint32_t)len + (1u << p.rows_shift) - 1) >> p.rows_shift : 0;
+      const uint32_t units = tiles * (uint32_t)group;
+      uint32_t incl = units;
+#pragma unroll
+      for (int d = 1; d < 64; d <<= 1) {
+        const uint32_t below = __shfl_up(incl, d, 64);
+        if (lane_id >= d) incl += below;
+      }
+      const uint32_t chunk_total = __builtin_amdgcn_readlane(incl, 63);
+      if (unit < carry + chunk_total) {  // (the same for every lane)
+        const uint64_t past = __builtin_amdgcn_ballot_w64(carry + incl > unit);  // lanes whose units end behind this one
+        const int l0 = __builtin_amdgcn_readfirstlane(__builtin_ctzll(past));
+        b = b0 + l0;
+        up = (int)(unit - (carry + __builtin_amdgcn_readlane(incl, l0) - __builtin_amdgcn_readlane(units, l0)));
+        nz = (int)__builtin_amdgcn_readlane(tiles, l0);
+        break;
+      }
+      carry += chunk_total;
+    }
+    if (b < 0) return;  // past the last unit that exists
+    cut = 0;
+  } else {
+    j = div_by(j1, p.d_second);
+    const int r2 = (int)(j1 - j * p.n_second);
+    up = p.tile_major ? r2 : r1;
+    slot = p.tile_major ? r1 : r2;
+    // (sequence, cut of its KV chunk): j < batch * kv_cuts for every workgroup of the grid
+    b = (int)div_by(j, p.d_cuts);
+    cut = (int)j - b * p.kv_cuts;
+  }
   // The request's six numbers, all requested before the first of them is used (one memory latency instead of three on
   // the way to the first tile load; a workgroup's start-up is what a short launch is made of).
   const int q_len = p.q_len[b], kv_len_all = p.kv_len[b], qf = p.q_first[b], kf_all = p.kv_first[b];
@@ -279,9 +323,9 @@ __global__ __launch_bounds__(HALF ? NWAVE * 32 : NWAVE * 64, HALF ? 2 : 1) void 
   const int vh = xcd + 8 * slot;  // (KV head, slice) pair: always < hkv * slices
   const int kvh = (int)div_by((uint32_t)vh, p.d_slices);
   const int u = up * p.slices + (vh - kvh * p.slices);
-  if (u >= group * p.nz) return;
+  if (u >= group * nz) return;
   const int zr = (int)div_by((uint32_t)u, p.d_group), gq = u - zr * group;
-  const int z = p.nz - 1 - zr;
+  const int z = nz - 1 - zr;
 
   // The workgroup's rows: 1 << pack_shift query heads of the KV head side by side, BMW >> pack_shift query positions of
   // each (grouped-query attention: the heads of a group read the same K/V, so a workgroup of several of them walks the
@@ -1131,11 +1175,28 @@ static int launch_prefill_rows(const lsattn_prefill_args* a, bool tile_major, co
   const int64_t wgs = (int64_t)8 * p.units_per_slice * p.kv_slots * a->batch * p.kv_cuts;
   if (wgs > 0x7fffffff) return LSATTN_ERR_INVALID_ARG;
   p.fold_from = p.fold_sum = 0;
+  p.listed = 0;
+  p.rows_shift = (SPLIT || HALF ? 7 : 8) - p.pack_shift;
+  // A grid of the units that can exist instead of one sized by the longest request (see the kernel), when the caller
+  // bounds the rows of all requests together and that grid is at most half of the other: a skewed batch.  (One KV head
+  // or slot per XCD index only, and no cuts along the keys.)
+  int64_t wgs_launch = wgs;
+  if (a->total_q_rows > 0 && p.slices == 1 && p.kv_cuts == 1 && a->batch <= kListedMaxBatch && wgs >= kListedFromWorkgroups) {
+    const int64_t rows_wg = BMW >> p.pack_shift;
+    const int64_t units_max = (int64_t)group * ((a->total_q_rows + rows_wg - 1) / rows_wg + a->batch);
+    const int64_t wgs_listed = 8 * p.kv_slots * units_max;
+    if (wgs_listed * 2 <= wgs) {
+      p.listed = 1;
+      p.n_first = p.kv_slots;
+      p.d_first = fast_div((uint32_t)p.n_first);
+      wgs_launch = wgs_listed;
+    }
+  }
   if (HALF && fold && wgs > 2 * kCUs / 2 && wgs <= 2 * kCUs) {
     p.fold_from = (int32_t)(kCUs / 8);
     p.fold_sum = p.fold_from + (int32_t)(wgs / 8) - 1;
   }
-  hipLaunchKernelGGL((prefill_kernel<T, MODE, DV, SPLIT, HALF>), dim3((unsigned)wgs), dim3(HALF ? NWAVE * 32 : NWAVE * 64), 0, st, p);
+  hipLaunchKernelGGL((prefill_kernel<T, MODE, DV, SPLIT, HALF>), dim3((unsigned)wgs_launch), dim3(HALF ? NWAVE * 32 : NWAVE * 64), 0, st, p);
   return check_launch();
 }
 
@@ -1157,7 +1218,14 @@ template <typename T, int MODE, bool DV> static int launch_prefill(const lsattn_
   const int64_t nz256 = (a->max_q_len + BM - 1) / BM;
   const int ps = pack_shift_for(a, false, tn);  // (the workgroups of several heads are shorter: less padding past a short chunk)
   const int64_t cuts = a->kv_cuts > 1 ? a->kv_cuts : 1;
-  const int64_t wgs256 = cuts * a->batch * (a->num_q_heads >> ps) * ((a->max_q_len + (BM >> ps) - 1) / (BM >> ps));
+  // query tiles of `rows` positions over the whole batch: the longest request's times the batch, or fewer if the caller
+  // bounds the rows of all requests together
+  auto tiles_of = [&](int64_t rows) {
+    const int64_t by_longest = a->batch * ((a->max_q_len + rows - 1) / rows);
+    const int64_t by_total = a->total_q_rows > 0 ? (a->total_q_rows + rows - 1) / rows + a->batch : by_longest;
+    return by_total < by_longest ? by_total : by_longest;
+  };
+  const int64_t wgs256 = cuts * (a->num_q_heads >> ps) * tiles_of(BM >> ps);
   bool tile_major = wgs256 < kTileMajorBelowWorkgroups;
   if (tn.prefill_order == LSATTN_PREFILL_ORDER_TILE) tile_major = true;
   if (tn.prefill_order == LSATTN_PREFILL_ORDER_HEAD) tile_major = false;
@@ -1172,7 +1240,7 @@ template <typename T, int MODE, bool DV> static int launch_prefill(const lsattn_
     // one of short chunks against long K/V (which the host cannot tell apart) would run on half the CUs.  Not for
     // launches that write their rows elsewhere either (the step cut along the keys: few, long workgroups).
     const int ph = pack_shift_for(a, true, tn);
-    const int64_t wgs128 = cuts * a->batch * (a->num_q_heads >> ph) * ((a->max_q_len + (BM / 2 >> ph) - 1) / (BM / 2 >> ph));
+    const int64_t wgs128 = cuts * (a->num_q_heads >> ph) * tiles_of(BM / 2 >> ph);
     bool half = a->max_q_len <= (ph ? 1024 : 1536) && !a->o_b_start_loc && a->kv_cuts <= 1 && wgs128 >= 3 * kCUs;
     if (tn.prefill_rows == LSATTN_PREFILL_ROWS_128) split = true, half = false;
     if (tn.prefill_rows == LSATTN_PREFILL_ROWS_256) split = false, half = false;
@@ -1195,7 +1263,7 @@ static int validate(const lsattn_prefill_args* a, int mode) {
   if (!a->q_b_start_loc || !a->q_b_seq_len || !a->q_first_token_global_idx || !a->kv_b_start_loc || !a->kv_b_seq_len ||
       !a->kv_first_token_global_idx)
     return LSATTN_ERR_INVALID_ARG;
-  if (a->batch < 0 || a->num_q_heads <= 0 || a->num_kv_heads <= 0 || a->sp_peers < 1 || a->max_q_len < 0)
+  if (a->batch < 0 || a->num_q_heads <= 0 || a->num_kv_heads <= 0 || a->sp_peers < 1 || a->max_q_len < 0 || a->total_q_rows < 0)
     return LSATTN_ERR_INVALID_ARG;
   if (a->num_q_heads % a->num_kv_heads) return LSATTN_ERR_INVALID_ARG;
   if (a->head_dim != 128) return LSATTN_ERR_UNSUPPORTED;

@@ -100,7 +100,7 @@ def _pad_head_dim(t: torch.Tensor) -> torch.Tensor:
 def _prefill_args(q, k, v, o, q_b_start_loc, q_b_seq_len, q_first, kv_b_start_loc, kv_b_seq_len, kv_first,
                   peers: int, max_q_len: int, sm_scale: Optional[float], v_f16: Optional[torch.Tensor] = None,
                   v_f16_valid: bool = False, o_b_start_loc: Optional[torch.Tensor] = None,
-                  cuts: Optional[Tuple[int, int, int]] = None) -> _lib.PrefillArgs:
+                  cuts: Optional[Tuple[int, int, int]] = None, total_q_len: Optional[int] = None) -> _lib.PrefillArgs:
     for t, n in ((q, "q"), (k, "k"), (v, "v"), (o, "o")):
         _dev(t, n)
         if t.dim() != 3:
@@ -154,6 +154,10 @@ def _prefill_args(q, k, v, o, q_b_start_loc, q_b_seq_len, q_first, kv_b_start_lo
         a.o_b_start_loc = o_b_start_loc.data_ptr()
     if cuts is not None:
         a.kv_cuts, a.kv_cut_len, a.o_cut_rows = int(cuts[0]), int(cuts[1]), int(cuts[2])
+    if total_q_len is not None:
+        if int(total_q_len) < 0:
+            raise ValueError("total_q_len must be >= 0")
+        a.total_q_rows = int(total_q_len)
     return a
 
 
@@ -224,7 +228,7 @@ def context_attention_fwd(q, k, v, o, q_b_start_loc, q_b_seq_len, q_first_token_
                           kv_b_start_loc, kv_b_seq_len, kv_first_token_global_idx,
                           logical_sp_peers_num: int, max_q_b_seq_len: int, m, l, *, v_f16: Optional[torch.Tensor] = None,
                           v_f16_valid: bool = False, workspace=None, max_kv_len: Optional[int] = None,
-                          kv_splits: Optional[int] = None) -> None:
+                          kv_splits: Optional[int] = None, total_q_len: Optional[int] = None) -> None:
     """One ring-attention step folded in place into (o, m, l); signature of RING:191-206.
 
     Keyword-only additions for bfloat16 inputs (the reference is fp16 only): the kernel multiplies P and V in fp16, so V is
@@ -240,6 +244,11 @@ def context_attention_fwd(q, k, v, o, q_b_start_loc, q_b_seq_len, q_first_token_
     upper bound of every chunk's length, replaces the rows of the k buffer there: in the layer k is a view of a buffer
     sized for the longest batch), capped by what the workspace holds; kv_splits forces it.  Without a workspace the call
     is the reference's: one launch, no scratch.  (m, l) stay opaque: a step folded this way enters as (its LSE, 1).
+
+    Keyword-only, for batches that mix long and short requests: total_q_len, an upper bound of the sum of q_b_seq_len
+    (q.shape[0] when q is packed and no two sequences share rows).  The launch is sized by max_q_b_seq_len times the batch
+    (RING:262), all the host knows; with the bound it is sized by the query tiles that can exist when those are at most half
+    as many.  A bound below the real sum leaves rows uncomputed.
 
     Call it repeatedly with the same local q/o/m/l and a different kv chunk each time.
     Start from m = -inf, l = 0 (o need not be zeroed).  After k calls o is the
@@ -279,7 +288,7 @@ def context_attention_fwd(q, k, v, o, q_b_start_loc, q_b_seq_len, q_first_token_
         return
     a = _prefill_args(q, k, v, o, q_b_start_loc, q_b_seq_len, q_first_token_global_idx, kv_b_start_loc,
                       kv_b_seq_len, kv_first_token_global_idx, logical_sp_peers_num, max_q_b_seq_len,
-                      1.0 / (D ** 0.5), v_f16 if o_user is None else None, v_f16_valid and o_user is None)
+                      1.0 / (D ** 0.5), v_f16 if o_user is None else None, v_f16_valid and o_user is None, total_q_len=total_q_len)
     a.m, a.l = m.data_ptr(), l.data_ptr()
     a.ml_stride_t, a.ml_stride_h = m.stride(0), m.stride(1)
     _lib.check(_lib.load().lsattn_prefill_step_merge(C.byref(a), _stream()), "lsattn_prefill_step_merge")
@@ -294,7 +303,8 @@ def prefill_attention_step(q, k, v, q_b_start_loc, q_b_seq_len, q_first_token_gl
                            out: Optional[torch.Tensor] = None, lse: Optional[torch.Tensor] = None,
                            sm_scale: Optional[float] = None, accumulate: bool = False, v_f16: Optional[torch.Tensor] = None,
                            v_f16_valid: bool = False, kv_splits: Optional[int] = None,
-                           kv_split_workspace=None, max_kv_len: Optional[int] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+                           kv_split_workspace=None, max_kv_len: Optional[int] = None,
+                           total_q_len: Optional[int] = None) -> Tuple[torch.Tensor, torch.Tensor]:
     """One step as a mergeable partial: (O fp32 [Tq,Hq,D] normalised, LSE fp32 [Tq,Hq]).
     v_f16 / v_f16_valid: as in context_attention_fwd (the caller's buffer for the fp16 copy of a bfloat16 v).
     kv_splits: short query chunks against a long KV chunk give the launch too few workgroups for the chip (one per 128
@@ -305,6 +315,7 @@ def prefill_attention_step(q, k, v, q_b_start_loc, q_b_seq_len, q_first_token_gl
     (out, lse): kv_split_workspace passes the caller's memory for them (as context_attention_fwd's workspace).
 
     Same inputs as context_attention_fwd; rows that see no key get O = 0, LSE = -inf.
+    total_q_len: as in context_attention_fwd (an upper bound of the rows of all sequences together, for skewed batches).
     With accumulate=True the step is LSE-merged into the (out, lse) passed in (a running partial of earlier steps over
     other keys; lse = -inf marks an empty row) in the kernel's epilogue, instead of being written from the empty state;
     rows that see no key in this step keep what they hold.
@@ -346,7 +357,7 @@ def prefill_attention_step(q, k, v, q_b_start_loc, q_b_seq_len, q_first_token_gl
         return out, lse
     a = _prefill_args(q, k, v, out, q_b_start_loc, q_b_seq_len, q_first_token_global_idx, kv_b_start_loc,
                       kv_b_seq_len, kv_first_token_global_idx, logical_sp_peers_num, max_q_b_seq_len, sm_scale,
-                      v_f16 if out_user is None else None, v_f16_valid and out_user is None)
+                      v_f16 if out_user is None else None, v_f16_valid and out_user is None, total_q_len=total_q_len)
     a.lse = lse.data_ptr()
     if accumulate:
         _lib.check(_lib.load().lsattn_prefill_step_accumulate(C.byref(a), _stream()), "lsattn_prefill_step_accumulate")

@@ -53,7 +53,7 @@ def ring_prefill(q, chunks: Sequence[KVChunk], q_b_start_loc, q_b_seq_len, q_fir
     for c in chunks:
         context_attention_fwd(q, c.k(num_kv_heads), c.v(num_kv_heads), o, q_b_start_loc, q_b_seq_len,
                               q_first_token_global_idx, c.b_start_loc, c.b_seq_len, c.first_token_global_idx,
-                              logical_sp_peers_num, max_q_len, m, l)
+                              logical_sp_peers_num, max_q_len, m, l, total_q_len=q.shape[0])  # (q is packed: its rows bound the batch)
     return o, m, l
 
 
@@ -67,7 +67,8 @@ def ring_prefill_partials(q, chunks: Sequence[KVChunk], q_b_start_loc, q_b_seq_l
         ob, lb = bufs[i] if bufs is not None else (None, None)
         parts.append(prefill_attention_step(q, c.k(num_kv_heads), c.v(num_kv_heads), q_b_start_loc, q_b_seq_len,
                                             q_first_token_global_idx, c.b_start_loc, c.b_seq_len,
-                                            c.first_token_global_idx, logical_sp_peers_num, max_q_len, ob, lb))
+                                            c.first_token_global_idx, logical_sp_peers_num, max_q_len, ob, lb,
+                                            total_q_len=q.shape[0]))
     return lse_merge(parts, out, lse)
 
 
@@ -79,7 +80,7 @@ def ring_prefill_accumulate(q, chunks: Sequence[KVChunk], q_b_start_loc, q_b_seq
     for i, c in enumerate(chunks):
         out, lse = prefill_attention_step(q, c.k(num_kv_heads), c.v(num_kv_heads), q_b_start_loc, q_b_seq_len,
                                           q_first_token_global_idx, c.b_start_loc, c.b_seq_len, c.first_token_global_idx,
-                                          logical_sp_peers_num, max_q_len, out, lse, accumulate=i > 0)
+                                          logical_sp_peers_num, max_q_len, out, lse, accumulate=i > 0, total_q_len=q.shape[0])
     return out, lse
 
 
@@ -102,7 +103,7 @@ def ring_prefill_with_migration(q, chunks: Sequence[KVChunk], q_b_start_loc, q_b
     for c in chunks:
         context_attention_fwd(q, c.k(num_kv_heads), c.v(num_kv_heads), o, q_b_start_loc, q_b_seq_len,
                               q_first_token_global_idx, c.b_start_loc, c.b_seq_len, c.first_token_global_idx,
-                              logical_sp_peers_num, max_q_len, m, l)
+                              logical_sp_peers_num, max_q_len, m, l, total_q_len=q.shape[0])
         kv_range_begin, kv_range_end, new_kv_cache_len = pre_copy_and_register_kv(
             kv_cache_index_begin, kv_cache_index_end, c.first_token_global_idx, logical_sp_peers_num)
         new_kv_cache_len_sum = torch.cumsum(new_kv_cache_len, dim=0, dtype=torch.int64)

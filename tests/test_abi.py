@@ -46,7 +46,8 @@ int main(void) {
   printf("%zu %zu\n", sizeof(lsattn_decode_migration_args), offsetof(lsattn_decode_migration_args, b_seq_len));
   printf("%zu %zu\n", sizeof(lsattn_rotary_kv_write_args), offsetof(lsattn_rotary_kv_write_args, register_mode));
   printf("%zu %zu\n", sizeof(lsattn_tuning), offsetof(lsattn_tuning, decode_listed));
-  printf("%zu %zu %zu\n", sizeof(lsattn_merge_cuts_args), offsetof(lsattn_merge_cuts_args, ml_stride_h), offsetof(lsattn_prefill_args, o_cut_rows));
+  printf("%zu %zu %zu %zu\n", sizeof(lsattn_merge_cuts_args), offsetof(lsattn_merge_cuts_args, ml_stride_h), offsetof(lsattn_prefill_args, o_cut_rows),
+         offsetof(lsattn_prefill_args, total_q_rows));
   printf("%zu %zu %zu %zu %zu %zu\n", offsetof(lsattn_prefill_args, sm_scale), offsetof(lsattn_prefill_args, ml_stride_h),
          offsetof(lsattn_decode_stage1_args, req_to_tokens), offsetof(lsattn_decode_stage2_args, block_seq),
          offsetof(lsattn_kv_copy_register_args, req_to_tokens), offsetof(lsattn_kv_copy_register_args, should_register));
@@ -62,9 +63,10 @@ int main(void) {
     mig = [int(x) for x in out[5:7]]
     rot = [int(x) for x in out[7:9]]
     tun = [int(x) for x in out[9:11]]
-    cuts = [int(x) for x in out[11:14]]
-    offs = [int(x) for x in out[14:]]
-    assert cuts == [C.sizeof(_lib.MergeCutsArgs), _lib.MergeCutsArgs.ml_stride_h.offset, _lib.PrefillArgs.o_cut_rows.offset]
+    cuts = [int(x) for x in out[11:15]]
+    offs = [int(x) for x in out[15:]]
+    assert cuts == [C.sizeof(_lib.MergeCutsArgs), _lib.MergeCutsArgs.ml_stride_h.offset, _lib.PrefillArgs.o_cut_rows.offset,
+                    _lib.PrefillArgs.total_q_rows.offset]
     assert tun == [C.sizeof(_lib.Tuning), _lib.Tuning.decode_listed.offset]
     assert rot == [C.sizeof(_lib.RotaryKvWriteArgs), _lib.RotaryKvWriteArgs.register_mode.offset]
     assert mig == [C.sizeof(_lib.DecodeMigrationArgs), _lib.DecodeMigrationArgs.b_seq_len.offset]

@@ -469,6 +469,59 @@ def test_short_queries_against_long_kv_split_along_the_keys(lsa, dtype, P):
     assert bool((l_run.cpu()[~seen] == float("-inf")).all())
 
 
+@pytest.mark.parametrize("dtype,Hq,Hkv", [(torch.float16, 32, 8), (torch.bfloat16, 16, 16), (torch.float16, 8, 8)])
+def test_skewed_batch_with_a_bound_on_its_rows_walks_the_units_that_exist(lsa, prefill_geometry, dtype, Hq, Hkv):
+    """One request of 6000 rows among 69 of 0 to 300 (two of them empty) with total_q_len = the rows of the packed q: the
+    grid sized by the longest request would be 70 x 24 query tiles per head group and nearly all of them empty, so the
+    launch numbers the tiles that exist (every workgroup finds its request from q_b_seq_len; 70 requests: two steps of 64).
+    All three epilogues, against the oracle; a second, shifted KV chunk through the folding ones; every forced
+    workgroup shape.  A batch the bound does not shrink by half (all requests alike) takes the ordinary grid."""
+    import random
+    rng = random.Random(Hq)
+    lens = [rng.randint(1, 300) for _ in range(70)]
+    lens[0] = lens[33] = 0
+    lens[65] = 6000
+    T = sum(lens)
+    q = rand_t((T, Hq, 128), 4701, dtype)
+    k, v = rand_t((T, Hkv, 128), 4702, dtype), rand_t((T, Hkv, 128), 4703, dtype)
+    m = meta(lens)
+    o_ref, lse_ref = orc.attn_step(q, k, v, *m, *m, 1)
+    dq, dk, dv = q.to(DEV), k.to(DEV), v.to(DEV)
+    dm = _dev(*m)
+    o, lse = lsa.prefill_attention_step(dq, dk, dv, *dm, *dm, 1, max(lens), total_q_len=T)
+    torch.cuda.synchronize()
+    assert_o_close(o, o_ref, "O")
+    assert_lse_close(lse, lse_ref, "LSE")
+    # an earlier chunk of 40 keys per request, all visible (positions before the queries'), folded in by both folding epilogues
+    klens = [40 if n else 0 for n in lens]
+    k0, v0 = rand_t((sum(klens), Hkv, 128), 4704, dtype), rand_t((sum(klens), Hkv, 128), 4705, dtype)
+    qm, km0 = meta(lens, [40] * len(lens)), meta(klens)
+    kml = meta(lens, [40] * len(lens))
+    p0 = orc.attn_step(q, k0, v0, *qm, *km0, 1)
+    p1 = orc.attn_step(q, k, v, *qm, *kml, 1)
+    o2_ref, l2_ref = orc.lse_merge([p0, p1])
+    dqm = _dev(*qm)
+    out, l2 = lsa.prefill_attention_step(dq, k0.to(DEV), v0.to(DEV), *dqm, *_dev(*km0), 1, max(lens), total_q_len=T)
+    lsa.prefill_attention_step(dq, dk, dv, *dqm, *_dev(*kml), 1, max(lens), out=out, lse=l2, accumulate=True, total_q_len=T)
+    torch.cuda.synchronize()
+    seen = torch.isfinite(l2_ref)
+    assert_o_close(out.cpu()[seen], o2_ref[seen], "accumulated O")
+    assert_lse_close(l2, l2_ref, "accumulated LSE")
+    o_st = torch.zeros((T, Hq, 128), dtype=dtype, device=DEV)
+    m_st = torch.full((T, Hq), float("-inf"), device=DEV)
+    l_st = torch.zeros((T, Hq), device=DEV)
+    lsa.context_attention_fwd(dq, k0.to(DEV), v0.to(DEV), o_st, *dqm, *_dev(*km0), 1, max(lens), m_st, l_st, total_q_len=T)
+    lsa.context_attention_fwd(dq, dk, dv, o_st, *dqm, *_dev(*kml), 1, max(lens), m_st, l_st, total_q_len=T)
+    torch.cuda.synchronize()
+    assert_lse_close(orc.state_lse(m_st.cpu(), l_st.cpu()).float(), l2_ref, "state LSE")
+    bar = dict(max_abs=2e-3, rel=1.5e-3) if dtype == torch.float16 else dict(max_abs=2e-2, rel=6e-3)
+    assert_o_close(o_st.cpu()[seen], o2_ref[seen], "in-place o", **bar)
+    # a loose bound (twice the rows) is as good; a uniform batch keeps the ordinary grid and the same answer
+    o3, l3 = lsa.prefill_attention_step(dq, dk, dv, *dm, *dm, 1, max(lens), total_q_len=2 * T + 5)
+    torch.cuda.synchronize()
+    assert torch.equal(o3, o) and torch.equal(l3, lse)
+
+
 def test_kv_cuts_leave_rows_outside_the_sequences_alone(lsa):
     """Rows of q / out that belong to no sequence (a gap between two sequences and a tail) keep what they hold on the
     route cut along the keys, as on the unsplit one, with and without accumulate; the partials' workspace starts as NaN.
