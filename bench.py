@@ -410,20 +410,22 @@ class VarlenPrefill:
         self.flops = 4 * D * Hq * self.pairs
         self.scatter_bytes = T * 2 * Hkv * D * 2 * 2  # read + write of every K/V row
         self.v_f16 = torch.empty((T, Hkv, D), dtype=torch.float16, device=DEV)  # the caller's buffer for the fp16 copy of V
+        self.bound_rows = True  # pass total_q_len = the rows of the packed q (the batch is skewed: 1 K to 200 K tokens)
 
     def attention(self):
         import loongserve_amd as lsa
         self.m.fill_(float("-inf"))
         self.l.zero_()
         lsa.context_attention_fwd(self.q, self.kv[:, :self.Hkv], self.kv[:, self.Hkv:], self.o, self.start, self.len, self.first,
-                                  self.start, self.len, self.first, 1, self.max_len, self.m, self.l, v_f16=self.v_f16)
+                                  self.start, self.len, self.first, 1, self.max_len, self.m, self.l, v_f16=self.v_f16,
+                                  total_q_len=self.T if self.bound_rows else None)
 
     def attention_kernel_only(self):
         """The attention launch alone: (m, l) not reset (the result is not used), V's fp16 copy taken as it stands."""
         import loongserve_amd as lsa
         lsa.context_attention_fwd(self.q, self.kv[:, :self.Hkv], self.kv[:, self.Hkv:], self.o, self.start, self.len, self.first,
                                   self.start, self.len, self.first, 1, self.max_len, self.m, self.l, v_f16=self.v_f16,
-                                  v_f16_valid=True)
+                                  v_f16_valid=True, total_q_len=self.T if self.bound_rows else None)
 
     def persist(self):
         import loongserve_amd as lsa

@@ -275,7 +275,7 @@ __global__ __launch_bounds__(HALF ? NWAVE * 32 : NWAVE * 64, HALF ? 2 : 1) void 
     uint32_t carry = 0;
     b = -1;
     up = 0;
-    for (int b0 = 0; b0 < p.batch; b0 += 64) {
+    for (int b0 = 0; b0 < p.batch && b < 0; b0 += 64) {  // (until the unit's request is found)
       const int bb = b0 + lane_id;
       const int len = bb < p.batch ? p.q_len[bb] : 0;
       const uint32_t tiles = len > 0 ? ((uint32_t)len + (1u << p.rows_shift) - 1) >> p.rows_shift : 0;
@@ -293,7 +293,6 @@ __global__ __launch_bounds__(HALF ? NWAVE * 32 : NWAVE * 64, HALF ? 2 : 1) void 
         b = b0 + l0;
         up = (int)(unit - (carry + __builtin_amdgcn_readlane(incl, l0) - __builtin_amdgcn_readlane(units, l0)));
         nz = (int)__builtin_amdgcn_readlane(tiles, l0);
-        break;
       }
       carry += chunk_total;
     }

@@ -147,7 +147,8 @@ def _kernels(text):
 
 
 def _loops(lines):
-    """(first line index, last line index) of every loop: a label and a later branch back to it."""
+    """(first line index, last line index) of every loop: a label and a later branch back to it.  (A block that only ends
+    the program, placed early in the text and branched back to by later exits, is no loop.)"""
     labels = {}
     loops = []
     for i, raw in enumerate(lines):
@@ -156,7 +157,9 @@ def _loops(lines):
             labels[m.group(1)] = i
         m = re.match(r"^\s+s_cbranch_\w+\s+(\.LBB\d+_\d+)", raw) or re.match(r"^\s+s_branch\s+(\.LBB\d+_\d+)", raw)
         if m and m.group(1) in labels:
-            loops.append((labels[m.group(1)], i))
+            first = next((l.split(";")[0].strip() for l in lines[labels[m.group(1)] + 1:] if l.split(";")[0].strip()), "")
+            if first != "s_endpgm":
+                loops.append((labels[m.group(1)], i))
     return loops
 
 
