@@ -1249,8 +1249,11 @@ template <typename T, int MODE, bool DV> static int launch_prefill(const lsattn_
     // grid running backwards (see the kernel), each CU one heavy and one light workgroup side by side, instead of the
     // split shape's two rounds.  Longer chunks keep the rules above (the pairs' work is then long against what a
     // workgroup costs besides its tiles, and the shape's rings of two tiles are the slower ones per tile).
-    const bool fold = a->batch == 1 && cuts == 1 && !a->o_b_start_loc && a->max_q_len <= 2048 && wgs128 > kCUs && wgs128 <= 2 * kCUs &&
-                      tn.prefill_rows == 0;
+    // (measured, one sequence, MHA 32: 2048 tokens = 512 workgroups 45.7 us against 47.1 split and 47.3 unfolded; 1792 tokens
+    // = 448 39.6 against 40.5; 1536 = 384 34.2 against 33.5 and 1280 = 320 29.7 against 27.4: the fold pays from seven
+    // eighths of two workgroups per CU on, below that the split shape's two rounds do)
+    const bool fold = a->batch == 1 && cuts == 1 && !a->o_b_start_loc && a->max_q_len <= 2048 && wgs128 * 8 >= 7 * 2 * kCUs &&
+                      wgs128 <= 2 * kCUs && tn.prefill_rows == 0;
     if (fold) return launch_prefill_rows<T, MODE, true, false, true>(a, true, tn, st, true);
     if (half) return launch_prefill_rows<T, MODE, true, false, true>(a, true, tn, st);
     return split ? launch_prefill_rows<T, MODE, true, true>(a, true, tn, st) : launch_prefill_rows<T, MODE, true, false>(a, tile_major, tn, st);
