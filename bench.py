@@ -600,7 +600,7 @@ def chunked_prefill_step():
     m = torch.full((Tq, Hq), float("-inf"), device=DEV)
     l = torch.zeros((Tq, Hq), device=DEV)
     from loongserve_amd.ops import kv_split_count
-    S = kv_split_count(1, Hq, Tq, Tk)
+    S = kv_split_count(1, Hq, Tq, Tk, Hkv)
     ws = torch.empty(S * Tq * Hq * (D + 1), dtype=torch.float32, device=DEV)
     step = lambda: lsa.prefill_attention_step(q, kv[:, :Hkv], kv[:, Hkv:], *qm, *km, 1, Tq, out=o32, lse=l32, kv_split_workspace=ws)  # noqa: E731
     op_ws = lambda: lsa.context_attention_fwd(q, kv[:, :Hkv], kv[:, Hkv:], o16, *qm, *km, 1, Tq, m, l, workspace=ws)  # noqa: E731

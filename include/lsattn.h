@@ -39,6 +39,7 @@ extern "C" {
 #define LSATTN_F32 2
 
 #define LSATTN_MAX_PARTS 16
+#define LSATTN_MAX_KV_CUTS 64 /* cuts of a KV chunk inside one prefill launch (lsattn_prefill_args.kv_cuts) */
 
 /*
  * One ring / context-parallel prefill attention step: local Q chunk against one KV chunk.
@@ -91,7 +92,7 @@ typedef struct lsattn_prefill_args {
    * kv_b_start_loc / kv_b_seq_len / kv_first_token_global_idx and its own output rows), which lsattn_lse_merge then
    * joins: short query chunks against long KV fill the chip that way.  Zero the struct before filling it in. */
   const int32_t* o_b_start_loc;
-  /* Optional (0 or 1: off), lsattn_prefill_step only; no counterpart in the reference.  kv_cuts = S in 2..LSATTN_MAX_PARTS
+  /* Optional (0 or 1: off), lsattn_prefill_step only; no counterpart in the reference.  kv_cuts = S in 2..LSATTN_MAX_KV_CUTS
    * enters every sequence S times into the launch: entry c attends to keys [c * kv_cut_len, (c + 1) * kv_cut_len) of the
    * sequence's KV chunk (kv_cut_len a multiple of 64) and writes the partial (o, lse) of its rows o_cut_rows * c rows
    * further down than entry 0 does, so o and lse hold S * o_cut_rows rows (o_cut_rows >= the rows of q).  A short query
@@ -162,7 +163,7 @@ typedef struct lsattn_merge_cuts_args {
   const float* o_parts;
   const float* lse_parts;
   int64_t part_rows;
-  int32_t n_parts;     /* 1..LSATTN_MAX_PARTS */
+  int32_t n_parts;     /* 1..LSATTN_MAX_KV_CUTS */
   int32_t mode;        /* 0, 1, 2 as above */
   int32_t batch;
   int32_t num_q_heads;

@@ -15,6 +15,7 @@ LIB_PATH = os.environ.get("LSATTN_LIB_PATH") or os.path.join(os.path.dirname(os.
 
 LSATTN_F16, LSATTN_BF16, LSATTN_F32 = 0, 1, 2
 LSATTN_MAX_PARTS = 16
+LSATTN_MAX_KV_CUTS = 64
 LSATTN_STATIC_SCRATCH_BYTES = 64 * 1024 * 1024
 
 _vp, _i32, _i64, _f32 = C.c_void_p, C.c_int32, C.c_int64, C.c_float

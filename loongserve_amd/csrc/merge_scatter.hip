@@ -369,7 +369,7 @@ extern "C" int lsattn_lse_merge(const lsattn_merge_args* a, void* stream) {
 
 extern "C" int lsattn_prefill_merge_cuts(const lsattn_merge_cuts_args* a, void* stream) {
   if (!a || !a->o_parts || !a->lse_parts || !a->q_b_start_loc || !a->q_b_seq_len || !a->o) return LSATTN_ERR_INVALID_ARG;
-  if (a->n_parts < 1 || a->n_parts > LSATTN_MAX_PARTS || a->part_rows < 0 || a->batch < 0 || a->num_q_heads <= 0 || a->max_q_len < 0)
+  if (a->n_parts < 1 || a->n_parts > LSATTN_MAX_KV_CUTS || a->part_rows < 0 || a->batch < 0 || a->num_q_heads <= 0 || a->max_q_len < 0)
     return LSATTN_ERR_INVALID_ARG;
   if (a->head_dim != 128) return LSATTN_ERR_UNSUPPORTED;
   if (a->mode < 0 || a->mode > 2) return LSATTN_ERR_INVALID_ARG;

@@ -1232,6 +1232,16 @@ template <typename T, int MODE, bool DV> static int launch_prefill(const lsattn_
     return launch_prefill_rows<T, MODE, false, false>(a, tile_major, tn, st);
   } else {
     bool split = wgs256 <= kCUs / 2 || (wgs256 <= kCUs && nz256 >= 5);
+    // Short chunks that a 256-row workgroup pads much further than a 128-row one (100 rows of one head: 256 against 128): the
+    // 128-row shapes walk the same tiles for at most four fifths of the rows (100 rows x 131072 keys in 15 cuts, MHA 32:
+    // 507 -> 376 us).  Per row and tile they are 5 to 10 % behind the 256-row shape, hence the margin.
+    {
+      // (query positions the longest chunk is padded to; the heads side by side in a workgroup cancel out)
+      const int64_t padded256 = ((a->max_q_len + (BM >> ps) - 1) / (BM >> ps)) * (BM >> ps);
+      const int ph0 = pack_shift_for(a, true, tn);
+      const int64_t padded128 = ((a->max_q_len + (BM / 2 >> ph0) - 1) / (BM / 2 >> ph0)) * (BM / 2 >> ph0);
+      if (padded128 * 5 <= padded256 * 4) split = true;
+    }
     // The four-wave shape (two workgroups per CU) for chunks of up to 1024 rows (1536 with one head per workgroup),
     // whose workgroups walk a few tiles each and spend as long starting and ending as working, from three workgroups
     // per CU on: 3 to 17 % shorter launches on batches of 4 to 32 requests of 128 to 1536 tokens.  Smaller launches keep
@@ -1273,7 +1283,7 @@ static int validate(const lsattn_prefill_args* a, int mode) {
   if (a->v_is_f16 != 0 && (a->v_is_f16 != 1 || a->dtype != LSATTN_BF16)) return LSATTN_ERR_INVALID_ARG;
   // the chunk cut along the keys: a multiple of the 64-key tile per cut, the cuts' outputs apart (fp32 partials only),
   // and key positions that stay within 31 bits
-  if (a->kv_cuts < 0 || a->kv_cuts > LSATTN_MAX_PARTS) return LSATTN_ERR_INVALID_ARG;
+  if (a->kv_cuts < 0 || a->kv_cuts > LSATTN_MAX_KV_CUTS) return LSATTN_ERR_INVALID_ARG;
   if (a->kv_cuts > 1 && (mode != 0 || a->kv_cut_len < 64 || a->kv_cut_len % 64 || a->o_cut_rows <= 0 ||
                          (int64_t)a->kv_cut_len * a->kv_cuts > 0x7fffffff))
     return LSATTN_ERR_INVALID_ARG;

@@ -185,7 +185,7 @@ def _cut_workspace(workspace, S: int, Tq: int, Hq: int, D: int, device):
 def _workspace_cuts(workspace, Tq: int, Hq: int, D: int) -> int:
     """How many cuts' partials a single-tensor workspace holds."""
     if workspace is None or isinstance(workspace, (tuple, list)) or Tq == 0:
-        return _lib.LSATTN_MAX_PARTS
+        return _lib.LSATTN_MAX_KV_CUTS
     return workspace.numel() // (Tq * Hq * (D + 1))
 
 
@@ -208,14 +208,22 @@ KV_SPLIT_BELOW_WORKGROUPS = 192
 KV_SPLIT_MIN_KEYS = 8192
 
 
-def kv_split_count(batch: int, num_q_heads: int, max_q_len: int, kv_rows: int) -> int:
-    """KV cuts the prefill operators use by themselves: enough for about two workgroups per CU, cuts of at least 2048
-    keys (kv_rows bounds every sequence's chunk: max_kv_len where the caller gives it, else the rows of the k buffer;
-    the lengths themselves live on the device)."""
-    wgs = batch * num_q_heads * ((max_q_len + 127) // 128)
+def kv_split_count(batch: int, num_q_heads: int, max_q_len: int, kv_rows: int, num_kv_heads: Optional[int] = None) -> int:
+    """KV cuts the prefill operators use by themselves: enough for a good round of workgroups (about 320), cuts of at
+    least 4096 keys (kv_rows bounds every sequence's chunk: max_kv_len where the caller gives it, else the rows of the k buffer;
+    the lengths themselves live on the device).  The launch's size without cuts is counted in 128-row workgroups as the
+    kernel forms them: up to four query heads of a KV head side by side (num_kv_heads given), 128 / that many positions each."""
+    pack = 1
+    if num_kv_heads:
+        group = num_q_heads // num_kv_heads
+        while pack < 4 and group % (2 * pack) == 0:
+            pack *= 2
+    wgs = batch * (num_q_heads // pack) * ((max_q_len + 128 // pack - 1) // (128 // pack))
     if wgs <= 0 or wgs >= KV_SPLIT_BELOW_WORKGROUPS or kv_rows < KV_SPLIT_MIN_KEYS:
         return 1
-    return max(1, min(_lib.LSATTN_MAX_PARTS - 1, 512 // wgs, kv_rows // 2048))
+    # (measured, GQA 32/8 unless said: 16 rows x 131072 keys 32 cuts 124 us against 134 with 16 and 160 with 64; 100 x 131072
+    # 16 cuts 243 against 252 with 8 and 270 with 32, MHA 8 cuts 388 against 412; 128 x 32768 8 cuts 80 against 84 with 16)
+    return max(1, min(_lib.LSATTN_MAX_KV_CUTS, 320 // wgs, kv_rows // 4096))
 
 
 def _cut_len(kv_rows: int, S: int) -> int:
@@ -272,8 +280,8 @@ def context_attention_fwd(q, k, v, o, q_b_start_loc, q_b_seq_len, q_first_token_
     S = 1
     if workspace is not None and o_user is None and q.dim() == 3:
         kv_rows = k.shape[0] if max_kv_len is None else int(max_kv_len)
-        S = kv_split_count(q_b_seq_len.shape[0], q.shape[1], int(max_q_b_seq_len), kv_rows) if kv_splits is None else int(kv_splits)
-        S = min(S, _workspace_cuts(workspace, q.shape[0], q.shape[1], D), _lib.LSATTN_MAX_PARTS)
+        S = kv_split_count(q_b_seq_len.shape[0], q.shape[1], int(max_q_b_seq_len), kv_rows, k.shape[1]) if kv_splits is None else int(kv_splits)
+        S = min(S, _workspace_cuts(workspace, q.shape[0], q.shape[1], D), _lib.LSATTN_MAX_KV_CUTS)
     if S > 1:
         Tq = q.shape[0]
         po, pl = _cut_workspace(workspace, S, Tq, q.shape[1], D, q.device)
@@ -337,10 +345,10 @@ def prefill_attention_step(q, k, v, q_b_start_loc, q_b_seq_len, q_first_token_gl
         if sm_scale is None:
             sm_scale = 1.0 / (D ** 0.5)
     kv_rows = k.shape[0] if max_kv_len is None else int(max_kv_len)
-    S = kv_split_count(q_b_seq_len.shape[0], q.shape[1], int(max_q_b_seq_len), kv_rows) if kv_splits is None else int(kv_splits)
+    S = kv_split_count(q_b_seq_len.shape[0], q.shape[1], int(max_q_b_seq_len), kv_rows, k.shape[1]) if kv_splits is None else int(kv_splits)
     if S > 1:
-        if S > _lib.LSATTN_MAX_PARTS:
-            raise ValueError("at most %d KV slices" % _lib.LSATTN_MAX_PARTS)
+        if S > _lib.LSATTN_MAX_KV_CUTS:
+            raise ValueError("at most %d KV slices" % _lib.LSATTN_MAX_KV_CUTS)
         if out.dim() != 3 or out.stride(2) != 1 or tuple(out.shape) != tuple(q.shape):
             raise ValueError("out must have q's shape and be contiguous in head_dim")
         Tq = q.shape[0]

@@ -138,8 +138,8 @@ def test_validation_rejects_bad_arguments_without_gpu():
     assert lib.lsattn_prefill_step(C.byref(a), None) == -1          # not a multiple of 64 keys
     a.kv_cut_len, a.o_cut_rows = 128, 0
     assert lib.lsattn_prefill_step(C.byref(a), None) == -1          # no room between the cuts' outputs
-    a.o_cut_rows, a.kv_cuts = 8, 17
-    assert lib.lsattn_prefill_step(C.byref(a), None) == -1          # more cuts than LSATTN_MAX_PARTS
+    a.o_cut_rows, a.kv_cuts = 8, 65
+    assert lib.lsattn_prefill_step(C.byref(a), None) == -1          # more cuts than LSATTN_MAX_KV_CUTS
     a.kv_cuts = 4
     assert lib.lsattn_prefill_step_accumulate(C.byref(a), None) == -1  # the folding steps take no cuts
     mc = _lib.MergeCutsArgs()
@@ -152,7 +152,7 @@ def test_validation_rejects_bad_arguments_without_gpu():
     assert lib.lsattn_prefill_merge_cuts(C.byref(mc), None) == -2   # head_dim
     mc.head_dim, mc.mode = 128, 1
     assert lib.lsattn_prefill_merge_cuts(C.byref(mc), None) == -1   # mode 1 needs m, l and a 16-bit o
-    mc.mode, mc.n_parts = 0, 17
+    mc.mode, mc.n_parts = 0, 65
     assert lib.lsattn_prefill_merge_cuts(C.byref(mc), None) == -1
     # the fused decode call refuses argument blocks that do not describe the same partials
     s1, s2 = _lib.DecodeStage1Args(), _lib.DecodeStage2Args()
@@ -267,8 +267,11 @@ def test_kv_split_count_from_shapes():
     from loongserve_amd.ops import kv_split_count
     assert kv_split_count(1, 32, 16384, 16384) == 1          # config 2: 4096 workgroups
     assert kv_split_count(1, 32, 2048, 2048) == 1            # config 1: enough workgroups, few keys
-    assert kv_split_count(1, 32, 100, 131072) == 15          # one 100-row chunk against 131072 keys
-    assert kv_split_count(1, 8, 100, 20000) == 9             # slices of at least 2048 keys
-    assert kv_split_count(4, 32, 128, 100000) == 4           # 128 workgroups: four slices fill two rounds
+    assert kv_split_count(1, 32, 100, 131072) == 10          # one 100-row chunk against 131072 keys: 32 workgroups -> 320
+    assert kv_split_count(1, 32, 100, 131072, 8) == 10       # GQA 32/8: four heads side by side, 8 x 4 workgroups of 32 positions
+    assert kv_split_count(1, 32, 16, 131072, 8) == 32        # 16 rows: 8 workgroups; cuts of at least 4096 keys
+    assert kv_split_count(1, 32, 16, 20000, 8) == 4
+    assert kv_split_count(1, 8, 100, 20000) == 4             # cuts of at least 4096 keys
+    assert kv_split_count(4, 32, 128, 100000) == 2           # 128 workgroups: two cuts
     assert kv_split_count(1, 32, 100, 4096) == 1             # short KV
     assert kv_split_count(0, 32, 100, 100000) == 1

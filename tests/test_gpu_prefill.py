@@ -449,7 +449,7 @@ def test_short_queries_against_long_kv_split_along_the_keys(lsa, dtype, P):
     dqm, dkm = [t.to(DEV) for t in qm], [t.to(DEV) for t in km]
     assert ops.kv_split_count(len(qlens), Hq, max(qlens), k.shape[0]) > 1
     o1, l1 = lsa.prefill_attention_step(dq, dk, dv, *dqm, *dkm, P, max(qlens), kv_splits=1)
-    for S in (None, 2, 7, 15):
+    for S in (None, 2, 7, 15, 33, 64):
         o, l = lsa.prefill_attention_step(dq, dk, dv, *dqm, *dkm, P, max(qlens), kv_splits=S)
         torch.cuda.synchronize()
         assert_o_close(o, o_ref, "O, %s slices" % S)
