@@ -557,6 +557,8 @@ def config5(details=None):
 
 
 def _causal_case(N, Hq, Hkv, B):
+    """A batch of B causal prompts of N tokens: the fp32-partial call, the reference operator's in-place call on rows in
+    their start state with the call that resets them (m = -inf, l = 0), flops, and the bytes either route has to move."""
     q = _randn_half((B * N, Hq, D), 4100 + N + B)
     kv = _randn_half((B * N, 2 * Hkv, D), 4200 + N + B)
     st = torch.arange(B, dtype=torch.int32, device=DEV) * N
@@ -564,20 +566,42 @@ def _causal_case(N, Hq, Hkv, B):
     z = torch.zeros(B, dtype=torch.int32, device=DEV)
     o = torch.empty((B * N, Hq, D), dtype=torch.float32, device=DEV)
     lse = torch.empty((B * N, Hq), dtype=torch.float32, device=DEV)
+    o16 = torch.zeros((B * N, Hq, D), dtype=torch.float16, device=DEV)
+    m = torch.full((B * N, Hq), float("-inf"), device=DEV)
+    l = torch.zeros((B * N, Hq), device=DEV)
     import loongserve_amd as lsa
     fn = lambda: lsa.prefill_attention_step(q, kv[:, :Hkv], kv[:, Hkv:], st, ln, z, st, ln, z, 1, N, out=o, lse=lse, kv_splits=1)  # noqa: E731
-    return fn, 4.0 * D * Hq * B * N * (N + 1) / 2
+
+    def reset():
+        m.fill_(float("-inf"))
+        l.zero_()
+
+    def inplace():
+        reset()
+        lsa.context_attention_fwd(q, kv[:, :Hkv], kv[:, Hkv:], o16, st, ln, z, st, ln, z, 1, N, m, l)
+
+    rows = B * N * Hq
+    bytes_partial = 2 * (q.numel() + kv.numel()) + 4 * rows * (D + 1)
+    bytes_inplace = 2 * (q.numel() + kv.numel()) + 2 * rows * D + 4 * 4 * rows  # (o written, m and l read and written)
+    return fn, 4.0 * D * Hq * B * N * (N + 1) / 2, inplace, reset, bytes_partial, bytes_inplace
 
 
 def short_prompts():
     """Batches of short prompts (outside the five configs; the regime of the reference's published 1 x 100 / 1 x 1000
-    token rows): causal, fp16, device time per launch from a HIP graph of 20 launches, median of 10 replays."""
+    token rows): causal, fp16, device time per launch from a HIP graph of 20 launches, median of 10 replays.  `us` is the
+    fp32-partial call, `inplace_us` the reference's operator (o in fp16, (m, l) in place) on rows in their start state,
+    with the time of the two fills that reset them taken off.  The smaller launches move more bytes than they
+    compute: `hbm_frac` is the bytes either route has to move over 8 TB/s against its time, `frac` the MFMA fraction."""
     rows = {}
     for name, (N, Hq, Hkv, B) in (("16x256_mha", (256, 32, 32, 16)), ("8x512_gqa", (512, 32, 8, 8)), ("32x1024_gqa", (1024, 32, 8, 32)),
                                   ("6x2048_gqa", (2048, 32, 8, 6)), ("1x4096_mha", (4096, 32, 32, 1)), ("1x8192_gqa", (8192, 32, 8, 1))):
-        fn, fl = _causal_case(N, Hq, Hkv, B)
+        fn, fl, inplace, reset, by_p, by_i = _causal_case(N, Hq, Hkv, B)
         ms = _time_graph(fn, launches=20, reps=10, warm_reps=3)
-        rows[name] = {"us": _r(ms * 1e3, 1), "frac": _r(fl / (ms * 1e-3) / 1e12 / PEAK_MFMA_TFLOPS)}
+        ms_i = _time_graph(inplace, launches=20, reps=10, warm_reps=3) - _time_graph(reset, launches=20, reps=10, warm_reps=3)
+        rows[name] = {"us": _r(ms * 1e3, 1), "frac": _r(fl / (ms * 1e-3) / 1e12 / PEAK_MFMA_TFLOPS),
+                      "hbm_frac": _r(by_p / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS), "inplace_us": _r(ms_i * 1e3, 1),
+                      "inplace_frac": _r(fl / (ms_i * 1e-3) / 1e12 / PEAK_MFMA_TFLOPS),
+                      "inplace_hbm_frac": _r(by_i / (ms_i * 1e-3) / 1e9 / PEAK_HBM_GBS)}
         torch.cuda.empty_cache()
     return rows
 
@@ -635,7 +659,7 @@ def prefill_launch_sizes(tile_us):
     try:
         for N, Hq, Hkv, B in ((1024, 32, 8, 1), (2048, 32, 32, 1), (512, 32, 8, 8), (4096, 32, 32, 1), (2048, 32, 8, 6), (1024, 32, 8, 32),
                               (256, 32, 32, 16), (8192, 32, 8, 1)):
-            fn, fl = _causal_case(N, Hq, Hkv, B)
+            fn, fl = _causal_case(N, Hq, Hkv, B)[:2]
             row = {"tokens": N, "requests": B, "q_heads": Hq, "kv_heads": Hkv, "workgroups_of_256_rows": B * Hq * ((N + 255) // 256)}
             _time_graph(fn, launches=5, reps=2)  # first touch of the new buffers
             # (the library's choice is timed last: the first timing after new buffers reads a few per cent long)

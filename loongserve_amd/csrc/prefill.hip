@@ -241,7 +241,9 @@ __global__ __launch_bounds__(HALF ? NWAVE * 32 : NWAVE * 64, HALF ? 2 : 1) void 
   // anything but references the optimiser can see through is kept in memory, with every scalar operand it feeds)
   constexpr int RING = kRingOf<HALF>;            // tiles per ring
   constexpr int LDSV = kLdsVOf<HALF>;            // the V ring behind the K ring
-  __shared__ __attribute__((aligned(1024))) char lds[2 * RING * kTileBytes];
+  // (behind the rings, for the epilogue that folds into (o, m, l): a kilobyte per wave for the old m and l of its rows)
+  constexpr int kStateOff = 2 * RING * kTileBytes;
+  __shared__ __attribute__((aligned(1024))) char lds[kStateOff + (MODE == 1 ? (HALF ? NWAVE / 2 : NWAVE) * 1024 : 0)];
   constexpr int BMW = SPLIT || HALF ? BM / 2 : BM;  // query rows of this workgroup
 
   // Workgroup ids go to the 8 XCDs round-robin.  The (query head, query tile) units of one KV head are dealt to p.slices
@@ -353,6 +355,24 @@ __global__ __launch_bounds__(HALF ? NWAVE * 32 : NWAVE * 64, HALF ? 2 : 1) void 
   const int nt = (visible_keys(qf + m_hi * P) + BN - 1) / BN;  // tiles the workgroup walks
 
   const int m_w0 = m_lo + (wrow & ((1 << wph_shift) - 1)) * 32;
+
+  // The old m and l of the wave's rows (MODE 1) are asked for first of all and go straight into LDS, a float per lane:
+  // they have landed when Q has (loads return in order), cost no register over the loops, and the epilogue knows without
+  // a trip to memory whether a row is still in its start state (the first step of a ring, a prefill on one GPU), whose
+  // old o is never read.
+  if (MODE == 1) {
+#pragma unroll
+    for (int qb = 0; qb < 2; qb++) {
+      const int m = m_w0 + 16 * qb + qc;
+      const int64_t at = (o_start + (m < q_len ? m : 0)) * p.ml_st + (int64_t)h * p.ml_sh;
+      const float* pm = p.m + at;
+      const float* pl = p.l + at;
+      const int dst = (int)(uintptr_t)(__attribute__((address_space(3))) char*)lds + kStateOff + wave * 1024 + qb * 256;
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %2, off\n\t"
+                   "s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %3, off" ::"s"(dst), "s"(dst + 512), "v"(pm), "v"(pl)
+                   : "m0", "memory");
+    }
+  }
 
   // Q as B operands: qreg[qb][ks] = Q[row 16 qb + qc][32 ks + 8g .. +7]; cnt[qb] = keys that row sees (0 past the end)
   u32x4 qreg[2][4];
@@ -915,9 +935,9 @@ __global__ __launch_bounds__(HALF ? NWAVE * 32 : NWAVE * 64, HALF ? 2 : 1) void 
     for (int qb = 0; qb < 2; qb++) {
       const int m = m_w0 + 16 * qb + qc;
       const int64_t tok = o_start + (m < q_len ? m : 0);
-      if (MODE == 1) {
-        st_a[qb] = p.m[tok * p.ml_st + (int64_t)h * p.ml_sh];
-        st_b[qb] = p.l[tok * p.ml_st + (int64_t)h * p.ml_sh];
+      if (MODE == 1) {  // (fetched into the wave's LDS at the start)
+        st_a[qb] = *(const float*)(lds + kStateOff + wave * 1024 + qb * 256 + lane * 4);
+        st_b[qb] = *(const float*)(lds + kStateOff + wave * 1024 + 512 + qb * 256 + lane * 4);
       }
       if (MODE == 2) st_a[qb] = p.lse[tok * p.hq + h] * kLog2e;
     }
@@ -996,16 +1016,29 @@ __global__ __launch_bounds__(HALF ? NWAVE * 32 : NWAVE * 64, HALF ? 2 : 1) void 
         float l_tot[NB];
         u32x2 old[NB][NDB];
         bool in_range[NB];
+        bool has_old = false;  // some row of these blocks carries an earlier step's result
 #pragma unroll
         for (int i = 0; i < NB; i++) {
           const int qb = qb0 + i;
-          const int m = m_w0 + 16 * qb + qc;
           l_tot[i] = column_sum(l_run[qb]);
-          in_range[i] = m < q_len;
-          const int64_t tok = o_start + (in_range[i] ? m : 0);
-          const uint16_t* orow = (const uint16_t*)p.o + tok * p.o_st + (int64_t)h * p.o_sh;
+          in_range[i] = m_w0 + 16 * qb + qc < q_len;
+          has_old |= in_range[i] && st_a[qb] != -INFINITY && st_b[qb] != 0.f;
+        }
+        // (the same for every lane: a wave none of whose rows has an old result does not read o at all)
+        const bool read_old = __builtin_amdgcn_ballot_w64(has_old) != 0;
 #pragma unroll
-          for (int d = 0; d < NDB; d++) old[i][d] = *(const u32x2*)(orow + (DB0 + d) * 16 + 4 * g);
+        for (int i = 0; i < NB; i++)
+#pragma unroll
+          for (int d = 0; d < NDB; d++) old[i][d] = u32x2{0u, 0u};
+        if (read_old) {
+#pragma unroll
+          for (int i = 0; i < NB; i++) {
+            const int m = m_w0 + 16 * (qb0 + i) + qc;
+            const int64_t tok = o_start + (in_range[i] ? m : 0);
+            const uint16_t* orow = (const uint16_t*)p.o + tok * p.o_st + (int64_t)h * p.o_sh;
+#pragma unroll
+            for (int d = 0; d < NDB; d++) old[i][d] = *(const u32x2*)(orow + (DB0 + d) * 16 + 4 * g);
+          }
         }
 #pragma unroll
         for (int i = 0; i < NB; i++) {

@@ -142,6 +142,51 @@ def test_ring_inplace_state_matches_monolithic(lsa, dtype):
     assert_lse_close(orc.state_lse(ms.cpu(), ls.cpu()).float(), orc.state_lse(m_c, l_c).float(), "state vs oracle state")
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("Hq,Hkv", [(8, 2), (4, 4)])
+def test_inplace_step_over_rows_in_their_start_state_beside_rows_that_carry_one(lsa, dtype, Hq, Hkv):
+    # The in-place operator reads a row's old o only if the row carries an earlier step's result (m > -inf, l > 0); rows
+    # in their start state may hold anything there.  Both kinds side by side in the blocks of sixteen rows the kernel
+    # works in, in whole blocks of either kind, in a whole sequence of either kind; o of the start-state rows is NaN on
+    # the device and zero for the oracle.
+    lens = [700, 333, 64]
+    T, D = sum(lens), 128
+    q, k, v = rand_t((T, Hq, D), 61, dtype), rand_t((T, Hkv, D), 62, dtype), rand_t((T, Hkv, D), 63, dtype)
+    qm = meta(lens, [5000, 5000, 5000])
+    # an earlier step over other keys (positions below every query's) gives every row a state ...
+    k0, v0 = rand_t((T, Hkv, D), 64, dtype), rand_t((T, Hkv, D), 65, dtype)
+    o_ref = torch.zeros((T, Hq, D), dtype=dtype)
+    m_ref, l_ref = torch.full((T, Hq), float("-inf")), torch.zeros(T, Hq)
+    km0 = meta(lens)
+    orc.context_attention_fwd(q, k0, v0, o_ref, *qm, *km0, 1, max(lens), m_ref, l_ref)
+    assert torch.isfinite(m_ref).all()
+    # ... which these rows lose again: a ragged stretch, whole blocks, single rows, all of the last sequence
+    fresh = torch.zeros(T, dtype=torch.bool)
+    fresh[5:23] = True
+    fresh[64:192] = True
+    fresh[300:700:7] = True
+    fresh[700 + 100:700 + 333] = True
+    fresh[700 + 333:] = True
+    o_ref[fresh] = 0
+    m_ref[fresh] = float("-inf")
+    l_ref[fresh] = 0
+    o_d, m_d, l_d = _dev(o_ref.clone(), m_ref.clone(), l_ref.clone())
+    o_d[fresh.to(DEV)] = float("nan")
+    qd, kd, vd = _dev(q, k, v)
+    qs, ql, qf = _dev(*qm)
+    lsa.context_attention_fwd(qd, kd, vd, o_d, qs, ql, qf, qs, ql, qf, 1, max(lens), m_d, l_d)
+    torch.cuda.synchronize()
+    o_exact, lse_now = orc.attn_step(q, k, v, *qm, *qm, 1)
+    o_prev, lse_prev = orc.attn_step(q, k0, v0, *qm, *km0, 1)
+    orc.context_attention_fwd(q, k, v, o_ref, *qm, *qm, 1, max(lens), m_ref, l_ref)
+    assert torch.isfinite(o_d.float()).all()
+    # the exact answer: this step alone for the fresh rows, both steps merged for the others
+    both_o, both_lse = orc.lse_merge([(o_prev, lse_prev), (o_exact, lse_now)])
+    exact = torch.where(fresh[:, None, None], o_exact, both_o)
+    assert_inplace_o_close(o_d.cpu(), o_ref, exact, "o")
+    assert_lse_close(orc.state_lse(m_d.cpu(), l_d.cpu()).float(), torch.where(fresh[:, None], lse_now, both_lse), "state LSE")
+
+
 def test_striped_ring_equals_full_sequence(lsa):
     from loongserve_amd.simulate import KVChunk, ring_prefill_partials
     T, Hq, Hkv, D, P = 1531, 4, 2, 128, 4
