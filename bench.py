@@ -1011,6 +1011,13 @@ def main():
     if only is None:
         summary["short_prompts"] = short_prompts()
         summary["chunked_prefill_step"] = chunked_prefill_step()
+        # decode batches of one long request beside many short ones: the two stages as a decode step's master calls them
+        # (one partial per 256 tokens) and the fused call, as fractions of the HBM peak
+        summary["decode_mixed_lengths"] = {
+            c["batch"].replace(" tokens", "").replace(" ", ""): {
+                "two_stages_ms": _r(c["chosen"]["two_stages_ms"]), "two_stages_frac": _r(c["chosen"]["two_stages_gbs"] / PEAK_HBM_GBS),
+                "fused_ms": _r(c["chosen"]["fused_ms"]), "fused_frac": _r(c["chosen"]["fused_gbs"] / PEAK_HBM_GBS)}
+            for c in decode_mixed_lengths(full=False)["cases"]}
         summary["ceiling"] = {"mfma_tflops": _r(roof.get("sustained_peak"), 1), "read_gbs": _r(roof.get("decode_sustained_peak_gbs"), 1)}
     if args.sweeps:
         details["prefill_launch_sizes"] = prefill_launch_sizes(tile_us)

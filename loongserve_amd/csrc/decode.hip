@@ -777,8 +777,10 @@ __global__ __launch_bounds__(kMfmaWaves * 64, 2) void decode_stage1_mfma_listed_
 }
 
 // ------------------------------------------------------------------------------------
-// Stage 2: grid (batch, heads); SL slices of D/4 lanes walk the block axis in parallel
-// (the reference walks it serially, flash_decoding_stage2.cu:38-48), then merge through LDS.
+// Stage 2: one workgroup per (request, head), the heads of a request next to each other in the grid (a request much
+// longer than the others then has all its workgroups start together, wherever it stands in the batch, instead of its
+// last head at the very end of the launch); SL slices of D/4 lanes walk the block axis in parallel (the reference walks
+// it serially, flash_decoding_stage2.cu:38-48), then merge through LDS.
 // ------------------------------------------------------------------------------------
 struct Stage2Params {
   void* o;
@@ -805,8 +807,7 @@ template <typename OT, int D, int NT>
 __global__ __launch_bounds__(NT) void decode_stage2_kernel(Stage2Params p) {
   constexpr int LPR = D / 4;      // lanes per row (float4 each)
   constexpr int SL = NT / LPR;    // slices walking the block axis
-  constexpr int U = 8;            // rows a slice has in flight
-  const int64_t b = blockIdx.x, h = blockIdx.y;
+  const int64_t b = blockIdx.x / (uint32_t)p.heads, h = blockIdx.x % (uint32_t)p.heads;
   const int slice = threadIdx.x / LPR, c = threadIdx.x % LPR;
   const int64_t len = p.b_seqlen[b];
   int64_t n = len <= 0 ? 0 : (len + p.block_seq - 1) / p.block_seq;
@@ -831,6 +832,7 @@ __global__ __launch_bounds__(NT) void decode_stage2_kernel(Stage2Params p) {
   // long request's merge is a chain of them.  Positions past the request's last block repeat that block and are
   // dropped; an empty partial's row is loaded like any other (it may hold anything: stage 1 leaves the rows it merged
   // into another one untouched) and dropped by its log-sum-exp.
+  constexpr int U = 8;  // rows a slice has in flight (sixteen measured slower: the many short requests of a batch then ask for rows they drop)
   for (int64_t i = slice; i < n; i += U * SL) {
     float lse[U];
     f32x4 tv[U];
@@ -1068,7 +1070,7 @@ extern "C" int lsattn_decode_stage1(const lsattn_decode_stage1_args* a, void* st
 template <typename OT> static int dispatch_stage2(const Stage2Params& p, int64_t D, dim3 grid, int64_t live_blocks, hipStream_t st) {
   // few (batch, head) pairs with many partials each (long contexts at small batch): 1024 threads walk the block axis in 32
   // slices instead of 8, or the merge takes a fifth of the time of the gather it follows
-  const bool wide = D == 128 && live_blocks >= 64 && (int64_t)grid.x * grid.y < 2048;
+  const bool wide = D == 128 && live_blocks >= 64 && ((int64_t)grid.x < 2048 || (live_blocks >= 1024 && (int64_t)grid.x < 8192));
   switch (D) {
     case 32: hipLaunchKernelGGL((decode_stage2_kernel<OT, 32, 256>), grid, dim3(256), 0, st, p); break;
     case 64: hipLaunchKernelGGL((decode_stage2_kernel<OT, 64, 256>), grid, dim3(256), 0, st, p); break;
@@ -1087,12 +1089,12 @@ static int decode_stage2(const lsattn_decode_stage2_args* a, int64_t live_blocks
   if (((uintptr_t)a->o | (uintptr_t)a->mid_o) & 15) return LSATTN_ERR_INVALID_ARG;
   if (a->head_dim != 32 && a->head_dim != 64 && a->head_dim != 128) return LSATTN_ERR_UNSUPPORTED;
   if (a->batch == 0) return LSATTN_OK;
-  if (a->num_heads > 65535) return LSATTN_ERR_INVALID_ARG;
+  if (a->batch * a->num_heads > 0x7fffffff) return LSATTN_ERR_INVALID_ARG;
   Stage2Params p{a->o, a->out_logexpsum, a->b_seqlen, a->mid_o, a->mid_o_logexpsum,
                  a->batch, a->num_heads, a->num_seq_blocks, a->block_seq,
                  a->partials_by_request ? a->num_heads : a->batch * a->num_heads,
                  a->partials_by_request ? a->num_seq_blocks * a->num_heads : a->num_heads};
-  dim3 grid((unsigned)a->batch, (unsigned)a->num_heads);
+  dim3 grid((unsigned)(a->batch * a->num_heads));
   hipStream_t st = (hipStream_t)stream;
   switch (a->o_dtype) {
     case LSATTN_F32: return dispatch_stage2<float>(p, a->head_dim, grid, live_blocks, st);

@@ -205,13 +205,15 @@ def _merge_cuts(po, pl, S: int, Tq: int, q_b_start_loc, q_b_seq_len, max_q_len: 
 # Launches below this many 128-row workgroups (batch x query heads x ceil(max_q / 128)) are cut along the keys when the
 # KV chunks may hold at least KV_SPLIT_MIN_KEYS keys: 256 CUs run one workgroup each.
 KV_SPLIT_BELOW_WORKGROUPS = 192
+KV_SPLIT_ROUND = 256  # workgroups of a cut launch that run at once: one per CU
 KV_SPLIT_MIN_KEYS = 8192
 
 
 def kv_split_count(batch: int, num_q_heads: int, max_q_len: int, kv_rows: int, num_kv_heads: Optional[int] = None) -> int:
-    """KV cuts the prefill operators use by themselves: enough for a good round of workgroups (about 320), cuts of at
-    least 4096 keys (kv_rows bounds every sequence's chunk: max_kv_len where the caller gives it, else the rows of the k buffer;
-    the lengths themselves live on the device).  The launch's size without cuts is counted in 128-row workgroups as the
+    """KV cuts the prefill operators use by themselves: the count that leaves the longest chain of tiles on a CU shortest
+    when the launch's workgroups run in rounds of 256 (one per CU), the smaller count on ties, with cuts of at least 4096
+    keys (kv_rows bounds every sequence's chunk: max_kv_len where the caller gives it, else the rows of the k buffer; the
+    lengths themselves live on the device).  The launch's size without cuts is counted in 128-row workgroups as the
     kernel forms them: up to four query heads of a KV head side by side (num_kv_heads given), 128 / that many positions each."""
     pack = 1
     if num_kv_heads:
@@ -221,9 +223,16 @@ def kv_split_count(batch: int, num_q_heads: int, max_q_len: int, kv_rows: int, n
     wgs = batch * (num_q_heads // pack) * ((max_q_len + 128 // pack - 1) // (128 // pack))
     if wgs <= 0 or wgs >= KV_SPLIT_BELOW_WORKGROUPS or kv_rows < KV_SPLIT_MIN_KEYS:
         return 1
-    # (measured, GQA 32/8 unless said: 16 rows x 131072 keys 32 cuts 124 us against 134 with 16 and 160 with 64; 100 x 131072
-    # 16 cuts 243 against 252 with 8 and 270 with 32, MHA 8 cuts 388 against 412; 128 x 32768 8 cuts 80 against 84 with 16)
-    return max(1, min(_lib.LSATTN_MAX_KV_CUTS, 320 // wgs, kv_rows // 4096))
+    # rounds(S) / S of the uncut chain is what a CU walks with S cuts.  (measured, GQA 32/8 unless said: 16 rows x 131072 keys
+    # 32 cuts 124 us against 134 with 16 and 160 with 64; 100 x 131072 8 cuts 252, 10 cuts 285, 16 cuts 243, 32 cuts 270, MHA 8 cuts 388
+    # against 412 with 16; 128 x 32768 8 cuts 80 against 84 with 16)
+    best, best_cost = 1, None
+    for S in range(1, max(1, min(_lib.LSATTN_MAX_KV_CUTS, kv_rows // 4096)) + 1):
+        # (and every cut adds a part to write and to merge: about a thousandth of the uncut chain each in the cases above)
+        cost = (-(-wgs * S // KV_SPLIT_ROUND)) / S + 0.001 * S
+        if best_cost is None or cost < best_cost - 1e-9:
+            best, best_cost = S, cost
+    return best
 
 
 def _cut_len(kv_rows: int, S: int) -> int:

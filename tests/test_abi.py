@@ -267,11 +267,12 @@ def test_kv_split_count_from_shapes():
     from loongserve_amd.ops import kv_split_count
     assert kv_split_count(1, 32, 16384, 16384) == 1          # config 2: 4096 workgroups
     assert kv_split_count(1, 32, 2048, 2048) == 1            # config 1: enough workgroups, few keys
-    assert kv_split_count(1, 32, 100, 131072) == 10          # one 100-row chunk against 131072 keys: 32 workgroups -> 320
-    assert kv_split_count(1, 32, 100, 131072, 8) == 10       # GQA 32/8: four heads side by side, 8 x 4 workgroups of 32 positions
+    assert kv_split_count(1, 32, 100, 131072) == 8           # one 100-row chunk against 131072 keys: 32 workgroups -> one round of 256
+    assert kv_split_count(1, 32, 100, 131072, 8) == 8        # GQA 32/8: four heads side by side, 8 x 4 workgroups of 32 positions
     assert kv_split_count(1, 32, 16, 131072, 8) == 32        # 16 rows: 8 workgroups; cuts of at least 4096 keys
     assert kv_split_count(1, 32, 16, 20000, 8) == 4
     assert kv_split_count(1, 8, 100, 20000) == 4             # cuts of at least 4096 keys
     assert kv_split_count(4, 32, 128, 100000) == 2           # 128 workgroups: two cuts
+    assert kv_split_count(1, 100, 128, 100000) == 5          # 100 workgroups: two rounds of five cuts walk less than one round of two
     assert kv_split_count(1, 32, 100, 4096) == 1             # short KV
     assert kv_split_count(0, 32, 100, 100000) == 1
