@@ -70,7 +70,7 @@ typedef struct lsattn_prefill_args {
   int32_t batch;
   int32_t num_q_heads;
   int32_t num_kv_heads;
-  int32_t head_dim;   /* 128 */
+  int32_t head_dim;   /* 128; 16, 32 and 64 (RING:248-250) run a plainer kernel of their own, which takes no kv_cuts */
   int32_t dtype;      /* LSATTN_F16 or LSATTN_BF16 (q, k, v) */
   int32_t sp_peers;   /* logical_sp_peers_num, >= 1 */
   int32_t max_q_len;  /* max over q_b_seq_len (sizes the launch, RING:262) */
@@ -135,7 +135,7 @@ int lsattn_prefill_step_accumulate(const lsattn_prefill_args* a, void* stream);
  */
 typedef struct lsattn_merge_args {
   int32_t n_parts; /* 1..LSATTN_MAX_PARTS */
-  int32_t head_dim;
+  int32_t head_dim; /* 16, 32, 64 or 128 */
   int64_t rows;    /* tokens * heads */
   const float* o_parts[LSATTN_MAX_PARTS];
   const float* lse_parts[LSATTN_MAX_PARTS];

@@ -15,7 +15,7 @@ ROOT = os.path.dirname(PKG_DIR)
 CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_PATH = os.path.join(PKG_DIR, "liblsattn.so")
 CEILING_LIB_PATH = os.path.join(PKG_DIR, "libls_ceiling.so")  # measurement aids of bench.py (include/ls_ceiling.h)
-SOURCES = ["prefill.hip", "decode.hip", "merge_scatter.hip", "elementwise.hip", "pool.hip"]
+SOURCES = ["prefill.hip", "prefill_small.hip", "decode.hip", "merge_scatter.hip", "elementwise.hip", "pool.hip"]
 # elementwise.hip reproduces the reference's half arithmetic operation by operation: no fused multiply-adds
 # other than the ones it writes
 FILE_FLAGS = {

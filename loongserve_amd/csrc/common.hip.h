@@ -79,6 +79,10 @@ struct Tuning {
 };
 Tuning tuning();
 
+// The prefill step for head sizes 16, 32 and 64 (prefill_small.hip); `mode`: 0 fp32 partial, 1 in-place (o, m, l), 2 merge into a
+// running fp32 partial.  Arguments validated by the caller.
+int launch_prefill_small(const lsattn_prefill_args* a, int mode, hipStream_t st);
+
 inline int check_launch() { return hipGetLastError() == hipSuccess ? LSATTN_OK : LSATTN_ERR_LAUNCH; }
 
 }  // namespace lsattn

@@ -332,6 +332,7 @@ template <typename OT> static int launch_merge(const MergeParams& p, int D, hipS
   const int64_t blocks = (threads + 255) / 256;
   if (blocks > 0x7fffffff) return LSATTN_ERR_INVALID_ARG;
   switch (D) {
+    case 16: hipLaunchKernelGGL((lse_merge_kernel<OT, 16>), dim3((unsigned)blocks), dim3(256), 0, st, p); break;
     case 32: hipLaunchKernelGGL((lse_merge_kernel<OT, 32>), dim3((unsigned)blocks), dim3(256), 0, st, p); break;
     case 64: hipLaunchKernelGGL((lse_merge_kernel<OT, 64>), dim3((unsigned)blocks), dim3(256), 0, st, p); break;
     case 128: hipLaunchKernelGGL((lse_merge_kernel<OT, 128>), dim3((unsigned)blocks), dim3(256), 0, st, p); break;

@@ -1311,7 +1311,8 @@ static int validate(const lsattn_prefill_args* a, int mode) {
   if (a->batch < 0 || a->num_q_heads <= 0 || a->num_kv_heads <= 0 || a->sp_peers < 1 || a->max_q_len < 0 || a->total_q_rows < 0)
     return LSATTN_ERR_INVALID_ARG;
   if (a->num_q_heads % a->num_kv_heads) return LSATTN_ERR_INVALID_ARG;
-  if (a->head_dim != 128) return LSATTN_ERR_UNSUPPORTED;
+  if (a->head_dim != 128 && a->head_dim != 64 && a->head_dim != 32 && a->head_dim != 16) return LSATTN_ERR_UNSUPPORTED;
+  if (a->head_dim != 128 && a->kv_cuts > 1) return LSATTN_ERR_UNSUPPORTED;  // (the cut along the keys is the 128-wide kernel's)
   if (a->dtype != LSATTN_F16 && a->dtype != LSATTN_BF16) return LSATTN_ERR_UNSUPPORTED;
   if (a->v_is_f16 != 0 && (a->v_is_f16 != 1 || a->dtype != LSATTN_BF16)) return LSATTN_ERR_INVALID_ARG;
   // the chunk cut along the keys: a multiple of the 64-key tile per cut, the cuts' outputs apart (fp32 partials only),
@@ -1343,6 +1344,7 @@ extern "C" int lsattn_prefill_step(const lsattn_prefill_args* a, void* stream) {
   const int rc = validate(a, 0);
   if (rc != LSATTN_OK) return rc;
   if (a->batch == 0 || a->max_q_len == 0) return LSATTN_OK;
+  if (a->head_dim != 128) return launch_prefill_small(a, 0, (hipStream_t)stream);
   if (a->dtype == LSATTN_F16) return launch_prefill<F16, 0, true>(a, (hipStream_t)stream);
   return a->v_is_f16 ? launch_prefill<BF16, 0, true>(a, (hipStream_t)stream) : launch_prefill<BF16, 0, false>(a, (hipStream_t)stream);
 }
@@ -1351,6 +1353,7 @@ extern "C" int lsattn_prefill_step_merge(const lsattn_prefill_args* a, void* str
   const int rc = validate(a, 1);
   if (rc != LSATTN_OK) return rc;
   if (a->batch == 0 || a->max_q_len == 0) return LSATTN_OK;
+  if (a->head_dim != 128) return launch_prefill_small(a, 1, (hipStream_t)stream);
   if (a->dtype == LSATTN_F16) return launch_prefill<F16, 1, true>(a, (hipStream_t)stream);
   return a->v_is_f16 ? launch_prefill<BF16, 1, true>(a, (hipStream_t)stream) : launch_prefill<BF16, 1, false>(a, (hipStream_t)stream);
 }
@@ -1359,6 +1362,7 @@ extern "C" int lsattn_prefill_step_accumulate(const lsattn_prefill_args* a, void
   const int rc = validate(a, 2);
   if (rc != LSATTN_OK) return rc;
   if (a->batch == 0 || a->max_q_len == 0) return LSATTN_OK;
+  if (a->head_dim != 128) return launch_prefill_small(a, 2, (hipStream_t)stream);
   if (a->dtype == LSATTN_F16) return launch_prefill<F16, 2, true>(a, (hipStream_t)stream);
   return a->v_is_f16 ? launch_prefill<BF16, 2, true>(a, (hipStream_t)stream) : launch_prefill<BF16, 2, false>(a, (hipStream_t)stream);
 }

@@ -86,15 +86,7 @@ def _v_as_f16(v: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tens
     return out
 
 
-KERNEL_HEAD_DIM = 128
-
-
-def _pad_head_dim(t: torch.Tensor) -> torch.Tensor:
-    """[tokens, heads, D] with D < 128 -> a new [tokens, heads, 128] tensor, zeros beyond D.  Zero columns leave q.k
-    unchanged and give zero output columns, so the 128-wide kernel computes the D-wide attention exactly."""
-    out = t.new_zeros((t.shape[0], t.shape[1], KERNEL_HEAD_DIM))
-    out[..., :t.shape[-1]] = t
-    return out
+KERNEL_HEAD_DIM = 128  # the tuned kernel's head size (and the only one whose KV chunks are cut); 16, 32 and 64 take the plain kernel
 
 
 def _prefill_args(q, k, v, o, q_b_start_loc, q_b_seq_len, q_first, kv_b_start_loc, kv_b_seq_len, kv_first,
@@ -126,7 +118,8 @@ def _prefill_args(q, k, v, o, q_b_start_loc, q_b_seq_len, q_first, kv_b_start_lo
                  (kv_b_start_loc, "kv_b_start_loc"), (kv_b_seq_len, "kv_b_seq_len"), (kv_first, "kv_first_token_global_idx")):
         _i32vec(t, n, B)
     a = _lib.PrefillArgs()
-    if q.dtype == torch.bfloat16 and (PRECONVERT_BF16_V or v_f16 is not None):
+    # (the kernel for head sizes below 128 converts V as it stages it, at no cost: no copy unless the caller brings one)
+    if q.dtype == torch.bfloat16 and ((PRECONVERT_BF16_V and Lq == KERNEL_HEAD_DIM) or v_f16 is not None):
         if v_f16_valid:
             if v_f16 is None or v_f16.dtype != torch.float16 or v_f16.shape != v.shape or v_f16.stride(2) != 1:
                 raise ValueError("v_f16_valid needs v_f16, the float16 copy of v")
@@ -274,12 +267,6 @@ def context_attention_fwd(q, k, v, o, q_b_start_loc, q_b_seq_len, q_first_token_
     if o.dtype != q.dtype:
         raise ValueError("o must have the dtype of q")
     D = q.shape[-1]
-    o_user = None
-    if q.dim() == 3 and D in (16, 32, 64) and k.shape[-1] == D and v.shape[-1] == D and o.shape == q.shape:
-        # head sizes below 128 (RING:250 admits them): run the 128-wide kernel on zero-padded copies, old o included
-        # (the step folds into it), and copy the first D columns back
-        o_user, o = o, _pad_head_dim(o)
-        q, k, v = _pad_head_dim(q), _pad_head_dim(k), _pad_head_dim(v)
     for t, n in ((m, "m"), (l, "l")):
         _dev(t, n)
         if t.dtype != torch.float32 or t.dim() != 2 or tuple(t.shape) != (q.shape[0], q.shape[1]):
@@ -287,7 +274,7 @@ def context_attention_fwd(q, k, v, o, q_b_start_loc, q_b_seq_len, q_first_token_
     if m.stride() != l.stride():
         raise ValueError("m and l must share strides")
     S = 1
-    if workspace is not None and o_user is None and q.dim() == 3:
+    if workspace is not None and D == KERNEL_HEAD_DIM and q.dim() == 3:
         kv_rows = k.shape[0] if max_kv_len is None else int(max_kv_len)
         S = kv_split_count(q_b_seq_len.shape[0], q.shape[1], int(max_q_b_seq_len), kv_rows, k.shape[1]) if kv_splits is None else int(kv_splits)
         S = min(S, _workspace_cuts(workspace, q.shape[0], q.shape[1], D), _lib.LSATTN_MAX_KV_CUTS)
@@ -305,12 +292,10 @@ def context_attention_fwd(q, k, v, o, q_b_start_loc, q_b_seq_len, q_first_token_
         return
     a = _prefill_args(q, k, v, o, q_b_start_loc, q_b_seq_len, q_first_token_global_idx, kv_b_start_loc,
                       kv_b_seq_len, kv_first_token_global_idx, logical_sp_peers_num, max_q_b_seq_len,
-                      1.0 / (D ** 0.5), v_f16 if o_user is None else None, v_f16_valid and o_user is None, total_q_len=total_q_len)
+                      1.0 / (D ** 0.5), v_f16, v_f16_valid, total_q_len=total_q_len)
     a.m, a.l = m.data_ptr(), l.data_ptr()
     a.ml_stride_t, a.ml_stride_h = m.stride(0), m.stride(1)
     _lib.check(_lib.load().lsattn_prefill_step_merge(C.byref(a), _stream()), "lsattn_prefill_step_merge")
-    if o_user is not None:
-        o_user.copy_(o[..., :D])
 
 
 @torch.inference_mode()
@@ -346,15 +331,10 @@ def prefill_attention_step(q, k, v, q_b_start_loc, q_b_seq_len, q_first_token_gl
         lse = torch.empty(q.shape[:2], dtype=torch.float32, device=q.device)
     if out.dtype != torch.float32 or lse.dtype != torch.float32 or not lse.is_contiguous():
         raise ValueError("out and lse must be float32, lse contiguous")
-    out_user = None
-    if q.dim() == 3 and D in (16, 32, 64) and k.shape[-1] == D and v.shape[-1] == D and out.shape == q.shape:
-        out_user, out = out, (_pad_head_dim(out) if accumulate else
-                              torch.empty(q.shape[:2] + (KERNEL_HEAD_DIM,), dtype=torch.float32, device=q.device))
-        q, k, v = _pad_head_dim(q), _pad_head_dim(k), _pad_head_dim(v)
-        if sm_scale is None:
-            sm_scale = 1.0 / (D ** 0.5)
     kv_rows = k.shape[0] if max_kv_len is None else int(max_kv_len)
     S = kv_split_count(q_b_seq_len.shape[0], q.shape[1], int(max_q_b_seq_len), kv_rows, k.shape[1]) if kv_splits is None else int(kv_splits)
+    if D != KERNEL_HEAD_DIM:
+        S = 1  # (the cut along the keys is the 128-wide kernel's)
     if S > 1:
         if S > _lib.LSATTN_MAX_KV_CUTS:
             raise ValueError("at most %d KV slices" % _lib.LSATTN_MAX_KV_CUTS)
@@ -364,25 +344,19 @@ def prefill_attention_step(q, k, v, q_b_start_loc, q_b_seq_len, q_first_token_gl
         po, pl = _cut_workspace(kv_split_workspace, S, Tq, q.shape[1], q.shape[2], q.device)
         a = _prefill_args(q, k, v, po, q_b_start_loc, q_b_seq_len, q_first_token_global_idx, kv_b_start_loc, kv_b_seq_len,
                           kv_first_token_global_idx, logical_sp_peers_num, max_q_b_seq_len, sm_scale,
-                          v_f16 if out_user is None else None, v_f16_valid and out_user is None, cuts=(S, _cut_len(kv_rows, S), Tq))
+                          v_f16, v_f16_valid, cuts=(S, _cut_len(kv_rows, S), Tq))
         a.lse = pl.data_ptr()
         _lib.check(_lib.load().lsattn_prefill_step(C.byref(a), _stream()), "lsattn_prefill_step")
         _merge_cuts(po, pl, S, Tq, q_b_start_loc, q_b_seq_len, max_q_b_seq_len, 2 if accumulate else 0, out, lse=lse)
-        if out_user is not None:
-            out_user.copy_(out[..., :D])
-            out = out_user
         return out, lse
     a = _prefill_args(q, k, v, out, q_b_start_loc, q_b_seq_len, q_first_token_global_idx, kv_b_start_loc,
                       kv_b_seq_len, kv_first_token_global_idx, logical_sp_peers_num, max_q_b_seq_len, sm_scale,
-                      v_f16 if out_user is None else None, v_f16_valid and out_user is None, total_q_len=total_q_len)
+                      v_f16, v_f16_valid, total_q_len=total_q_len)
     a.lse = lse.data_ptr()
     if accumulate:
         _lib.check(_lib.load().lsattn_prefill_step_accumulate(C.byref(a), _stream()), "lsattn_prefill_step_accumulate")
     else:
         _lib.check(_lib.load().lsattn_prefill_step(C.byref(a), _stream()), "lsattn_prefill_step")
-    if out_user is not None:
-        out_user.copy_(out[..., :D])
-        out = out_user
     return out, lse
 
 

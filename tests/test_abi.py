@@ -119,9 +119,13 @@ def test_validation_rejects_bad_arguments_without_gpu():
     for f in ("q", "k", "v", "o", "lse", "q_b_start_loc", "q_b_seq_len", "q_first_token_global_idx", "kv_b_start_loc",
               "kv_b_seq_len", "kv_first_token_global_idx"):
         setattr(a, f, fake)
-    a.batch, a.num_q_heads, a.num_kv_heads, a.head_dim, a.sp_peers, a.max_q_len = 1, 4, 2, 64, 1, 8
+    a.batch, a.num_q_heads, a.num_kv_heads, a.head_dim, a.sp_peers, a.max_q_len = 1, 4, 2, 48, 1, 8
     a.o_dtype = _lib.LSATTN_F32
     assert lib.lsattn_prefill_step(C.byref(a), None) == -2
+    # head sizes 16, 32 and 64 have a kernel of their own, which does not cut the KV chunk
+    a.head_dim, a.kv_cuts, a.kv_cut_len, a.o_cut_rows = 64, 2, 64, 8
+    assert lib.lsattn_prefill_step(C.byref(a), None) == -2
+    a.kv_cuts = a.kv_cut_len = a.o_cut_rows = 0
     a.head_dim, a.num_kv_heads = 128, 3
     assert lib.lsattn_prefill_step(C.byref(a), None) == -1
     # K/V token strides must be positive and keep a 64-row tile within a 32-bit byte offset

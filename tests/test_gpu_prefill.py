@@ -368,8 +368,8 @@ def test_bf16_to_f16_rows_is_exact_in_range_and_saturates(lsa):
 
 @pytest.mark.parametrize("D", [16, 32, 64])
 def test_head_sizes_below_128(lsa, D):
-    """RING:250 admits head sizes 16, 32 and 64; the operators run them through the 128-wide kernel on zero-padded
-    copies.  One partial step, and two in-place steps whose second one folds into the first one's o."""
+    """RING:250 admits head sizes 16, 32 and 64; they have a kernel of their own.  One partial step, and two in-place
+    steps whose second one folds into the first one's o."""
     print("case D", D, flush=True)
     lens, Hq, Hkv = [300, 77], 4, 2
     T = sum(lens)
@@ -385,7 +385,7 @@ def test_head_sizes_below_128(lsa, D):
     k0, v0 = rand_t((sum(klens), Hkv, D), 44), rand_t((sum(klens), Hkv, D), 45)
     qm = meta(lens, [150, 40])
     km0 = meta(klens)
-    od = torch.empty(T, Hq, D, dtype=torch.float16, device=DEV)
+    od = torch.full((T, Hq, D), float("nan"), dtype=torch.float16, device=DEV)  # (rows in their start state may hold anything)
     md = torch.full((T, Hq), float("-inf"), device=DEV)
     ld = torch.zeros(T, Hq, device=DEV)
     oc, mc, lc = torch.zeros(T, Hq, D, dtype=torch.float16), torch.full((T, Hq), float("-inf")), torch.zeros(T, Hq)
@@ -395,6 +395,77 @@ def test_head_sizes_below_128(lsa, D):
     torch.cuda.synchronize()
     assert_o_close(od, oc.float(), "in-place o")
     assert_lse_close(orc.state_lse(md.cpu(), ld.cpu()).float(), orc.state_lse(mc, lc).float(), "state")
+
+
+@pytest.mark.parametrize("D", [16, 32, 64])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_head_sizes_below_128_over_a_striped_ring(lsa, D, dtype):
+    """The kernel of the small head sizes through everything the 128-wide one is asked: ragged batches with an empty
+    request, grouped heads (7 query heads on 1 KV head, 6 on 3), a ring of P = 3 striped shards taken as separate fp32
+    partials, folded into a running partial by the epilogue, and folded in place into (o, m, l); strided K/V views of one
+    buffer; for bfloat16 the V converted by the kernel and brought as an fp16 copy."""
+    print("case D", D, dtype, flush=True)
+    from loongserve_amd.simulate import KVChunk, ring_prefill, ring_prefill_accumulate, ring_prefill_partials
+    P = 3
+    for lens, Hq, Hkv in (([257, 0, 64, 1], 7, 1), ([130, 333], 6, 3)):
+        T = sum(lens)
+        q, kv = rand_t((T, Hq, D), 71, dtype), rand_t((T, 2 * Hkv, D), 72, dtype)
+        k, v = kv[:, :Hkv], kv[:, Hkv:]
+        m = meta(lens)
+        o_ref, lse_ref = orc.attn_step(q, k, v, *m, *m, 1)
+        # shard r of the striped ring holds tokens r, r + P, ... of every sequence
+        chunks, shards = [], []
+        for r in range(P):
+            idx, st, ln = [], [], []
+            for s0, n in zip(m[0].tolist(), lens):
+                ids = list(range(s0 + r, s0 + n, P))
+                st.append(len(idx))
+                ln.append(len(ids))
+                idx += ids
+            it = torch.tensor(idx, dtype=torch.long)
+            km = (torch.tensor(st, dtype=torch.int32), torch.tensor(ln, dtype=torch.int32), torch.full((len(lens),), r, dtype=torch.int32))
+            shards.append((kv[it], km))
+            chunks.append(KVChunk(kv[it].to(DEV), *(t.to(DEV) for t in km)))
+        # the queries of shard 1: tokens 1, 1 + P, ...
+        qi, qst, qln = [], [], []
+        for s0, n in zip(m[0].tolist(), lens):
+            ids = list(range(s0 + 1, s0 + n, P))
+            qst.append(len(qi))
+            qln.append(len(ids))
+            qi += ids
+        qit = torch.tensor(qi, dtype=torch.long)
+        qm = (torch.tensor(qst, dtype=torch.int32), torch.tensor(qln, dtype=torch.int32), torch.full((len(lens),), 1, dtype=torch.int32))
+        ql_q = q[qit]
+        qs_d, qn_d, qf_d = _dev(*qm)
+        maxq = max(qln)
+        order = [1, 0, 2]
+        o1, lse1 = ring_prefill_partials(ql_q.to(DEV), [chunks[i] for i in order], qs_d, qn_d, qf_d, P, maxq, Hkv)
+        o2, lse2 = ring_prefill_accumulate(ql_q.to(DEV), [chunks[i] for i in order], qs_d, qn_d, qf_d, P, maxq, Hkv)
+        o3, m3, l3 = ring_prefill(ql_q.to(DEV), [chunks[i] for i in order], qs_d, qn_d, qf_d, P, maxq, Hkv)
+        torch.cuda.synchronize()
+        assert_o_close(o1, o_ref[qit], "partials O")
+        assert_lse_close(lse1, lse_ref[qit], "partials LSE")
+        assert_o_close(o2, o_ref[qit], "accumulated O")
+        assert_lse_close(lse2, lse_ref[qit], "accumulated LSE")
+        o_st = torch.zeros((len(qi), Hq, D), dtype=dtype)
+        m_st, l_st = torch.full((len(qi), Hq), float("-inf")), torch.zeros(len(qi), Hq)
+        for i in order:
+            kvs, km = shards[i]
+            orc.context_attention_fwd(ql_q, kvs[:, :Hkv], kvs[:, Hkv:], o_st, *qm, *km, P, maxq, m_st, l_st)
+        assert_inplace_o_close(o3.cpu(), o_st, o_ref[qit], "ring o")
+        assert_lse_close(orc.state_lse(m3.cpu(), l3.cpu()).float(), lse_ref[qit], "state LSE")
+        if dtype == torch.bfloat16:
+            # the caller's fp16 copy of V instead of the conversion inside the kernel
+            c = chunks[0]
+            vf = torch.empty((c.kv.shape[0], Hkv, D), dtype=torch.float16, device=DEV)
+            o4, lse4 = lsa.prefill_attention_step(ql_q.to(DEV), c.kv[:, :Hkv], c.kv[:, Hkv:], qs_d, qn_d, qf_d, c.b_start_loc, c.b_seq_len, c.first_token_global_idx,
+                                                  P, maxq, v_f16=vf)
+            o5, lse5 = lsa.prefill_attention_step(ql_q.to(DEV), c.kv[:, :Hkv], c.kv[:, Hkv:], qs_d, qn_d, qf_d, c.b_start_loc, c.b_seq_len, c.first_token_global_idx, P, maxq)
+            torch.cuda.synchronize()
+            vsrc = c.kv[:, Hkv:].cpu().float()
+            normal = vsrc.abs() >= 2.0 ** -14  # (exact in fp16's normal range)
+            assert torch.equal(vf.cpu().float()[normal], vsrc[normal])
+            assert torch.equal(o4, o5) and torch.equal(lse4, lse5)
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
