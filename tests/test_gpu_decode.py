@@ -384,6 +384,34 @@ def test_stage2_alone_over_few_and_many_partials(lsa, nblk):
         assert_lse_close(l, l_ref, "lse", rel=1e-5)
 
 
+@pytest.mark.parametrize("B,H,nblk", [(70, 32, 1030), (300, 8, 520), (9, 5, 1024)])
+def test_stage2_of_one_long_request_among_many_short_ones(lsa, B, H, nblk):
+    """The merge of a batch in which one request has a thousand partials and the others a few: more (request, head) pairs
+    than the narrow launch's bound for the wide one, with enough partials for the wide launch all the same (70 x 32), too
+    many pairs for it (300 x 8), and a small batch; the long request in the middle of the batch, so that the heads of a
+    request and the requests of a head are both told apart in the grid."""
+    print("case", B, H, nblk, flush=True)
+    D, BS = 128, 16
+    g = torch.Generator().manual_seed(B * 1000 + nblk)
+    mo = torch.randn(nblk, B, H, D, generator=g)
+    ml = torch.randn(nblk, B, H, generator=g) * 5
+    ml[torch.rand(nblk, B, H, generator=g) < 0.1] = float("-inf")
+    lens = torch.randint(1, 4 * BS, (B,), generator=g).to(torch.int32)
+    lens[B // 2] = nblk * BS - 3
+    lens[0] = 0
+    o_ref = torch.empty(B, H, D)
+    l_ref = torch.empty(B, H)
+    orc.decode_stage2(mo, ml, lens, o_ref, l_ref, BS)
+    o = torch.full((B, H, D), 9.0, device=DEV)
+    l = torch.full((B, H), 9.0, device=DEV)
+    lsa.longserve_flash_decode_stage2(mo.to(DEV), ml.to(DEV), lens.to(DEV), o, l, BS)
+    torch.cuda.synchronize()
+    dead = torch.isinf(l_ref) & (l_ref < 0)
+    assert torch.equal(torch.isinf(l.cpu()) & (l.cpu() < 0), dead)
+    assert_o_close(o, torch.where(dead[..., None], torch.zeros(()), o_ref), "o", max_abs=2e-5, rel=1e-5)
+    assert_lse_close(l, l_ref, "lse", rel=1e-5)
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_peaked_softmax_keeps_the_bars(lsa, dtype):
     """Scores of magnitude up to ~64: a few tokens carry each request."""
