@@ -54,6 +54,12 @@ FUSED_MIN_WORKGROUPS = 256
 # (config 3, lengths 4096..32768: 903 us at 1024, 947 at 2048).
 FUSED_LONG_SPLIT_TOKENS = 4096
 FUSED_LONG_MIN_BLOCKS = 64
+# ... and only in batches of at most this many requests.  What the coarser split wins is a few percent and only if the
+# requests are about as long as each other (64 x 65536 tokens 2.78 ms at 1024, 2.58 at 4096; 32 x 131072 2.65 at 2048,
+# 2.58 at 4096); what it loses when one long request stands among many short ones is more (131072 + 255 x 512 tokens:
+# 0.181 ms at 1024, 0.198 at 2048, 0.238 at 4096; 131072 + 63 x 2048: 0.207 / 0.217 / 0.275; but 524288 + 63 x 2048, where the
+# long request is four fifths of all tokens: 0.447 / 0.429 / 0.416), and the larger the batch the likelier the latter.
+FUSED_LONG_MAX_BATCH = 64
 
 
 @functools.lru_cache(maxsize=4096)
@@ -64,7 +70,7 @@ def _fused_block_seq(block_seq: int, batch_size: int, max_len_in_batch: int, num
         blocks = (int(max_len_in_batch) + 2 * bs - 1) // (2 * bs)
         if int(batch_size) * blocks * task_groups < FUSED_MIN_WORKGROUPS:
             break
-        if bs * 2 > FUSED_SPLIT_TOKENS and blocks < FUSED_LONG_MIN_BLOCKS:
+        if bs * 2 > FUSED_SPLIT_TOKENS and (blocks < FUSED_LONG_MIN_BLOCKS or int(batch_size) > FUSED_LONG_MAX_BATCH):
             break
         bs *= 2
     return bs

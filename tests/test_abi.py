@@ -250,6 +250,8 @@ def test_fused_decode_split_rule():
     assert _fused_block_seq(256, 4, 131072, 32) == 2048
     assert _fused_block_seq(256, 16, 32768, 8) == 1024
     assert _fused_block_seq(2048, 64, 32768, 8) == 2048          # never below what the caller asked for
+    assert _fused_block_seq(256, 64, 524288, 8) == 4096          # up to 64 requests may go beyond 1024
+    assert _fused_block_seq(256, 256, 131072, 8) == 1024         # larger batches stay there: the likelier to hold one long request among short ones
     assert _fused_block_seq(16, 4096, 16, 8) == 16
     for bs in (1, 16, 64, 256):
         got = _fused_block_seq(bs, 1 << 14, 1 << 20, 32)
