@@ -724,6 +724,13 @@ __global__ __launch_bounds__(kMfmaWaves * 64, 2) void decode_stage1_mfma_kernel(
 // neighbouring units, which run at the same time on neighbouring workgroups (all KV heads of a token are fetched together).
 constexpr int kListedMaxBatch = 1024;
 constexpr int64_t kListedFromWorkgroups = 32768;  // launches of the plain grid from which the list is walked instead
+// ... and from a quarter of that when a partial covers 1024 tokens and more (the fused call's splits): with units that long
+// a skewed batch has few of them, one to a CU at best, and the plain grid's empty workgroups stand in their way (131072 +
+// 63 x 2048 tokens at 2048 per partial, 8192 workgroups: 0.217 -> 0.167 ms; at 1024, 16384 workgroups: 0.207 -> 0.176);
+// batches of one length lose under one percent (64 x 65536 at 1024: 2.777 -> 2.80 ms).  At 256 tokens per partial the
+// list costs an even batch more than that (config 3, 16384 workgroups: 947 -> 962 us) and stays with the larger grids.
+constexpr int64_t kListedFromWorkgroupsCoarse = 8192;
+constexpr int64_t kListedCoarseTokens = 1024;
 constexpr int64_t kCUs = 256;                     // compute units of the MI355X
 template <typename T>
 __global__ __launch_bounds__(kMfmaWaves * 64, 2) void decode_stage1_mfma_listed_kernel(Stage1Params p) {
@@ -1010,7 +1017,7 @@ template <typename T> static int launch_stage1_mfma(const lsattn_decode_stage1_a
   // is empty whenever the batch mixes long and short requests, which the host cannot see.
   // lsattn_set_tuning overrides the choice (tuning and tests).
   const int64_t wgs_total = wgs_x * wgs_y * a->batch;
-  bool listed = wgs_total >= kListedFromWorkgroups;
+  bool listed = wgs_total >= kListedFromWorkgroups || (a->seq_block_size >= kListedCoarseTokens && wgs_total >= kListedFromWorkgroupsCoarse);
   if (tn.decode_listed == LSATTN_DECODE_LISTED_OFF) listed = false;
   if (tn.decode_listed == LSATTN_DECODE_LISTED_ON) listed = true;
   if (listed && a->batch <= kListedMaxBatch && wgs_total <= 0x7fffffff) {
