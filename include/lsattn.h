@@ -252,6 +252,11 @@ int lsattn_decode_stage2(const lsattn_decode_stage2_args* a, void* stream);
  * longserve_token_decode_attention_flash_decoding (FDPY:12-27) back to back on `stream`.  Both argument blocks must name
  * the same mid_o, mid_o_logexpsum, b_seqlen, batch, heads, block count, head_dim, block size and layout of the partials (else
  * LSATTN_ERR_INVALID_ARG); everything else as in the two calls it stands for.
+ * mid_o and mid_o_logexpsum are scratch to this call, as they are to the reference's function (FDPY:12-27 hands neither
+ * out): the call may cut the contexts otherwise than seq_block_size says.  Launches of eight and more requests with
+ * enough tokens deal the blocks of all requests (256 tokens each, or the smallest multiple of that by a power of two
+ * whose rows the buffers hold) in equal shares to the waves, whatever the lengths of the requests are, and leave one
+ * partial per share and request; (o, out_logexpsum) are the same softmax merged from other pieces.
  */
 int lsattn_decode_attention(const lsattn_decode_stage1_args* s1, const lsattn_decode_stage2_args* s2, void* stream);
 
@@ -263,7 +268,9 @@ int lsattn_decode_attention(const lsattn_decode_stage1_args* s1, const lsattn_de
  * mid_o_logexpsum must be NULL in both; num_blocks (= num_seq_blocks) is the number of partial rows the caller would
  * have allocated, and min(num_blocks, ceil(max_len_in_batch / seq_block_size)) * batch * Hq * (D + 1) * 4 bytes must not
  * exceed LSATTN_STATIC_SCRATCH_BYTES (else LSATTN_ERR_WORKSPACE); merge_blocks must be 0 or 1.  Results are those of
- * lsattn_decode_attention bit for bit.  The call allocates and frees nothing.  Each GPU has one such array (held until
+ * lsattn_decode_attention: the same kernels; bit for bit whenever both calls cut the contexts alike, which they do
+ * unless the launch is dealt in equal shares and the array holds fewer rows for the batch than the caller's buffers would
+ * (then the shares are counted in larger blocks and the sums are added in another order).  The call allocates and frees nothing.  Each GPU has one such array (held until
  * the process ends) and every call on that GPU uses it: calls that overlap on one GPU (two streams, two threads) race;
  * calls in stream order on one stream do not.  Nothing needs clearing between calls: stage 2 reads only rows that
  * stage 1 of the same call has written.  The first call on a device looks the array's address up
@@ -515,6 +522,7 @@ int lsattn_bf16_to_f16_rows(const void* src, int64_t src_stride, void* dst, int6
 #define LSATTN_DECODE_STAGE1_SPLIT 3 /* the matrix-pipe kernel, the four waves of a workgroup on one block          */
 #define LSATTN_DECODE_LISTED_OFF 1   /* stage 1's grid sized by the longest request                                */
 #define LSATTN_DECODE_LISTED_ON 2    /* a fixed grid walks the list of units that exist                            */
+#define LSATTN_DECODE_LISTED_SHARES 3 /* lsattn_decode_attention deals the blocks in equal shares whatever the size   */
 typedef struct lsattn_tuning {
   int32_t prefill_rows;
   int32_t prefill_order;

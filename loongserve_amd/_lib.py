@@ -90,7 +90,7 @@ TUNING_VALUES = {
     "prefill_order": {None: 0, "tile": 1, "head": 2},
     "prefill_pack": {None: 0, "off": 1},
     "decode_stage1": {None: 0, "lane": 1, "mfma": 2, "split": 3},
-    "decode_listed": {None: 0, "off": 1, "on": 2},
+    "decode_listed": {None: 0, "off": 1, "on": 2, "shares": 3},
 }
 LSATTN_VERSION = 3  # of include/lsattn.h, which the argument blocks above mirror
 
@@ -182,7 +182,7 @@ def load():
 
 def set_tuning(**choices) -> None:
     """Force launch choices of the library process-wide (lsattn_set_tuning): prefill_rows "128" | "256" | "half",
-    prefill_order "tile" | "head", prefill_pack "off", decode_stage1 "lane" | "mfma" | "split", decode_listed "off" | "on";
+    prefill_order "tile" | "head", prefill_pack "off", decode_stage1 "lane" | "mfma" | "split", decode_listed "off" | "on" | "shares";
     fields not named (or None) go back to the library's own choice, so set_tuning() restores all of them."""
     t = Tuning()
     for name, value in choices.items():

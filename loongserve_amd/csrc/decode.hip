@@ -418,9 +418,13 @@ constexpr int kMfmaStage = kMfmaBatch * (kMfmaKRow + kMfmaVRow);  // LDS bytes p
 // fourth batch of its tokens and merge their partials through LDS: four times the waves of the plain shape, each short.
 // One unit of work of a workgroup: request b, task group bid_t, chunk group bid_c (of n_cgroups in the grid; LISTED: the
 // unit comes from a list of the units that exist, and its chunk group is taken as it is).
-template <typename T, bool WS, bool LISTED>
+// RANGE: the wave's unit is blocks [r_lo, r_hi) of the request instead (r_lo < r_hi <= the request's blocks), computed into
+// one partial, which goes to row r_lo; the rows of the other blocks are left alone (the merge behind it knows which rows
+// hold a partial).
+template <typename T, bool WS, bool LISTED, bool RANGE = false>
 __device__ __forceinline__ void stage1_mfma_unit(const Stage1Params& p, char* lds, const int lane, const int wave, const int64_t b,
-                                                 const unsigned bid_t, const unsigned bid_c, const unsigned n_cgroups) {
+                                                 const unsigned bid_t, const unsigned bid_c, const unsigned n_cgroups,
+                                                 const int64_t r_lo = 0, const int64_t r_hi = 0) {
   const int n = lane & 15, g = lane >> 4;  // query head (column) or 16-byte chunk of a row / token group or row of four
   // The waves of a workgroup: tw of them on neighbouring tasks (KV heads: their rows of a token lie side by side in memory
   // and are then fetched at about the same time), the rest on consecutive chunks of tokens.
@@ -443,8 +447,8 @@ __device__ __forceinline__ void stage1_mfma_unit(const Stage1Params& p, char* ld
   const unsigned n_chunks = n_cgroups * cw;
   const unsigned wave_chunk = bid_c * cw + (WS ? 0 : wave >> (tw == 4 ? 2 : tw == 2 ? 1 : 0));
   const unsigned chunk = LISTED ? wave_chunk : (wave_chunk + (unsigned)b) % n_chunks;  // (rotated by the request, as above)
-  const int64_t blk_begin = (int64_t)chunk * p.blocks_per_wg;  // (WS: one block per workgroup)
-  int64_t blk_end = blk_begin + p.blocks_per_wg;
+  const int64_t blk_begin = RANGE ? r_lo : (int64_t)chunk * p.blocks_per_wg;  // (WS: one block per workgroup)
+  int64_t blk_end = RANGE ? r_hi : blk_begin + p.blocks_per_wg;
   if (blk_end > nblk) blk_end = nblk;
   if (blk_begin >= blk_end) return;  // (WS: the same for the four waves, which meet at a barrier below)
   const int bs = (int)p.block_seq;                    // a multiple of 32 (checked on the host)
@@ -542,9 +546,11 @@ __device__ __forceinline__ void stage1_mfma_unit(const Stage1Params& p, char* ld
 #pragma unroll
       for (int db = 0; db < 8; db++) *(f32x4*)(dst + 16 * db) = oacc[db] * inv;
       if (g == 0) p.mid_lse[row] = (m + __builtin_amdgcn_logf(lt)) * kLn2;
-      // the rows of the blocks merged into this partial (row_mul <= 16: lane group g takes every fourth of them)
-      for (int r = 1 + g; r < p.row_mul; r += 4)
-        if (blk * p.row_mul + r < fine_nblk) p.mid_lse[(blk * p.row_mul + r) * p.blk_rows + b * p.req_rows + qh0 + n] = -INFINITY;
+      if (!RANGE) {
+        // the rows of the blocks merged into this partial (row_mul <= 16: lane group g takes every fourth of them)
+        for (int r = 1 + g; r < p.row_mul; r += 4)
+          if (blk * p.row_mul + r < fine_nblk) p.mid_lse[(blk * p.row_mul + r) * p.blk_rows + b * p.req_rows + qh0 + n] = -INFINITY;
+      }
     }
   };
   // one batch whose rows have arrived in kr / vr
@@ -621,6 +627,10 @@ __device__ __forceinline__ void stage1_mfma_unit(const Stage1Params& p, char* ld
   };
   auto finish_batch = [&](int t0) __attribute__((always_inline)) {
     if (WS) return;  // (the block's partial is merged from the four waves after the loop)
+    if (RANGE) {  // (one partial for the whole range)
+      if (t0 + kMfmaBatch >= t_end) flush(blk_begin);
+      return;
+    }
     if ((t0 + kMfmaBatch - t_begin) % bs == 0 || t0 + kMfmaBatch >= t_end) {
       flush(blk_begin + (t0 - t_begin) / bs);
       reset();
@@ -732,6 +742,8 @@ constexpr int64_t kListedFromWorkgroups = 32768;  // launches of the plain grid 
 constexpr int64_t kListedFromWorkgroupsCoarse = 8192;
 constexpr int64_t kListedCoarseTokens = 1024;
 constexpr int64_t kCUs = 256;                     // compute units of the MI355X
+constexpr int64_t kSharesMinBatch = 8;            // ... and from this many requests on (a few long requests: 4 x 131072 and 1 x 1048576 tokens measured 1 % behind the grids)
+constexpr int64_t kSharesMinBlocks = 4;           // equal shares from this many blocks per worker on (an upper bound from the longest request)
 template <typename T>
 __global__ __launch_bounds__(kMfmaWaves * 64, 2) void decode_stage1_mfma_listed_kernel(Stage1Params p) {
   __shared__ __attribute__((aligned(1024))) char lds[kMfmaWaves * kMfmaStage];
@@ -783,6 +795,76 @@ __global__ __launch_bounds__(kMfmaWaves * 64, 2) void decode_stage1_mfma_listed_
   }
 }
 
+// The plain shape with the work dealt in equal shares (the fused call, whose partials are scratch).  All blocks of all
+// requests, request after request, form one line; the workgroups of a task group cut it into as many contiguous shares
+// as they have waves that walk tokens, and a wave computes its share of every request it touches into ONE partial (row
+// = the share's first block of that request).  Every wave gets the same number of blocks to
+// within one whatever the lengths are, a request long or short costs one partial per share it touches instead of one
+// per block (the partials, written while the gather saturates the memory system, cost eight times their bytes), and no
+// split size has to be guessed from the longest request.  Neighbouring workgroups hold the task groups of the same
+// share (all KV heads of a token are fetched at about the same time).  The merge that follows (decode_stage2_kernel with
+// SHARES) works out the same shares from the lengths and visits the rows that hold a partial, nothing else.
+template <typename T>
+__global__ __launch_bounds__(kMfmaWaves * 64, 2) void decode_stage1_mfma_range_kernel(Stage1Params p) {
+  __shared__ __attribute__((aligned(1024))) char lds[kMfmaWaves * kMfmaStage];
+  __shared__ uint32_t first_block[kListedMaxBatch + 1];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int tw = p.tasks_on_x & 7, cw = kMfmaWaves / tw;
+  const uint32_t task_groups = (uint32_t)((p.tasks + tw - 1) / tw);
+  const int batch = (int)p.batch;  // <= kListedMaxBatch (checked on the host)
+  if (wave == 0) {
+    uint32_t carry = 0;
+    for (int b0 = 0; b0 < batch; b0 += 64) {
+      const int bb = b0 + lane;
+      uint32_t blocks = 0;
+      if (bb < batch) {
+        const int len = p.b_seqlen[bb];
+        int64_t nblk = len <= 0 ? 0 : ((int64_t)len + p.block_seq - 1) / p.block_seq;  // (the same clamps as in the unit)
+        if (nblk > p.grid_blocks) nblk = p.grid_blocks;
+        if (nblk > p.num_blocks) nblk = p.num_blocks;
+        blocks = (uint32_t)nblk;
+      }
+      uint32_t incl = blocks;  // inclusive prefix sum over the 64 lanes
+#pragma unroll
+      for (int d = 1; d < 64; d <<= 1) {
+        const uint32_t up = __shfl_up(incl, d, 64);
+        if (lane >= d) incl += up;
+      }
+      if (bb < batch) first_block[bb] = carry + incl - blocks;
+      carry += __builtin_amdgcn_readlane(incl, 63);
+    }
+    if (lane == 0) first_block[batch] = carry;
+  }
+  __syncthreads();
+  const uint64_t total = first_block[batch];
+  // the wave's share: worker v of V, over the workgroups of its task group and their waves that walk tokens
+  const uint32_t tg = blockIdx.x % task_groups;
+  const uint64_t V = (uint64_t)(gridDim.x / task_groups) * cw;
+  const uint64_t v = (uint64_t)(blockIdx.x / task_groups) * cw + (wave / tw);
+  uint32_t x = (uint32_t)(v * total / V);
+  const uint32_t hi_all = (uint32_t)((v + 1) * total / V);
+  if (x >= hi_all) return;
+  // the request that holds block x: first_block[lo] <= x < first_block[hi] throughout (requests without blocks are skipped)
+  int lo = 0, hi = batch;
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    const uint32_t f = __builtin_amdgcn_readfirstlane(first_block[mid]);
+    if (f <= x) lo = mid;
+    else hi = mid;
+  }
+  int r = lo;
+  while (x < hi_all) {
+    const uint32_t r0 = __builtin_amdgcn_readfirstlane(first_block[r]), r1 = __builtin_amdgcn_readfirstlane(first_block[r + 1]);
+    if (r1 > x) {
+      const uint32_t end = r1 < hi_all ? r1 : hi_all;
+      stage1_mfma_unit<T, false, true, true>(p, lds, lane, wave, r, tg, 0, 0, (int64_t)(x - r0), (int64_t)(end - r0));
+      x = end;
+    }
+    r++;
+  }
+}
+
 // ------------------------------------------------------------------------------------
 // Stage 2: one workgroup per (request, head), the heads of a request next to each other in the grid (a request much
 // longer than the others then has all its workgroups start together, wherever it stands in the batch, instead of its
@@ -797,6 +879,8 @@ struct Stage2Params {
   const float* mid_lse;
   int64_t batch, heads, num_seq_blocks, block_seq;
   int64_t blk_rows, req_rows;  // rows of mid_o between consecutive blocks / requests
+  int64_t grid_blocks;         // (SHARES) stage 1's bound on a request's blocks, from the longest request
+  int64_t shares_workers;      // (SHARES) the shares stage 1 dealt the blocks of all requests in
 };
 
 template <typename OT> __device__ __forceinline__ void store4(void* base, int64_t elem, const f32x4& v);
@@ -810,15 +894,60 @@ template <> __device__ __forceinline__ void store4<BF16>(void* base, int64_t ele
   *(u32x2*)((uint16_t*)base + elem) = u32x2{pack2<BF16>(v[0], v[1]), pack2<BF16>(v[2], v[3])};
 }
 
-template <typename OT, int D, int NT>
+// SHARES: behind decode_stage1_mfma_range_kernel, which dealt the blocks of all requests, request after request, in
+// shares_workers equal shares and left one partial per share and request, at the row of the share's first block of the
+// request.  The workgroup counts the blocks in front of its request and in all (the same clamps as stage 1), lists the
+// shares that begin inside its request, and visits those rows (and row 0, where the share that reaches into the
+// request from the one before it, or begins with it, left its partial).
+template <typename OT, int D, int NT, bool SHARES = false>
 __global__ __launch_bounds__(NT) void decode_stage2_kernel(Stage2Params p) {
   constexpr int LPR = D / 4;      // lanes per row (float4 each)
   constexpr int SL = NT / LPR;    // slices walking the block axis
   const int64_t b = blockIdx.x / (uint32_t)p.heads, h = blockIdx.x % (uint32_t)p.heads;
   const int slice = threadIdx.x / LPR, c = threadIdx.x % LPR;
-  const int64_t len = p.b_seqlen[b];
-  int64_t n = len <= 0 ? 0 : (len + p.block_seq - 1) / p.block_seq;
-  if (n > p.num_seq_blocks) n = p.num_seq_blocks;
+  auto blocks_of = [&](int64_t len) -> int64_t {
+    int64_t nb = len <= 0 ? 0 : (len + p.block_seq - 1) / p.block_seq;
+    if (nb > p.num_seq_blocks) nb = p.num_seq_blocks;
+    if (SHARES && nb > p.grid_blocks) nb = p.grid_blocks;
+    return nb;
+  };
+  int64_t n = blocks_of(p.b_seqlen[b]);
+  // SHARES: entry i of the rows to visit is row 0 for i = 0, else the first block of share v_lo + i - 1 (its distance from
+  // the request's first block); an entry whose share is empty (more shares than blocks) holds nothing
+  uint64_t first = 0, total = 1, v_lo = 0;
+  const uint64_t V = SHARES ? (uint64_t)p.shares_workers : 1;
+  if (SHARES) {
+    uint32_t pre = 0, tot = 0;
+    for (int64_t i = threadIdx.x; i < p.batch; i += NT) {
+      const uint32_t nb = (uint32_t)blocks_of(p.b_seqlen[i]);
+      tot += nb;
+      if (i < b) pre += nb;
+    }
+#pragma unroll
+    for (int d = 32; d > 0; d >>= 1) {
+      pre += __shfl_xor(pre, d, 64);
+      tot += __shfl_xor(tot, d, 64);
+    }
+    __shared__ uint32_t red[2][NT / 64];
+    if ((threadIdx.x & 63) == 0) {
+      red[0][threadIdx.x >> 6] = pre;
+      red[1][threadIdx.x >> 6] = tot;
+    }
+    __syncthreads();
+    pre = tot = 0;
+#pragma unroll
+    for (int w = 0; w < NT / 64; w++) {
+      pre += red[0][w];
+      tot += red[1][w];
+    }
+    first = pre;
+    total = tot > 0 ? tot : 1;
+    if (n > 0) {
+      v_lo = ((first + 1) * V + total - 1) / total;                        // the first share that begins behind block 0 of the request
+      const uint64_t v_end = ((first + (uint64_t)n) * V + total - 1) / total;  // one past the last share that begins inside it
+      n = 1 + (int64_t)(v_end > v_lo ? v_end - v_lo : 0);
+    }
+  }
   const int64_t row_stride = p.blk_rows;
   const int64_t row0 = b * p.req_rows + h;
   const int64_t out_row = b * p.heads + h;
@@ -843,16 +972,25 @@ __global__ __launch_bounds__(NT) void decode_stage2_kernel(Stage2Params p) {
   for (int64_t i = slice; i < n; i += U * SL) {
     float lse[U];
     f32x4 tv[U];
+    bool holds[U];
 #pragma unroll
     for (int u = 0; u < U; u++) {
-      const int64_t blk = i + u * SL < n ? i + u * SL : n - 1;
+      const int64_t e = i + u * SL < n ? i + u * SL : n - 1;
+      int64_t blk = e;
+      holds[u] = i + u * SL < n;
+      if (SHARES && e > 0) {
+        const uint64_t v = v_lo + (uint64_t)e - 1;
+        const uint64_t x = v * total / V;
+        blk = (int64_t)(x - first);
+        holds[u] = holds[u] && (v + 1) * total / V > x;  // (an empty share left nothing)
+      }
       const int64_t row = blk * row_stride + row0;
       lse[u] = p.mid_lse[row];
       tv[u] = *(const f32x4*)(p.mid_o + row * D + c * 4);
     }
 #pragma unroll
     for (int u = 0; u < U; u++)
-      if (i + u * SL < n) fold(lse[u], tv[u]);
+      if (holds[u]) fold(lse[u], tv[u]);
   }
   __shared__ float sM[SL], sL[SL];
   __shared__ f32x4 sAcc[SL][LPR];
@@ -946,7 +1084,8 @@ static int launch_stage1(const lsattn_decode_stage1_args* a, hipStream_t st) {
 
 // Large launches: the matrix-pipe kernel, when its conditions hold (blocks a multiple of 32 tokens, enough waves to fill
 // the chip); lsattn_set_tuning forces the choice where the conditions allow it (tuning, tests).
-template <typename T> static int launch_stage1_mfma(const lsattn_decode_stage1_args* a, hipStream_t st, bool* taken) {
+// `shares`: deal the blocks in equal shares (decode_stage1_mfma_range_kernel) or launch nothing (*taken stays false).
+template <typename T> static int launch_stage1_mfma(const lsattn_decode_stage1_args* a, hipStream_t st, bool* taken, int64_t* shares = nullptr) {
   *taken = false;
   const int group = (int)(a->num_q_heads / a->num_kv_heads);
   Stage1Params p;
@@ -999,6 +1138,24 @@ template <typename T> static int launch_stage1_mfma(const lsattn_decode_stage1_a
   if (tn.decode_stage1 == LSATTN_DECODE_STAGE1_LANE) use = split_waves = false;
   if (tn.decode_stage1 == LSATTN_DECODE_STAGE1_MFMA) use = true, split_waves = false;
   if (tn.decode_stage1 == LSATTN_DECODE_STAGE1_SPLIT && can_split) use = false, split_waves = true;
+  if (shares) {
+    // only where the plain shape would run, on launches with at least kSharesMinBlocks blocks of 256 tokens and more per
+    // worker to deal (fewer: the grids above, whose workgroups the hardware hands out as they finish)
+    const int tws = p.tasks >= 4 ? 4 : p.tasks >= 2 ? 2 : 1;
+    const int64_t task_groups = (p.tasks + tws - 1) / tws;
+    int64_t per_group = 2 * kCUs / task_groups;  // workgroups per task group: two workgroups per CU in all
+    const bool forced = tn.decode_listed == LSATTN_DECODE_LISTED_SHARES;  // (tests: whatever the launch's size)
+    if (tn.decode_listed == LSATTN_DECODE_LISTED_OFF || tn.decode_listed == LSATTN_DECODE_LISTED_ON) return LSATTN_OK;
+    if (per_group < 1 || p.row_mul != 1 || a->batch > kListedMaxBatch || nblk * a->batch > 0x7fffffff) return LSATTN_OK;
+    const int64_t workers = per_group * (kMfmaWaves / tws);
+    if (!forced && (!use || split_waves || a->seq_block_size < 256 || a->batch < kSharesMinBatch || nblk * a->batch < kSharesMinBlocks * workers)) return LSATTN_OK;
+    *taken = true;
+    *shares = workers;
+    p.tasks_on_x = tws;
+    p.blocks_per_wg = 1;
+    hipLaunchKernelGGL((decode_stage1_mfma_range_kernel<T>), dim3((unsigned)(per_group * task_groups)), dim3(kMfmaWaves * 64), 0, st, p);
+    return check_launch();
+  }
   if (split_waves) {
     *taken = true;
     p.blocks_per_wg = 1;
@@ -1031,8 +1188,12 @@ template <typename T> static int launch_stage1_mfma(const lsattn_decode_stage1_a
   return check_launch();
 }
 
-template <typename T> static int dispatch_stage1(const lsattn_decode_stage1_args* a, hipStream_t st) {
+template <typename T> static int dispatch_stage1(const lsattn_decode_stage1_args* a, hipStream_t st, int64_t* shares = nullptr) {
   const int group = (int)(a->num_q_heads / a->num_kv_heads);
+  if (shares) {  // (in equal shares or not at all: *shares is their number, or stays 0)
+    bool taken;
+    return launch_stage1_mfma<T>(a, st, &taken, shares);
+  }
   {
     bool taken;
     const int rc = launch_stage1_mfma<T>(a, st, &taken);
@@ -1051,7 +1212,9 @@ template <typename T> static int dispatch_stage1(const lsattn_decode_stage1_args
 
 using namespace lsattn;
 
-extern "C" int lsattn_decode_stage1(const lsattn_decode_stage1_args* a, void* stream) {
+// `shares` (the fused call): launch stage 1 in equal shares if the launch is one for them (*shares: how many) or nothing.
+static int decode_stage1(const lsattn_decode_stage1_args* a, void* stream, int64_t* shares) {
+  if (shares) *shares = 0;
   if (!a || !a->mid_o || !a->mid_o_logexpsum || !a->q || !a->k || !a->v || !a->req_to_tokens || !a->b_req_idx ||
       !a->b_seqlen)
     return LSATTN_ERR_INVALID_ARG;
@@ -1067,14 +1230,24 @@ extern "C" int lsattn_decode_stage1(const lsattn_decode_stage1_args* a, void* st
   if (a->head_dim != 128) return LSATTN_ERR_UNSUPPORTED;  // as flash_decoding_stage1.cu:210
   if (a->batch == 0 || a->num_blocks == 0 || a->max_len_in_batch == 0) return LSATTN_OK;
   hipStream_t st = (hipStream_t)stream;
-  if (a->dtype == LSATTN_F16) return dispatch_stage1<F16>(a, st);
-  if (a->dtype == LSATTN_BF16) return dispatch_stage1<BF16>(a, st);
+  if (a->dtype == LSATTN_F16) return dispatch_stage1<F16>(a, st, shares);
+  if (a->dtype == LSATTN_BF16) return dispatch_stage1<BF16>(a, st, shares);
   return LSATTN_ERR_UNSUPPORTED;
 }
+
+extern "C" int lsattn_decode_stage1(const lsattn_decode_stage1_args* a, void* stream) { return decode_stage1(a, stream, nullptr); }
 
 // `live_blocks`: an upper bound of the partial rows any request has (the rows of the buffer, or fewer when the caller
 // knows the longest request); it picks the shape of the merge, which decides the order of its additions.
 template <typename OT> static int dispatch_stage2(const Stage2Params& p, int64_t D, dim3 grid, int64_t live_blocks, hipStream_t st) {
+  if (p.shares_workers > 0) {
+    if (D != 128) return LSATTN_ERR_UNSUPPORTED;
+    // (a request's partials: at most one per share and one more, and no more than it has blocks)
+    const int64_t most = live_blocks < p.shares_workers + 1 ? live_blocks : p.shares_workers + 1;
+    if (most >= 64 && (int64_t)grid.x < 2048) hipLaunchKernelGGL((decode_stage2_kernel<OT, 128, 1024, true>), grid, dim3(1024), 0, st, p);
+    else hipLaunchKernelGGL((decode_stage2_kernel<OT, 128, 256, true>), grid, dim3(256), 0, st, p);
+    return check_launch();
+  }
   // few (batch, head) pairs with many partials each (long contexts at small batch): 1024 threads walk the block axis in 32
   // slices instead of 8, or the merge takes a fifth of the time of the gather it follows
   const bool wide = D == 128 && live_blocks >= 64 && ((int64_t)grid.x < 2048 || (live_blocks >= 1024 && (int64_t)grid.x < 8192));
@@ -1090,7 +1263,7 @@ template <typename OT> static int dispatch_stage2(const Stage2Params& p, int64_t
   return check_launch();
 }
 
-static int decode_stage2(const lsattn_decode_stage2_args* a, int64_t live_blocks, void* stream) {
+static int decode_stage2(const lsattn_decode_stage2_args* a, int64_t live_blocks, void* stream, int64_t shares_workers = 0, int64_t grid_blocks = 0) {
   if (!a || !a->o || !a->out_logexpsum || !a->b_seqlen || !a->mid_o || !a->mid_o_logexpsum) return LSATTN_ERR_INVALID_ARG;
   if (a->batch < 0 || a->num_heads <= 0 || a->num_seq_blocks < 0 || a->block_seq < 1) return LSATTN_ERR_INVALID_ARG;
   if (((uintptr_t)a->o | (uintptr_t)a->mid_o) & 15) return LSATTN_ERR_INVALID_ARG;
@@ -1100,7 +1273,7 @@ static int decode_stage2(const lsattn_decode_stage2_args* a, int64_t live_blocks
   Stage2Params p{a->o, a->out_logexpsum, a->b_seqlen, a->mid_o, a->mid_o_logexpsum,
                  a->batch, a->num_heads, a->num_seq_blocks, a->block_seq,
                  a->partials_by_request ? a->num_heads : a->batch * a->num_heads,
-                 a->partials_by_request ? a->num_seq_blocks * a->num_heads : a->num_heads};
+                 a->partials_by_request ? a->num_seq_blocks * a->num_heads : a->num_heads, grid_blocks, shares_workers};
   dim3 grid((unsigned)(a->batch * a->num_heads));
   hipStream_t st = (hipStream_t)stream;
   switch (a->o_dtype) {
@@ -1122,6 +1295,25 @@ extern "C" int lsattn_decode_attention(const lsattn_decode_stage1_args* s1, cons
       s1->batch != s2->batch || s1->num_q_heads != s2->num_heads || s1->num_blocks != s2->num_seq_blocks ||
       s1->head_dim != s2->head_dim || s1->seq_block_size != s2->block_seq || !s1->partials_by_request != !s2->partials_by_request)
     return LSATTN_ERR_INVALID_ARG;
+  // Large launches deal the tokens in equal shares (decode_stage1_mfma_range_kernel), however coarse the split asked
+  // for: the partials are scratch here, and a share leaves one partial per request it touches whatever the block size.
+  // The blocks the shares are counted in: 256 tokens, or the smallest multiple by a power of two whose rows the buffers hold
+  // (a share's partial goes to the row of its first block).
+  if (s1->merge_blocks <= 1 && s1->seq_block_size >= 256 && s1->max_len_in_batch > 0 && s1->num_blocks > 0) {
+    int64_t g = 256;
+    while ((s1->max_len_in_batch + g - 1) / g > s1->num_blocks) g *= 2;
+    lsattn_decode_stage1_args a1 = *s1;
+    a1.seq_block_size = g;
+    int64_t shares = 0;
+    const int rc1 = decode_stage1(&a1, stream, &shares);
+    if (rc1 != LSATTN_OK) return rc1;
+    if (shares > 0) {
+      lsattn_decode_stage2_args a2 = *s2;
+      a2.block_seq = g;
+      const int64_t rows = (s1->max_len_in_batch + g - 1) / g;
+      return decode_stage2(&a2, rows, stream, shares, rows);
+    }
+  }
   const int rc = lsattn_decode_stage1(s1, stream);
   if (rc != LSATTN_OK) return rc;
   // the merge's shape from the rows the longest request can reach, not from the rows the buffer happens to have: the
@@ -1177,8 +1369,14 @@ extern "C" int lsattn_decode_attention_static(const lsattn_decode_stage1_args* s
   if (rows > s1->num_blocks) rows = s1->num_blocks;
   const int64_t per_row = s1->batch * s1->num_q_heads;  // (request, head) pairs per block row
   if (per_row > 0 && rows > (int64_t)LSATTN_STATIC_SCRATCH_BYTES / 4 / 129 / per_row) return LSATTN_ERR_WORKSPACE;
+  if ((uint64_t)(rows * per_row * 129) * 4 > (uint64_t)LSATTN_STATIC_SCRATCH_BYTES) return LSATTN_ERR_WORKSPACE;
+  // The array is laid out for as many rows as it holds for this batch, up to one per 256 tokens of the longest request:
+  // the fused call below counts its equal shares in the smallest blocks whose rows it is given.
+  int64_t rows_laid = (s1->max_len_in_batch + 255) / 256;
+  if (per_row > 0 && rows_laid > (int64_t)LSATTN_STATIC_SCRATCH_BYTES / 4 / 129 / per_row) rows_laid = (int64_t)LSATTN_STATIC_SCRATCH_BYTES / 4 / 129 / per_row;
+  if (rows_laid < rows) rows_laid = rows;
+  rows = rows_laid;
   const int64_t o_floats = rows * per_row * 128;         // a multiple of 128 floats: the LSE part stays 16-byte aligned
-  if ((uint64_t)(o_floats + rows * per_row) * 4 > (uint64_t)LSATTN_STATIC_SCRATCH_BYTES) return LSATTN_ERR_WORKSPACE;
   float* base = (float*)scratch_on_current_device();
   if (!base) return LSATTN_ERR_LAUNCH;
   lsattn_decode_stage1_args a1 = *s1;

@@ -519,7 +519,7 @@ extern "C" int lsattn_set_tuning(const lsattn_tuning* t) {
   if (!t) t = &z;
   if (t->prefill_rows < 0 || t->prefill_rows > LSATTN_PREFILL_ROWS_HALF || t->prefill_order < 0 || t->prefill_order > LSATTN_PREFILL_ORDER_HEAD ||
       t->prefill_pack < 0 || t->prefill_pack > LSATTN_PREFILL_PACK_OFF || t->decode_stage1 < 0 || t->decode_stage1 > LSATTN_DECODE_STAGE1_SPLIT ||
-      t->decode_listed < 0 || t->decode_listed > LSATTN_DECODE_LISTED_ON || t->reserved[0] || t->reserved[1] || t->reserved[2])
+      t->decode_listed < 0 || t->decode_listed > LSATTN_DECODE_LISTED_SHARES || t->reserved[0] || t->reserved[1] || t->reserved[2])
     return LSATTN_ERR_INVALID_ARG;
   const int32_t v[5] = {t->prefill_rows, t->prefill_order, t->prefill_pack, t->decode_stage1, t->decode_listed};
   for (int i = 0; i < 5; i++) lsattn::g_tuning[i].store(v[i], std::memory_order_relaxed);

@@ -41,6 +41,8 @@ def longserve_flash_decode_stage2(mid_out, mid_out_logexpsum, B_Seqlen, O, out_l
 # cut more coarsely than BLOCK_SEQ: fewer fp32 block partials are written while the gather saturates the memory system
 # (every MB of them costs about as much as 8 MB of reads).  The result is the same softmax, merged from fewer pieces.
 # longserve_flash_decode_stage1 / _stage2 called on their own always split at the block_seq they are given.
+# (Launches of eight and more requests with enough tokens do not use the split at all: lsattn_decode_attention deals their
+# blocks in equal shares to the waves, one partial per share and request.  The split below is what smaller launches get.)
 FUSED_SPLIT_TOKENS = 1024
 # Do not coarsen below this many (upper-bound estimate of) stage-1 workgroups: one per CU.  Measured on 131072 tokens in
 # all (1 x 131072 ... 16 x 8192, 8 KV heads): 92-95 us at 256 workgroups of 1024 tokens against 100-104 us at 1024 of 256.

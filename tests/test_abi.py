@@ -191,14 +191,14 @@ def test_tuning_block_is_validated_and_named_values_match_the_header():
             ("prefill_order", "head"): "LSATTN_PREFILL_ORDER_HEAD", ("prefill_pack", "off"): "LSATTN_PREFILL_PACK_OFF",
             ("decode_stage1", "lane"): "LSATTN_DECODE_STAGE1_LANE", ("decode_stage1", "mfma"): "LSATTN_DECODE_STAGE1_MFMA",
             ("decode_stage1", "split"): "LSATTN_DECODE_STAGE1_SPLIT", ("decode_listed", "off"): "LSATTN_DECODE_LISTED_OFF",
-            ("decode_listed", "on"): "LSATTN_DECODE_LISTED_ON"}
+            ("decode_listed", "on"): "LSATTN_DECODE_LISTED_ON", ("decode_listed", "shares"): "LSATTN_DECODE_LISTED_SHARES"}
     assert len(num) == len(want)
     for (field, name), macro in want.items():
         assert _lib.TUNING_VALUES[field][name] == num[macro]
         assert _lib.TUNING_VALUES[field][None] == 0
     try:
         t = _lib.Tuning()
-        for field, top in (("prefill_rows", 3), ("prefill_order", 2), ("prefill_pack", 1), ("decode_stage1", 3), ("decode_listed", 2)):
+        for field, top in (("prefill_rows", 3), ("prefill_order", 2), ("prefill_pack", 1), ("decode_stage1", 3), ("decode_listed", 3)):
             for bad in (-1, top + 1):
                 t = _lib.Tuning()
                 setattr(t, field, bad)

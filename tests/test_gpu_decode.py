@@ -471,6 +471,91 @@ def test_one_request_of_a_million_tokens(lsa):
     assert_o_close(o2[0], o_ref.cpu(), "peaked o")
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("Hq,Hkv,BS,lens", [
+    (32, 8, 256, [5000, 1, 256, 257, 0, 9000, 300]),          # two task groups of four KV heads
+    (8, 1, 256, [3000, 700, 12000, 256]),                     # one KV head: the four waves of a workgroup hold four shares
+    (16, 2, 512, [100, 5000, 2049, 17, 1024, 1, 999]),        # two KV heads: two waves on tasks, two shares per workgroup
+    (40, 5, 256, [4097, 130, 0, 0, 6000]),                    # five KV heads: the second task group half empty
+    (17, 1, 1024, [40000, 3, 2048]),                          # a second task with one live row; a split of 1024 dealt in blocks of 256
+])
+def test_fused_call_in_equal_shares(lsa, tuning, dtype, Hq, Hkv, BS, lens):
+    """The fused call with stage 1 dealt in equal shares of blocks (forced: these launches are far smaller than the ones
+    the library deals that way by itself): shares that end inside a request, requests inside a share, requests without
+    tokens, more workers than blocks; the partials' buffers start as NaN (every row the merge reads must have been
+    written, as a partial or as an empty row) and are as tall as the caller's BLOCK_SEQ of 256 makes them."""
+    tuning(decode_listed="shares")
+    B, D = len(lens), 128
+    q, kv, table, b_req, b_len = decode_case(500 + Hq + len(lens), B, Hq, Hkv, D, lens, sum(lens) + 500, dtype)
+    o_ref, l_ref = orc.decode_full(q, kv[:, :Hkv], kv[:, Hkv:], table, b_req, b_len)
+    kvd = kv.to(DEV)
+    nblk = (max(lens) + 255) // 256
+    mo_d = torch.full((nblk, B, Hq, D), float("nan"), device=DEV)
+    ml_d = torch.full((nblk, B, Hq), float("nan"), device=DEV)
+    o_d = torch.full((B, Hq, D), float("nan"), device=DEV)
+    l_d = torch.full((B, Hq), float("nan"), device=DEV)
+    lsa.longserve_cuda_kernels.flash_decoding(mo_d, ml_d, q.to(DEV), kvd[:, :Hkv], kvd[:, Hkv:], table.to(DEV), b_req.to(DEV), b_len.to(DEV),
+                                              max(lens), o_d, l_d, BS)
+    torch.cuda.synchronize()
+    assert_o_close(o_d, o_ref, "o")
+    assert_lse_close(l_d, l_ref, "lse")
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_large_batch_that_is_dealt_in_equal_shares_by_itself(lsa, dtype):
+    """48 requests of 1 to 9000 tokens, 32 query heads on 8 KV heads: 48 x 36 blocks of 256 tokens at most, enough for the
+    library to deal them in equal shares by itself (nothing forced) in the fused call; the two stages on their own keep
+    one partial per block."""
+    lsa.set_tuning()
+    import random
+    rng = random.Random(17)
+    B, Hq, Hkv, D, BS = 48, 32, 8, 128, 256
+    lens = [rng.randint(1, 9000) for _ in range(B)]
+    lens[5] = 9000
+    lens[6] = 0
+    q, kv, table, b_req, b_len = decode_case(79, B, Hq, Hkv, D, lens, sum(lens) + 1000, dtype)
+    o_ref, l_ref = orc.decode_full(q, kv[:, :Hkv], kv[:, Hkv:], table, b_req, b_len)
+    kvd = kv.to(DEV)
+    nblk = (max(lens) + BS - 1) // BS
+    mo_d = torch.full((nblk, B, Hq, D), float("nan"), device=DEV)
+    ml_d = torch.full((nblk, B, Hq), float("nan"), device=DEV)
+    o_d = torch.empty(B, Hq, D, device=DEV)
+    l_d = torch.empty(B, Hq, device=DEV)
+    lsa.longserve_token_decode_attention_flash_decoding(q.to(DEV), table.to(DEV), b_req.to(DEV), b_len.to(DEV), mo_d, ml_d, B, max(lens),
+                                                        Hq, D, kvd[:, :Hkv], kvd[:, Hkv:], BS, o_d, l_d)
+    torch.cuda.synchronize()
+    assert_o_close(o_d, o_ref, "o, fused call")
+    assert_lse_close(l_d, l_ref, "lse, fused call")
+    # (in equal shares a request has far fewer partials than blocks: most rows of the buffer are never written)
+    ml = ml_d.cpu()
+    assert int(torch.isnan(ml).sum()) > int(torch.isfinite(ml).sum()) > 0
+    # the entry point that brings its own partials takes the same route (its array holds a row per 256 tokens here)
+    o_s = torch.full((B, Hq, D), float("nan"), device=DEV)
+    l_s = torch.full((B, Hq), float("nan"), device=DEV)
+    lsa.longserve_cuda_kernels.flash_decoding_static(q.to(DEV), kvd[:, :Hkv], kvd[:, Hkv:], table.to(DEV), b_req.to(DEV), b_len.to(DEV),
+                                                     max(lens), o_s, l_s, 1024)
+    torch.cuda.synchronize()
+    assert torch.equal(o_s, o_d) and torch.equal(l_s, l_d)
+    # recorded in a HIP graph and replayed on new queries: every replay against the eager call
+    qd = q.to(DEV).clone()
+    td, rd, ld = table.to(DEV), b_req.to(DEV), b_len.to(DEV)
+    o_g = torch.empty(B, Hq, D, device=DEV)
+    l_g = torch.empty(B, Hq, device=DEV)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        lsa.longserve_token_decode_attention_flash_decoding(qd, td, rd, ld, mo_d, ml_d, B, max(lens), Hq, D, kvd[:, :Hkv], kvd[:, Hkv:], BS, o_g, l_g)
+    for rep in range(3):
+        qd.copy_((torch.randn(q.shape, generator=torch.Generator().manual_seed(900 + rep)) * 0.5).to(dtype))
+        o_g.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        o_e = torch.empty(B, Hq, D, device=DEV)
+        l_e = torch.empty(B, Hq, device=DEV)
+        lsa.longserve_token_decode_attention_flash_decoding(qd, td, rd, ld, mo_d, ml_d, B, max(lens), Hq, D, kvd[:, :Hkv], kvd[:, Hkv:], BS, o_e, l_e)
+        torch.cuda.synchronize()
+        assert torch.equal(o_g, o_e) and torch.equal(l_g, l_e), "replay %d" % rep
+
+
 @pytest.mark.parametrize("seed", [3, 11, 42])
 def test_random_decode_shapes_on_both_stage1_kernels(lsa, tuning, seed):
     """Seeded random sweep of stage 1 + stage 2 against the oracle, once with the library's own choice of stage-1 kernel
