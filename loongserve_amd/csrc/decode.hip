@@ -881,6 +881,7 @@ struct Stage2Params {
   int64_t blk_rows, req_rows;  // rows of mid_o between consecutive blocks / requests
   int64_t grid_blocks;         // (SHARES) stage 1's bound on a request's blocks, from the longest request
   int64_t shares_workers;      // (SHARES) the shares stage 1 dealt the blocks of all requests in
+  uint32_t workers_mul, workers_shr;  // (SHARES) n / shares_workers = umulhi(n, mul) >> shr for n < 2^31 (mul = 0: shares_workers = 1)
 };
 
 template <typename OT> __device__ __forceinline__ void store4(void* base, int64_t elem, const f32x4& v);
@@ -916,6 +917,12 @@ __global__ __launch_bounds__(NT) void decode_stage2_kernel(Stage2Params p) {
   // the request's first block); an entry whose share is empty (more shares than blocks) holds nothing
   uint64_t first = 0, total = 1, v_lo = 0;
   const uint64_t V = SHARES ? (uint64_t)p.shares_workers : 1;
+  uint64_t per_share = 0;  // total / V ...
+  uint32_t rest = 0;       // ... and total % V: share v begins at block v * per_share + v * rest / V (v * rest < V * V: 32 bits)
+  auto share_begin = [&](uint64_t v) -> uint64_t {
+    const uint32_t t = (uint32_t)v * rest;
+    return v * per_share + (p.workers_mul ? __umulhi(t, p.workers_mul) >> p.workers_shr : t);
+  };
   if (SHARES) {
     uint32_t pre = 0, tot = 0;
     for (int64_t i = threadIdx.x; i < p.batch; i += NT) {
@@ -942,6 +949,8 @@ __global__ __launch_bounds__(NT) void decode_stage2_kernel(Stage2Params p) {
     }
     first = pre;
     total = tot > 0 ? tot : 1;
+    per_share = total / V;
+    rest = (uint32_t)(total - per_share * V);
     if (n > 0) {
       v_lo = ((first + 1) * V + total - 1) / total;                        // the first share that begins behind block 0 of the request
       const uint64_t v_end = ((first + (uint64_t)n) * V + total - 1) / total;  // one past the last share that begins inside it
@@ -980,9 +989,9 @@ __global__ __launch_bounds__(NT) void decode_stage2_kernel(Stage2Params p) {
       holds[u] = i + u * SL < n;
       if (SHARES && e > 0) {
         const uint64_t v = v_lo + (uint64_t)e - 1;
-        const uint64_t x = v * total / V;
+        const uint64_t x = share_begin(v);
         blk = (int64_t)(x - first);
-        holds[u] = holds[u] && (v + 1) * total / V > x;  // (an empty share left nothing)
+        holds[u] = holds[u] && share_begin(v + 1) > x;  // (an empty share left nothing)
       }
       const int64_t row = blk * row_stride + row0;
       lse[u] = p.mid_lse[row];
@@ -1273,7 +1282,13 @@ static int decode_stage2(const lsattn_decode_stage2_args* a, int64_t live_blocks
   Stage2Params p{a->o, a->out_logexpsum, a->b_seqlen, a->mid_o, a->mid_o_logexpsum,
                  a->batch, a->num_heads, a->num_seq_blocks, a->block_seq,
                  a->partials_by_request ? a->num_heads : a->batch * a->num_heads,
-                 a->partials_by_request ? a->num_seq_blocks * a->num_heads : a->num_heads, grid_blocks, shares_workers};
+                 a->partials_by_request ? a->num_seq_blocks * a->num_heads : a->num_heads, grid_blocks, shares_workers, 0, 0};
+  if (shares_workers > 1) {  // (shares_workers <= 2048: v * rest stays far below 2^31)
+    uint32_t L = 0;
+    while ((1u << L) < (uint32_t)shares_workers) L++;
+    p.workers_mul = (uint32_t)((((uint64_t)1 << (31 + L)) + shares_workers - 1) / shares_workers);
+    p.workers_shr = L - 1;
+  }
   dim3 grid((unsigned)(a->batch * a->num_heads));
   hipStream_t st = (hipStream_t)stream;
   switch (a->o_dtype) {
