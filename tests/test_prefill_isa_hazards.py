@@ -391,8 +391,9 @@ _ZN6lsattn4demoEv:
 @pytest.mark.skipif(shutil.which(HIPCC) is None, reason="hipcc not available")
 def test_decode_matrix_pipe_kernel_touches_no_register_of_a_load_in_flight():
     res = loads_in_flight_violations(_decode_asm(), "decode_stage1_mfma_")
-    # fp16 and bf16: plain, with the waves of a workgroup splitting a block, and the plain shape over a list of units
-    assert len(res) == 6 and sum("listed" in name for name in res) == 2, list(res)
+    # fp16 and bf16: plain, with the waves of a workgroup splitting a block, the plain shape over a list of units, and the
+    # plain shape over every wave's equal share of the blocks
+    assert len(res) == 8 and sum("listed" in name for name in res) == 2 and sum("range" in name for name in res) == 2, list(res)
     for name, (n, bad) in res.items():
         assert n >= 3 * 8 + 3 * 16, (name, n)             # slot and row loads of the prologue and of both halves of the loop
         assert not bad, name + "\n" + "\n".join(bad[:20])
