@@ -131,6 +131,10 @@ class Ceiling:
         self.lib.ls_ceiling_mfma_f16_flop.argtypes = [ctypes.c_int, ctypes.c_int]
         self.lib.ls_ceiling_read.restype = ctypes.c_int
         self.lib.ls_ceiling_read.argtypes = [vp, ctypes.c_uint64, vp, vp]
+        self.lib.ls_ceiling_read_with_stores.restype = ctypes.c_int
+        self.lib.ls_ceiling_read_with_stores.argtypes = [vp, ctypes.c_uint64, vp, ctypes.c_uint32, ctypes.c_int, vp, vp]
+        self.lib.ls_ceiling_read_with_stores_bytes.restype = ctypes.c_uint64
+        self.lib.ls_ceiling_read_with_stores_bytes.argtypes = [ctypes.c_uint64, ctypes.c_uint32]
 
     def mfma_tflops(self, iters=60000, workgroups=256, launches=24, warm=8):
         """A stream of v_mfma_f32_16x16x32_f16 on random fp16 operands, one wave per SIMD, nothing else; launches of
@@ -162,6 +166,27 @@ class Ceiling:
         del src
         torch.cuda.empty_cache()
         return nbytes / (med * 1e-3) / 1e9, med
+
+
+    def read_with_stores_gbs(self, every=64, nbytes=4 << 30, launches=20, warm=5):
+        """The same read with 8 KB stores mixed into one of every `every` trips of a wave (64: 1.6 % of the bytes, what one
+        fp32 partial per 256 tokens is to config 3's gather): GB/s of the read with ordinary stores and with stores that
+        are written through to memory as they are issued (what the decode kernel's partials use)."""
+        src = torch.empty(nbytes, dtype=torch.uint8, device=DEV)
+        src.view(torch.int32).random_(0, 1 << 30)
+        dst = torch.empty(int(self.lib.ls_ceiling_read_with_stores_bytes(nbytes, every)), dtype=torch.uint8, device=DEV)
+        sink = torch.zeros(256, dtype=torch.int32, device=DEV)
+        st = torch.cuda.current_stream().cuda_stream
+        out = []
+        for system_scope in (0, 1):
+            def call():
+                if self.lib.ls_ceiling_read_with_stores(src.data_ptr(), nbytes, dst.data_ptr(), every, system_scope, sink.data_ptr(), st) != 0:
+                    raise RuntimeError("ls_ceiling_read_with_stores failed")
+            ms = _time_events(call, launches, warm)
+            out.append(nbytes / (sorted(ms)[len(ms) // 2] * 1e-3) / 1e9)
+        del src, dst
+        torch.cuda.empty_cache()
+        return out[0], out[1], 1.0 / every
 
 
 def _roof(kernel, bound, achieved, per_launch_ms, traffic_key, **extra):
@@ -957,6 +982,7 @@ def main():
         sep = _stats(_time_events(d.step_separate_stages, 50, 10))
         sepm = _stats(_time_events(d.step_separate_stages_merged, 30, 5))
         read_peak, _ = ceil.read_gbs()
+        read_stores_plain, read_stores_through, _ = ceil.read_with_stores_gbs(64)
         gbs = d.bytes / (st["median_ms"] * 1e-3) / 1e9
         # The fused call is two launches from one library call, timed together (HIP events around the call): stage 1 in equal
         # shares (decode_stage1_mfma_range_kernel, all but a few microseconds of it) and the merge of the shares' partials.
@@ -968,13 +994,17 @@ def main():
                  "decode_achieved_gbs": ach, "decode_frac": ach / PEAK_HBM_GBS,
                  "decode_per_launch_ms": st["median_ms"], "decode_traffic": TRAFFIC_BYTES["config3"], "decode_algorithmic_gb": d.bytes / 1e9,
                  "decode_sustained_peak_gbs": read_peak, "decode_frac_of_sustained": ach / read_peak,
-                 "decode_plain_grid_stage1_ms": s1["median_ms"], "decode_plain_grid_stage1_frac": plain / PEAK_HBM_GBS}
+                 "decode_plain_grid_stage1_ms": s1["median_ms"], "decode_plain_grid_stage1_frac": plain / PEAK_HBM_GBS,
+                 # the streaming read of the ceiling library with 1.6 % of stores mixed in (the share of one fp32 partial per
+                 # 256 tokens in this gather): ordinary stores / stores written through as they are issued (the kernel's)
+                 "decode_read_with_partial_stores_gbs": read_stores_plain, "decode_read_with_partial_stores_written_through_gbs": read_stores_through}
         summary["config3"] = {"value": _r(gbs, 1), "unit": "GB/s", "frac": _r(gbs / PEAK_HBM_GBS), "ms": _r(st["median_ms"]),
                               "p10_ms": _r(st["p10_ms"]), "p90_ms": _r(st["p90_ms"]), "kernel": "decode_stage1_mfma_range_kernel<F16> + decode_stage2_kernel",
                               "frac_of_sustained": _r(gbs / read_peak), "plain_grid_stage1_frac": _r(plain / PEAK_HBM_GBS),
                               "two_stages_reference_buffers_ms": _r(sep["median_ms"]),
                               "two_stages_reference_buffers_frac": _r(d.bytes / (sep["median_ms"] * 1e-3) / 1e9 / PEAK_HBM_GBS),
                               "two_stages_merged_blocks_frac": _r(d.bytes / (sepm["median_ms"] * 1e-3) / 1e9 / PEAK_HBM_GBS),
+                              "two_stages_frac_of_read_with_as_many_stores": _r(d.bytes / (sep["median_ms"] * 1e-3) / 1e9 / read_stores_through),
                               "workload": "config 3: batch 64, ctx U[4096,32768], GQA 32/8, fp16, 2.5M-slot scattered pool; fused call, BLOCK_SEQ %d, "
                                           "stage 1 in equal shares of 256-token blocks" % d.BS}
         if only == "decode":
@@ -1011,7 +1041,9 @@ def main():
         mfma_peak, mfma_ms = ceil.mfma_tflops()
         read_peak, read_ms = ceil.read_gbs()
         line.update({"value": mfma_peak, "unit": "TFLOP/s", "ms_per_step": mfma_ms, "config": {"workload": "ceilings: MFMA stream, 4 GiB read"}})
-        summary["ceiling"] = {"mfma_tflops": _r(mfma_peak, 1), "mfma_ms": _r(mfma_ms), "read_gbs": _r(read_peak, 1), "read_ms": _r(read_ms)}
+        summary["ceiling"] = {"mfma_tflops": _r(mfma_peak, 1), "mfma_ms": _r(mfma_ms), "read_gbs": _r(read_peak, 1), "read_ms": _r(read_ms),
+                              "read_with_stores_gbs": {"%.2f %% of the bytes stored" % (100.0 / e): dict(zip(("plain", "written_through"), (_r(a, 1), _r(b, 1))))
+                                                       for e in (1024, 256, 64, 16) for a, b, _ in (ceil.read_with_stores_gbs(e),)}}
     if only == "chunked":
         summary["chunked_prefill_step"] = c = chunked_prefill_step()
         line.update({"value": c["kv_gbs_workspace_route"], "unit": "GB/s", "ms_per_step": c["context_attention_fwd_workspace_us"] * 1e-3,
@@ -1026,7 +1058,9 @@ def main():
                 "two_stages_ms": _r(c["chosen"]["two_stages_ms"]), "two_stages_frac": _r(c["chosen"]["two_stages_gbs"] / PEAK_HBM_GBS),
                 "fused_ms": _r(c["chosen"]["fused_ms"]), "fused_frac": _r(c["chosen"]["fused_gbs"] / PEAK_HBM_GBS)}
             for c in decode_mixed_lengths(full=False)["cases"]}
-        summary["ceiling"] = {"mfma_tflops": _r(roof.get("sustained_peak"), 1), "read_gbs": _r(roof.get("decode_sustained_peak_gbs"), 1)}
+        summary["ceiling"] = {"mfma_tflops": _r(roof.get("sustained_peak"), 1), "read_gbs": _r(roof.get("decode_sustained_peak_gbs"), 1),
+                              "read_with_1.6pct_stores_gbs": [_r(roof.get("decode_read_with_partial_stores_gbs"), 1),
+                                                             _r(roof.get("decode_read_with_partial_stores_written_through_gbs"), 1)]}
     if args.sweeps:
         details["prefill_launch_sizes"] = prefill_launch_sizes(tile_us)
         details["decode_latency"] = decode_latency()

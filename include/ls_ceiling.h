@@ -24,6 +24,15 @@ double ls_ceiling_mfma_f16_flop(int iters, int workgroups);
  * 4096 workgroups of 256 lanes.  sink: 1024 bytes (practically never written). */
 int ls_ceiling_read(const void* src, uint64_t bytes, void* sink, void* stream);
 
+/* The same read with stores mixed in (what the partials of a split-K decode do to its gather): in one of every `every`
+ * trips of a wave's loop over 8 KB of reads, spread evenly over the waves and the launch, the wave also writes 8 KB to
+ * dst (sixteen rows of 512 bytes, a store instruction a 64-byte piece of each).  every = 64: 1.6 % of the bytes, the
+ * share of one fp32 partial per 256 tokens and 32 query heads on 8 KV heads.  system_scope != 0: the stores are written
+ * through to memory as they are issued (sc0 sc1) instead of being written back from the L2 later.
+ * dst: ls_ceiling_read_with_stores_bytes(bytes, every) bytes, 16-byte aligned. */
+int ls_ceiling_read_with_stores(const void* src, uint64_t bytes, void* dst, uint32_t every, int system_scope, void* sink, void* stream);
+uint64_t ls_ceiling_read_with_stores_bytes(uint64_t bytes, uint32_t every);
+
 #ifdef __cplusplus
 }
 #endif

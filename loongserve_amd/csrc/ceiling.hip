@@ -62,6 +62,42 @@ __global__ __launch_bounds__(256) void read_stream_kernel(const u32x4* __restric
   if ((x[0] ^ x[1] ^ x[2] ^ x[3]) == 0x9e3779b9u) sink[threadIdx.x] = x[0];  // (keeps the loads; practically never taken)
 }
 
+// The same read with stores mixed in, as a split-K decode mixes its partials into its gather: in one of every `every`
+// trips (spread evenly over the waves and over the launch) the wave also writes 8 KB, as sixteen rows of 512 bytes of
+// which a store instruction writes a 64-byte piece each (the shape of a partial's row stores).  SYSTEM: the stores carry
+// the system-scope bits (sc0 sc1: written through to memory as they are issued) instead of waiting in the L2 as dirty
+// lines that are written back later.
+template <bool SYSTEM>
+__global__ __launch_bounds__(256) void read_with_stores_kernel(const u32x4* __restrict__ src, uint64_t n16, u32x4* __restrict__ dst, uint32_t every,
+                                                               uint32_t* __restrict__ sink) {
+  const uint64_t stride = (uint64_t)gridDim.x * 256;
+  uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+  const uint32_t wave = (blockIdx.x * 256 + threadIdx.x) >> 6;
+  const uint32_t trips = (uint32_t)(n16 / (8 * stride));  // full trips of a wave
+  const int lane = threadIdx.x & 63;
+  u32x4 x = {0, 0, 0, 0};
+  uint32_t t = 0;
+  for (; i + 7 * stride < n16; i += 8 * stride, t++) {
+    u32x4 w[8];
+#pragma unroll
+    for (int u = 0; u < 8; u++) w[u] = __builtin_nontemporal_load(src + i + u * stride);
+#pragma unroll
+    for (int u = 0; u < 8; u++) x ^= w[u];
+    const uint32_t event = wave * trips + t;
+    if (t < trips && event % every == 0) {
+      u32x4* base = dst + (uint64_t)(event / every) * 512 + (lane & 15) * 32 + (lane >> 4);  // 8 KB = 512 x 16 B per event
+#pragma unroll
+      for (int u = 0; u < 8; u++) {
+        // (a vector instruction may not overwrite the data of a store of more than 64 bits in the two cycles behind it)
+        if (SYSTEM) asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1\n\ts_nop 1" : : "v"(base + 4 * u), "v"(x) : "memory");
+        else asm volatile("global_store_dwordx4 %0, %1, off\n\ts_nop 1" : : "v"(base + 4 * u), "v"(x) : "memory");
+      }
+    }
+  }
+  for (; i < n16; i += stride) x ^= __builtin_nontemporal_load(src + i);
+  if ((x[0] ^ x[1] ^ x[2] ^ x[3]) == 0x9e3779b9u) sink[threadIdx.x] = x[0];  // (keeps the loads; practically never taken)
+}
+
 }  // namespace
 
 extern "C" int ls_ceiling_mfma_f16(const void* operands, void* sink, int iters, int workgroups, void* stream) {
@@ -78,5 +114,22 @@ extern "C" double ls_ceiling_mfma_f16_flop(int iters, int workgroups) {
 extern "C" int ls_ceiling_read(const void* src, uint64_t bytes, void* sink, void* stream) {
   if (!src || !sink || bytes < 16 || ((uintptr_t)src & 15)) return -1;
   hipLaunchKernelGGL(read_stream_kernel, dim3(256 * 16), dim3(256), 0, (hipStream_t)stream, (const u32x4*)src, bytes / 16, (uint32_t*)sink);
+  return hipGetLastError() == hipSuccess ? 0 : -3;
+}
+
+extern "C" uint64_t ls_ceiling_read_with_stores_bytes(uint64_t bytes, uint32_t every) {
+  if (every < 1) return 0;
+  const uint64_t waves = 256 * 16 * 4, trips = bytes / 16 / (8ull * 256 * 16 * 256);
+  return (waves * trips + every - 1) / every * 8192;
+}
+
+extern "C" int ls_ceiling_read_with_stores(const void* src, uint64_t bytes, void* dst, uint32_t every, int system_scope, void* sink, void* stream) {
+  if (!src || !dst || !sink || bytes < 16 || every < 1 || (((uintptr_t)src | (uintptr_t)dst) & 15)) return -1;
+  if (system_scope)
+    hipLaunchKernelGGL(read_with_stores_kernel<true>, dim3(256 * 16), dim3(256), 0, (hipStream_t)stream, (const u32x4*)src, bytes / 16, (u32x4*)dst,
+                       every, (uint32_t*)sink);
+  else
+    hipLaunchKernelGGL(read_with_stores_kernel<false>, dim3(256 * 16), dim3(256), 0, (hipStream_t)stream, (const u32x4*)src, bytes / 16, (u32x4*)dst,
+                       every, (uint32_t*)sink);
   return hipGetLastError() == hipSuccess ? 0 : -3;
 }

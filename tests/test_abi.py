@@ -16,6 +16,18 @@ def _declared_symbols():
     return sorted(set(re.findall(r"\b(lsattn_[a-z0-9_]+)\s*\(", text)))
 
 
+def test_ceiling_library_exports_every_declared_symbol():
+    """libls_ceiling.so (bench.py's measurement aids) exports what include/ls_ceiling.h declares."""
+    import ctypes
+    text = open(os.path.join(ROOT, "include", "ls_ceiling.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    names = sorted(set(re.findall(r"\b(ls_ceiling_[a-z0-9_]+)\s*\(", text)))
+    assert len(names) == 5, names
+    lib = ctypes.CDLL(os.path.join(ROOT, "loongserve_amd", "libls_ceiling.so"))
+    for n in names:
+        assert getattr(lib, n) is not None
+
+
 def test_library_exports_every_declared_symbol():
     from loongserve_amd import _lib
     lib = _lib.load()

@@ -397,3 +397,26 @@ def test_decode_matrix_pipe_kernel_touches_no_register_of_a_load_in_flight():
     for name, (n, bad) in res.items():
         assert n >= 3 * 8 + 3 * 16, (name, n)             # slot and row loads of the prologue and of both halves of the loop
         assert not bad, name + "\n" + "\n".join(bad[:20])
+
+
+@pytest.mark.skipif(shutil.which(HIPCC) is None, reason="hipcc not available")
+def test_inline_assembly_stores_of_a_partial_keep_their_data_registers_for_two_cycles():
+    """The matrix-pipe decode kernel stores a partial's row from inline assembly (the compiler has no plain store with the
+    system-scope bits).  A vector instruction may not overwrite the data registers of a store of more than 64 bits in
+    the two cycles behind it; the compiler's hazard recogniser covers its own stores only, so every such store must be
+    followed by `s_nop 1` (or more) inside the same assembly block."""
+    for src in ("decode.hip", "ceiling.hip"):
+        raw = _device_asm(src).split("\n")
+        lines = [ln.split(";")[0].strip() for ln in raw]
+        seen, in_asm = 0, False
+        for i, ins in enumerate(lines):
+            if "#ASMSTART" in raw[i]:
+                in_asm = True
+            if "#ASMEND" in raw[i]:
+                in_asm = False
+            if in_asm and ins.startswith("global_store_dwordx"):
+                seen += 1
+                nxt = next(x for x in lines[i + 1:] if x)
+                m = re.match(r"s_nop (\d+)", nxt)
+                assert m and int(m.group(1)) >= 1, "%s line %d: %s is followed by %s" % (src, i + 1, ins, nxt)
+        assert seen >= 8, (src, seen)
