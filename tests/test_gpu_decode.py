@@ -556,6 +556,51 @@ def test_large_batch_that_is_dealt_in_equal_shares_by_itself(lsa, dtype):
         assert torch.equal(o_g, o_e) and torch.equal(l_g, l_e), "replay %d" % rep
 
 
+@pytest.mark.parametrize("seed", [5, 19, 77])
+def test_random_fused_calls_in_equal_shares(lsa, tuning, seed):
+    """Seeded random sweep of the fused call with stage 1 forced into equal shares, and of the entry point that brings
+    its own partials on the same inputs (bit for bit the same where the caller's buffers are tall enough for blocks of
+    256 tokens, which is what that entry point always deals): 1 to 40 requests of 0 to 9000 tokens (several empty,
+    of one token, of exactly a block), groups of 1 to 20 query heads on 1 to 8 KV heads, both dtypes, the caller's
+    BLOCK_SEQ 256 to 2048, buffers as tall as that makes them."""
+    import random
+    rng = random.Random(seed)
+    tuning(decode_listed="shares")
+    for case in range(8):
+        dtype = rng.choice([torch.float16, torch.bfloat16])
+        Hkv = rng.choice([1, 2, 3, 5, 8])
+        Hq = Hkv * rng.choice([1, 2, 4, 5, 8, 16, 17, 20])
+        BS = rng.choice([256, 512, 1024, 2048])
+        B = rng.choice([1, 2, 3, 9, 17, 40])
+        lens = [rng.choice([0, 1, 2, 255, 256, 257, 511, 512, 1000, 2049, 4096, 9000, rng.randint(1, 9000)]) for _ in range(B)]
+        if max(lens) == 0:
+            lens[0] = 300
+        print("case", seed, case, dtype, Hq, Hkv, BS, lens, flush=True)
+        D = 128
+        q, kv, table, b_req, b_len = decode_case(7000 + 100 * seed + case, B, Hq, Hkv, D, lens, sum(lens) + 300, dtype)
+        o_ref, l_ref = orc.decode_full(q, kv[:, :Hkv], kv[:, Hkv:], table, b_req, b_len)
+        kvd, qd, td, rd, ld = kv.to(DEV), q.to(DEV), table.to(DEV), b_req.to(DEV), b_len.to(DEV)
+        nblk = (max(lens) + BS - 1) // BS
+        mo_d = torch.full((nblk, B, Hq, D), float("nan"), device=DEV)
+        ml_d = torch.full((nblk, B, Hq), float("nan"), device=DEV)
+        o_d = torch.full((B, Hq, D), float("nan"), device=DEV)
+        l_d = torch.full((B, Hq), float("nan"), device=DEV)
+        lsa.longserve_cuda_kernels.flash_decoding(mo_d, ml_d, qd, kvd[:, :Hkv], kvd[:, Hkv:], td, rd, ld, max(lens), o_d, l_d, BS)
+        torch.cuda.synchronize()
+        what = "seed %d case %d" % (seed, case)
+        live = torch.tensor(lens) > 0
+        assert_o_close(o_d[live.to(DEV)], o_ref[live], "o, " + what)
+        assert_lse_close(l_d, l_ref, "lse, " + what)
+        o_s = torch.full((B, Hq, D), float("nan"), device=DEV)
+        l_s = torch.full((B, Hq), float("nan"), device=DEV)
+        lsa.longserve_cuda_kernels.flash_decoding_static(qd, kvd[:, :Hkv], kvd[:, Hkv:], td, rd, ld, max(lens), o_s, l_s, BS)
+        torch.cuda.synchronize()
+        assert_o_close(o_s[live.to(DEV)], o_ref[live], "o, own partials, " + what)
+        assert_lse_close(l_s, l_ref, "lse, own partials, " + what)
+        if nblk >= (max(lens) + 255) // 256:  # (both calls then deal blocks of 256 tokens: the same sums in the same order)
+            assert torch.equal(o_s[live.to(DEV)], o_d[live.to(DEV)]) and torch.equal(l_s, l_d), "own partials, " + what
+
+
 @pytest.mark.parametrize("seed", [3, 11, 42])
 def test_random_decode_shapes_on_both_stage1_kernels(lsa, tuning, seed):
     """Seeded random sweep of stage 1 + stage 2 against the oracle, once with the library's own choice of stage-1 kernel
