@@ -21,11 +21,11 @@ int ls_ceiling_mfma_f16(const void* operands, void* sink, int iters, int workgro
 double ls_ceiling_mfma_f16_flop(int iters, int workgroups);
 
 /* Reads `bytes` bytes at src (16-byte aligned) once, 16 bytes per lane and load, eight loads in flight per lane,
- * 4096 workgroups of 256 lanes.  sink: 1024 bytes (practically never written). */
+ * a wave 8 KB side by side at a time, 4096 workgroups of 256 lanes.  sink: 1024 bytes (practically never written). */
 int ls_ceiling_read(const void* src, uint64_t bytes, void* sink, void* stream);
 
 /* The same read with stores mixed in (what the partials of a split-K decode do to its gather): in one of every `every`
- * trips of a wave's loop over 8 KB of reads, spread evenly over the waves and the launch, the wave also writes 8 KB to
+ * trips of a wave's loop over 8 KB of reads, spread over the waves and the launch, the wave also writes 8 KB to
  * dst (sixteen rows of 512 bytes, a store instruction a 64-byte piece of each).  every = 64: 1.6 % of the bytes, the
  * share of one fp32 partial per 256 tokens and 32 query heads on 8 KV heads.  system_scope != 0: the stores are written
  * through to memory as they are issued (sc0 sc1) instead of being written back from the L2 later.
