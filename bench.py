@@ -36,11 +36,11 @@ if ROOT not in sys.path:
 # which is regenerated with the kernels (the JSON line says so in "traffic_source").
 TRAFFIC_SOURCE = "profiles/bench_default_hbm_traffic.txt (rocprofv3 --pmc, scaled by a 1 GiB copy); constants of bench.py, not measured in this run"
 TRAFFIC_BYTES = {
-    "config2": 1305.7e6,    # per launch, averaged over the four launches of a ring step (one diagonal + three full)
+    "config2": 1305.9e6,    # per launch, averaged over the four launches of a ring step (one diagonal + three full)
     "config3": 5186.9e6,    # the fused call: stage 1 in equal shares (5180.2) + the merge behind it (6.7)
     "config1": 92.6e6,
-    "config4": 8614.2e6,    # stage 1 over one instance's 4 x 131072 tokens
-    "config5": 104980.9e6,    # the attention launch (K/V re-fetched from HBM about 25 times)
+    "config4": 8614.1e6,    # stage 1 over one instance's 4 x 131072 tokens
+    "config5": 104980.5e6,    # the attention launch (K/V re-fetched from HBM about 25 times)
     "decode_8_1": 657.6e6,  # stage 1 of the large-group cases
     "decode_16_2": 1308.9e6,
     "decode_64_8": 5222.4e6,
