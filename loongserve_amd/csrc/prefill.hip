@@ -73,6 +73,7 @@ struct PrefillParams {
   int32_t pack_shift, heads_per_kv;  // 1 << pack_shift query heads of a KV head side by side in a workgroup; query heads per KV head
   int32_t fold_from, fold_sum;       // (ids >> 3) from fold_from on run backwards: j -> fold_sum - j (0: the whole grid runs forwards)
   int32_t listed, rows_shift;        // the grid numbers the (request, query tile, head group) units that exist (see the kernel); log2 of a workgroup's query positions
+  int32_t store_through;             // epilogue 0 writes O through to memory as the stores are issued (launches of one round; the fp16 o of epilogue 1 gains nothing from it)
   int32_t kv_cuts, kv_cut_len;       // every sequence entered kv_cuts times, entry c taking keys [c, c + 1) * kv_cut_len of its chunk
   int64_t o_cut_rows;                // and writing its rows o_cut_rows * c further down
   FastDiv d_peers, d_first, d_second, d_slices, d_group, d_cuts;
@@ -233,6 +234,13 @@ __device__ __forceinline__ const char* uniform_ptr(const char* ptr) {
 // HALF: four waves and 128 query rows, 32 per wave and every key, with rings of two tiles (64 KB of LDS): two such
 // workgroups fit a CU, and one's start-up, finish and turn-over run beside the other's tiles.  For launches whose
 // workgroups are short (a few tiles each): there a workgroup that fills the CU spends as long starting and ending as working.
+// A 16-byte store that goes through to memory as it is issued (system-scope bits) instead of waiting in the L2 as a dirty
+// line until the end of the launch.  From inline assembly (the compiler has no such store that is not atomic); the
+// s_nop keeps vector instructions off the data registers for the two cycles a store of more than 64 bits needs.
+__device__ __forceinline__ void store16_through(float* addr, const f32x4 v) {
+  asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1\n\ts_nop 1" : : "v"(addr), "v"(v) : "memory");
+}
+
 template <typename T, int MODE, bool DV, bool SPLIT, bool HALF = false>
 __global__ __launch_bounds__(HALF ? NWAVE * 32 : NWAVE * 64, HALF ? 2 : 1) void prefill_kernel(PrefillParams p) {
   static_assert(DV || !SPLIT, "the split variant takes fp16 V tiles only");
@@ -993,20 +1001,31 @@ __global__ __launch_bounds__(HALF ? NWAVE * 32 : NWAVE * 64, HALF ? 2 : 1) void 
   auto finish = [&](auto db0_tag) __attribute__((always_inline)) {
     constexpr int DB0 = decltype(db0_tag)::value;
     if (MODE == 0) {
-      // the step's partial from the empty state
+      // the step's partial from the empty state.  THROUGH (a launch of one round: every workgroup stores as the launch
+      // ends, and what the L2s hold then is written back before the launch counts as done): the stores go through to
+      // memory as they are issued, 1 x 2048 tokens 46.9 -> 45.9 us.  In launches of several rounds that costs the L2's
+      // joining of a line's halves while other workgroups compute (32 x 1024 tokens 398 -> 417 us): plain stores there.
+      auto write_partial = [&](auto through_tag) __attribute__((always_inline)) {
+        constexpr bool THROUGH = decltype(through_tag)::value;
 #pragma unroll
-      for (int qb = 0; qb < 2; qb++) {
-        const int m = m_w0 + 16 * qb + qc;
-        const float l_tot = column_sum(l_run[qb]);
-        if (m < q_len) {
-          const int64_t tok = o_start + m;
-          const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
-          float* orow = (float*)p.o + tok * p.o_st + (int64_t)h * p.o_sh;
+        for (int qb = 0; qb < 2; qb++) {
+          const int m = m_w0 + 16 * qb + qc;
+          const float l_tot = column_sum(l_run[qb]);
+          if (m < q_len) {
+            const int64_t tok = o_start + m;
+            const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+            float* orow = (float*)p.o + tok * p.o_st + (int64_t)h * p.o_sh;
 #pragma unroll
-          for (int i = 0; i < NDB; i++) *(f32x4*)(orow + (DB0 + i) * 16 + 4 * g) = oacc[DB0 + i][qb] * inv;
-          if (g == 0 && DB0 == 0) p.lse[tok * p.hq + h] = l_tot > 0.f ? (m_run[qb] + __builtin_amdgcn_logf(l_tot)) * kLn2 : -INFINITY;
+            for (int i = 0; i < NDB; i++) {
+              if (THROUGH) store16_through(orow + (DB0 + i) * 16 + 4 * g, oacc[DB0 + i][qb] * inv);
+              else *(f32x4*)(orow + (DB0 + i) * 16 + 4 * g) = oacc[DB0 + i][qb] * inv;
+            }
+            if (g == 0 && DB0 == 0) p.lse[tok * p.hq + h] = l_tot > 0.f ? (m_run[qb] + __builtin_amdgcn_logf(l_tot)) * kLn2 : -INFINITY;
+          }
         }
-      }
+      };
+      if (p.store_through) write_partial(std::true_type{});
+      else write_partial(std::false_type{});
     }
     if (MODE == 1) {
       // the reference's update of (o, m, l) (RING:171-188).  NB row blocks at a time: all reads of their old o are in
@@ -1228,6 +1247,7 @@ static int launch_prefill_rows(const lsattn_prefill_args* a, bool tile_major, co
     p.fold_from = (int32_t)(kCUs / 8);
     p.fold_sum = p.fold_from + (int32_t)(wgs / 8) - 1;
   }
+  p.store_through = MODE == 0 && wgs_launch <= (HALF ? 2 * kCUs : kCUs);  // (resident together: two four-wave workgroups per CU, one of the others)
   hipLaunchKernelGGL((prefill_kernel<T, MODE, DV, SPLIT, HALF>), dim3((unsigned)wgs_launch), dim3(HALF ? NWAVE * 32 : NWAVE * 64), 0, st, p);
   return check_launch();
 }

@@ -405,7 +405,7 @@ def test_inline_assembly_stores_of_a_partial_keep_their_data_registers_for_two_c
     system-scope bits).  A vector instruction may not overwrite the data registers of a store of more than 64 bits in
     the two cycles behind it; the compiler's hazard recogniser covers its own stores only, so every such store must be
     followed by `s_nop 1` (or more) inside the same assembly block."""
-    for src in ("decode.hip", "ceiling.hip"):
+    for src in ("decode.hip", "ceiling.hip", "prefill.hip"):
         raw = _device_asm(src).split("\n")
         lines = [ln.split(";")[0].strip() for ln in raw]
         seen, in_asm = 0, False
