@@ -73,7 +73,7 @@ struct PrefillParams {
   int32_t pack_shift, heads_per_kv;  // 1 << pack_shift query heads of a KV head side by side in a workgroup; query heads per KV head
   int32_t fold_from, fold_sum;       // (ids >> 3) from fold_from on run backwards: j -> fold_sum - j (0: the whole grid runs forwards)
   int32_t listed, rows_shift;        // the grid numbers the (request, query tile, head group) units that exist (see the kernel); log2 of a workgroup's query positions
-  int32_t store_through;             // epilogue 0 writes O through to memory as the stores are issued (launches of one round; the fp16 o of epilogue 1 gains nothing from it)
+  int32_t store_through;             // epilogue 0 writes O through to memory as the stores are issued (launches of at most two rounds; the fp16 o of epilogue 1 gains nothing from it)
   int32_t kv_cuts, kv_cut_len;       // every sequence entered kv_cuts times, entry c taking keys [c, c + 1) * kv_cut_len of its chunk
   int64_t o_cut_rows;                // and writing its rows o_cut_rows * c further down
   FastDiv d_peers, d_first, d_second, d_slices, d_group, d_cuts;
@@ -1001,9 +1001,9 @@ __global__ __launch_bounds__(HALF ? NWAVE * 32 : NWAVE * 64, HALF ? 2 : 1) void 
   auto finish = [&](auto db0_tag) __attribute__((always_inline)) {
     constexpr int DB0 = decltype(db0_tag)::value;
     if (MODE == 0) {
-      // the step's partial from the empty state.  THROUGH (a launch of one round: every workgroup stores as the launch
+      // the step's partial from the empty state.  THROUGH (a launch of one or two rounds: every workgroup stores as the launch
       // ends, and what the L2s hold then is written back before the launch counts as done): the stores go through to
-      // memory as they are issued, 1 x 2048 tokens 46.9 -> 45.9 us.  In launches of several rounds that costs the L2's
+      // memory as they are issued, 1 x 2048 tokens 46.9 -> 45.9 us.  In launches of many rounds that costs the L2's
       // joining of a line's halves while other workgroups compute (32 x 1024 tokens 398 -> 417 us): plain stores there.
       auto write_partial = [&](auto through_tag) __attribute__((always_inline)) {
         constexpr bool THROUGH = decltype(through_tag)::value;
@@ -1247,7 +1247,9 @@ static int launch_prefill_rows(const lsattn_prefill_args* a, bool tile_major, co
     p.fold_from = (int32_t)(kCUs / 8);
     p.fold_sum = p.fold_from + (int32_t)(wgs / 8) - 1;
   }
-  p.store_through = MODE == 0 && wgs_launch <= (HALF ? 2 * kCUs : kCUs);  // (resident together: two four-wave workgroups per CU, one of the others)
+  // (a round: two four-wave workgroups per CU, one of the others.  Two rounds still gain: 16 x 256 tokens 38.0 -> 36.8 us,
+  // 1 x 4096 129.0 -> 127.7; six rounds lose 1-3 %, sixteen 5 %.)
+  p.store_through = MODE == 0 && wgs_launch <= 2 * (HALF ? 2 * kCUs : kCUs);
   hipLaunchKernelGGL((prefill_kernel<T, MODE, DV, SPLIT, HALF>), dim3((unsigned)wgs_launch), dim3(HALF ? NWAVE * 32 : NWAVE * 64), 0, st, p);
   return check_launch();
 }
