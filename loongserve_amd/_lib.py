@@ -163,6 +163,10 @@ def load():
     global _lib
     if _lib is not None:
         return _lib
+    # PyTorch-ROCm ships a HIP runtime of its own.  Loaded first, it is the one this library's `libamdhip64.so.*`
+    # dependency resolves to (same soname), and the process has one runtime; loaded second, the process would hold
+    # two, and the library's launches would find no device in theirs (hipErrorNoDevice on the first launch).
+    import torch  # noqa: F401
     if not os.path.exists(LIB_PATH):
         raise ImportError(
             "loongserve_amd: %s is missing; there is no fallback implementation. "

@@ -103,6 +103,7 @@ __global__ __launch_bounds__(256) void read_with_stores_kernel(const u32x4* __re
 
 extern "C" int ls_ceiling_mfma_f16(const void* operands, void* sink, int iters, int workgroups, void* stream) {
   if (!operands || !sink || iters < 1 || workgroups < 1 || ((uintptr_t)operands & 15)) return -1;
+  (void)hipGetLastError();  // (an earlier call of the host program may have left an error that is not this launch's)
   hipLaunchKernelGGL(mfma_stream_kernel, dim3((unsigned)workgroups), dim3(256), 0, (hipStream_t)stream, (const u32x4*)operands,
                      (float*)sink, iters);
   return hipGetLastError() == hipSuccess ? 0 : -3;
@@ -114,6 +115,7 @@ extern "C" double ls_ceiling_mfma_f16_flop(int iters, int workgroups) {
 
 extern "C" int ls_ceiling_read(const void* src, uint64_t bytes, void* sink, void* stream) {
   if (!src || !sink || bytes < 16 || ((uintptr_t)src & 15)) return -1;
+  (void)hipGetLastError();  // (an earlier call of the host program may have left an error that is not this launch's)
   hipLaunchKernelGGL(read_stream_kernel, dim3(256 * 16), dim3(256), 0, (hipStream_t)stream, (const u32x4*)src, bytes / 16, (uint32_t*)sink);
   return hipGetLastError() == hipSuccess ? 0 : -3;
 }
@@ -126,6 +128,7 @@ extern "C" uint64_t ls_ceiling_read_with_stores_bytes(uint64_t bytes, uint32_t e
 
 extern "C" int ls_ceiling_read_with_stores(const void* src, uint64_t bytes, void* dst, uint32_t every, int system_scope, void* sink, void* stream) {
   if (!src || !dst || !sink || bytes < 16 || every < 1 || (((uintptr_t)src | (uintptr_t)dst) & 15)) return -1;
+  (void)hipGetLastError();  // (an earlier call of the host program may have left an error that is not this launch's)
   if (system_scope)
     hipLaunchKernelGGL(read_with_stores_kernel<true>, dim3(256 * 16), dim3(256), 0, (hipStream_t)stream, (const u32x4*)src, bytes / 16, (u32x4*)dst,
                        every, (uint32_t*)sink);

@@ -83,6 +83,14 @@ Tuning tuning();
 // running fp32 partial.  Arguments validated by the caller.
 int launch_prefill_small(const lsattn_prefill_args* a, int mode, hipStream_t st);
 
+// check_launch reports what the launch in front of it left in the host thread's last-error slot, so every launch first
+// empties that slot: an earlier runtime call of the host program may have left something there that is not this
+// library's to report (hipEventQuery's "not ready", which a framework's copy engine polls with, among them).
+#define LSATTN_LAUNCH_KERNEL(...)   \
+  do {                              \
+    (void)hipGetLastError();        \
+    hipLaunchKernelGGL(__VA_ARGS__); \
+  } while (0)
 inline int check_launch() { return hipGetLastError() == hipSuccess ? LSATTN_OK : LSATTN_ERR_LAUNCH; }
 
 }  // namespace lsattn

@@ -1097,15 +1097,15 @@ static int launch_stage1(const lsattn_decode_stage1_args* a, hipStream_t st) {
     p.tasks_on_x = chunks <= 65535;
     dim3 grid = p.tasks_on_x ? dim3((unsigned)p.tasks, (unsigned)chunks, (unsigned)a->batch)
                              : dim3((unsigned)chunks, (unsigned)p.tasks, (unsigned)a->batch);
-    if (once) hipLaunchKernelGGL((decode_stage1_kernel<T, GT, NW, true, true, HR>), grid, dim3(NW * 64), 0, st, p);
-    else hipLaunchKernelGGL((decode_stage1_kernel<T, GT, NW, true, false, HR>), grid, dim3(NW * 64), 0, st, p);
+    if (once) LSATTN_LAUNCH_KERNEL((decode_stage1_kernel<T, GT, NW, true, true, HR>), grid, dim3(NW * 64), 0, st, p);
+    else LSATTN_LAUNCH_KERNEL((decode_stage1_kernel<T, GT, NW, true, false, HR>), grid, dim3(NW * 64), 0, st, p);
     return check_launch();
   }
   p.tasks_on_x = wgs_y <= 2 && chunks <= 65535;  // with more task groups per chunk (MHA, 32 KV heads) it measured 2 % slower
   dim3 grid = p.tasks_on_x ? dim3((unsigned)wgs_y, (unsigned)chunks, (unsigned)a->batch)
                            : dim3((unsigned)chunks, (unsigned)wgs_y, (unsigned)a->batch);
-  if (once) hipLaunchKernelGGL((decode_stage1_kernel<T, GT, NW, false, true, HR>), grid, dim3(NW * 64), 0, st, p);
-  else hipLaunchKernelGGL((decode_stage1_kernel<T, GT, NW, false, false, HR>), grid, dim3(NW * 64), 0, st, p);
+  if (once) LSATTN_LAUNCH_KERNEL((decode_stage1_kernel<T, GT, NW, false, true, HR>), grid, dim3(NW * 64), 0, st, p);
+  else LSATTN_LAUNCH_KERNEL((decode_stage1_kernel<T, GT, NW, false, false, HR>), grid, dim3(NW * 64), 0, st, p);
   return check_launch();
 }
 
@@ -1180,14 +1180,14 @@ template <typename T> static int launch_stage1_mfma(const lsattn_decode_stage1_a
     *shares = workers;
     p.tasks_on_x = tws;
     p.blocks_per_wg = 1;
-    hipLaunchKernelGGL((decode_stage1_mfma_range_kernel<T>), dim3((unsigned)(per_group * task_groups)), dim3(kMfmaWaves * 64), 0, st, p);
+    LSATTN_LAUNCH_KERNEL((decode_stage1_mfma_range_kernel<T>), dim3((unsigned)(per_group * task_groups)), dim3(kMfmaWaves * 64), 0, st, p);
     return check_launch();
   }
   if (split_waves) {
     *taken = true;
     p.blocks_per_wg = 1;
     p.tasks_on_x = 1;
-    hipLaunchKernelGGL((decode_stage1_mfma_kernel<T, true>), dim3((unsigned)nblk, (unsigned)p.tasks, (unsigned)a->batch), dim3(kMfmaWaves * 64),
+    LSATTN_LAUNCH_KERNEL((decode_stage1_mfma_kernel<T, true>), dim3((unsigned)nblk, (unsigned)p.tasks, (unsigned)a->batch), dim3(kMfmaWaves * 64),
                        0, st, p);
     return check_launch();
   }
@@ -1206,12 +1206,12 @@ template <typename T> static int launch_stage1_mfma(const lsattn_decode_stage1_a
   if (tn.decode_listed == LSATTN_DECODE_LISTED_ON) listed = true;
   if (listed && a->batch <= kListedMaxBatch && wgs_total <= 0x7fffffff) {
     const int64_t resident = 2 * kCUs;  // two workgroups of this kernel per CU
-    hipLaunchKernelGGL((decode_stage1_mfma_listed_kernel<T>), dim3((unsigned)(wgs_total < resident ? wgs_total : resident)),
+    LSATTN_LAUNCH_KERNEL((decode_stage1_mfma_listed_kernel<T>), dim3((unsigned)(wgs_total < resident ? wgs_total : resident)),
                        dim3(kMfmaWaves * 64), 0, st, p);
     return check_launch();
   }
   const dim3 grid = tasks_first ? dim3((unsigned)wgs_y, (unsigned)wgs_x, (unsigned)a->batch) : dim3((unsigned)wgs_x, (unsigned)wgs_y, (unsigned)a->batch);
-  hipLaunchKernelGGL((decode_stage1_mfma_kernel<T, false>), grid, dim3(kMfmaWaves * 64), 0, st, p);
+  LSATTN_LAUNCH_KERNEL((decode_stage1_mfma_kernel<T, false>), grid, dim3(kMfmaWaves * 64), 0, st, p);
   return check_launch();
 }
 
@@ -1271,19 +1271,19 @@ template <typename OT> static int dispatch_stage2(const Stage2Params& p, int64_t
     if (D != 128) return LSATTN_ERR_UNSUPPORTED;
     // (a request's partials: at most one per share and one more, and no more than it has blocks)
     const int64_t most = live_blocks < p.shares_workers + 1 ? live_blocks : p.shares_workers + 1;
-    if (most >= 64 && (int64_t)grid.x < 2048) hipLaunchKernelGGL((decode_stage2_kernel<OT, 128, 1024, true>), grid, dim3(1024), 0, st, p);
-    else hipLaunchKernelGGL((decode_stage2_kernel<OT, 128, 256, true>), grid, dim3(256), 0, st, p);
+    if (most >= 64 && (int64_t)grid.x < 2048) LSATTN_LAUNCH_KERNEL((decode_stage2_kernel<OT, 128, 1024, true>), grid, dim3(1024), 0, st, p);
+    else LSATTN_LAUNCH_KERNEL((decode_stage2_kernel<OT, 128, 256, true>), grid, dim3(256), 0, st, p);
     return check_launch();
   }
   // few (batch, head) pairs with many partials each (long contexts at small batch): 1024 threads walk the block axis in 32
   // slices instead of 8, or the merge takes a fifth of the time of the gather it follows
   const bool wide = D == 128 && live_blocks >= 64 && ((int64_t)grid.x < 2048 || (live_blocks >= 1024 && (int64_t)grid.x < 8192));
   switch (D) {
-    case 32: hipLaunchKernelGGL((decode_stage2_kernel<OT, 32, 256>), grid, dim3(256), 0, st, p); break;
-    case 64: hipLaunchKernelGGL((decode_stage2_kernel<OT, 64, 256>), grid, dim3(256), 0, st, p); break;
+    case 32: LSATTN_LAUNCH_KERNEL((decode_stage2_kernel<OT, 32, 256>), grid, dim3(256), 0, st, p); break;
+    case 64: LSATTN_LAUNCH_KERNEL((decode_stage2_kernel<OT, 64, 256>), grid, dim3(256), 0, st, p); break;
     case 128:
-      if (wide) hipLaunchKernelGGL((decode_stage2_kernel<OT, 128, 1024>), grid, dim3(1024), 0, st, p);
-      else hipLaunchKernelGGL((decode_stage2_kernel<OT, 128, 256>), grid, dim3(256), 0, st, p);
+      if (wide) LSATTN_LAUNCH_KERNEL((decode_stage2_kernel<OT, 128, 1024>), grid, dim3(1024), 0, st, p);
+      else LSATTN_LAUNCH_KERNEL((decode_stage2_kernel<OT, 128, 256>), grid, dim3(256), 0, st, p);
       break;
     default: return LSATTN_ERR_UNSUPPORTED;
   }

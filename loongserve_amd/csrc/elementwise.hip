@@ -251,7 +251,7 @@ extern "C" int lsattn_bf16_to_f16_rows(const void* src, int64_t src_stride, void
   if (n_rows == 0) return LSATTN_OK;
   const int64_t blocks = (n_rows * (row_elems / 8) + 255) / 256;
   if (blocks > 0x7fffffff) return LSATTN_ERR_INVALID_ARG;
-  hipLaunchKernelGGL(bf16_to_f16_rows_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (const uint16_t*)src,
+  LSATTN_LAUNCH_KERNEL(bf16_to_f16_rows_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (const uint16_t*)src,
                      src_stride, (uint16_t*)dst, dst_stride, n_rows, row_elems / 8);
   return check_launch();
 }
@@ -263,7 +263,7 @@ extern "C" int lsattn_rms_norm(void* out, const void* in, const void* weight, in
   if (num_tokens == 0) return LSATTN_OK;
   const int64_t blocks = (num_tokens + 3) / 4;
   if (blocks > 0x7fffffff) return LSATTN_ERR_INVALID_ARG;
-  hipLaunchKernelGGL(rms_norm_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (uint16_t*)out,
+  LSATTN_LAUNCH_KERNEL(rms_norm_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (uint16_t*)out,
                      (const uint16_t*)in, (const uint16_t*)weight, num_tokens, hidden_size, eps);
   return check_launch();
 }
@@ -274,7 +274,7 @@ extern "C" int lsattn_silu_and_mul_inplace(void* io, int64_t num_tokens, int64_t
   if (num_tokens == 0) return LSATTN_OK;
   const int64_t blocks = (num_tokens * (ffn_inter_dim / 8) + 255) / 256;
   if (blocks > 0x7fffffff) return LSATTN_ERR_INVALID_ARG;
-  hipLaunchKernelGGL(silu_and_mul_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (uint16_t*)io, num_tokens,
+  LSATTN_LAUNCH_KERNEL(silu_and_mul_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (uint16_t*)io, num_tokens,
                      ffn_inter_dim);
   return check_launch();
 }
@@ -287,7 +287,7 @@ extern "C" int lsattn_rotary_emb(void* x, const void* cos, const void* sin, int6
   if (num_tokens == 0) return LSATTN_OK;
   const int64_t blocks = (num_tokens * num_heads * (head_dim / 16) + 255) / 256;
   if (blocks > 0x7fffffff) return LSATTN_ERR_INVALID_ARG;
-  hipLaunchKernelGGL(rotary_emb_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (uint16_t*)x,
+  LSATTN_LAUNCH_KERNEL(rotary_emb_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (uint16_t*)x,
                      (const uint16_t*)cos, (const uint16_t*)sin, x_stride_t, x_stride_h, num_tokens, num_heads, head_dim);
   return check_launch();
 }
@@ -342,6 +342,6 @@ extern "C" int lsattn_rotary_kv_write(const lsattn_rotary_kv_write_args* a, void
   const int64_t blocks = p.data_blocks + reg_blocks;
   if (blocks == 0) return LSATTN_OK;
   if (blocks > 0x7fffffff) return LSATTN_ERR_INVALID_ARG;
-  hipLaunchKernelGGL(rotary_kv_write_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, p);
+  LSATTN_LAUNCH_KERNEL(rotary_kv_write_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, p);
   return check_launch();
 }

@@ -323,7 +323,7 @@ template <bool SEND> static int launch_migration(const lsattn_decode_migration_a
   p.rows_per_block = cpr >= 256 ? 1 : (int32_t)(256 / cpr);  // one 16-byte piece per lane and layer
   const int64_t blocks = (a->max_num_tokens + p.rows_per_block - 1) / p.rows_per_block;
   if (blocks > 0x7fffffff) return LSATTN_ERR_INVALID_ARG;
-  hipLaunchKernelGGL((decode_migration_kernel<SEND>), dim3((unsigned)blocks, (unsigned)a->batch), dim3(256), 0, st, p);
+  LSATTN_LAUNCH_KERNEL((decode_migration_kernel<SEND>), dim3((unsigned)blocks, (unsigned)a->batch), dim3(256), 0, st, p);
   return check_launch();
 }
 
@@ -332,10 +332,10 @@ template <typename OT> static int launch_merge(const MergeParams& p, int D, hipS
   const int64_t blocks = (threads + 255) / 256;
   if (blocks > 0x7fffffff) return LSATTN_ERR_INVALID_ARG;
   switch (D) {
-    case 16: hipLaunchKernelGGL((lse_merge_kernel<OT, 16>), dim3((unsigned)blocks), dim3(256), 0, st, p); break;
-    case 32: hipLaunchKernelGGL((lse_merge_kernel<OT, 32>), dim3((unsigned)blocks), dim3(256), 0, st, p); break;
-    case 64: hipLaunchKernelGGL((lse_merge_kernel<OT, 64>), dim3((unsigned)blocks), dim3(256), 0, st, p); break;
-    case 128: hipLaunchKernelGGL((lse_merge_kernel<OT, 128>), dim3((unsigned)blocks), dim3(256), 0, st, p); break;
+    case 16: LSATTN_LAUNCH_KERNEL((lse_merge_kernel<OT, 16>), dim3((unsigned)blocks), dim3(256), 0, st, p); break;
+    case 32: LSATTN_LAUNCH_KERNEL((lse_merge_kernel<OT, 32>), dim3((unsigned)blocks), dim3(256), 0, st, p); break;
+    case 64: LSATTN_LAUNCH_KERNEL((lse_merge_kernel<OT, 64>), dim3((unsigned)blocks), dim3(256), 0, st, p); break;
+    case 128: LSATTN_LAUNCH_KERNEL((lse_merge_kernel<OT, 128>), dim3((unsigned)blocks), dim3(256), 0, st, p); break;
     default: return LSATTN_ERR_UNSUPPORTED;
   }
   return check_launch();
@@ -386,10 +386,10 @@ extern "C" int lsattn_prefill_merge_cuts(const lsattn_merge_cuts_args* a, void* 
   if (blocks > 0x7fffffff) return LSATTN_ERR_INVALID_ARG;
   const dim3 grid((unsigned)blocks, (unsigned)a->batch);
   hipStream_t st = (hipStream_t)stream;
-  if (a->mode == 0) hipLaunchKernelGGL((merge_cuts_kernel<float, 0>), grid, dim3(256), 0, st, p);
-  else if (a->mode == 2) hipLaunchKernelGGL((merge_cuts_kernel<float, 2>), grid, dim3(256), 0, st, p);
-  else if (a->o_dtype == LSATTN_F16) hipLaunchKernelGGL((merge_cuts_kernel<F16, 1>), grid, dim3(256), 0, st, p);
-  else hipLaunchKernelGGL((merge_cuts_kernel<BF16, 1>), grid, dim3(256), 0, st, p);
+  if (a->mode == 0) LSATTN_LAUNCH_KERNEL((merge_cuts_kernel<float, 0>), grid, dim3(256), 0, st, p);
+  else if (a->mode == 2) LSATTN_LAUNCH_KERNEL((merge_cuts_kernel<float, 2>), grid, dim3(256), 0, st, p);
+  else if (a->o_dtype == LSATTN_F16) LSATTN_LAUNCH_KERNEL((merge_cuts_kernel<F16, 1>), grid, dim3(256), 0, st, p);
+  else LSATTN_LAUNCH_KERNEL((merge_cuts_kernel<BF16, 1>), grid, dim3(256), 0, st, p);
   return check_launch();
 }
 
@@ -402,7 +402,7 @@ extern "C" int lsattn_kv_scatter(const void* src, int64_t src_stride_bytes, void
   const int64_t cpr = row_bytes / 16;
   const int64_t blocks = (n_rows * cpr + 255) / 256;
   if (blocks > 0x7fffffff || cpr > 0x7fffffff) return LSATTN_ERR_INVALID_ARG;
-  hipLaunchKernelGGL(kv_scatter_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (const char*)src,
+  LSATTN_LAUNCH_KERNEL(kv_scatter_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (const char*)src,
                      src_stride_bytes, (char*)dst, dst_stride_bytes, dest_index, n_rows, (int32_t)cpr);
   return check_launch();
 }
@@ -416,7 +416,7 @@ extern "C" int lsattn_register_tokens(int32_t* req_to_tokens, int64_t max_seq_le
   if (batch == 0 || max_len_in_batch == 0) return LSATTN_OK;
   if (batch > 65535) return LSATTN_ERR_INVALID_ARG;
   dim3 grid((unsigned)((max_len_in_batch + 255) / 256), (unsigned)batch);
-  hipLaunchKernelGGL(register_tokens_kernel, grid, dim3(256), 0, (hipStream_t)stream, req_to_tokens, max_seq_len,
+  LSATTN_LAUNCH_KERNEL(register_tokens_kernel, grid, dim3(256), 0, (hipStream_t)stream, req_to_tokens, max_seq_len,
                      b_req_idx, b_start_loc, b_seq_len, mem_index);
   return check_launch();
 }
@@ -431,10 +431,10 @@ extern "C" int lsattn_register_decode_tokens(int32_t* req_to_tokens, int64_t max
   const int64_t blocks = (batch + 255) / 256;
   if (blocks > 0x7fffffff) return LSATTN_ERR_INVALID_ARG;
   if (mem_index_is_i64)
-    hipLaunchKernelGGL(register_decode_tokens_kernel<int64_t>, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+    LSATTN_LAUNCH_KERNEL(register_decode_tokens_kernel<int64_t>, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
                        req_to_tokens, max_seq_len, b_req_idx, b_seq_len, (const int64_t*)mem_index, batch);
   else
-    hipLaunchKernelGGL(register_decode_tokens_kernel<int32_t>, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+    LSATTN_LAUNCH_KERNEL(register_decode_tokens_kernel<int32_t>, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
                        req_to_tokens, max_seq_len, b_req_idx, b_seq_len, (const int32_t*)mem_index, batch);
   return check_launch();
 }
@@ -448,7 +448,7 @@ extern "C" int lsattn_kv_ranges(const int32_t* kv_cache_index_begin, const int32
   if (batch == 0) return LSATTN_OK;
   const int64_t blocks = (batch + 255) / 256;
   if (blocks > 0x7fffffff) return LSATTN_ERR_INVALID_ARG;
-  hipLaunchKernelGGL(kv_ranges_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, kv_cache_index_begin,
+  LSATTN_LAUNCH_KERNEL(kv_ranges_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, kv_cache_index_begin,
                      kv_cache_index_end, kv_first_token_global_idx, sp_peers, batch, kv_range_begin, kv_range_end,
                      new_kv_cache_len);
   return check_launch();
@@ -490,7 +490,7 @@ extern "C" int lsattn_kv_copy_register(const lsattn_kv_copy_register_args* a, vo
   if (blocks > 0x7fffffff) return LSATTN_ERR_INVALID_ARG;
   p.chunks_per_row = (int32_t)cpr;
   p.should_register = a->should_register;
-  hipLaunchKernelGGL(kv_copy_register_kernel, dim3((unsigned)blocks, (unsigned)a->batch), dim3(256), 0, (hipStream_t)stream, p);
+  LSATTN_LAUNCH_KERNEL(kv_copy_register_kernel, dim3((unsigned)blocks, (unsigned)a->batch), dim3(256), 0, (hipStream_t)stream, p);
   return check_launch();
 }
 

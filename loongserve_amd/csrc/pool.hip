@@ -370,12 +370,12 @@ extern "C" int lsattn_pool_alloc(int32_t* mem_state, int64_t pool_size, int64_t 
   if (need > 0 && !out_index) return LSATTN_ERR_INVALID_ARG;
   hipStream_t st = (hipStream_t)stream;
   const PoolWorkspace w = pool_carve(workspace, pool_size);
-  hipLaunchKernelGGL(pool_summarise_kernel, dim3((unsigned)w.nb), dim3(kPoolThreads), 0, st, mem_state, pool_size, w.blk_free,
+  LSATTN_LAUNCH_KERNEL(pool_summarise_kernel, dim3((unsigned)w.nb), dim3(kPoolThreads), 0, st, mem_state, pool_size, w.blk_free,
                      w.blk_last_used);
-  hipLaunchKernelGGL(pool_scan_summaries_kernel, dim3(1), dim3(1024), 0, st, w.blk_free, w.blk_last_used, w.nb, w.free_before,
+  LSATTN_LAUNCH_KERNEL(pool_scan_summaries_kernel, dim3(1), dim3(1024), 0, st, w.blk_free, w.blk_last_used, w.nb, w.free_before,
                      w.last_used_before, w.cells, need, out_index, (int64_t*)nullptr);
   if (need > 0)
-    hipLaunchKernelGGL(pool_take_kernel, dim3((unsigned)w.nb), dim3(kPoolThreads), 0, st, mem_state, pool_size, w.free_before,
+    LSATTN_LAUNCH_KERNEL(pool_take_kernel, dim3((unsigned)w.nb), dim3(kPoolThreads), 0, st, mem_state, pool_size, w.free_before,
                        need, out_index);
   return check_launch();
 }
@@ -387,11 +387,11 @@ extern "C" int lsattn_pool_find_contiguous(const int32_t* mem_state, int64_t poo
   if (!out_start || need <= 0) return LSATTN_ERR_INVALID_ARG;
   hipStream_t st = (hipStream_t)stream;
   const PoolWorkspace w = pool_carve(workspace, pool_size);
-  hipLaunchKernelGGL(pool_summarise_kernel, dim3((unsigned)w.nb), dim3(kPoolThreads), 0, st, mem_state, pool_size, w.blk_free,
+  LSATTN_LAUNCH_KERNEL(pool_summarise_kernel, dim3((unsigned)w.nb), dim3(kPoolThreads), 0, st, mem_state, pool_size, w.blk_free,
                      w.blk_last_used);
-  hipLaunchKernelGGL(pool_scan_summaries_kernel, dim3(1), dim3(1024), 0, st, w.blk_free, w.blk_last_used, w.nb, w.free_before,
+  LSATTN_LAUNCH_KERNEL(pool_scan_summaries_kernel, dim3(1), dim3(1024), 0, st, w.blk_free, w.blk_last_used, w.nb, w.free_before,
                      w.last_used_before, w.cells, (int64_t)0, (int64_t*)nullptr, out_start);
-  hipLaunchKernelGGL(pool_first_fit_kernel, dim3((unsigned)w.nb), dim3(kPoolThreads), 0, st, mem_state, pool_size,
+  LSATTN_LAUNCH_KERNEL(pool_first_fit_kernel, dim3((unsigned)w.nb), dim3(kPoolThreads), 0, st, mem_state, pool_size,
                      w.last_used_before, need, out_start);
   return check_launch();
 }
@@ -408,10 +408,10 @@ extern "C" int lsattn_pool_update_refs(int32_t* mem_state, int64_t pool_size, co
   int64_t* blk_counts = (int64_t*)workspace;
   int32_t* old_state = (int32_t*)(blk_counts + 2 * nblk);
   if (n > 0)
-    hipLaunchKernelGGL(pool_refs_gather_kernel, dim3((unsigned)nblk), dim3(256), 0, st, mem_state, pool_size, index, n, delta,
+    LSATTN_LAUNCH_KERNEL(pool_refs_gather_kernel, dim3((unsigned)nblk), dim3(256), 0, st, mem_state, pool_size, index, n, delta,
                        old_state, blk_counts);
   // with n == 0 one workgroup still runs, to write counted = {0, 0}
-  hipLaunchKernelGGL(pool_refs_apply_kernel, dim3((unsigned)(nblk > 0 ? nblk : 1)), dim3(256), 0, st, mem_state, pool_size, index,
+  LSATTN_LAUNCH_KERNEL(pool_refs_apply_kernel, dim3((unsigned)(nblk > 0 ? nblk : 1)), dim3(256), 0, st, mem_state, pool_size, index,
                      n, delta, old_state, blk_counts, nblk, counted);
   return check_launch();
 }

@@ -1250,7 +1250,7 @@ static int launch_prefill_rows(const lsattn_prefill_args* a, bool tile_major, co
   // (a round: two four-wave workgroups per CU, one of the others.  Two rounds still gain: 16 x 256 tokens 38.0 -> 36.8 us,
   // 1 x 4096 129.0 -> 127.7; six rounds lose 1-3 %, sixteen 5 %.)
   p.store_through = MODE == 0 && wgs_launch <= 2 * (HALF ? 2 * kCUs : kCUs);
-  hipLaunchKernelGGL((prefill_kernel<T, MODE, DV, SPLIT, HALF>), dim3((unsigned)wgs_launch), dim3(HALF ? NWAVE * 32 : NWAVE * 64), 0, st, p);
+  LSATTN_LAUNCH_KERNEL((prefill_kernel<T, MODE, DV, SPLIT, HALF>), dim3((unsigned)wgs_launch), dim3(HALF ? NWAVE * 32 : NWAVE * 64), 0, st, p);
   return check_launch();
 }
 

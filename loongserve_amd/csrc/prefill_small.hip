@@ -336,7 +336,7 @@ __global__ __launch_bounds__(kWaves * 64) void prefill_small_kernel(SmallParams 
 template <typename T, int D, int MODE> int launch(const SmallParams& p, const lsattn_prefill_args* a, hipStream_t st) {
   const int64_t tiles = (a->max_q_len + kRows - 1) / kRows;  // workgroups per head and request
   if (tiles > 0x7fffffff || a->num_q_heads > 65535 || a->batch > 65535) return LSATTN_ERR_INVALID_ARG;
-  hipLaunchKernelGGL((prefill_small_kernel<T, D, MODE>), dim3((unsigned)tiles, (unsigned)a->num_q_heads, (unsigned)a->batch),
+  LSATTN_LAUNCH_KERNEL((prefill_small_kernel<T, D, MODE>), dim3((unsigned)tiles, (unsigned)a->num_q_heads, (unsigned)a->batch),
                      dim3(kWaves * 64), 0, st, p);
   return check_launch();
 }

@@ -16,6 +16,19 @@ def _declared_symbols():
     return sorted(set(re.findall(r"\b(lsattn_[a-z0-9_]+)\s*\(", text)))
 
 
+def test_importing_the_package_first_leaves_one_hip_runtime_in_the_process():
+    """PyTorch-ROCm ships its own libamdhip64; the library links the system's.  Whatever the program imports first, the
+    process must end up with one runtime (two: the library's launches find no device in theirs)."""
+    import subprocess
+    import sys
+    code = ("import loongserve_amd, torch\n"
+            "print(sorted({l.split()[-1] for l in open('/proc/self/maps') if 'libamdhip64' in l}))")
+    out = subprocess.run([sys.executable, "-c", code], cwd=ROOT, capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0, out.stderr[-2000:]
+    paths = eval(out.stdout.strip().splitlines()[-1])
+    assert len(paths) == 1, paths
+
+
 def test_ceiling_library_exports_every_declared_symbol():
     """libls_ceiling.so (bench.py's measurement aids) exports what include/ls_ceiling.h declares."""
     import ctypes

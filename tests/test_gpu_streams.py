@@ -63,3 +63,34 @@ def test_two_threads_two_streams(lsa):
     for b in got:
         assert torch.equal(b[0], ref[0]) and torch.equal(b[1], ref[1])
         assert torch.equal(b[4], ref[4]) and torch.equal(b[5], ref[5])
+
+
+def test_an_error_left_behind_by_the_host_program_is_not_reported_as_a_launch_failure(lsa):
+    """The runtime keeps the last error of a host thread until somebody asks for it, harmless ones included (a framework's
+    copy engine polls events and gets "not ready"; here: a device number that does not exist).  The library's launches
+    report their own outcome, not what was there before them."""
+    import ctypes
+    hip = ctypes.CDLL("libamdhip64.so")
+    hip.hipSetDevice.argtypes = [ctypes.c_int]
+    hip.hipPeekAtLastError.restype = ctypes.c_int
+    Hq, Hkv, D, BS = 8, 2, 128, 64
+    lens = [300]
+    q, k, v = [rand_t(s, 40 + i).to(DEV) for i, s in enumerate(((300, Hq, D), (300, Hkv, D), (300, Hkv, D)))]
+    m = [t.to(DEV) for t in meta(lens)]
+    o_ok, lse_ok = lsa.prefill_attention_step(q, k, v, *m, *m, 1, 300)
+    dq, dkv, table, b_req, b_len = [t.to(DEV) for t in decode_case(78, 2, Hq, Hkv, D, [500, 70], 2000)]
+    mo = torch.empty(8, 2, Hq, D, device=DEV)
+    ml = torch.empty(8, 2, Hq, device=DEV)
+    d_ok = lsa.longserve_token_decode_attention_flash_decoding(dq, table, b_req, b_len, mo, ml, 2, 500, Hq, D, dkv[:, :Hkv], dkv[:, Hkv:], BS)
+    torch.cuda.synchronize()
+    for call in ("prefill", "decode"):
+        assert hip.hipSetDevice(12345) != 0      # fails, changes nothing, and stays behind as the thread's last error
+        assert hip.hipPeekAtLastError() != 0
+        if call == "prefill":
+            o, lse = lsa.prefill_attention_step(q, k, v, *m, *m, 1, 300)
+            torch.cuda.synchronize()
+            assert torch.equal(o, o_ok) and torch.equal(lse, lse_ok)
+        else:
+            d = lsa.longserve_token_decode_attention_flash_decoding(dq, table, b_req, b_len, mo, ml, 2, 500, Hq, D, dkv[:, :Hkv], dkv[:, Hkv:], BS)
+            torch.cuda.synchronize()
+            assert torch.equal(d[0], d_ok[0]) and torch.equal(d[1], d_ok[1])
