@@ -14,8 +14,19 @@ DEV = "cuda:0"
 
 @pytest.mark.parametrize("seed", [1, 7, 23])
 def test_random_steps_match_the_oracle(lsa, seed):
+    _sweep(lsa, seed, 16, [128])
+
+
+@pytest.mark.parametrize("seed", [2, 9])
+def test_random_steps_of_head_sizes_below_128_match_the_oracle(lsa, seed):
+    """The same sweep over the head sizes 16, 32 and 64 (a kernel of their own)."""
+    _sweep(lsa, seed, 12, [16, 32, 64])
+
+
+def _sweep(lsa, seed, cases, head_sizes):
     rng = random.Random(seed)
-    for case in range(16):
+    for case in range(cases):
+        D = rng.choice(head_sizes)
         dtype = rng.choice([torch.float16, torch.bfloat16])
         Hkv = rng.choice([1, 2, 3])
         Hq = Hkv * rng.choice([1, 2, 4])
@@ -25,11 +36,11 @@ def test_random_steps_match_the_oracle(lsa, seed):
         klens = [rng.choice([0, 1, 63, 64, 200, 256, 448, 511, 512, 700, 1300, 2500]) for _ in range(B)]
         qf = [rng.choice([0, 1, 5, 300, 1000, 4000]) for _ in range(B)]
         kf = [rng.choice([0, 1, 2, 3, 100, 700]) for _ in range(B)]
-        print("case", seed, case, dtype, Hq, Hkv, P, qlens, qf, klens, kf, flush=True)
+        print("case", seed, case, D, dtype, Hq, Hkv, P, qlens, qf, klens, kf, flush=True)
         Tq, Tk = sum(qlens), max(sum(klens), 1)
-        q = rand_t((Tq, Hq, 128), 1000 * seed + case, dtype)
-        k = rand_t((Tk, Hkv, 128), 1000 * seed + 100 + case, dtype)
-        v = rand_t((Tk, Hkv, 128), 1000 * seed + 200 + case, dtype)
+        q = rand_t((Tq, Hq, D), 1000 * seed + case, dtype)
+        k = rand_t((Tk, Hkv, D), 1000 * seed + 100 + case, dtype)
+        v = rand_t((Tk, Hkv, D), 1000 * seed + 200 + case, dtype)
         qm, km = meta(qlens, qf), meta(klens, kf)
         o_ref, lse_ref = orc.attn_step(q, k, v, *qm, *km, P)
         o, lse = lsa.prefill_attention_step(q.to(DEV), k.to(DEV), v.to(DEV), *[t.to(DEV) for t in qm], *[t.to(DEV) for t in km],
@@ -43,17 +54,17 @@ def test_random_steps_match_the_oracle(lsa, seed):
         klens2 = [rng.choice([0, 1, 64, 130, 512, 700, 1300]) for _ in range(B)]
         kf2 = [rng.choice([0, 2, 50, 900]) for _ in range(B)]
         Tk2 = max(sum(klens2), 1)
-        k2 = rand_t((Tk2, Hkv, 128), 1000 * seed + 300 + case, dtype)
-        v2 = rand_t((Tk2, Hkv, 128), 1000 * seed + 400 + case, dtype)
+        k2 = rand_t((Tk2, Hkv, D), 1000 * seed + 300 + case, dtype)
+        v2 = rand_t((Tk2, Hkv, D), 1000 * seed + 400 + case, dtype)
         km2 = meta(klens2, kf2)
         o2_ref, lse2_ref = orc.lse_merge([(o_ref, lse_ref), orc.attn_step(q, k2, v2, *qm, *km2, P)])
         qd, qmd = q.to(DEV), [t.to(DEV) for t in qm]
         lsa.prefill_attention_step(qd, k2.to(DEV), v2.to(DEV), *qmd, *[t.to(DEV) for t in km2], P, max(qlens), o, lse,
                                    accumulate=True)
-        od = torch.full((Tq, Hq, 128), float("nan"), dtype=dtype, device=DEV)
+        od = torch.full((Tq, Hq, D), float("nan"), dtype=dtype, device=DEV)
         md = torch.full((Tq, Hq), float("-inf"), device=DEV)
         ld = torch.zeros(Tq, Hq, device=DEV)
-        o_st = torch.zeros((Tq, Hq, 128), dtype=dtype)  # the oracle's in-place state over the same two steps
+        o_st = torch.zeros((Tq, Hq, D), dtype=dtype)  # the oracle's in-place state over the same two steps
         m_st, l_st = torch.full((Tq, Hq), float("-inf")), torch.zeros(Tq, Hq)
         for kk, vv, kmm in ((k, v, km), (k2, v2, km2)):
             lsa.context_attention_fwd(qd, kk.to(DEV), vv.to(DEV), od, *qmd, *[t.to(DEV) for t in kmm], P, max(qlens), md, ld)
