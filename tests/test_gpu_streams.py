@@ -70,7 +70,10 @@ def test_an_error_left_behind_by_the_host_program_is_not_reported_as_a_launch_fa
     copy engine polls events and gets "not ready"; here: a device number that does not exist).  The library's launches
     report their own outcome, not what was there before them."""
     import ctypes
-    hip = ctypes.CDLL("libamdhip64.so")
+    # (the runtime this process already runs on, by the path it was loaded from: a bare library name could bring in a second one)
+    loaded = sorted({ln.split()[-1] for ln in open("/proc/self/maps") if "libamdhip64" in ln})
+    assert len(loaded) == 1, loaded
+    hip = ctypes.CDLL(loaded[0])
     hip.hipSetDevice.argtypes = [ctypes.c_int]
     hip.hipPeekAtLastError.restype = ctypes.c_int
     Hq, Hkv, D, BS = 8, 2, 128, 64
