@@ -32,6 +32,7 @@ def test_importing_the_package_first_leaves_one_hip_runtime_in_the_process():
 def test_ceiling_library_exports_every_declared_symbol():
     """libls_ceiling.so (bench.py's measurement aids) exports what include/ls_ceiling.h declares."""
     import ctypes
+    import torch  # noqa: F401  (first, so that this process keeps to one HIP runtime: see the test above)
     text = open(os.path.join(ROOT, "include", "ls_ceiling.h")).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     names = sorted(set(re.findall(r"\b(ls_ceiling_[a-z0-9_]+)\s*\(", text)))
